@@ -1,0 +1,125 @@
+// Shared device/host helpers for the gfx950 graph-primitive kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/graphiler_amd.h"
+
+namespace ga {
+
+constexpr int kWave = 64;      // CDNA wavefront width
+constexpr int kBlock = 256;    // threads per workgroup used by the row kernels
+
+typedef uint16_t bf16_t;  // raw bf16 storage
+
+__device__ __forceinline__ float bf16_lo(uint32_t packed) {
+  return __uint_as_float(packed << 16);
+}
+__device__ __forceinline__ float bf16_hi(uint32_t packed) {
+  return __uint_as_float(packed & 0xffff0000u);
+}
+// fp32 -> bf16, round to nearest even, NaN kept quiet (same rounding as
+// PyTorch's float -> bfloat16 conversion).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// Row fragment I/O: VEC consecutive features of element type T, widened to
+// fp32 registers.  VEC > 1 uses one 16-byte access.
+template <typename T, int VEC>
+struct Frag;
+
+template <>
+struct Frag<float, 4> {
+  typedef float4 raw_t;
+  static __device__ __forceinline__ raw_t load(const float *p) {
+    return *reinterpret_cast<const float4 *>(p);
+  }
+  static __device__ __forceinline__ void widen(const raw_t &r, float (&f)[4]) {
+    f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w;
+  }
+  static __device__ __forceinline__ void store(float *p, const float (&f)[4]) {
+    *reinterpret_cast<float4 *>(p) = make_float4(f[0], f[1], f[2], f[3]);
+  }
+};
+
+template <>
+struct Frag<float, 1> {
+  typedef float raw_t;
+  static __device__ __forceinline__ raw_t load(const float *p) { return *p; }
+  static __device__ __forceinline__ void widen(const raw_t &r, float (&f)[1]) {
+    f[0] = r;
+  }
+  static __device__ __forceinline__ void store(float *p, const float (&f)[1]) {
+    *p = f[0];
+  }
+};
+
+template <>
+struct Frag<bf16_t, 8> {
+  typedef uint4 raw_t;
+  static __device__ __forceinline__ raw_t load(const bf16_t *p) {
+    return *reinterpret_cast<const uint4 *>(p);
+  }
+  static __device__ __forceinline__ void widen(const raw_t &r, float (&f)[8]) {
+    f[0] = bf16_lo(r.x); f[1] = bf16_hi(r.x);
+    f[2] = bf16_lo(r.y); f[3] = bf16_hi(r.y);
+    f[4] = bf16_lo(r.z); f[5] = bf16_hi(r.z);
+    f[6] = bf16_lo(r.w); f[7] = bf16_hi(r.w);
+  }
+  static __device__ __forceinline__ void store(bf16_t *p, const float (&f)[8]) {
+    uint4 r;
+    r.x = pack_bf16(f[0], f[1]);
+    r.y = pack_bf16(f[2], f[3]);
+    r.z = pack_bf16(f[4], f[5]);
+    r.w = pack_bf16(f[6], f[7]);
+    *reinterpret_cast<uint4 *>(p) = r;
+  }
+};
+
+template <>
+struct Frag<bf16_t, 1> {
+  typedef bf16_t raw_t;
+  static __device__ __forceinline__ raw_t load(const bf16_t *p) { return *p; }
+  static __device__ __forceinline__ void widen(const raw_t &r, float (&f)[1]) {
+    f[0] = bf16_lo(r);
+  }
+  static __device__ __forceinline__ void store(bf16_t *p, const float (&f)[1]) {
+    *p = (bf16_t)f32_to_bf16_bits(f[0]);
+  }
+};
+
+// ---- host side -----------------------------------------------------------
+
+inline int ilog2_floor(uint64_t x) {
+  int s = 0;
+  while (x > 1) { x >>= 1; ++s; }
+  return s;
+}
+inline int ilog2_ceil(uint64_t x) {
+  int s = ilog2_floor(x);
+  return ((uint64_t)1 << s) < x ? s + 1 : s;
+}
+inline bool aligned(const void *p, size_t a) {
+  return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? GA_OK : (int)e;
+}
+
+// log2 of the slots per run of the load-balanced row reductions.  Every lane
+// group walks exactly one run, so the value trades scheduling slack and
+// workspace (two partial rows per run) against per-run overhead.  It depends
+// on the edge count and the feature width only, so the workspace query and the
+// launch agree.
+int run_shift_for(int64_t n_edges, int64_t feat);
+
+}  // namespace ga

@@ -1,0 +1,231 @@
+"""Graph container and host-side preparation.
+
+``DGLGraph`` mirrors the reference's custom class
+(include/dglgraph.h:7-75, registered in src/dglgraph.cpp:5-24): the same ten
+constructor arguments, the same four setters and the same public fields, so the
+operator wrappers in :mod:`graphiler_amd.ops` read it exactly as the
+reference's operators read theirs.  On top of that it caches what the gfx950
+kernels need once per graph: the slot->row maps of both adjacencies, whether
+the edge-id columns are the identity, and a reusable workspace.
+
+``prepare_graph`` mirrors python/graphiler/utils/setup.py:116-146: in- and
+out-adjacency with int32 pointer / neighbour / edge-id columns and int64 COO
+columns, built here from a plain (src, dst) edge list instead of a DGL graph.
+Inside one node's group the edges keep ascending edge-id order.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+import torch
+
+from . import capi
+
+
+@dataclass
+class GraphArrays:
+    """Host (numpy) form of the arrays ``prepare_graph`` produces."""
+    num_nodes: int
+    in_pointer: np.ndarray
+    in_node_indices: np.ndarray
+    in_edge_indices: np.ndarray
+    out_pointer: np.ndarray
+    out_node_indices: np.ndarray
+    out_edge_indices: np.ndarray
+    COO_src: np.ndarray
+    COO_dst: np.ndarray
+
+
+def _group(n_nodes: int, key: np.ndarray, other: np.ndarray):
+    """Stable grouping of edge ids by ``key`` -> (pointer, neighbour, edge id)."""
+    order = np.argsort(key, kind="stable")
+    counts = np.bincount(key, minlength=n_nodes)
+    pointer = np.zeros(n_nodes + 1, np.int64)
+    np.cumsum(counts, out=pointer[1:])
+    return (pointer.astype(np.int32), other[order].astype(np.int32),
+            order.astype(np.int32))
+
+
+def build_graph_arrays(src, dst, num_nodes: int) -> GraphArrays:
+    """CSR-by-destination and CSR-by-source of an edge list (host, numpy)."""
+    src = np.ascontiguousarray(src, dtype=np.int64)
+    dst = np.ascontiguousarray(dst, dtype=np.int64)
+    if src.shape != dst.shape or src.ndim != 1:
+        raise ValueError("src and dst must be 1-D arrays of equal length")
+    if src.shape[0] >= 2 ** 31 or num_nodes >= 2 ** 31:
+        raise ValueError("graphs are limited to int32 node and edge ids")
+    if src.size and (min(src.min(), dst.min()) < 0 or
+                     max(src.max(), dst.max()) >= num_nodes):
+        raise ValueError("edge endpoint outside [0, num_nodes)")
+    ip, inb, ie = _group(num_nodes, dst, src)
+    op, onb, oe = _group(num_nodes, src, dst)
+    return GraphArrays(num_nodes, ip, inb, ie, op, onb, oe, src, dst)
+
+
+def type_pointer(type_of, num_types: int) -> np.ndarray:
+    """int32 running sum of items per type; ``type_of`` must be sorted
+    (ids of one type are contiguous, include/dglgraph.h:68-69)."""
+    type_of = np.asarray(type_of, dtype=np.int64)
+    if type_of.size and np.any(np.diff(type_of) < 0):
+        raise ValueError("items must be sorted by type")
+    ptr = np.zeros(num_types + 1, np.int64)
+    np.cumsum(np.bincount(type_of, minlength=num_types), out=ptr[1:])
+    return ptr.astype(np.int32)
+
+
+def sort_edges_by_type(src, dst, etype):
+    """Stable reorder of an edge list so edge ids of one type are contiguous.
+    Returns (src, dst, etype, order) with ``order`` the applied permutation."""
+    etype = np.asarray(etype, dtype=np.int64)
+    order = np.argsort(etype, kind="stable")
+    return (np.asarray(src)[order], np.asarray(dst)[order], etype[order], order)
+
+
+def _check_index(t: torch.Tensor, dtype: torch.dtype, name: str):
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} must be {dtype}")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+class DGLGraph:
+    """Drop-in for ``torch.classes.my_classes.DGLGraph``."""
+
+    def __init__(self, in_pointer, in_node_indices, in_edge_indices,
+                 out_pointer, out_node_indices, out_edge_indices, COO_src,
+                 COO_dst, ntype_pointer: Optional[torch.Tensor] = None,
+                 etype_pointer: Optional[torch.Tensor] = None):
+        for name, t in (("in_pointer", in_pointer),
+                        ("in_node_indices", in_node_indices),
+                        ("in_edge_indices", in_edge_indices),
+                        ("out_pointer", out_pointer),
+                        ("out_node_indices", out_node_indices),
+                        ("out_edge_indices", out_edge_indices)):
+            _check_index(t, torch.int32, name)
+        _check_index(COO_src, torch.int64, "COO_src")
+        _check_index(COO_dst, torch.int64, "COO_dst")
+        self.in_pointer = in_pointer
+        self.in_node_indices = in_node_indices
+        self.in_edge_indices = in_edge_indices
+        self.out_pointer = out_pointer
+        self.out_node_indices = out_node_indices
+        self.out_edge_indices = out_edge_indices
+        self.COO_src = COO_src
+        self.COO_dst = COO_dst
+        self.ntype_pointer = None
+        self.etype_pointer = None
+        self.ntype_COO = None
+        self.etype_COO = None
+        # include/dglgraph.h:22-27
+        self.num_nodes = int(in_pointer.size(0)) - 1
+        self.num_edges = int(in_node_indices.size(0))
+        self.num_ntypes = 1
+        self.num_etypes = 1
+        self.SetNtypePointer(ntype_pointer)
+        self.SetEtypePointer(etype_pointer)
+        self._cache = {}
+
+    # -- setters (include/dglgraph.h:29-46) ---------------------------------
+    def SetNtypePointer(self, pointer):
+        if pointer is not None:
+            _check_index(pointer, torch.int32, "ntype_pointer")
+        self.ntype_pointer = pointer
+        self.num_ntypes = int(pointer.size(0)) - 1 if pointer is not None else 1
+
+    def SetEtypePointer(self, pointer):
+        if pointer is not None:
+            _check_index(pointer, torch.int32, "etype_pointer")
+        self.etype_pointer = pointer
+        self.num_etypes = int(pointer.size(0)) - 1 if pointer is not None else 1
+
+    def SetNtypeCOO(self, column):
+        _check_index(column, torch.int64, "ntype_COO")
+        if column.size(0) != self.num_nodes:
+            raise RuntimeError("ntype_COO must have one entry per node")
+        self.ntype_COO = column
+
+    def SetEtypeCOO(self, column):
+        _check_index(column, torch.int64, "etype_COO")
+        if column.size(0) != self.num_edges:
+            raise RuntimeError("etype_COO must have one entry per edge")
+        self.etype_COO = column
+
+    # -- derived data the kernels schedule with -----------------------------
+    @property
+    def device(self):
+        return self.in_pointer.device
+
+    def _row_ids(self, pointer: torch.Tensor) -> torch.Tensor:
+        rows = torch.empty(self.num_edges, dtype=torch.int32, device=self.device)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        capi.check(capi.load().ga_csr_row_ids(
+            pointer.data_ptr(), self.num_nodes, self.num_edges,
+            rows.data_ptr(), stream), "ga_csr_row_ids")
+        return rows
+
+    @property
+    def in_row_of_slot(self) -> torch.Tensor:
+        """Destination node of every slot of the in-adjacency (int32, E)."""
+        if "in_rows" not in self._cache:
+            self._cache["in_rows"] = self._row_ids(self.in_pointer)
+        return self._cache["in_rows"]
+
+    @property
+    def out_row_of_slot(self) -> torch.Tensor:
+        """Source node of every slot of the out-adjacency (int32, E)."""
+        if "out_rows" not in self._cache:
+            self._cache["out_rows"] = self._row_ids(self.out_pointer)
+        return self._cache["out_rows"]
+
+    def _identity(self, key: str, column: torch.Tensor) -> bool:
+        if key not in self._cache:
+            n = column.numel()
+            ar = torch.arange(n, dtype=torch.int32, device=column.device)
+            self._cache[key] = bool(torch.equal(column, ar))
+        return self._cache[key]
+
+    @property
+    def in_eid_is_identity(self) -> bool:
+        """True when edge ids already are in-adjacency slot numbers."""
+        return self._identity("in_ident", self.in_edge_indices)
+
+    @property
+    def out_eid_is_identity(self) -> bool:
+        return self._identity("out_ident", self.out_edge_indices)
+
+    def workspace(self, nbytes: int) -> torch.Tensor:
+        """Scratch buffer reused across calls on this graph (grows on demand).
+        Calls that use it are ordered on the current stream."""
+        ws = self._cache.get("ws")
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8,
+                             device=self.device)
+            self._cache["ws"] = ws
+        return ws
+
+
+def prepare_graph(src, dst, num_nodes: int, device="cuda:0",
+                  ntype_of=None, num_ntypes: int = 0, etype_of=None,
+                  num_etypes: int = 0) -> DGLGraph:
+    """Build the device graph from an edge list (setup.py:116-146); when type
+    columns are given also install the type pointers and type COO columns the
+    way load_data does for heterogeneous graphs (setup.py:87-100)."""
+    arr = build_graph_arrays(src, dst, num_nodes)
+    dev = torch.device(device)
+
+    def up(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    g = DGLGraph(up(arr.in_pointer), up(arr.in_node_indices),
+                 up(arr.in_edge_indices), up(arr.out_pointer),
+                 up(arr.out_node_indices), up(arr.out_edge_indices),
+                 up(arr.COO_src), up(arr.COO_dst), None, None)
+    if ntype_of is not None:
+        g.SetNtypePointer(up(type_pointer(ntype_of, num_ntypes)))
+        g.SetNtypeCOO(up(np.asarray(ntype_of, dtype=np.int64)))
+    if etype_of is not None:
+        g.SetEtypePointer(up(type_pointer(etype_of, num_etypes)))
+        g.SetEtypeCOO(up(np.asarray(etype_of, dtype=np.int64)))
+    return g

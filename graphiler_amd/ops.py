@@ -1,0 +1,327 @@
+"""Operator wrappers: the reference's ``torch.ops.my_ops.*`` surface over the C ABI.
+
+Every function keeps the name, argument order and argument meaning of the
+operator it replaces (schemas in src/ops/dgl_primitives/spmm.cu:391-406,
+sddmm.cu:131-134, segment_softmax/segment_softmax.cu:27-30,
+segment_mm/segment_mm.cu:35-42, broadcast/broadcast.cu:102-122).  The unused
+``dim / keep_dim / dtype`` arguments exist in the reference because its builder
+relabels an ``aten::sum`` / ``aten::softmax`` node (src/builder/builder.cpp:141-143);
+they are accepted and ignored here too, except ``dim == 1`` for the softmax.
+
+The wrappers own allocation and argument checking (CUDA + contiguous, raising
+``RuntimeError`` like the reference's CHECK_INPUT, src/ops/ops.cuh:14-20) and
+hand raw device pointers plus the current HIP stream to the library.  There is
+no CPU path: tensors that are not on the GPU are rejected.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+
+from . import capi
+from .graph import DGLGraph
+
+_DTYPES = {torch.float32: capi.GA_F32, torch.bfloat16: capi.GA_BF16}
+_REDUCE = {"sum": capi.GA_SUM, "max": capi.GA_MAX, "min": capi.GA_MIN}
+
+
+def _check_input(x: torch.Tensor, name: str) -> None:
+    if not x.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not x.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _feat_dtype(x: torch.Tensor, name: str) -> int:
+    if x.dtype not in _DTYPES:
+        raise RuntimeError(f"{name} must be float32 or bfloat16")
+    return _DTYPES[x.dtype]
+
+
+def _stream(x: torch.Tensor) -> int:
+    return torch.cuda.current_stream(x.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def get_feat_dim(features: torch.Tensor) -> int:
+    """broadcast.cu:3-9: product of the sizes of all dimensions after the first."""
+    d = 1
+    for s in features.shape[1:]:
+        d *= int(s)
+    return d
+
+
+def _out_shape(rows: int, x: torch.Tensor):
+    return (rows,) + (tuple(x.shape[1:]) if x.dim() > 1 else (1,))
+
+
+# ----------------------------------------------------------------- SpMM ----
+def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
+         w: Optional[torch.Tensor] = None, reverse: bool = False) -> torch.Tensor:
+    """Generalised SpMM over the in-adjacency (``reverse``: the out-adjacency).
+
+    op: "copy_u" (u is (N, ...)), "copy_e" (u is (E, ...)), "u_mul_e"
+    (w is (E,), (E, 1) or (E, H) fp32).  reduce: "sum" | "max" | "min".
+    """
+    _check_input(u, "features")
+    dt = _feat_dtype(u, "features")
+    if reverse:
+        pointer, nbr, eid = g.out_pointer, g.out_node_indices, g.out_edge_indices
+        rows, ident = g.out_row_of_slot, g.out_eid_is_identity
+    else:
+        pointer, nbr, eid = g.in_pointer, g.in_node_indices, g.in_edge_indices
+        rows, ident = g.in_row_of_slot, g.in_eid_is_identity
+    feat = get_feat_dim(u)
+    heads = 1
+    code = {"copy_u": capi.GA_COPY_U, "copy_e": capi.GA_COPY_E,
+            "u_mul_e": capi.GA_U_MUL_E}[op]
+    if op == "u_mul_e":
+        _check_input(w, "edge weights")
+        if w.dtype != torch.float32:
+            raise RuntimeError("edge weights must be float32")
+        if w.shape[0] != g.num_edges:
+            raise RuntimeError("edge weights must have one row per edge")
+        heads = get_feat_dim(w)
+        if feat % heads:
+            raise RuntimeError("feature width is not a multiple of the heads")
+    n_src = g.num_edges if op == "copy_e" else g.num_nodes
+    if u.shape[0] != n_src:
+        raise RuntimeError("features have the wrong number of rows")
+    out = torch.empty(_out_shape(g.num_nodes, u), dtype=u.dtype, device=u.device)
+    lib = capi.load()
+    ws_bytes = lib.ga_spmm_workspace_bytes(g.num_edges, feat)
+    ws = g.workspace(ws_bytes)
+    capi.check(lib.ga_spmm_csr(
+        pointer.data_ptr(), rows.data_ptr(), nbr.data_ptr(),
+        None if ident else eid.data_ptr(), u.data_ptr(), _ptr(w),
+        out.data_ptr(), g.num_nodes, g.num_edges, feat, heads, code,
+        _REDUCE[reduce], dt, ws.data_ptr(), ws.numel(), _stream(u)),
+        "ga_spmm_csr")
+    return out
+
+
+def SpMMSrc(features, dims: Sequence[int], keep_dim: bool, dtype,
+            graph: DGLGraph) -> torch.Tensor:
+    """spmm.cu:375-389: out[v] = sum over in-edges of features[src]."""
+    return spmm(graph, "copy_u", "sum", features)
+
+
+def SpMMEdge(features, dims: Sequence[int], keep_dim: bool, dtype,
+             graph: DGLGraph) -> torch.Tensor:
+    """spmm.cu:359-373: out[v] = sum over in-edges of features[edge id]."""
+    return spmm(graph, "copy_e", "sum", features)
+
+
+def gspmm_src_mul_e_sum(ufeature, efeature, dims: Sequence[int], keep_dim: bool,
+                        dtype, graph: DGLGraph) -> torch.Tensor:
+    """spmm.cu:286-320: out[v] = sum over in-edges of ufeature[src] * efeature[e]."""
+    return spmm(graph, "u_mul_e", "sum", ufeature, efeature)
+
+
+def gspmm_dst_mul_e_sum(ufeature, efeature, dims: Sequence[int], keep_dim: bool,
+                        dtype, graph: DGLGraph) -> torch.Tensor:
+    """spmm.cu:322-356: the same contraction over the out-adjacency:
+    out[v] = sum over out-edges of ufeature[dst] * efeature[e]."""
+    return spmm(graph, "u_mul_e", "sum", ufeature, efeature, reverse=True)
+
+
+# ---------------------------------------------------------------- SDDMM ----
+def _edge_columns(g: DGLGraph):
+    """(lhs, rhs, bits) giving source and destination of every edge in edge-id
+    order: the int32 in-adjacency columns when edge ids are slot numbers (half
+    the index traffic), the int64 COO columns otherwise."""
+    if g.in_eid_is_identity:
+        return g.in_node_indices, g.in_row_of_slot, 32
+    return g.COO_src, g.COO_dst, 64
+
+
+def gsddmm_u_add_v_mul_alpha(src_feature, dst_feature, alpha: int,
+                             graph: DGLGraph) -> torch.Tensor:
+    """sddmm.cu:118-129: out[e] = src_feature[src[e]] + dst_feature[dst[e]]
+    in edge-id order, fp32 (E, feat).  ``alpha`` is ignored, as in the reference."""
+    _check_input(src_feature, "src_feature")
+    _check_input(dst_feature, "dst_feature")
+    dt = _feat_dtype(src_feature, "src_feature")
+    if dst_feature.dtype != src_feature.dtype:
+        raise RuntimeError("src_feature and dst_feature must share a dtype")
+    feat = get_feat_dim(src_feature)
+    if get_feat_dim(dst_feature) != feat:
+        raise RuntimeError("src_feature and dst_feature must share a width")
+    out = torch.empty(_out_shape(graph.num_edges, src_feature),
+                      dtype=torch.float32, device=src_feature.device)
+    lhs, rhs, bits = _edge_columns(graph)
+    capi.check(capi.load().ga_sddmm_u_add_v(
+        lhs.data_ptr(), rhs.data_ptr(), bits, src_feature.data_ptr(),
+        dst_feature.data_ptr(), out.data_ptr(), graph.num_edges, feat, dt,
+        _stream(out)), "ga_sddmm_u_add_v")
+    return out
+
+
+def gsddmm_u_dot_v(src_feature, dst_feature, graph: DGLGraph) -> torch.Tensor:
+    """u_dot_v over the last dimension (functor.cuh:103-116, sddmm.cuh:80-120):
+    (N, H, D) x (N, H, D) -> (E, H) fp32; 2-D inputs are one head."""
+    _check_input(src_feature, "src_feature")
+    _check_input(dst_feature, "dst_feature")
+    dt = _feat_dtype(src_feature, "src_feature")
+    if dst_feature.dtype != src_feature.dtype or \
+            dst_feature.shape[1:] != src_feature.shape[1:]:
+        raise RuntimeError("src_feature and dst_feature must share dtype and shape")
+    if src_feature.dim() == 2:
+        heads, dim = 1, int(src_feature.shape[1])
+    elif src_feature.dim() == 3:
+        heads, dim = int(src_feature.shape[1]), int(src_feature.shape[2])
+    else:
+        raise RuntimeError("u_dot_v expects (N, D) or (N, H, D) features")
+    out = torch.empty((graph.num_edges, heads), dtype=torch.float32,
+                      device=src_feature.device)
+    lhs, rhs, bits = _edge_columns(graph)
+    capi.check(capi.load().ga_sddmm_u_dot_v(
+        lhs.data_ptr(), rhs.data_ptr(), bits, src_feature.data_ptr(),
+        dst_feature.data_ptr(), out.data_ptr(), graph.num_edges, heads, dim, dt,
+        _stream(out)), "ga_sddmm_u_dot_v")
+    return out
+
+
+# -------------------------------------------------------------- softmax ----
+def SegmentSoftmax(features, dim: int, dtype, graph: DGLGraph) -> torch.Tensor:
+    """segment_softmax.cu:3-24: softmax of the per-edge logits over each
+    destination's in-edges; (E,), (E, 1) or (E, H) fp32."""
+    _check_input(features, "features")
+    if dim != 1:
+        raise RuntimeError("SegmentSoftmax reduces over dim 1 of the mailbox")
+    if features.dtype != torch.float32:
+        raise RuntimeError("features must be float32")
+    if features.shape[0] != graph.num_edges:
+        raise RuntimeError("features must have one row per edge")
+    heads = get_feat_dim(features)
+    ident = graph.in_eid_is_identity
+    # every edge id occurs in exactly one segment, so all of y is written
+    y = torch.empty_like(features)
+    capi.check(capi.load().ga_segment_softmax(
+        graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
+        None if ident else graph.in_edge_indices.data_ptr(),
+        features.data_ptr(), y.data_ptr(), graph.num_nodes, graph.num_edges,
+        heads, _stream(y)), "ga_segment_softmax")
+    return y
+
+
+# ----------------------------------------------------------- segment_mm ----
+def _segment_mm(features, weights, type_pointer, num_types, rows_expected):
+    _check_input(features, "features")
+    _check_input(weights, "weights")
+    dt = _feat_dtype(features, "features")
+    if weights.dtype != features.dtype:
+        raise RuntimeError("features and weights must share a dtype")
+    if type_pointer is None:
+        raise RuntimeError("the graph has no type pointer for this operator")
+    if weights.dim() == 3:
+        heads = 1
+    elif weights.dim() == 4:
+        heads = int(weights.shape[1])
+    else:
+        raise RuntimeError("weights must be (T, K, M) or (T, H, K, M)")
+    K, M = int(weights.shape[-2]), int(weights.shape[-1])
+    if int(weights.shape[0]) != num_types:
+        raise RuntimeError("weights must have one matrix per type")
+    rows = int(features.shape[0])
+    if rows != rows_expected or get_feat_dim(features) != heads * K:
+        raise RuntimeError("features must be (rows, heads*K)")
+    out = torch.empty((rows, heads * M), dtype=features.dtype,
+                      device=features.device)
+    capi.check(capi.load().ga_segment_mm(
+        type_pointer.data_ptr(), num_types, features.data_ptr(),
+        weights.data_ptr(), out.data_ptr(), rows, heads, K, M, dt,
+        _stream(out)), "ga_segment_mm")
+    return out
+
+
+def SegmentMMNode(features, weights, graph: DGLGraph) -> torch.Tensor:
+    """segment_mm.cu:23-27: per-node-type linear, nodes sorted by type."""
+    return _segment_mm(features, weights, graph.ntype_pointer,
+                       graph.num_ntypes, graph.num_nodes)
+
+
+def SegmentMMEdge(features, weights, graph: DGLGraph) -> torch.Tensor:
+    """segment_mm.cu:29-33: per-edge-type linear, edges sorted by type."""
+    return _segment_mm(features, weights, graph.etype_pointer,
+                       graph.num_etypes, graph.num_edges)
+
+
+# ------------------------------------------------------------ broadcast ----
+def _gather(features: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    _check_input(features, "features")
+    row_bytes = get_feat_dim(features) * features.element_size()
+    out = torch.empty((index.shape[0],) + tuple(features.shape[1:]),
+                      dtype=features.dtype, device=features.device)
+    capi.check(capi.load().ga_gather_rows(
+        index.data_ptr(), 64 if index.dtype == torch.int64 else 32,
+        features.data_ptr(), out.data_ptr(), index.shape[0], row_bytes,
+        _stream(out)), "ga_gather_rows")
+    return out
+
+
+def BroadcastSrcNode(features, graph: DGLGraph) -> torch.Tensor:
+    """broadcast.cu:58-63: features[COO_src]."""
+    return _gather(features, graph.COO_src)
+
+
+def BroadcastDstNode(features, graph: DGLGraph) -> torch.Tensor:
+    """broadcast.cu:64-69: features[COO_dst]."""
+    return _gather(features, graph.COO_dst)
+
+
+def BroadcastNodeType(features, graph: DGLGraph) -> torch.Tensor:
+    """broadcast.cu:71-79: features[ntype_COO]."""
+    if graph.ntype_COO is None:
+        raise RuntimeError("the graph has no node-type column")
+    return _gather(features, graph.ntype_COO)
+
+
+def BroadcastSrcNodeType(features, graph: DGLGraph) -> torch.Tensor:
+    """broadcast.cu:81-84."""
+    return BroadcastSrcNode(BroadcastNodeType(features, graph), graph)
+
+
+def BroadcastDstNodeType(features, graph: DGLGraph) -> torch.Tensor:
+    """broadcast.cu:86-89."""
+    return BroadcastDstNode(BroadcastNodeType(features, graph), graph)
+
+
+def BroadcastEdgeType(features, graph: DGLGraph) -> torch.Tensor:
+    """broadcast.cu:91-100: features[etype_COO]."""
+    if graph.etype_COO is None:
+        raise RuntimeError("the graph has no edge-type column")
+    return _gather(features, graph.etype_COO)
+
+
+# ----------------------------------------------------------- fused GAT ----
+def gat_aggregate(el, er, z, graph: DGLGraph, negative_slope: float = 0.01):
+    """u_add_v -> leaky_relu -> edge softmax -> u_mul_e sum in one pass
+    (the four-operator chain of examples/GAT/GAT.py:25-36 at opt level 2).
+    el, er: (N, H) fp32 attention terms of source / destination; z: (N, H*D)."""
+    _check_input(el, "el")
+    _check_input(er, "er")
+    _check_input(z, "z")
+    dt = _feat_dtype(z, "z")
+    if el.dtype != torch.float32 or er.dtype != torch.float32:
+        raise RuntimeError("el and er must be float32")
+    heads = get_feat_dim(el)
+    feat = get_feat_dim(z)
+    if get_feat_dim(er) != heads or feat % heads:
+        raise RuntimeError("inconsistent head count")
+    out = torch.empty(_out_shape(graph.num_nodes, z), dtype=z.dtype,
+                      device=z.device)
+    lib = capi.load()
+    ws_bytes = lib.ga_gat_workspace_bytes(graph.num_edges, feat, heads)
+    ws = graph.workspace(ws_bytes)
+    capi.check(lib.ga_gat_aggregate(
+        graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
+        graph.in_node_indices.data_ptr(), el.data_ptr(), er.data_ptr(),
+        z.data_ptr(), out.data_ptr(), graph.num_nodes, graph.num_edges, heads,
+        feat // heads, float(negative_slope), dt, ws.data_ptr(), ws.numel(),
+        _stream(out)), "ga_gat_aggregate")
+    return out

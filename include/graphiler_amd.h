@@ -1,0 +1,166 @@
+/*
+ * graphiler_amd.h -- C ABI of the MI355X (gfx950) sparse graph-primitive layer.
+ *
+ * These entry points are what the operator wrappers behind the reference's
+ * TorchScript boundary (torch.ops.my_ops.* / torch.classes.my_classes.DGLGraph)
+ * bind to.  Each declaration cites the reference function it replaces
+ * (paths relative to the reference repository).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says "host";
+ *   - sizes are int64_t, graph index arrays keep the reference's layout
+ *     (include/dglgraph.h:54-74): int32 row pointer / neighbour id / edge id,
+ *     int64 COO endpoints and type columns;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all
+ *     work is enqueued on it and nothing synchronises;
+ *   - entry points never allocate, never throw and return GA_OK (0), a negative
+ *     GA_E* code for rejected arguments, or a positive hipError_t from a launch;
+ *   - feature matrices are row-major and contiguous; GA_BF16 data is read and
+ *     written as bf16, accumulated in fp32; per-edge scalars (attention logits
+ *     and weights) are always fp32;
+ *   - results are deterministic: no atomics are used, and the order of every
+ *     floating-point reduction is a function of the graph and sizes only.
+ */
+#ifndef GRAPHILER_AMD_H_
+#define GRAPHILER_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GA_OK 0
+#define GA_EINVAL (-1)       /* null / negative / inconsistent argument      */
+#define GA_EUNSUPPORTED (-2) /* valid request this build has no kernel for   */
+#define GA_EWORKSPACE (-3)   /* workspace missing, too small or misaligned   */
+#define GA_EALIGN (-4)       /* pointer not aligned to its element size      */
+
+typedef void *ga_stream_t;
+
+enum ga_dtype { GA_F32 = 0, GA_BF16 = 1 };
+/* message = u[nbr] | e[eid] | u[nbr] * w[eid]   (functor.cuh:18-121)         */
+enum ga_spmm_op { GA_COPY_U = 0, GA_COPY_E = 1, GA_U_MUL_E = 2 };
+/* functor.cuh:125-213: sum starts at 0, max at -inf, min at +inf             */
+enum ga_reduce { GA_SUM = 0, GA_MAX = 1, GA_MIN = 2 };
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ga_version(void);
+/* Static, human-readable text for a return code of this library. */
+const char *ga_error_string(int code);
+
+/* ------------------------------------------------------------------ graph --
+ * Slot -> row map of a grouped adjacency: row_of_slot[i] = v for every
+ * i in [pointer[v], pointer[v+1]).  It is the schedule every row-reduction
+ * kernel below balances its work with (equal-sized runs of slots instead of
+ * whole rows), built once per graph next to the arrays that
+ * python/graphiler/utils/setup.py:116-146 (prepare_graph) fills in.
+ */
+int ga_csr_row_ids(const int32_t *pointer, int64_t n_rows, int64_t n_edges,
+                   int32_t *row_of_slot, ga_stream_t stream);
+
+/* ------------------------------------------------------------------- SpMM --
+ * out[v, h, d] = reduce_{i in [pointer[v], pointer[v+1])} msg_i[h, d]
+ * Replaces SpMMSrc (spmm.cu:375-389; op GA_COPY_U, gather by nbr),
+ * SpMMEdge (spmm.cu:359-373; op GA_COPY_E, gather rows of the (E, feat) matrix
+ * `u` by eid), src_mul_e_sum / dst_mul_e_sum (spmm.cu:286-356; op GA_U_MUL_E,
+ * pass the in- or the out-adjacency) and the generic SpMMCsrKernel with the
+ * Max / Min reducers (spmm.cuh:30-71).
+ *   pointer      (n_rows+1) int32     nbr (n_edges) int32, unused for COPY_E
+ *   row_of_slot  (n_edges)  int32     from ga_csr_row_ids
+ *   eid          (n_edges)  int32 or NULL when eid[i] == i
+ *   u            (n_src, feat)  or (n_edges, feat) for COPY_E, `dtype`
+ *   w            (n_edges, heads) fp32, U_MUL_E only; feat % heads == 0
+ *   out          (n_rows, feat) `dtype`; every row is written (rows without
+ *                edges get 0, -inf or +inf by reducer)
+ *   workspace    ga_spmm_workspace_bytes() bytes, 16-byte aligned
+ */
+size_t ga_spmm_workspace_bytes(int64_t n_edges, int64_t feat);
+int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
+                const int32_t *nbr, const int32_t *eid, const void *u,
+                const float *w, void *out, int64_t n_rows, int64_t n_edges,
+                int64_t feat, int64_t heads, int op, int reduce, int dtype,
+                void *workspace, size_t workspace_bytes, ga_stream_t stream);
+
+/* ------------------------------------------------------------------ SDDMM --
+ * out[i, k] = u[lhs[i], k] + v[rhs[i], k], fp32 output (E, feat).
+ * Replaces SDDMMCoo_u_add_v_mul_alpha (sddmm.cu:118-129, kernel
+ * sddmm.cuh:34-71); `alpha` of the reference is accepted by the operator
+ * wrapper and ignored there, as in the reference.  (lhs, rhs) are either the
+ * int64 COO columns (idx_bits 64: output in edge-id order) or the int32
+ * (nbr, row_of_slot) columns of an adjacency (idx_bits 32: output in slot
+ * order, equal to edge-id order when eid[i] == i).
+ */
+int ga_sddmm_u_add_v(const void *lhs, const void *rhs, int idx_bits,
+                     const void *u, const void *v, float *out, int64_t n_edges,
+                     int64_t feat, int dtype, ga_stream_t stream);
+
+/* out[i, h] = sum_d u[lhs[i], h, d] * v[rhs[i], h, d], fp32 output (E, heads).
+ * The Dot functor (functor.cuh:103-116) with the reduction over the last
+ * dimension (bcast.cc:37-39,57-60; kernel sddmm.cuh:80-120), which the
+ * reference compiles but never registers. */
+int ga_sddmm_u_dot_v(const void *lhs, const void *rhs, int idx_bits,
+                     const void *u, const void *v, float *out, int64_t n_edges,
+                     int64_t heads, int64_t dim, int dtype, ga_stream_t stream);
+
+/* ---------------------------------------------------------- edge softmax --
+ * y[e, h] = softmax of x[., h] over the edges e = eid[i] (or i when eid is
+ * NULL), i in [pointer[v], pointer[v+1]), for every row v.  fp32 in and out.
+ * Replaces SegmentSoftmaxForward / softmax_v (segment_softmax.cu:3-24,
+ * segment_softmax_kernel.cu:4-49) and supplies the multi-head case the
+ * reference leaves empty (softmax_m, segment_softmax_kernel.cu:52-53).
+ * Uses the true segment maximum (the reference clamps it at >= 0, which only
+ * changes results once every logit of a segment is below about -87).
+ * y entries of edges that belong to no row are left untouched: pass y zeroed
+ * to match the reference's zeros_like output when eid is not a permutation.
+ */
+int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
+                       const int32_t *eid, const float *x, float *y,
+                       int64_t n_rows, int64_t n_edges, int64_t heads,
+                       ga_stream_t stream);
+
+/* ------------------------------------------------------------ segment_mm --
+ * Y[r, h, :] = X[r, h, :] @ W[t, h, :, :] for r in [type_pointer[t],
+ * type_pointer[t+1]).  Replaces SegmentMMBase / SegmentMMNode / SegmentMMEdge
+ * (segment_mm.cu:4-33) for heads == 1; heads > 1 applies one K x M block per
+ * head.  type_pointer stays on the device (the reference copies it to the host
+ * every call, segment_mm.cu:10).  X (rows, heads*K), W (n_types, heads, K, M),
+ * Y (rows, heads*M), all `dtype`; fp32 accumulation on the matrix cores.
+ */
+int ga_segment_mm(const int32_t *type_pointer, int64_t n_types, const void *X,
+                  const void *W, void *Y, int64_t rows, int64_t heads,
+                  int64_t K, int64_t M, int dtype, ga_stream_t stream);
+
+/* ---------------------------------------------------------------- gather --
+ * y[i, :] = x[idx[i], :], a bit-exact row copy of row_bytes bytes.
+ * Replaces BroadcastSrcNode / DstNode / NodeType / EdgeType
+ * (broadcast.cu:58-100: features.index({COO_src | COO_dst | ntype_COO |
+ * etype_COO})).  idx is int64 (idx_bits 64) or int32 (idx_bits 32); entries
+ * must lie in [0, n_in) -- they are not checked on the device.
+ */
+int ga_gather_rows(const void *idx, int idx_bits, const void *x, void *y,
+                   int64_t n_out, int64_t row_bytes, ga_stream_t stream);
+
+/* ------------------------------------------------- fused GAT aggregation --
+ * The chain the reference's optimised GAT plan executes as four operators
+ * (examples/GAT/GAT.py:25-36 after fusion.cpp:37-47,67-77):
+ * gsddmm_u_add_v -> leaky_relu -> SegmentSoftmax -> gspmm_src_mul_e_sum,
+ *   s_i = leaky_relu(el[nbr[i], h] + er[v, h], slope),  a = softmax_v(s),
+ *   out[v, h, :] = sum_i a_i * z[nbr[i], h, :]
+ * in one pass over the edges without materialising per-edge tensors.
+ * el, er (n, heads) fp32; z, out (n, heads*dim) `dtype`.  Rows without edges
+ * get 0.  workspace: ga_gat_workspace_bytes() bytes, 16-byte aligned.
+ */
+size_t ga_gat_workspace_bytes(int64_t n_edges, int64_t feat, int64_t heads);
+int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
+                     const int32_t *nbr, const float *el, const float *er,
+                     const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                     int64_t heads, int64_t dim, float slope, int dtype,
+                     void *workspace, size_t workspace_bytes,
+                     ga_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GRAPHILER_AMD_H_ */

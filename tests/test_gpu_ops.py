@@ -1,0 +1,219 @@
+"""Parity of the HIP operators (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from graphiler_amd import datasets, ops, prepare_graph
+from graphiler_amd.graph import build_graph_arrays
+from helpers import (TOL_BF16, TOL_F32, assert_close, random_graph,
+                     skewed_graph, to_bf16_f32)
+
+pytestmark = pytest.mark.gpu
+
+
+def _graphs():
+    rng = np.random.default_rng(11)
+    dbg = datasets.debug_graph()
+    out = {"debug": (dbg.src, dbg.dst, 3)}
+    s, d = random_graph(rng, 300, 2000)
+    out["uniform"] = (s, d, 300)
+    s, d = skewed_graph(rng, 1000, 6000, 9000)
+    out["skewed"] = (s, d, 1000)
+    wl = datasets.gat_rmat(num_nodes=5000, n_edges=150_000, scale=13, seed=5)
+    out["rmat_by_dst"] = (wl.src, wl.dst, wl.num_nodes)
+    out["no_edges"] = (np.zeros(0, np.int64), np.zeros(0, np.int64), 17)
+    out["one_row"] = (rng.integers(0, 5, 4000, dtype=np.int64),
+                      np.zeros(4000, np.int64), 5)
+    return out
+
+
+GRAPHS = _graphs()
+
+
+@pytest.fixture(scope="module", params=list(GRAPHS))
+def graph(request, device):
+    src, dst, n = GRAPHS[request.param]
+    g = prepare_graph(src, dst, n, device=device)
+    return request.param, g, build_graph_arrays(src, dst, n)
+
+
+def _dev(a, device, bf16=False):
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    return t.to(torch.bfloat16) if bf16 else t
+
+
+def test_row_ids_bit_exact(graph):
+    name, g, arr = graph
+    want = np.repeat(np.arange(arr.num_nodes, dtype=np.int32),
+                     np.diff(arr.in_pointer))
+    assert np.array_equal(g.in_row_of_slot.cpu().numpy(), want)
+    want = np.repeat(np.arange(arr.num_nodes, dtype=np.int32),
+                     np.diff(arr.out_pointer))
+    assert np.array_equal(g.out_row_of_slot.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("feat", [1, 3, 16, 64, 100, 256, 602])
+@pytest.mark.parametrize("op", ["copy_u", "copy_e"])
+def test_spmm_copy_sum_f32(graph, device, feat, op):
+    name, g, arr = graph
+    rng = np.random.default_rng(feat)
+    rows = arr.num_nodes if op == "copy_u" else arr.COO_src.shape[0]
+    x = rng.standard_normal((rows, feat), dtype=np.float32)
+    fn = ops.SpMMSrc if op == "copy_u" else ops.SpMMEdge
+    got = fn(_dev(x, device), [1], False, None, g).cpu().numpy()
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      x, op=op)
+    assert_close(got, ref, TOL_F32, f"{op} sum {name} F={feat}")
+    # rows without in-edges are exactly zero
+    empty = np.diff(arr.in_pointer) == 0
+    assert not got[empty].any()
+
+
+@pytest.mark.parametrize("feat,heads", [(1, 1), (5, 1), (64, 1), (64, 4),
+                                        (128, 8), (256, 4), (12, 3)])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_spmm_u_mul_e_sum_f32(graph, device, feat, heads, reverse):
+    name, g, arr = graph
+    rng = np.random.default_rng(feat * 7 + heads)
+    e = arr.COO_src.shape[0]
+    x = rng.standard_normal((arr.num_nodes, feat), dtype=np.float32)
+    w = rng.standard_normal((e, heads), dtype=np.float32)
+    fn = ops.gspmm_dst_mul_e_sum if reverse else ops.gspmm_src_mul_e_sum
+    got = fn(_dev(x, device), _dev(w, device), [1], False, None, g).cpu().numpy()
+    if reverse:
+        ref = oracle.spmm(arr.out_pointer, arr.out_node_indices,
+                          arr.out_edge_indices, x, w, op="u_mul_e", heads=heads)
+    else:
+        ref = oracle.spmm(arr.in_pointer, arr.in_node_indices,
+                          arr.in_edge_indices, x, w, op="u_mul_e", heads=heads)
+    assert_close(got, ref, TOL_F32, f"u_mul_e {name} F={feat} H={heads}")
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+@pytest.mark.parametrize("op,feat,heads", [("copy_u", 64, 1), ("copy_u", 7, 1),
+                                           ("copy_e", 32, 1),
+                                           ("u_mul_e", 64, 2)])
+def test_spmm_max_min_f32(graph, device, reduce, op, feat, heads):
+    name, g, arr = graph
+    rng = np.random.default_rng(3)
+    e = arr.COO_src.shape[0]
+    rows = e if op == "copy_e" else arr.num_nodes
+    x = rng.standard_normal((rows, feat), dtype=np.float32)
+    w = rng.standard_normal((e, heads), dtype=np.float32) if op == "u_mul_e" else None
+    got = ops.spmm(g, op, reduce, _dev(x, device),
+                   None if w is None else _dev(w, device)).cpu().numpy()
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      x, w, op=op, reduce=reduce, heads=heads)
+    # a max / min of fp32 products is exact: compare bit for bit
+    assert np.array_equal(got, ref), f"{op} {reduce} {name}"
+
+
+@pytest.mark.parametrize("feat,heads", [(64, 1), (128, 8), (256, 4), (24, 3),
+                                        (7, 1)])
+def test_spmm_bf16(graph, device, feat, heads):
+    name, g, arr = graph
+    rng = np.random.default_rng(feat)
+    e = arr.COO_src.shape[0]
+    x = to_bf16_f32(rng.standard_normal((arr.num_nodes, feat), dtype=np.float32))
+    w = rng.standard_normal((e, heads), dtype=np.float32)
+    got = ops.gspmm_src_mul_e_sum(_dev(x, device, True), _dev(w, device), [1],
+                                  False, None, g)
+    assert got.dtype == torch.bfloat16
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      x, w, op="u_mul_e", heads=heads)
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16,
+                 f"bf16 u_mul_e {name} F={feat}")
+    got = ops.SpMMSrc(_dev(x, device, True), [1], False, None, g)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      x, op="copy_u")
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16, f"bf16 copy_u {name}")
+
+
+@pytest.mark.parametrize("feat", [1, 4, 8, 5])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_sddmm_u_add_v_bit_exact(graph, device, feat, bf16):
+    name, g, arr = graph
+    rng = np.random.default_rng(feat)
+    u = rng.standard_normal((arr.num_nodes, feat), dtype=np.float32)
+    v = rng.standard_normal((arr.num_nodes, feat), dtype=np.float32)
+    if bf16:
+        u, v = to_bf16_f32(u), to_bf16_f32(v)
+    got = ops.gsddmm_u_add_v_mul_alpha(_dev(u, device, bf16), _dev(v, device, bf16),
+                                       1, g)
+    assert got.dtype == torch.float32 and got.shape == (arr.COO_src.shape[0], feat)
+    ref = oracle.sddmm_u_add_v(arr.COO_src, arr.COO_dst, u, v)
+    assert np.array_equal(got.cpu().numpy(), ref), f"u_add_v {name} F={feat}"
+
+
+@pytest.mark.parametrize("heads,dim", [(1, 64), (8, 16), (4, 64), (3, 5),
+                                       (1, 1), (2, 256)])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_sddmm_u_dot_v(graph, device, heads, dim, bf16):
+    name, g, arr = graph
+    rng = np.random.default_rng(heads * 100 + dim)
+    u = rng.standard_normal((arr.num_nodes, heads, dim), dtype=np.float32)
+    v = rng.standard_normal((arr.num_nodes, heads, dim), dtype=np.float32)
+    if bf16:
+        u, v = to_bf16_f32(u), to_bf16_f32(v)
+    got = ops.gsddmm_u_dot_v(_dev(u, device, bf16), _dev(v, device, bf16), g)
+    ref = oracle.sddmm_u_dot_v(arr.COO_src, arr.COO_dst, u, v)
+    # bf16 inputs are exact in fp32; the products are accumulated in fp32
+    assert_close(got.cpu().numpy(), ref, TOL_F32, f"u_dot_v {name} {heads}x{dim}")
+
+
+@pytest.mark.parametrize("heads", [1, 4, 8, 3, 64])
+def test_segment_softmax(graph, device, heads):
+    name, g, arr = graph
+    rng = np.random.default_rng(heads)
+    e = arr.COO_src.shape[0]
+    x = (rng.standard_normal((e, heads)) * 4.0).astype(np.float32)
+    got = ops.SegmentSoftmax(_dev(x, device), 1, None, g).cpu().numpy()
+    ref = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, x)
+    assert_close(got, ref, TOL_F32, f"softmax {name} H={heads}")
+    if e:
+        # each non-empty segment sums to one, per head
+        sums = oracle.spmm(arr.in_pointer, arr.in_node_indices,
+                           arr.in_edge_indices, got.astype(np.float32),
+                           op="copy_e")
+        nonempty = np.diff(arr.in_pointer) > 0
+        assert np.abs(sums[nonempty] - 1.0).max() < 1e-5
+
+
+def test_segment_softmax_1d_input(graph, device):
+    name, g, arr = graph
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal(arr.COO_src.shape[0]).astype(np.float32)
+    got = ops.SegmentSoftmax(_dev(x, device), 1, None, g)
+    assert got.shape == x.shape
+    ref = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, x)
+    assert_close(got.cpu().numpy(), ref, TOL_F32, f"softmax 1-D {name}")
+
+
+@pytest.mark.parametrize("shape,dtype", [((64,), np.float32), ((1,), np.float32),
+                                         ((3, 5), np.float32), ((7,), np.int64),
+                                         ((128,), np.float16), ((3,), np.uint8)])
+def test_broadcast_bit_exact(graph, device, shape, dtype):
+    name, g, arr = graph
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal((arr.num_nodes,) + shape) * 100).astype(dtype)
+    dx = _dev(x, device)
+    assert np.array_equal(ops.BroadcastSrcNode(dx, g).cpu().numpy(),
+                          oracle.gather_rows(arr.COO_src, x))
+    assert np.array_equal(ops.BroadcastDstNode(dx, g).cpu().numpy(),
+                          oracle.gather_rows(arr.COO_dst, x))
+
+
+def test_check_input_errors(device):
+    dbg = datasets.debug_graph()
+    g = prepare_graph(dbg.src, dbg.dst, 3, device=device)
+    x = torch.ones(3, 4)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        ops.SpMMSrc(x, [1], False, None, g)
+    xt = torch.ones(4, 3, device=device).t()
+    with pytest.raises(RuntimeError, match="must be contiguous"):
+        ops.SpMMSrc(xt, [1], False, None, g)
+    with pytest.raises(RuntimeError):
+        ops.SegmentSoftmax(torch.ones(6, 1, device=device), 0, None, g)
+    with pytest.raises(RuntimeError):
+        ops.BroadcastEdgeType(torch.ones(2, 2, device=device), g)
