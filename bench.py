@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one GAT layer forward on the Reddit-shaped R-MAT graph.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--path fused|plan]
+
+A step is one forward pass of a single-head GAT layer over the whole graph
+(232,965 nodes, 11.6 M edges, fp32 features 602 -> 64): the dense projection
+(torch.mm) followed by the graph-operator chain u_add_v -> leaky_relu(0.2) ->
+edge softmax -> u_mul_e sum, either as the four operators of the reference's
+compiled plan (--path plan) or as the single fused pass (--path fused).  All
+inputs are resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+# HBM bytes per dominant-kernel launch measured with rocprofv3 --pmc
+# (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); the summary
+# lives under profiles/.  None until measured for the kernel named below.
+MEASURED_TRAFFIC_BYTES = {"plan": None, "fused": None}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--path", choices=["fused", "plan"], default="fused")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 "
+                 "(the path is not sharded across devices)")
+
+    import numpy as np
+    import torch
+    import torch.nn.functional as F
+
+    from graphiler_amd import datasets, layers, ops, prepare_graph
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    slope = 0.2
+    in_dim, out_dim, heads = 602, 64, 1
+
+    wl = datasets.gat_rmat()                      # config 2, seed 1
+    N, E = wl.num_nodes, wl.num_edges
+    g = prepare_graph(wl.src, wl.dst, N, device=dev)
+    rng = np.random.default_rng(1)
+    x_h = rng.standard_normal((N, in_dim), dtype=np.float32)
+    w_h = datasets.glorot(rng, (in_dim, out_dim))
+    a_h = datasets.glorot(rng, (2, heads, out_dim // heads), fan_in=2 * out_dim, fan_out=1)
+    x, w, a = (torch.from_numpy(t).to(dev) for t in (x_h, w_h, a_h))
+    g.in_row_of_slot                              # per-graph schedule, built once
+    assert g.in_eid_is_identity
+
+    fused = args.path == "fused"
+
+    def step():
+        return layers.gat_layer(g, x, w, a, heads, slope, fused=fused)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- per-operator timing with events on the launch stream ---------------
+    def ev_time(fn, reps=20):
+        fn()
+        torch.cuda.synchronize()
+        s = torch.cuda.Event(enable_timing=True)
+        e = torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / reps
+
+    z, el, er = layers.gat_project(x, w, a, heads)
+    logits = F.leaky_relu_(ops.gsddmm_u_add_v_mul_alpha(el, er, 1, g), slope)
+    att = ops.SegmentSoftmax(logits, 1, None, g)
+    ops_ms = {
+        "dense_project": ev_time(lambda: layers.gat_project(x, w, a, heads)),
+        "sddmm_u_add_v": ev_time(lambda: ops.gsddmm_u_add_v_mul_alpha(el, er, 1, g)),
+        "leaky_relu": ev_time(lambda: F.leaky_relu_(logits, 1.0)),
+        "segment_softmax": ev_time(lambda: ops.SegmentSoftmax(logits, 1, None, g)),
+        "spmm_u_mul_e": ev_time(lambda: ops.gspmm_src_mul_e_sum(z, att, [1], False, None, g)),
+    }
+    b = 4
+    F_ = out_dim
+    alg = {
+        "spmm_u_mul_e": 4 * (N + 1) + E * (4 + 4 * heads + F_ * b) + N * F_ * b,
+        "sddmm_u_add_v": 4 * (N + 1) + E * (4 + heads * b + 4 * heads) + N * heads * b,
+        "segment_softmax": 4 * (N + 1) + 8 * E * heads,
+        "gat_fused": 4 * (N + 1) + E * (4 + heads * b + F_ * b) + N * (heads * b + F_ * b),
+    }
+    if fused:
+        ops_ms["gat_fused"] = ev_time(lambda: ops.gat_aggregate(el, er, z, g, slope))
+        dom = "gat_fused"
+    else:
+        dom = "spmm_u_mul_e"
+    sparse_ms = ops_ms["gat_fused"] if fused else (
+        ops_ms["sddmm_u_add_v"] + ops_ms["leaky_relu"] +
+        ops_ms["segment_softmax"] + ops_ms["spmm_u_mul_e"])
+    achieved = alg[dom] / (ops_ms[dom] * 1e-3) / 1e9
+    roofline = {
+        "kernel": dom, "bound": "hbm", "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES[args.path],
+        "algorithmic_bytes": alg[dom], "launch_ms": round(ops_ms[dom], 4),
+    }
+
+    # ---- CPU baseline: the oracle's fp32 port of the same layer -------------
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle
+        ptr = g.in_pointer.cpu().numpy()
+        nbr = g.in_node_indices.cpu().numpy()
+        xt, wt = torch.from_numpy(x_h), torch.from_numpy(w_h)
+
+        def cpu_layer():
+            zc = torch.mm(xt, wt).numpy()
+            zh = zc.reshape(N, heads, -1)
+            elc = (zh * a_h[0]).sum(-1).astype(np.float32)
+            erc = (zh * a_h[1]).sum(-1).astype(np.float32)
+            lg = oracle.sddmm_u_add_v(wl.src, wl.dst, elc, erc)
+            lg = np.where(lg >= 0, lg, np.float32(slope) * lg).astype(np.float32)
+            at = oracle.segment_softmax(ptr, None, lg, zero_floor=True)
+            return oracle.spmm_sum_f32(ptr, nbr, None, zc, at, op="u_mul_e", heads=heads)
+
+        cpu_layer()
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 10.0 and reps < 50):
+            ref = cpu_layer()
+            reps += 1
+        cpu_ms = (time.perf_counter() - t0) * 1e3 / reps
+        got = out.cpu().numpy().reshape(ref.shape)
+        err = float(np.abs(got - ref).max() / np.abs(ref).max())
+        cpu = {"value": round(E / (cpu_ms * 1e-3), 1), "unit": "edges/s",
+               "cores": oracle.num_threads(), "kind": "port",
+               "ms_per_step": round(cpu_ms, 2),
+               "sample": f"the full workload (all {E} edges), {reps} repetitions "
+                         "of the fp32 C port (OpenMP) + torch-CPU dense projection",
+               "max_rel_diff_vs_gpu": err}
+
+    line = {
+        "metric": "GAT layer fwd edges/s (1-head GAT, 232,965 nodes, 11.6M edges, 602->64 fp32)",
+        "value": round(E / (ms_per_step * 1e-3), 1),
+        "unit": "edges/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: R-MAT(a=.57,b=.19,c=.19, seed 1) N=232965 "
+                               "E=11600000 dst-CSR; X N(0,1) fp32 602; GAT 602->64, 1 head, "
+                               "leaky_relu 0.2; dense projection included in the step",
+                   "path": args.path, "num_nodes": N, "num_edges": E},
+        "sparse_path_ms": round(sparse_ms, 4),
+        "sparse_path_edges_per_s": round(E / (sparse_ms * 1e-3), 1),
+        "ops_ms": {k: round(v, 4) for k, v in ops_ms.items()},
+        "ops_alg_GBps": {k: round(alg[k] / (ops_ms[k] * 1e-3) / 1e9, 1)
+                         for k in alg if k in ops_ms},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

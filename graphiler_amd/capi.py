@@ -33,8 +33,9 @@ SIGNATURES = {
                                 _vp]),
     "ga_sddmm_u_dot_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64,
                                 _int, _vp]),
+    "ga_softmax_workspace_bytes": (_sz, [_i64, _i64]),
     "ga_segment_softmax": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
-                                  _vp]),
+                                  _vp, _sz, _vp]),
     "ga_segment_mm": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                              _int, _vp]),
     "ga_gather_rows": (_int, [_vp, _int, _vp, _vp, _i64, _i64, _vp]),

@@ -4,16 +4,18 @@
 // picked from the average segment size) handles one destination row, keeps up
 // to kCache elements per lane in registers so a typical segment is read once,
 // and reduces max / sum with a fixed xor-shuffle tree.  Rows longer than
-// kLongRow slots are skipped there and handled by one whole workgroup each
-// (found without any list: the workgroup whose first slot is the first multiple
-// of kLongRow inside the row owns it).  No atomics; order is fixed.
+// kLongRow slots are skipped there and cut into chunks at the multiples of
+// kLongRow, one workgroup per chunk (found without any list: the workgroup
+// looks up the row of its first slot): pass A writes per-chunk (max, sum-exp)
+// to the workspace, pass B merges them in chunk order and normalises.
+// No atomics; the order of every reduction is fixed.
 #include "common.h"
 
 namespace ga {
 namespace {
 
 constexpr int kCache = 4;
-constexpr int kLongRow = 2048;
+constexpr int kLongRow = 1024;
 
 // heads is a power of two <= S: lane -> fixed head (lane & (heads-1)).
 __global__ __launch_bounds__(kBlock) void softmax_rows_pow2_kernel(
@@ -128,33 +130,72 @@ __device__ __forceinline__ float block_reduce(float v, float *lds) {
   return r;
 }
 
-// One workgroup per row longer than kLongRow slots.
-__global__ __launch_bounds__(kBlock) void softmax_long_rows_kernel(
+// Rows longer than kLongRow slots are cut at the multiples of kLongRow; the
+// workgroup of chunk c owns the slots [c*kLongRow, (c+1)*kLongRow) of the long
+// row that contains slot c*kLongRow, and the first chunk of a row also takes
+// the row's slots before its first multiple.  Returns false when the chunk
+// holds no part of a long row.
+__device__ __forceinline__ bool long_chunk(const int32_t *pointer,
+                                           const int32_t *row_of_slot,
+                                           int64_t n_edges, int64_t &lo,
+                                           int64_t &hi, int64_t &c_first,
+                                           int64_t &c_last) {
+  const int64_t c = blockIdx.x;
+  const int row = row_of_slot[c * kLongRow];
+  const int64_t start = pointer[row], end = pointer[row + 1];
+  if (end - start <= kLongRow) return false;
+  c_first = (start + kLongRow - 1) / kLongRow;
+  c_last = (end - 1) / kLongRow;
+  lo = c == c_first ? start : c * kLongRow;
+  hi = min(end, (c + 1) * (int64_t)kLongRow);
+  return true;
+}
+
+// Pass A: per chunk and head, (max, sum of exp(x - max)) -> stats[c][h][2].
+__global__ __launch_bounds__(kBlock) void softmax_long_stats_kernel(
     const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
     const int32_t *__restrict__ eid, const float *__restrict__ x,
-    float *__restrict__ y, int heads) {
+    float *__restrict__ stats, int64_t n_edges, int heads) {
   __shared__ float lds[kBlock / kWave];
-  const int64_t first_slot = (int64_t)blockIdx.x * kLongRow;
-  const int row = row_of_slot[first_slot];
-  const int64_t start = pointer[row];
-  const int64_t deg = pointer[row + 1] - start;
-  // owner = the workgroup at the first multiple of kLongRow that is >= start
-  if (deg <= kLongRow || (start + kLongRow - 1) / kLongRow != blockIdx.x) return;
+  int64_t lo, hi, c_first, c_last;
+  if (!long_chunk(pointer, row_of_slot, n_edges, lo, hi, c_first, c_last)) return;
   for (int h = 0; h < heads; ++h) {
     float m = -INFINITY;
-    for (int64_t q = threadIdx.x; q < deg; q += kBlock) {
-      const int64_t e = eid ? (int64_t)eid[start + q] : start + q;
+    for (int64_t q = lo + threadIdx.x; q < hi; q += kBlock) {
+      const int64_t e = eid ? (int64_t)eid[q] : q;
       m = fmaxf(m, x[e * heads + h]);
     }
     m = block_reduce<true>(m, lds);
     float l = 0.0f;
-    for (int64_t q = threadIdx.x; q < deg; q += kBlock) {
-      const int64_t e = eid ? (int64_t)eid[start + q] : start + q;
+    for (int64_t q = lo + threadIdx.x; q < hi; q += kBlock) {
+      const int64_t e = eid ? (int64_t)eid[q] : q;
       l += expf(x[e * heads + h] - m);
     }
     l = block_reduce<false>(l, lds);
-    for (int64_t q = threadIdx.x; q < deg; q += kBlock) {
-      const int64_t e = eid ? (int64_t)eid[start + q] : start + q;
+    if (threadIdx.x == 0) {
+      stats[((int64_t)blockIdx.x * heads + h) * 2] = m;
+      stats[((int64_t)blockIdx.x * heads + h) * 2 + 1] = l;
+    }
+  }
+}
+
+// Pass B: merge the row's chunk statistics in chunk order, then normalise.
+__global__ __launch_bounds__(kBlock) void softmax_long_write_kernel(
+    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
+    const int32_t *__restrict__ eid, const float *__restrict__ x,
+    const float *__restrict__ stats, float *__restrict__ y, int64_t n_edges,
+    int heads) {
+  int64_t lo, hi, c_first, c_last;
+  if (!long_chunk(pointer, row_of_slot, n_edges, lo, hi, c_first, c_last)) return;
+  for (int h = 0; h < heads; ++h) {
+    float m = -INFINITY;
+    for (int64_t c = c_first; c <= c_last; ++c)
+      m = fmaxf(m, stats[(c * heads + h) * 2]);
+    float l = 0.0f;
+    for (int64_t c = c_first; c <= c_last; ++c)
+      l += stats[(c * heads + h) * 2 + 1] * expf(stats[(c * heads + h) * 2] - m);
+    for (int64_t q = lo + threadIdx.x; q < hi; q += kBlock) {
+      const int64_t e = eid ? (int64_t)eid[q] : q;
       y[e * heads + h] = expf(x[e * heads + h] - m) / l;
     }
   }
@@ -163,11 +204,19 @@ __global__ __launch_bounds__(kBlock) void softmax_long_rows_kernel(
 }  // namespace
 }  // namespace ga
 
-extern "C" int ga_segment_softmax(const int32_t *pointer,
-                                  const int32_t *row_of_slot,
-                                  const int32_t *eid, const float *x, float *y,
-                                  int64_t n_rows, int64_t n_edges,
-                                  int64_t heads, ga_stream_t stream) {
+extern "C" {
+
+size_t ga_softmax_workspace_bytes(int64_t n_edges, int64_t heads) {
+  if (n_edges <= ga::kLongRow || heads <= 0) return 0;
+  const int64_t chunks = (n_edges + ga::kLongRow - 1) / ga::kLongRow;
+  return (size_t)chunks * (size_t)heads * 2 * sizeof(float);
+}
+
+int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
+                       const int32_t *eid, const float *x, float *y,
+                       int64_t n_rows, int64_t n_edges, int64_t heads,
+                       void *workspace, size_t workspace_bytes,
+                       ga_stream_t stream) {
   using namespace ga;
   if (n_rows < 0 || n_edges < 0 || heads <= 0) return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || heads > 65536)
@@ -175,11 +224,16 @@ extern "C" int ga_segment_softmax(const int32_t *pointer,
   if (n_rows == 0 || n_edges == 0) return GA_OK;
   if (!pointer || !row_of_slot || !x || !y) return GA_EINVAL;
   if (!aligned(x, 4) || !aligned(y, 4)) return GA_EALIGN;
+  const size_t need = ga_softmax_workspace_bytes(n_edges, heads);
+  if (need && (!workspace || workspace_bytes < need || !aligned(workspace, 16)))
+    return GA_EWORKSPACE;
   hipStream_t s = (hipStream_t)stream;
 
+  // lanes per row: the register cache (kCache elements per lane) should cover
+  // an average segment, so that it is read from memory once
   const bool pow2 = (heads & (heads - 1)) == 0 && heads <= kWave;
   const int64_t avg = (n_edges * (pow2 ? heads : 1) + n_rows - 1) / n_rows;
-  int s_shift = ilog2_ceil((uint64_t)(avg < 1 ? 1 : avg));
+  int s_shift = ilog2_ceil((uint64_t)((avg + kCache - 1) / kCache));
   if (s_shift < 2) s_shift = 2;
   if (s_shift > 6) s_shift = 6;
   if (pow2 && (1 << s_shift) < heads) s_shift = ilog2_ceil((uint64_t)heads);
@@ -195,10 +249,16 @@ extern "C" int ga_segment_softmax(const int32_t *pointer,
                        dim3(kBlock), 0, s, pointer, eid, x, y, n_rows,
                        (int)heads, s_shift);
   if (n_edges > kLongRow) {
-    const int64_t lblocks = (n_edges + kLongRow - 1) / kLongRow;
-    hipLaunchKernelGGL(softmax_long_rows_kernel, dim3((unsigned)lblocks),
-                       dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, y,
-                       (int)heads);
+    const int64_t chunks = (n_edges + kLongRow - 1) / kLongRow;
+    float *stats = (float *)workspace;
+    hipLaunchKernelGGL(softmax_long_stats_kernel, dim3((unsigned)chunks),
+                       dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, stats,
+                       n_edges, (int)heads);
+    hipLaunchKernelGGL(softmax_long_write_kernel, dim3((unsigned)chunks),
+                       dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, stats, y,
+                       n_edges, (int)heads);
   }
   return launch_status();
 }
+
+}  // extern "C"

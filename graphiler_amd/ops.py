@@ -201,11 +201,13 @@ def SegmentSoftmax(features, dim: int, dtype, graph: DGLGraph) -> torch.Tensor:
     ident = graph.in_eid_is_identity
     # every edge id occurs in exactly one segment, so all of y is written
     y = torch.empty_like(features)
-    capi.check(capi.load().ga_segment_softmax(
+    lib = capi.load()
+    ws = graph.workspace(lib.ga_softmax_workspace_bytes(graph.num_edges, heads))
+    capi.check(lib.ga_segment_softmax(
         graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
         None if ident else graph.in_edge_indices.data_ptr(),
         features.data_ptr(), y.data_ptr(), graph.num_nodes, graph.num_edges,
-        heads, _stream(y)), "ga_segment_softmax")
+        heads, ws.data_ptr(), ws.numel(), _stream(y)), "ga_segment_softmax")
     return y
 
 

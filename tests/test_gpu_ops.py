@@ -217,3 +217,37 @@ def test_check_input_errors(device):
         ops.SegmentSoftmax(torch.ones(6, 1, device=device), 0, None, g)
     with pytest.raises(RuntimeError):
         ops.BroadcastEdgeType(torch.ones(2, 2, device=device), g)
+
+
+@pytest.mark.parametrize("heads,dim", [(1, 64), (4, 64), (8, 16), (1, 1),
+                                       (3, 5), (2, 100)])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_gat_aggregate_fused(graph, device, heads, dim, bf16):
+    name, g, arr = graph
+    rng = np.random.default_rng(heads * 31 + dim)
+    n = arr.num_nodes
+    el = rng.standard_normal((n, heads), dtype=np.float32) * 2
+    er = rng.standard_normal((n, heads), dtype=np.float32) * 2
+    z = rng.standard_normal((n, heads * dim), dtype=np.float32)
+    if bf16:
+        z = to_bf16_f32(z)
+    got = ops.gat_aggregate(_dev(el, device), _dev(er, device),
+                            _dev(z, device, bf16), g, 0.2)
+    ref = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er, z,
+                               heads=heads, slope=0.2)
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
+                 f"fused GAT {name} {heads}x{dim} bf16={bf16}")
+    assert not got.float().cpu().numpy()[np.diff(arr.in_pointer) == 0].any()
+
+
+def test_gat_layer_plan_equals_fused(graph, device):
+    from graphiler_amd import layers
+    name, g, arr = graph
+    rng = np.random.default_rng(5)
+    n = arr.num_nodes
+    h = torch.from_numpy(rng.standard_normal((n, 40), dtype=np.float32)).to(device)
+    w = torch.from_numpy(datasets.glorot(rng, (40, 32))).to(device)
+    a = torch.from_numpy(datasets.glorot(rng, (2, 2, 16))).to(device)
+    plan = layers.gat_layer(g, h, w, a, 2, 0.2, fused=False).cpu().numpy()
+    fused = layers.gat_layer(g, h, w, a, 2, 0.2, fused=True).cpu().numpy()
+    assert_close(fused, plan, 2 * TOL_F32, f"GAT layer plan vs fused {name}")
