@@ -33,6 +33,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--path", choices=["fused", "plan"], default="fused")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 1 GiB device-to-device elementwise copy "
+                         "(x.add(0)) so rocprofv3 --pmc counters can be scaled "
+                         "against a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 "
@@ -62,6 +66,12 @@ def main():
     assert g.in_eid_is_identity
 
     fused = args.path == "fused"
+    if args.calibrate_copy:
+        big = torch.zeros(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB
+        for _ in range(3):
+            big2 = big.add(0.0)        # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del big, big2
 
     def step():
         return layers.gat_layer(g, x, w, a, heads, slope, fused=fused)

@@ -1,0 +1,278 @@
+// Load-balanced row reduction over a grouped adjacency (shared by the SpMM and
+// the fused GAT aggregation).
+//
+// Schedule.  The slots [0, E) are cut into equal runs of 2^run_shift slots.  A
+// group of `tpr` adjacent lanes (tpr * VEC features = one feature-row tile,
+// 16 bytes per lane when VEC > 1) owns one run and walks it in slot order with
+// eight gathers in flight per lane; a workgroup of 256 lanes owns G = 256 / tpr
+// consecutive runs.  Rows that lie inside one run are written straight to the
+// output.  A row shared by neighbouring runs leaves partial states, which the
+// workgroup chains together in LDS; only a row that crosses the workgroup's
+// slot range leaves (at most two) partial states in the global workspace, and
+// a small second kernel combines those in workgroup order.  Work per lane group
+// is therefore identical whatever the degree distribution, no atomics are used
+// and the order of every combination depends on the graph and sizes only.
+//
+// A Policy supplies the per-lane state and arithmetic:
+//   kState                      floats of state per lane
+//   init(st)                    empty state
+//   absorb(st, ...)             done inside Policy::walk, which processes one
+//                               batch of slots
+//   merge(dst, src)             dst <- dst (+) src, dst precedes src in slot order
+//   finish(st, o)               state -> VEC output features
+//   empty_row(o)                output of a row without edges
+#pragma once
+
+#include "common.h"
+
+namespace ga {
+
+constexpr int kUnroll = 8;
+
+struct RunGeom {
+  int64_t n_edges;
+  int64_t n_runs;
+  int64_t n_rows;
+  int feat;
+  int run_shift;
+  int tpr_shift;
+  int lanes_total;  // ceil(feat / VEC): state slots per partial row
+};
+
+// Per-run bookkeeping shared through LDS.
+struct RunFlags {
+  int has_a;    // first segment began before this run
+  int a_open;   // ... and it also continues past the run's end
+  int has_b;    // last segment began inside this run and continues past its end
+  int row_a;
+  int row_b;
+};
+
+template <class Policy>
+__global__ __launch_bounds__(kBlock) void runs_kernel(
+    typename Policy::Args args, const int32_t *__restrict__ row_of_slot,
+    typename Policy::out_t *__restrict__ out, float *__restrict__ partial,
+    RunGeom geo) {
+  constexpr int VEC = Policy::kVec;
+  constexpr int SF = Policy::kState;
+  typedef Frag<typename Policy::out_t, VEC> OutIO;
+  // LDS: [run in block][A|B][lane in group][SF]
+  extern __shared__ float lds_state[];
+  __shared__ RunFlags flags[kBlock];
+
+  const int tpr = 1 << geo.tpr_shift;
+  const int G = kBlock >> geo.tpr_shift;
+  const int grp = threadIdx.x >> geo.tpr_shift;
+  const int lane = threadIdx.x & (tpr - 1);
+  const int64_t k = (int64_t)blockIdx.x * G + grp;
+  const int flane = (int)blockIdx.y * tpr + lane;   // feature lane index
+  const int f0 = flane * VEC;
+  const bool live = k < geo.n_runs && f0 < geo.feat;
+
+  float *my_a = lds_state + ((grp * 2 + 0) * tpr + lane) * SF;
+  float *my_b = lds_state + ((grp * 2 + 1) * tpr + lane) * SF;
+
+  float st[SF];
+  Policy::init(st);
+  bool has_a = false, a_open = false, has_b = false;
+  int row_a = 0, row_b = 0;
+
+  if (live) {
+    const int64_t a = k << geo.run_shift;
+    const int64_t b = min(a + ((int64_t)1 << geo.run_shift), geo.n_edges);
+    int cur = row_of_slot[a];
+    const bool began_before = a > 0 && row_of_slot[a - 1] == cur;
+    bool first_seg = true;
+
+    // closes the open segment: complete rows go to `out`, a first segment that
+    // began before the run becomes this run's A state
+    auto close_segment = [&]() {
+      if (first_seg && began_before) {
+        has_a = true;
+        row_a = cur;
+#pragma unroll
+        for (int i = 0; i < SF; ++i) my_a[i] = st[i];
+      } else {
+        float o[VEC];
+        Policy::finish(st, o);
+        OutIO::store(out + (int64_t)cur * geo.feat + f0, o);
+      }
+      first_seg = false;
+    };
+
+    Policy::walk(args, row_of_slot, a, b, f0, geo.feat, st, cur, close_segment);
+
+    const bool continues = b < geo.n_edges && row_of_slot[b] == cur;
+    if (first_seg && began_before) {
+      has_a = true;
+      a_open = continues;
+      row_a = cur;
+#pragma unroll
+      for (int i = 0; i < SF; ++i) my_a[i] = st[i];
+    } else if (continues) {
+      has_b = true;
+      row_b = cur;
+#pragma unroll
+      for (int i = 0; i < SF; ++i) my_b[i] = st[i];
+    } else {
+      float o[VEC];
+      Policy::finish(st, o);
+      OutIO::store(out + (int64_t)cur * geo.feat + f0, o);
+    }
+  }
+  if (lane == 0) {
+    flags[grp].has_a = has_a;
+    flags[grp].a_open = a_open;
+    flags[grp].has_b = has_b;
+    flags[grp].row_a = row_a;
+    flags[grp].row_b = row_b;
+  }
+  __syncthreads();
+  if (!live) return;
+
+  auto state_of = [&](int g, int slot) -> const float * {
+    return lds_state + ((g * 2 + slot) * tpr + lane) * SF;
+  };
+  // chain ending at run `i` (its A state included): walk back over runs the
+  // row passes straight through, then combine in ascending run order
+  auto chain_into = [&](int i, float (&acc)[SF]) -> bool {
+    int j = i - 1;
+    while (j >= 0 && flags[j].has_a && flags[j].a_open) --j;
+    const bool starts_inside = j >= 0;   // then run j holds the chain's B state
+    if (starts_inside) {
+      const float *p = state_of(j, 1);
+#pragma unroll
+      for (int q = 0; q < SF; ++q) acc[q] = p[q];
+    } else {
+      Policy::init(acc);
+    }
+    for (int g = j + 1; g <= i; ++g) Policy::merge(acc, state_of(g, 0));
+    return starts_inside;
+  };
+  float *const gp = partial + (int64_t)blockIdx.x * 2 * geo.lanes_total * SF;
+  const int64_t runs_left = geo.n_runs - (int64_t)blockIdx.x * G;
+  const int last = (int)(runs_left < G ? runs_left : G) - 1;
+
+  if (has_a && !a_open) {            // a row ends in my run
+    float acc[SF];
+    if (chain_into(grp, acc)) {
+      float o[VEC];
+      Policy::finish(acc, o);
+      OutIO::store(out + (int64_t)row_a * geo.feat + f0, o);
+    } else {                         // began before this workgroup: slot 0
+      float *p = gp + (int64_t)flane * SF;
+#pragma unroll
+      for (int q = 0; q < SF; ++q) p[q] = acc[q];
+    }
+  }
+  if (grp == last) {                 // what leaves the workgroup at its end
+    if (has_b) {
+      float *p = gp + ((int64_t)geo.lanes_total + flane) * SF;
+#pragma unroll
+      for (int q = 0; q < SF; ++q) p[q] = my_b[q];
+    } else if (has_a && a_open) {
+      float acc[SF];
+      const bool inside = chain_into(grp, acc);
+      float *p = gp + ((int64_t)(inside ? geo.lanes_total : 0) + flane) * SF;
+#pragma unroll
+      for (int q = 0; q < SF; ++q) p[q] = acc[q];
+    }
+  }
+}
+
+// Blocks [0, fix_blocks): one lane group per main-kernel workgroup q; the group
+// whose slot range holds the END of a row that began in an earlier workgroup
+// combines that row's global partial states in workgroup order.  Remaining
+// blocks: one lane group per row, rows without edges get Policy::empty_row.
+template <class Policy>
+__global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
+    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
+    const float *__restrict__ partial, typename Policy::out_t *__restrict__ out,
+    RunGeom geo, int64_t n_wg, int fix_blocks) {
+  constexpr int VEC = Policy::kVec;
+  constexpr int SF = Policy::kState;
+  typedef Frag<typename Policy::out_t, VEC> OutIO;
+  const int tpr = 1 << geo.tpr_shift;
+  const int G = kBlock >> geo.tpr_shift;
+  const int flane = (int)blockIdx.y * tpr + (threadIdx.x & (tpr - 1));
+  const int f0 = flane * VEC;
+  if (f0 >= geo.feat) return;
+  float o[VEC];
+  if ((int)blockIdx.x < fix_blocks) {
+    const int64_t q = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> geo.tpr_shift;
+    if (q >= n_wg) return;
+    const int wg_shift = geo.run_shift + (8 - geo.tpr_shift);  // log2(G * run)
+    const int64_t a = q << wg_shift;
+    const int64_t b = min(a + ((int64_t)1 << wg_shift), geo.n_edges);
+    const int row = row_of_slot[a];
+    const int64_t s = pointer[row], e = pointer[row + 1];
+    if (!(s < a && e <= b)) return;
+    const int64_t q_lo = s >> wg_shift;
+    float acc[SF];
+    const float *p = partial + ((q_lo * 2 + 1) * geo.lanes_total + flane) * SF;
+#pragma unroll
+    for (int i = 0; i < SF; ++i) acc[i] = p[i];
+    for (int64_t w = q_lo + 1; w <= q; ++w)
+      Policy::merge(acc, partial + ((w * 2) * geo.lanes_total + flane) * SF);
+    Policy::finish(acc, o);
+    OutIO::store(out + (int64_t)row * geo.feat + f0, o);
+    (void)G;
+  } else {
+    const int64_t row =
+        ((int64_t)(blockIdx.x - fix_blocks) * kBlock + threadIdx.x) >> geo.tpr_shift;
+    if (row >= geo.n_rows || pointer[row] != pointer[row + 1]) return;
+    Policy::empty_row(o);
+    OutIO::store(out + row * geo.feat + f0, o);
+  }
+}
+
+// Workspace bound that holds for every element type / vector width: at most
+// ceil(n_runs / 4) workgroups (tpr <= 64), two partial rows each.
+inline size_t runs_workspace_bytes(int64_t n_edges, int64_t feat,
+                                   int state_floats_per_feature) {
+  if (n_edges <= 0 || feat <= 0) return 0;
+  const int run_shift = run_shift_for(n_edges, feat);
+  const int64_t n_runs = (n_edges + ((int64_t)1 << run_shift) - 1) >> run_shift;
+  const int64_t n_wg = (n_runs + 3) / 4;
+  return (size_t)n_wg * 2 * (size_t)feat * state_floats_per_feature * sizeof(float);
+}
+
+template <class Policy>
+int launch_runs(typename Policy::Args args, const int32_t *pointer,
+                const int32_t *row_of_slot, void *out, int64_t n_rows,
+                int64_t n_edges, int feat, float *partial, hipStream_t stream) {
+  constexpr int VEC = Policy::kVec;
+  constexpr int SF = Policy::kState;
+  RunGeom geo;
+  const int lanes = (feat + VEC - 1) / VEC;
+  geo.tpr_shift = ilog2_ceil((uint64_t)(lanes > kWave ? kWave : lanes));
+  const int tpr = 1 << geo.tpr_shift;
+  const int ftiles = (lanes + tpr - 1) / tpr;
+  geo.run_shift = run_shift_for(n_edges, feat);
+  geo.n_runs = (n_edges + ((int64_t)1 << geo.run_shift) - 1) >> geo.run_shift;
+  geo.n_edges = n_edges;
+  geo.n_rows = n_rows;
+  geo.feat = feat;
+  geo.lanes_total = lanes;
+  const int G = kBlock >> geo.tpr_shift;
+  const int64_t n_wg = (geo.n_runs + G - 1) / G;
+  typedef typename Policy::out_t out_t;
+  if (n_wg > 0x7fffffff) return GA_EUNSUPPORTED;
+  if (n_wg > 0) {
+    const size_t lds = (size_t)kBlock * 2 * SF * sizeof(float);
+    hipLaunchKernelGGL((runs_kernel<Policy>), dim3((unsigned)n_wg, ftiles),
+                       dim3(kBlock), lds, stream, args, row_of_slot,
+                       (out_t *)out, partial, geo);
+  }
+  const int64_t fix_blocks = (n_wg + G - 1) / G;
+  const int64_t fill_blocks = (n_rows + G - 1) / G;
+  if (fix_blocks + fill_blocks > 0x7fffffff) return GA_EUNSUPPORTED;
+  if (fix_blocks + fill_blocks > 0)
+    hipLaunchKernelGGL((runs_fixup_kernel<Policy>),
+                       dim3((unsigned)(fix_blocks + fill_blocks), ftiles),
+                       dim3(kBlock), 0, stream, pointer, row_of_slot, partial,
+                       (out_t *)out, geo, n_wg, (int)fix_blocks);
+  return launch_status();
+}
+
+}  // namespace ga

@@ -1,15 +1,6 @@
-// Load-balanced CSR SpMM for gfx950 (copy_u / copy_e / u_mul_e x sum / max / min).
-//
-// Scheduling.  The adjacency's slots [0, E) are cut into equal runs of 2^s
-// slots.  A group of `tpr` adjacent lanes (tpr * VEC features cover one feature
-// row, 16 bytes per lane when VEC > 1) owns one run and walks it in slot order,
-// eight gathers in flight per lane.  Rows that lie inside one run are written
-// straight to the output; the (at most two) rows a run shares with its
-// neighbours are written as fp32 partial rows to the workspace and combined by
-// a second kernel in run order.  Work per lane group is therefore identical
-// whatever the degree distribution, no atomics are used, and the summation
-// order depends on the graph and sizes only.
-#include "common.h"
+// Load-balanced CSR SpMM for gfx950 (copy_u / copy_e / u_mul_e x sum / max / min)
+// on the run-based row-reduction schedule of row_runs.h.
+#include "row_runs.h"
 
 namespace ga {
 
@@ -27,8 +18,6 @@ int run_shift_for(int64_t n_edges, int64_t feat) {
 
 namespace {
 
-constexpr int kUnroll = 8;
-
 template <int RED>
 __device__ __forceinline__ float red_init() {
   return RED == GA_SUM ? 0.0f : (RED == GA_MAX ? -INFINITY : INFINITY);
@@ -41,160 +30,88 @@ __device__ __forceinline__ float red_apply(float acc, float m) {
   return acc > m ? m : acc;
 }
 
-// One lane group per run.  gidx: row of `u` gathered per slot (neighbour id, or
-// edge id for copy_e); nullptr means the slot index itself.
+// Row-reduction policy of the SpMM: the state is the VEC running reductions.
 template <typename T, int VEC, int RED, bool HASW>
-__global__ __launch_bounds__(kBlock) void spmm_runs_kernel(
-    const int32_t *__restrict__ row_of_slot, const int32_t *__restrict__ gidx,
-    const int32_t *__restrict__ eid, const T *__restrict__ u,
-    const float *__restrict__ w, T *__restrict__ out,
-    float *__restrict__ partial, int64_t n_edges, int64_t n_runs, int feat,
-    int heads, int dph, int run_shift, int tpr_shift) {
-  typedef Frag<T, VEC> IO;
-  const int tpr = 1 << tpr_shift;
-  const int64_t k = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> tpr_shift;
-  const int f0 = ((int)blockIdx.y * tpr + (threadIdx.x & (tpr - 1))) * VEC;
-  if (k >= n_runs || f0 >= feat) return;
-  const int h = HASW ? f0 / dph : 0;
+struct SpmmPolicy {
+  typedef T out_t;
+  static constexpr int kVec = VEC;
+  static constexpr int kState = VEC;
+  struct Args {
+    const int32_t *gidx;  // row of `u` gathered per slot (neighbour id, or edge
+                          // id for copy_e); nullptr: the slot index itself
+    const int32_t *eid;   // edge id per slot for `w`; nullptr: the slot index
+    const T *u;
+    const float *w;
+    int heads;
+    int dph;
+  };
+  static __device__ __forceinline__ void init(float (&st)[VEC]) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) st[v] = red_init<RED>();
+  }
+  static __device__ __forceinline__ void merge(float (&dst)[VEC], const float *src) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) dst[v] = red_apply<RED>(dst[v], src[v]);
+  }
+  static __device__ __forceinline__ void finish(const float (&st)[VEC], float (&o)[VEC]) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o[v] = st[v];
+  }
+  static __device__ __forceinline__ void empty_row(float (&o)[VEC]) { init(o); }
 
-  const int64_t a = k << run_shift;
-  const int64_t b = min(a + ((int64_t)1 << run_shift), n_edges);
-
-  int cur = row_of_slot[a];
-  const bool began_before = a > 0 && row_of_slot[a - 1] == cur;
-  bool first_seg = true;
-
-  float acc[VEC];
+  template <class Close>
+  static __device__ __forceinline__ void walk(const Args &A,
+                                              const int32_t *__restrict__ row_of_slot,
+                                              int64_t a, int64_t b, int f0, int feat,
+                                              float (&st)[VEC], int &cur,
+                                              Close &&close_segment) {
+    typedef Frag<T, VEC> IO;
+    const int h = HASW ? f0 / A.dph : 0;
+    for (int64_t j = a; j < b; j += kUnroll) {
+      int r[kUnroll];
+      int64_t g[kUnroll];
+      float ww[kUnroll];
+      typename IO::raw_t x[kUnroll];
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) acc[v] = red_init<RED>();
-
-  for (int64_t j = a; j < b; j += kUnroll) {
-    int r[kUnroll];
-    int64_t g[kUnroll];
-    float ww[kUnroll];
-    typename IO::raw_t x[kUnroll];
-#pragma unroll
-    for (int t = 0; t < kUnroll; ++t) {
-      const int64_t jj = j + t < b ? j + t : b - 1;
-      r[t] = row_of_slot[jj];
-      g[t] = gidx ? (int64_t)gidx[jj] : jj;
-      if (HASW) {
-        const int64_t e = eid ? (int64_t)eid[jj] : jj;
-        ww[t] = w[e * heads + h];
-      }
-    }
-#pragma unroll
-    for (int t = 0; t < kUnroll; ++t) x[t] = IO::load(u + g[t] * feat + f0);
-#pragma unroll
-    for (int t = 0; t < kUnroll; ++t) {
-      if (j + t < b) {
-        if (r[t] != cur) {
-          // the open row ended inside this run
-          if (first_seg && began_before) {
-            float *p = partial + (k * 2) * feat + f0;
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) p[v] = acc[v];
-          } else {
-            IO::store(out + (int64_t)cur * feat + f0, acc);
-          }
-          first_seg = false;
-          cur = r[t];
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) acc[v] = red_init<RED>();
+      for (int t = 0; t < kUnroll; ++t) {
+        const int64_t jj = j + t < b ? j + t : b - 1;
+        r[t] = row_of_slot[jj];
+        g[t] = A.gidx ? (int64_t)A.gidx[jj] : jj;
+        if (HASW) {
+          const int64_t e = A.eid ? (int64_t)A.eid[jj] : jj;
+          ww[t] = A.w[e * A.heads + h];
         }
-        float xf[VEC];
-        IO::widen(x[t], xf);
+      }
 #pragma unroll
-        for (int v = 0; v < VEC; ++v)
-          acc[v] = red_apply<RED>(acc[v], HASW ? xf[v] * ww[t] : xf[v]);
+      for (int t = 0; t < kUnroll; ++t) x[t] = IO::load(A.u + g[t] * feat + f0);
+#pragma unroll
+      for (int t = 0; t < kUnroll; ++t) {
+        if (j + t < b) {
+          if (r[t] != cur) {
+            close_segment();
+            cur = r[t];
+            init(st);
+          }
+          float xf[VEC];
+          IO::widen(x[t], xf);
+#pragma unroll
+          for (int v = 0; v < VEC; ++v)
+            st[v] = red_apply<RED>(st[v], HASW ? xf[v] * ww[t] : xf[v]);
+        }
       }
     }
   }
-  const bool continues = b < n_edges && row_of_slot[b] == cur;
-  if (first_seg ? (began_before || continues) : continues) {
-    float *p = partial + (k * 2 + (first_seg ? 0 : 1)) * feat + f0;
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) p[v] = acc[v];
-  } else {
-    IO::store(out + (int64_t)cur * feat + f0, acc);
-  }
-}
-
-// Blocks [0, fix_blocks): one lane group per run; the group whose run holds
-// the END of a row that began in an earlier run combines that row's partials
-// in run order.  Remaining blocks: one lane group per row, rows without edges
-// receive the reducer's start value.
-template <typename T, int VEC, int RED>
-__global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(
-    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
-    const float *__restrict__ partial, T *__restrict__ out, int64_t n_rows,
-    int64_t n_edges, int64_t n_runs, int feat, int run_shift, int tpr_shift,
-    int fix_blocks) {
-  typedef Frag<T, VEC> IO;
-  const int tpr = 1 << tpr_shift;
-  const int f0 = ((int)blockIdx.y * tpr + (threadIdx.x & (tpr - 1))) * VEC;
-  if (f0 >= feat) return;
-  float acc[VEC];
-  if ((int)blockIdx.x < fix_blocks) {
-    const int64_t k = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> tpr_shift;
-    if (k >= n_runs) return;
-    const int64_t a = k << run_shift;
-    const int64_t b = min(a + ((int64_t)1 << run_shift), n_edges);
-    const int row = row_of_slot[a];
-    const int64_t s = pointer[row], e = pointer[row + 1];
-    if (!(s < a && e <= b)) return;
-    const int64_t k_lo = s >> run_shift;
-    const int slot = (s == (k_lo << run_shift)) ? 0 : 1;
-    const float *p = partial + (k_lo * 2 + slot) * feat + f0;
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) acc[v] = p[v];
-    for (int64_t q = k_lo + 1; q <= k; ++q) {
-      const float *pq = partial + (q * 2) * feat + f0;
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) acc[v] = red_apply<RED>(acc[v], pq[v]);
-    }
-    IO::store(out + (int64_t)row * feat + f0, acc);
-  } else {
-    const int64_t row =
-        ((int64_t)(blockIdx.x - fix_blocks) * kBlock + threadIdx.x) >> tpr_shift;
-    if (row >= n_rows || pointer[row] != pointer[row + 1]) return;
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) acc[v] = red_init<RED>();
-    IO::store(out + row * feat + f0, acc);
-  }
-}
+};
 
 template <typename T, int VEC, int RED, bool HASW>
 int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
                 const int32_t *gidx, const int32_t *eid, const void *u,
                 const float *w, void *out, int64_t n_rows, int64_t n_edges,
                 int feat, int heads, float *partial, hipStream_t stream) {
-  const int lanes = (feat + VEC - 1) / VEC;
-  const int tpr_shift = ilog2_ceil((uint64_t)(lanes > kWave ? kWave : lanes));
-  const int tpr = 1 << tpr_shift;
-  const int ftiles = (lanes + tpr - 1) / tpr;
-  const int run_shift = run_shift_for(n_edges, feat);
-  const int64_t n_runs = (n_edges + ((int64_t)1 << run_shift) - 1) >> run_shift;
-  const int groups_per_block = kBlock >> tpr_shift;
-  if (n_runs > 0) {
-    const int64_t blocks = (n_runs + groups_per_block - 1) / groups_per_block;
-    if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-    hipLaunchKernelGGL((spmm_runs_kernel<T, VEC, RED, HASW>),
-                       dim3((unsigned)blocks, ftiles), dim3(kBlock), 0, stream,
-                       row_of_slot, gidx, eid, (const T *)u, w, (T *)out,
-                       partial, n_edges, n_runs, feat, heads, feat / heads,
-                       run_shift, tpr_shift);
-  }
-  const int64_t fix_blocks = (n_runs + groups_per_block - 1) / groups_per_block;
-  const int64_t fill_blocks = (n_rows + groups_per_block - 1) / groups_per_block;
-  if (fix_blocks + fill_blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-  if (fix_blocks + fill_blocks > 0)
-    hipLaunchKernelGGL((spmm_fixup_kernel<T, VEC, RED>),
-                       dim3((unsigned)(fix_blocks + fill_blocks), ftiles),
-                       dim3(kBlock), 0, stream, pointer, row_of_slot, partial,
-                       (T *)out, n_rows, n_edges, n_runs, feat, run_shift,
-                       tpr_shift, (int)fix_blocks);
-  return launch_status();
+  typedef SpmmPolicy<T, VEC, RED, HASW> P;
+  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads};
+  return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, feat,
+                        partial, stream);
 }
 
 template <typename T, int VEC, int RED>
@@ -265,10 +182,7 @@ int ga_csr_row_ids(const int32_t *pointer, int64_t n_rows, int64_t n_edges,
 }
 
 size_t ga_spmm_workspace_bytes(int64_t n_edges, int64_t feat) {
-  if (n_edges <= 0 || feat <= 0) return 0;
-  const int run_shift = ga::run_shift_for(n_edges, feat);
-  const int64_t n_runs = (n_edges + ((int64_t)1 << run_shift) - 1) >> run_shift;
-  return (size_t)n_runs * 2 * (size_t)feat * sizeof(float);
+  return ga::runs_workspace_bytes(n_edges, feat, 1);
 }
 
 int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,

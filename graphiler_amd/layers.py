@@ -33,13 +33,20 @@ def gat_project(h, fc_weight, attn_weight, heads: int = 1):
     """Dense part of the GAT plan (GAT.py:25-29 after the split and reorder
     passes): z = h @ W, el = <z, a_l>, er = <z, a_r> per head."""
     z = torch.mm(h, fc_weight)                               # (N, H*D)
-    n = z.shape[0]
-    d = z.shape[1] // heads
-    a_l, a_r = attn_weight[0], attn_weight[1]                # (H, D) each
-    zh = z.view(n, heads, d)
-    el = (zh * a_l).sum(-1).contiguous()                     # (N, H)
-    er = (zh * a_r).sum(-1).contiguous()
+    # per-head dot products as two skinny GEMMs with block-diagonal (H*D, H)
+    # matrices: the reference's mm(z2, attn_weight) after its split pass
+    el = torch.mm(z, _head_blocks(attn_weight[0]))           # (N, H)
+    er = torch.mm(z, _head_blocks(attn_weight[1]))
     return z, el, er
+
+
+def _head_blocks(a: torch.Tensor) -> torch.Tensor:
+    """(H, D) per-head vectors -> (H*D, H) block-diagonal matrix."""
+    heads, d = a.shape
+    m = torch.zeros(heads * d, heads, dtype=a.dtype, device=a.device)
+    for hd in range(heads):
+        m[hd * d:(hd + 1) * d, hd] = a[hd]
+    return m
 
 
 def gat_aggregate_plan(g: DGLGraph, z, el, er, negative_slope: float = 0.01):
