@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 # HBM bytes per dominant-kernel launch measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); the summary
 # lives under profiles/.  None until measured for the kernel named below.
-MEASURED_TRAFFIC_BYTES = {"plan": None, "fused": None}
+MEASURED_TRAFFIC_BYTES = {"plan": 1_480_080_486, "fused": 1_534_816_358}
 
 
 def main():
@@ -131,6 +131,9 @@ def main():
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES[args.path],
         "algorithmic_bytes": alg[dom], "launch_ms": round(ops_ms[dom], 4),
+        "note": ("algorithmic bytes credit no cache reuse (one gathered row per "
+                 "edge); a fraction above 1 means the gathers are cache-served: "
+                 "effective bandwidth, not HBM bandwidth"),
     }
 
     # ---- CPU baseline: the oracle's fp32 port of the same layer -------------
