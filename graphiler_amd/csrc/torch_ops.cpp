@@ -1,0 +1,469 @@
+// TorchScript boundary: torch.classes.my_classes.DGLGraph and torch.ops.my_ops.*
+// with the reference's class layout and operator schemas, so a compiled
+// Graphiler plan (a TorchScript graph of my_ops::* nodes) runs unchanged on the
+// gfx950 kernels.  This file is host-only glue over the C ABI of
+// include/graphiler_amd.h: it owns allocation, argument checks (raised as
+// c10::Error, i.e. RuntimeError in Python, like the reference's CHECK_INPUT in
+// src/ops/ops.cuh:14-20) and passes the current HIP stream down.
+//
+// Reference counterparts: include/dglgraph.h:7-75 and src/dglgraph.cpp:5-24
+// (class), the `static auto registry` blocks of src/ops/dgl_primitives/spmm.cu:391-406,
+// sddmm.cu:131-134, segment_softmax/segment_softmax.cu:27-30,
+// segment_mm/segment_mm.cu:35-42 and broadcast/broadcast.cu:102-122 (operators).
+#include <torch/custom_class.h>
+#include <torch/script.h>
+
+#include <c10/hip/HIPStream.h>
+
+#include <mutex>
+
+#include "../../include/graphiler_amd.h"
+
+namespace {
+
+void check_ga(int code, const char *where) {
+  TORCH_CHECK(code == GA_OK, where, ": ", ga_error_string(code), " (code ", code, ")");
+}
+
+void check_input(const torch::Tensor &x, const char *name) {
+  TORCH_CHECK(x.is_cuda(), name, " must be a CUDA tensor");
+  TORCH_CHECK(x.is_contiguous(), name, " must be contiguous");
+}
+
+void check_index(const torch::Tensor &x, at::ScalarType t, const char *name) {
+  check_input(x, name);
+  TORCH_CHECK(x.scalar_type() == t, name, " has the wrong integer type");
+}
+
+int feat_dtype(const torch::Tensor &x, const char *name) {
+  if (x.scalar_type() == at::kFloat) return GA_F32;
+  if (x.scalar_type() == at::kBFloat16) return GA_BF16;
+  TORCH_CHECK(false, name, " must be float32 or bfloat16");
+  return -1;
+}
+
+ga_stream_t current_stream(const torch::Tensor &x) {
+  return (ga_stream_t)c10::hip::getCurrentHIPStream(x.device().index()).stream();
+}
+
+int64_t feat_dim(const torch::Tensor &x) {
+  int64_t d = 1;
+  for (int64_t i = 1; i < x.dim(); ++i) d *= x.size(i);
+  return d;
+}
+
+std::vector<int64_t> out_shape(int64_t rows, const torch::Tensor &x) {
+  std::vector<int64_t> shape{rows};
+  if (x.dim() > 1)
+    for (int64_t i = 1; i < x.dim(); ++i) shape.push_back(x.size(i));
+  else
+    shape.push_back(1);
+  return shape;
+}
+
+}  // namespace
+
+// Same public members as the reference's struct; the private part caches what
+// the kernels schedule with (slot -> row maps, identity flags, workspace).
+struct DGLGraph : torch::CustomClassHolder {
+  DGLGraph(torch::Tensor in_pointer, torch::Tensor in_node_indices,
+           torch::Tensor in_edge_indices, torch::Tensor out_pointer,
+           torch::Tensor out_node_indices, torch::Tensor out_edge_indices,
+           torch::Tensor COO_src, torch::Tensor COO_dst,
+           at::optional<torch::Tensor> ntype_pointer,
+           at::optional<torch::Tensor> etype_pointer)
+      : in_pointer(in_pointer), in_node_indices(in_node_indices),
+        in_edge_indices(in_edge_indices), out_pointer(out_pointer),
+        out_node_indices(out_node_indices), out_edge_indices(out_edge_indices),
+        COO_src(COO_src), COO_dst(COO_dst) {
+    check_index(in_pointer, at::kInt, "in_pointer");
+    check_index(in_node_indices, at::kInt, "in_node_indices");
+    check_index(in_edge_indices, at::kInt, "in_edge_indices");
+    check_index(out_pointer, at::kInt, "out_pointer");
+    check_index(out_node_indices, at::kInt, "out_node_indices");
+    check_index(out_edge_indices, at::kInt, "out_edge_indices");
+    check_index(COO_src, at::kLong, "COO_src");
+    check_index(COO_dst, at::kLong, "COO_dst");
+    TORCH_CHECK(in_pointer.size(0) >= 1 && out_pointer.size(0) == in_pointer.size(0),
+                "pointers must have num_nodes + 1 entries");
+    num_nodes = in_pointer.size(0) - 1;
+    num_edges = in_node_indices.size(0);
+    TORCH_CHECK(in_edge_indices.size(0) == num_edges &&
+                    out_node_indices.size(0) == num_edges &&
+                    out_edge_indices.size(0) == num_edges &&
+                    COO_src.size(0) == num_edges && COO_dst.size(0) == num_edges,
+                "edge columns must all have num_edges entries");
+    SetNtypePointer(ntype_pointer);
+    SetEtypePointer(etype_pointer);
+  }
+  void SetNtypePointer(at::optional<torch::Tensor> pointer) {
+    if (pointer.has_value()) check_index(pointer.value(), at::kInt, "ntype_pointer");
+    ntype_pointer = pointer;
+    num_ntypes = pointer.has_value() ? pointer.value().size(0) - 1 : 1;
+  }
+  void SetEtypePointer(at::optional<torch::Tensor> pointer) {
+    if (pointer.has_value()) check_index(pointer.value(), at::kInt, "etype_pointer");
+    etype_pointer = pointer;
+    num_etypes = pointer.has_value() ? pointer.value().size(0) - 1 : 1;
+  }
+  void SetNtypeCOO(torch::Tensor column) {
+    check_index(column, at::kLong, "ntype_COO");
+    TORCH_CHECK(column.size(0) == num_nodes, "ntype_COO must have one entry per node");
+    ntype_COO = column;
+  }
+  void SetEtypeCOO(torch::Tensor column) {
+    check_index(column, at::kLong, "etype_COO");
+    TORCH_CHECK(column.size(0) == num_edges, "etype_COO must have one entry per edge");
+    etype_COO = column;
+  }
+
+  int64_t num_nodes, num_edges, num_ntypes, num_etypes;
+  torch::Tensor in_pointer, in_node_indices, in_edge_indices;
+  torch::Tensor out_pointer, out_node_indices, out_edge_indices;
+  torch::Tensor COO_src, COO_dst;
+  at::optional<torch::Tensor> ntype_pointer, etype_pointer, ntype_COO, etype_COO;
+
+  // ---- derived, built on first use ----------------------------------------
+  struct Side {
+    torch::Tensor rows;
+    bool identity = false;
+    bool ready = false;
+  };
+  const Side &side(bool reverse) {
+    std::lock_guard<std::mutex> lock(mu_);
+    Side &s = reverse ? out_side_ : in_side_;
+    if (!s.ready) {
+      const torch::Tensor &ptr = reverse ? out_pointer : in_pointer;
+      const torch::Tensor &eid = reverse ? out_edge_indices : in_edge_indices;
+      s.rows = torch::empty({num_edges}, ptr.options());
+      check_ga(ga_csr_row_ids(ptr.data_ptr<int>(), num_nodes, num_edges,
+                              s.rows.data_ptr<int>(), current_stream(ptr)),
+               "ga_csr_row_ids");
+      s.identity = num_edges == 0 ||
+                   torch::equal(eid, torch::arange(num_edges, eid.options()));
+      s.ready = true;
+    }
+    return s;
+  }
+  torch::Tensor workspace(size_t bytes) {
+    std::lock_guard<std::mutex> lock(mu_);
+    if (!ws_.defined() || (size_t)ws_.numel() < bytes)
+      ws_ = torch::empty({(int64_t)std::max<size_t>(bytes, 256)},
+                         in_pointer.options().dtype(at::kByte));
+    return ws_;
+  }
+
+ private:
+  std::mutex mu_;
+  Side in_side_, out_side_;
+  torch::Tensor ws_;
+};
+
+using GraphPtr = c10::intrusive_ptr<DGLGraph>;
+
+namespace {
+
+torch::Tensor spmm(const GraphPtr &g, int op, int reduce, const torch::Tensor &u,
+                   const at::optional<torch::Tensor> &w, bool reverse) {
+  check_input(u, "features");
+  const int dt = feat_dtype(u, "features");
+  const auto &side = g->side(reverse);
+  const torch::Tensor &ptr = reverse ? g->out_pointer : g->in_pointer;
+  const torch::Tensor &nbr = reverse ? g->out_node_indices : g->in_node_indices;
+  const torch::Tensor &eid = reverse ? g->out_edge_indices : g->in_edge_indices;
+  const int64_t feat = feat_dim(u);
+  int64_t heads = 1;
+  if (op == GA_U_MUL_E) {
+    TORCH_CHECK(w.has_value(), "edge weights are required");
+    check_input(w.value(), "edge weights");
+    TORCH_CHECK(w.value().scalar_type() == at::kFloat, "edge weights must be float32");
+    TORCH_CHECK(w.value().size(0) == g->num_edges, "edge weights must have one row per edge");
+    heads = feat_dim(w.value());
+    TORCH_CHECK(heads > 0 && feat % heads == 0,
+                "feature width is not a multiple of the heads");
+  }
+  TORCH_CHECK(u.size(0) == (op == GA_COPY_E ? g->num_edges : g->num_nodes),
+              "features have the wrong number of rows");
+  torch::Tensor out = torch::empty(out_shape(g->num_nodes, u), u.options());
+  const size_t ws_bytes = ga_spmm_workspace_bytes(g->num_edges, feat);
+  torch::Tensor ws = g->workspace(ws_bytes);
+  check_ga(ga_spmm_csr(ptr.data_ptr<int>(), side.rows.data_ptr<int>(),
+                       nbr.data_ptr<int>(),
+                       side.identity ? nullptr : eid.data_ptr<int>(), u.data_ptr(),
+                       w.has_value() ? w.value().data_ptr<float>() : nullptr,
+                       out.data_ptr(), g->num_nodes, g->num_edges, feat, heads, op,
+                       reduce, dt, ws.data_ptr(), (size_t)ws.numel(),
+                       current_stream(u)),
+           "ga_spmm_csr");
+  return out;
+}
+
+// spmm.cu:359-373
+torch::Tensor SpMMEdge(torch::Tensor features, std::vector<int64_t> dims,
+                       bool keep_dim, at::optional<int64_t> dtype,
+                       const GraphPtr &graph) {
+  return spmm(graph, GA_COPY_E, GA_SUM, features, at::nullopt, false);
+}
+// spmm.cu:375-389
+torch::Tensor SpMMSrc(torch::Tensor features, std::vector<int64_t> dims,
+                      bool keep_dim, at::optional<int64_t> dtype,
+                      const GraphPtr &graph) {
+  return spmm(graph, GA_COPY_U, GA_SUM, features, at::nullopt, false);
+}
+// spmm.cu:286-320
+torch::Tensor src_mul_e_sum(torch::Tensor ufeature, torch::Tensor efeature,
+                            std::vector<int64_t> dims, bool keep_dim,
+                            at::optional<int64_t> dtype,
+                            const GraphPtr &graph) {
+  return spmm(graph, GA_U_MUL_E, GA_SUM, ufeature, efeature, false);
+}
+// spmm.cu:322-356
+torch::Tensor dst_mul_e_sum(torch::Tensor ufeature, torch::Tensor efeature,
+                            std::vector<int64_t> dims, bool keep_dim,
+                            at::optional<int64_t> dtype,
+                            const GraphPtr &graph) {
+  return spmm(graph, GA_U_MUL_E, GA_SUM, ufeature, efeature, true);
+}
+// generic reducer entry (spmm.cuh:30-71 with functor.cuh:125-213)
+torch::Tensor gspmm(torch::Tensor ufeature, at::optional<torch::Tensor> efeature,
+                    std::string op, std::string reduce, const GraphPtr &graph) {
+  int o = op == "copy_u" ? GA_COPY_U : op == "copy_e" ? GA_COPY_E
+          : op == "u_mul_e" ? GA_U_MUL_E : -1;
+  int r = reduce == "sum" ? GA_SUM : reduce == "max" ? GA_MAX
+          : reduce == "min" ? GA_MIN : -1;
+  TORCH_CHECK(o >= 0, "Unsupported SpMM binary operator: ", op);
+  TORCH_CHECK(r >= 0, "Unsupported SpMM reducer: ", reduce);
+  return spmm(graph, o, r, ufeature, efeature, false);
+}
+
+struct EdgeColumns {
+  const void *lhs, *rhs;
+  int bits;
+};
+EdgeColumns edge_columns(const GraphPtr &g) {
+  const auto &side = g->side(false);
+  if (side.identity)
+    return {g->in_node_indices.data_ptr<int>(), side.rows.data_ptr<int>(), 32};
+  return {g->COO_src.data_ptr<int64_t>(), g->COO_dst.data_ptr<int64_t>(), 64};
+}
+
+// sddmm.cu:118-129 (alpha accepted and ignored, as there)
+torch::Tensor u_add_v_mul_alpha(torch::Tensor src_feature, torch::Tensor dst_feature,
+                                int64_t alpha, const GraphPtr &graph) {
+  check_input(src_feature, "src_feature");
+  check_input(dst_feature, "dst_feature");
+  const int dt = feat_dtype(src_feature, "src_feature");
+  TORCH_CHECK(dst_feature.scalar_type() == src_feature.scalar_type(),
+              "src_feature and dst_feature must share a dtype");
+  const int64_t feat = feat_dim(src_feature);
+  TORCH_CHECK(feat_dim(dst_feature) == feat,
+              "src_feature and dst_feature must share a width");
+  torch::Tensor out = torch::empty(out_shape(graph->num_edges, src_feature),
+                                   src_feature.options().dtype(at::kFloat));
+  const EdgeColumns c = edge_columns(graph);
+  check_ga(ga_sddmm_u_add_v(c.lhs, c.rhs, c.bits, src_feature.data_ptr(),
+                            dst_feature.data_ptr(), out.data_ptr<float>(),
+                            graph->num_edges, feat, dt, current_stream(out)),
+           "ga_sddmm_u_add_v");
+  return out;
+}
+
+// functor.cuh:103-116 + sddmm.cuh:80-120 (never registered by the reference)
+torch::Tensor u_dot_v(torch::Tensor src_feature, torch::Tensor dst_feature,
+                      const GraphPtr &graph) {
+  check_input(src_feature, "src_feature");
+  check_input(dst_feature, "dst_feature");
+  const int dt = feat_dtype(src_feature, "src_feature");
+  TORCH_CHECK(dst_feature.scalar_type() == src_feature.scalar_type() &&
+                  dst_feature.sizes().slice(1) == src_feature.sizes().slice(1),
+              "src_feature and dst_feature must share dtype and shape");
+  TORCH_CHECK(src_feature.dim() == 2 || src_feature.dim() == 3,
+              "u_dot_v expects (N, D) or (N, H, D) features");
+  const int64_t heads = src_feature.dim() == 3 ? src_feature.size(1) : 1;
+  const int64_t dim = src_feature.size(src_feature.dim() - 1);
+  torch::Tensor out = torch::empty({graph->num_edges, heads},
+                                   src_feature.options().dtype(at::kFloat));
+  const EdgeColumns c = edge_columns(graph);
+  check_ga(ga_sddmm_u_dot_v(c.lhs, c.rhs, c.bits, src_feature.data_ptr(),
+                            dst_feature.data_ptr(), out.data_ptr<float>(),
+                            graph->num_edges, heads, dim, dt, current_stream(out)),
+           "ga_sddmm_u_dot_v");
+  return out;
+}
+
+// segment_softmax.cu:3-24
+torch::Tensor SegmentSoftmaxForward(torch::Tensor features, int64_t dim,
+                                    at::optional<int64_t> dtype,
+                                    const GraphPtr &graph) {
+  check_input(features, "features");
+  TORCH_CHECK(dim == 1, "SegmentSoftmax reduces over dim 1 of the mailbox");
+  TORCH_CHECK(features.scalar_type() == at::kFloat, "features must be float32");
+  TORCH_CHECK(features.size(0) == graph->num_edges, "features must have one row per edge");
+  const int64_t heads = feat_dim(features);
+  const auto &side = graph->side(false);
+  torch::Tensor y = torch::empty_like(features);
+  torch::Tensor ws = graph->workspace(ga_softmax_workspace_bytes(graph->num_edges, heads));
+  check_ga(ga_segment_softmax(graph->in_pointer.data_ptr<int>(),
+                              side.rows.data_ptr<int>(),
+                              side.identity ? nullptr
+                                            : graph->in_edge_indices.data_ptr<int>(),
+                              features.data_ptr<float>(), y.data_ptr<float>(),
+                              graph->num_nodes, graph->num_edges, heads,
+                              ws.data_ptr(), (size_t)ws.numel(), current_stream(y)),
+           "ga_segment_softmax");
+  return y;
+}
+
+// segment_mm.cu:4-21
+torch::Tensor segment_mm(const torch::Tensor &features, const torch::Tensor &weights,
+                         const at::optional<torch::Tensor> &type_pointer,
+                         int64_t num_types, int64_t rows_expected) {
+  check_input(features, "features");
+  check_input(weights, "weights");
+  const int dt = feat_dtype(features, "features");
+  TORCH_CHECK(weights.scalar_type() == features.scalar_type(),
+              "features and weights must share a dtype");
+  TORCH_CHECK(type_pointer.has_value(), "the graph has no type pointer for this operator");
+  TORCH_CHECK(weights.dim() == 3 || weights.dim() == 4,
+              "weights must be (T, K, M) or (T, H, K, M)");
+  const int64_t heads = weights.dim() == 4 ? weights.size(1) : 1;
+  const int64_t K = weights.size(weights.dim() - 2), M = weights.size(weights.dim() - 1);
+  TORCH_CHECK(weights.size(0) == num_types, "weights must have one matrix per type");
+  const int64_t rows = features.size(0);
+  TORCH_CHECK(rows == rows_expected && feat_dim(features) == heads * K,
+              "features must be (rows, heads*K)");
+  torch::Tensor out = torch::empty({rows, heads * M}, features.options());
+  check_ga(ga_segment_mm(type_pointer.value().data_ptr<int>(), num_types,
+                         features.data_ptr(), weights.data_ptr(), out.data_ptr(),
+                         rows, heads, K, M, dt, current_stream(out)),
+           "ga_segment_mm");
+  return out;
+}
+// segment_mm.cu:23-27
+torch::Tensor SegmentMMNode(torch::Tensor features, torch::Tensor weights,
+                            const GraphPtr &graph) {
+  return segment_mm(features, weights, graph->ntype_pointer, graph->num_ntypes,
+                    graph->num_nodes);
+}
+// segment_mm.cu:29-33
+torch::Tensor SegmentMMEdge(torch::Tensor features, torch::Tensor weights,
+                            const GraphPtr &graph) {
+  return segment_mm(features, weights, graph->etype_pointer, graph->num_etypes,
+                    graph->num_edges);
+}
+
+torch::Tensor gather(const torch::Tensor &features, const torch::Tensor &index) {
+  check_input(features, "features");
+  std::vector<int64_t> shape{index.size(0)};
+  for (int64_t i = 1; i < features.dim(); ++i) shape.push_back(features.size(i));
+  torch::Tensor out = torch::empty(shape, features.options());
+  check_ga(ga_gather_rows(index.data_ptr(), 64, features.data_ptr(), out.data_ptr(),
+                          index.size(0), feat_dim(features) * features.element_size(),
+                          current_stream(out)),
+           "ga_gather_rows");
+  return out;
+}
+// broadcast.cu:58-100
+torch::Tensor BroadcastSrcNode(torch::Tensor features, const GraphPtr &graph) {
+  return gather(features, graph->COO_src);
+}
+torch::Tensor BroadcastDstNode(torch::Tensor features, const GraphPtr &graph) {
+  return gather(features, graph->COO_dst);
+}
+torch::Tensor BroadcastNodeType(torch::Tensor features, const GraphPtr &graph) {
+  TORCH_CHECK(graph->ntype_COO.has_value(), "the graph has no node-type column");
+  return gather(features, graph->ntype_COO.value());
+}
+torch::Tensor BroadcastSrcNodeType(torch::Tensor features, const GraphPtr &graph) {
+  return BroadcastSrcNode(BroadcastNodeType(features, graph), graph);
+}
+torch::Tensor BroadcastDstNodeType(torch::Tensor features, const GraphPtr &graph) {
+  return BroadcastDstNode(BroadcastNodeType(features, graph), graph);
+}
+torch::Tensor BroadcastEdgeType(torch::Tensor features, const GraphPtr &graph) {
+  TORCH_CHECK(graph->etype_COO.has_value(), "the graph has no edge-type column");
+  return gather(features, graph->etype_COO.value());
+}
+// broadcast.cu:3-9
+int64_t get_feat_dim(torch::Tensor features) { return feat_dim(features); }
+
+// fused u_add_v -> leaky_relu -> SegmentSoftmax -> src_mul_e_sum
+torch::Tensor gat_aggregate(torch::Tensor el, torch::Tensor er, torch::Tensor z,
+                            double negative_slope, const GraphPtr &graph) {
+  check_input(el, "el");
+  check_input(er, "er");
+  check_input(z, "z");
+  const int dt = feat_dtype(z, "z");
+  TORCH_CHECK(el.scalar_type() == at::kFloat && er.scalar_type() == at::kFloat,
+              "el and er must be float32");
+  const int64_t heads = feat_dim(el), feat = feat_dim(z);
+  TORCH_CHECK(feat_dim(er) == heads && heads > 0 && feat % heads == 0,
+              "inconsistent head count");
+  TORCH_CHECK(el.size(0) == graph->num_nodes && er.size(0) == graph->num_nodes &&
+                  z.size(0) == graph->num_nodes, "inputs must have one row per node");
+  const auto &side = graph->side(false);
+  torch::Tensor out = torch::empty(out_shape(graph->num_nodes, z), z.options());
+  torch::Tensor ws = graph->workspace(ga_gat_workspace_bytes(graph->num_edges, feat, heads));
+  check_ga(ga_gat_aggregate(graph->in_pointer.data_ptr<int>(),
+                            side.rows.data_ptr<int>(),
+                            graph->in_node_indices.data_ptr<int>(),
+                            el.data_ptr<float>(), er.data_ptr<float>(), z.data_ptr(),
+                            out.data_ptr(), graph->num_nodes, graph->num_edges, heads,
+                            feat / heads, (float)negative_slope, dt, ws.data_ptr(),
+                            (size_t)ws.numel(), current_stream(out)),
+           "ga_gat_aggregate");
+  return out;
+}
+
+}  // namespace
+
+TORCH_LIBRARY(my_classes, m) {
+  m.class_<DGLGraph>("DGLGraph")
+      .def(torch::init<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+                       torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+                       at::optional<torch::Tensor>, at::optional<torch::Tensor>>())
+      .def("SetNtypePointer", &DGLGraph::SetNtypePointer)
+      .def("SetEtypePointer", &DGLGraph::SetEtypePointer)
+      .def("SetNtypeCOO", &DGLGraph::SetNtypeCOO)
+      .def("SetEtypeCOO", &DGLGraph::SetEtypeCOO);
+}
+
+#define GRAPH_T "__torch__.torch.classes.my_classes.DGLGraph"
+
+static auto registry =
+    torch::RegisterOperators(
+        "my_ops::SpMMEdge(Tensor x, int[] dim, bool k, int? t, " GRAPH_T " g) -> Tensor y",
+        &SpMMEdge)
+        .op("my_ops::SpMMSrc(Tensor x, int[] dim, bool k, int? t, " GRAPH_T " g) -> Tensor y",
+            &SpMMSrc)
+        .op("my_ops::gspmm_src_mul_e_sum(Tensor x, Tensor y, int[] dim, bool k, int? t, "
+            GRAPH_T " g) -> Tensor z",
+            &src_mul_e_sum)
+        .op("my_ops::gspmm_dst_mul_e_sum(Tensor x, Tensor y, int[] dim, bool k, int? t, "
+            GRAPH_T " g) -> Tensor z",
+            &dst_mul_e_sum)
+        .op("my_ops::gsddmm_u_add_v_mul_alpha(Tensor x, Tensor y, int alpha, " GRAPH_T
+            " g) -> Tensor z",
+            &u_add_v_mul_alpha)
+        .op("my_ops::SegmentSoftmax(Tensor x, int dim, int? t, " GRAPH_T " g) -> Tensor y",
+            &SegmentSoftmaxForward)
+        .op("my_ops::SegmentMMNode(Tensor x, Tensor y, " GRAPH_T " g) -> Tensor z",
+            &SegmentMMNode)
+        .op("my_ops::SegmentMMEdge(Tensor x, Tensor y, " GRAPH_T " g) -> Tensor z",
+            &SegmentMMEdge)
+        .op("my_ops::BroadcastSrcNode(Tensor x, " GRAPH_T " g) -> Tensor y", &BroadcastSrcNode)
+        .op("my_ops::BroadcastDstNode(Tensor x, " GRAPH_T " g) -> Tensor y", &BroadcastDstNode)
+        .op("my_ops::BroadcastNodeType(Tensor x, " GRAPH_T " g) -> Tensor y", &BroadcastNodeType)
+        .op("my_ops::BroadcastSrcNodeType(Tensor x, " GRAPH_T " g) -> Tensor y",
+            &BroadcastSrcNodeType)
+        .op("my_ops::BroadcastDstNodeType(Tensor x, " GRAPH_T " g) -> Tensor y",
+            &BroadcastDstNodeType)
+        .op("my_ops::BroadcastEdgeType(Tensor x, " GRAPH_T " g) -> Tensor y", &BroadcastEdgeType)
+        .op("my_ops::get_feat_dim", &get_feat_dim)
+        // additions of this build (no counterpart registered by the reference)
+        .op("my_ops::gsddmm_u_dot_v(Tensor x, Tensor y, " GRAPH_T " g) -> Tensor z", &u_dot_v)
+        .op("my_ops::gspmm(Tensor x, Tensor? y, str op, str reduce, " GRAPH_T " g) -> Tensor z",
+            &gspmm)
+        .op("my_ops::gat_aggregate(Tensor el, Tensor er, Tensor z, float slope, " GRAPH_T
+            " g) -> Tensor y",
+            &gat_aggregate);
