@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import oracle
-from graphiler_amd import datasets, ops, prepare_graph
+from graphiler_amd import capi, datasets, ops, prepare_graph
 from graphiler_amd.graph import build_graph_arrays
 from helpers import (TOL_BF16, TOL_F32, assert_close, random_graph,
                      skewed_graph, to_bf16_f32)
@@ -251,3 +251,64 @@ def test_gat_layer_plan_equals_fused(graph, device):
     plan = layers.gat_layer(g, h, w, a, 2, 0.2, fused=False).cpu().numpy()
     fused = layers.gat_layer(g, h, w, a, 2, 0.2, fused=True).cpu().numpy()
     assert_close(fused, plan, 2 * TOL_F32, f"GAT layer plan vs fused {name}")
+
+
+def _typed_rows(rng, counts):
+    tp = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    return tp, int(tp[-1])
+
+
+@pytest.mark.parametrize("K,M,heads", [(16, 64, 1), (64, 8, 1), (64, 64, 1),
+                                       (128, 128, 1), (20, 12, 1), (6, 5, 1),
+                                       (16, 16, 8), (32, 48, 2), (8, 3, 3),
+                                       (256, 32, 1), (128, 200, 1)])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_segment_mm(device, K, M, heads, bf16):
+    rng = np.random.default_rng(K * 1000 + M + heads)
+    counts = [70, 0, 1, 333, 0, 0, 64, 15, 129, 2000, 0]
+    tp, rows = _typed_rows(rng, counts)
+    X = rng.standard_normal((rows, heads * K), dtype=np.float32)
+    W = (rng.standard_normal((len(counts), heads, K, M)) / np.sqrt(K)).astype(np.float32)
+    if bf16:
+        X, W = to_bf16_f32(X), to_bf16_f32(W)
+    lib = capi.load()
+    dX, dW = _dev(X, device, bf16), _dev(W, device, bf16)
+    dtp = _dev(tp, device)
+    Y = torch.full((rows, heads * M), float("nan"), dtype=dX.dtype, device=device)
+    rc = lib.ga_segment_mm(dtp.data_ptr(), len(counts), dX.data_ptr(), dW.data_ptr(),
+                           Y.data_ptr(), rows, heads, K, M,
+                           capi.GA_BF16 if bf16 else capi.GA_F32,
+                           torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    ref = oracle.segment_mm(tp, X, W, heads=heads)
+    assert_close(Y.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
+                 f"segment_mm K={K} M={M} H={heads} bf16={bf16}")
+
+
+def test_segment_mm_ops_and_rgcn_layer(device):
+    """SegmentMMEdge / SegmentMMNode through the operator wrappers, and the
+    RGCN plan BroadcastSrcNode -> SegmentMMEdge -> mul(norm) -> SpMMEdge."""
+    from graphiler_amd import layers
+    wl = datasets.rgcn_zipf(num_nodes=3000, n_edges=40_000, n_rel=60, seed=2)
+    ntype = np.sort(np.random.default_rng(0).integers(0, 4, wl.num_nodes))
+    g = prepare_graph(wl.src, wl.dst, wl.num_nodes, device=device,
+                      ntype_of=ntype, num_ntypes=4, etype_of=wl.etype, num_etypes=60)
+    arr = build_graph_arrays(wl.src, wl.dst, wl.num_nodes)
+    rng = np.random.default_rng(2)
+    h = rng.standard_normal((wl.num_nodes, 16), dtype=np.float32)
+    W = datasets.glorot(rng, (60, 16, 64))
+    deg = np.maximum(np.bincount(wl.dst, minlength=wl.num_nodes), 1)
+    norm = (1.0 / deg[wl.dst]).astype(np.float32)[:, None]
+    got = layers.rgcn_layer(g, _dev(h, device), _dev(W, device), _dev(norm, device))
+    etp = oracle.type_pointer(wl.etype, 60)
+    msg = oracle.segment_mm(etp, oracle.gather_rows(wl.src, h), W) * norm
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      msg.astype(np.float32), op="copy_e")
+    assert_close(got.cpu().numpy(), ref, 2 * TOL_F32, "RGCN layer")
+    Wn = datasets.glorot(rng, (4, 16, 32))
+    got = ops.SegmentMMNode(_dev(h, device), _dev(Wn, device), g)
+    ref = oracle.segment_mm(oracle.type_pointer(ntype, 4), h, Wn)
+    assert_close(got.cpu().numpy(), ref, TOL_F32, "SegmentMMNode")
+    with pytest.raises(RuntimeError, match="type pointer"):
+        g2 = prepare_graph(wl.src, wl.dst, wl.num_nodes, device=device)
+        ops.SegmentMMEdge(_dev(h[:1], device), _dev(W, device), g2)
