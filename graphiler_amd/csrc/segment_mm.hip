@@ -4,16 +4,24 @@
 //
 // Every configured shape (K, M <= 128) is bound by streaming X in and Y out, so
 // the kernel is organised around the row stream: a workgroup (4 waves) takes a
-// chunk of consecutive rows of ONE type, keeps that type's weights for all heads
-// in LDS, and each wave pushes 16-row tiles through MFMA with fp32 accumulation:
-//   fp32: v_mfma_f32_16x16x4_f32, one 16-byte X load per lane covers K = 16
-//         (the four components feed four MFMAs; the k order inside a block is
-//         permuted identically for X and W, which a dot product allows);
-//   bf16: v_mfma_f32_16x16x32_bf16, one 16-byte X load per lane covers K = 32.
-// The product is formed transposed (D = W^T X^T) so that each lane ends up with
-// four consecutive output columns of one row and stores them as one vector.
-// The type of a chunk is found on the device from type_pointer (block-wide
-// prefix sum of chunks per type): no host copy, no synchronisation.
+// chunk of consecutive rows of ONE type, keeps that type's weights in LDS, and
+// each wave pushes 16-row tiles through MFMA with fp32 accumulation:
+//   fp32          v_mfma_f32_16x16x4_f32; one 16-byte X load per lane covers
+//                 K = 16 (its four components feed four MFMAs; the k order
+//                 inside a block is permuted identically for X and W, which a
+//                 dot product allows);
+//   bf16, K%32==0 v_mfma_f32_16x16x32_bf16, one 16-byte X load covers K = 32;
+//   bf16, other   v_mfma_f32_16x16x16_bf16, one 8-byte X load covers K = 16.
+// Heads are folded into one product with a block-diagonal weight tile
+// (Kt = heads*K, Mt = heads*M, zeros off the diagonal): whole rows are loaded
+// with wide accesses; the MFMAs spent on zero blocks are far below the time the
+// row stream takes.  All X fragments of a
+// tile are loaded before its MFMAs.  Accumulators come out as D[row][column]
+// with 16 adjacent lanes holding 16 adjacent columns, so stores coalesce; for
+// bf16 two column blocks interleave their columns (even / odd) so a lane packs
+// two neighbouring outputs into one 4-byte store.  The type of a chunk is found
+// on the device from type_pointer (block-wide prefix sum of chunks per type):
+// no host copy, no synchronisation.
 #include "common.h"
 
 namespace ga {
@@ -21,28 +29,181 @@ namespace {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kTileRows = 16;              // rows per wave tile (MFMA N)
-constexpr int kWaves = kBlock / kWave;     // 4
+constexpr int kTileRows = 16;                   // rows per wave tile
+constexpr int kWaves = kBlock / kWave;          // 4
 constexpr int kTileBlock = kTileRows * kWaves;  // 64 rows per workgroup step
-constexpr int kMaxLds = 64 * 1024;
+constexpr int kMaxLds = 64 * 1024;          // default per-workgroup LDS limit
+constexpr int kMaxLdsOptIn = 158 * 1024;    // gfx950 has 160 KB per CU
 
-template <typename T>
-struct MmTraits;
+// Raises a kernel's dynamic LDS limit when a tile needs more than 64 KB.
+inline bool allow_lds(const void *kernel, size_t bytes) {
+  if (bytes <= (size_t)kMaxLds) return true;
+  if (bytes > (size_t)kMaxLdsOptIn) return false;
+  return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                             (int)bytes) == hipSuccess;
+}
+constexpr int kMaxFrags = 8;                    // X fragments preloaded per tile
+
+// Problem seen by one launch: rows of type t use the (Kt x Mt) block-diagonal
+// tile built from `hb` consecutive (K x M) head blocks of W[t].
+struct MmGeom {
+  int n_types;
+  int chunk_rows;
+  int K, M, hb;        // per-head sizes, heads folded into the tile
+  int Kt, Mt;          // hb*K, hb*M
+  int KB, MB;          // k blocks / 16-column blocks of the tile
+  int64_t ldx, ldy;    // row strides of X and Y (elements)
+  int64_t w_type_stride;  // elements between W[t] and W[t+1]
+};
+
+// Column of the tile held by lane column j of column block cb.
+template <bool PAIRED>
+__device__ __forceinline__ int tile_col(int cb, int j) {
+  return PAIRED ? ((cb >> 1) * 32 + 2 * j + (cb & 1)) : (cb * 16 + j);
+}
+
+template <typename T, int KBLK>
+struct Mma;
+
 template <>
-struct MmTraits<float> {
-  static constexpr int kColGroup = 4;  // 16-column blocks accumulated per pass
-  static __host__ __device__ int w_stride(int kb, int mb) { return mb * 16 + 4; }
-  static __host__ __device__ size_t lds_bytes(int heads, int kb, int mb) {
-    return (size_t)heads * kb * 16 * w_stride(kb, mb) * sizeof(float);
+struct Mma<float, 16> {          // LDS: [k][col], row stride ws floats
+  typedef float4 frag_t;
+  static constexpr bool kPaired = false;
+  static __host__ __device__ int mb_pad(int MB) { return MB; }
+  static __host__ __device__ int ws(int KB, int MB) { return MB * 16 + 4; }
+  static __host__ __device__ int tile_elems(int KB, int MB) { return KB * 16 * ws(KB, MB); }
+  static __device__ __forceinline__ frag_t zero() { return make_float4(0, 0, 0, 0); }
+  static __device__ __forceinline__ frag_t load(const float *p) {
+    return *reinterpret_cast<const float4 *>(p);
+  }
+  static __device__ __forceinline__ int k_of_lane(int lk) { return lk * 4; }
+  static __device__ __forceinline__ floatx4 mma(floatx4 acc, const float *tile, int wsv,
+                                                int kb, int cb, int lr, int lk,
+                                                const frag_t &x) {
+    const float *w = tile + (kb * 16 + lk * 4) * wsv + cb * 16 + lr;
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x.x, w[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x.y, w[wsv], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x.z, w[2 * wsv], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x.w, w[3 * wsv], acc, 0, 0, 0);
+    return acc;
+  }
+  // zero the padded tile, then copy the hb diagonal (K x M) blocks; no integer
+  // divisions: lanes run along the columns, waves along the rows
+  static __device__ void stage(const float *__restrict__ w, float *tile,
+                               const MmGeom &g) {
+    const int wsv = ws(g.KB, g.MB);
+    const int total4 = (g.KB * 16 * wsv) >> 2;          // wsv is a multiple of 4
+    for (int i = threadIdx.x; i < total4; i += kBlock)
+      reinterpret_cast<float4 *>(tile)[i] = make_float4(0, 0, 0, 0);
+    __syncthreads();
+    const int tx = threadIdx.x & (kWave - 1), ty = threadIdx.x / kWave;
+    const bool vec = (g.M & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
+    for (int h = 0; h < g.hb; ++h) {
+      const float *wh = w + (int64_t)h * g.K * g.M;
+      float *th = tile + (h * g.K) * wsv + h * g.M;
+      if (vec) {
+        for (int k = ty; k < g.K; k += kBlock / kWave)
+          for (int m = tx * 4; m < g.M; m += kWave * 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(wh + (int64_t)k * g.M + m);
+            float *d = th + k * wsv + m;       // 16-byte aligned only when h*M is
+            d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+          }
+      } else {
+        for (int k = ty; k < g.K; k += kBlock / kWave)
+          for (int m = tx; m < g.M; m += kWave)
+            th[k * wsv + m] = wh[(int64_t)k * g.M + m];
+      }
+    }
   }
 };
+
+// bf16 weights live transposed in LDS: [lane column][k], row stride ws elements,
+// so a lane's k-contiguous fragment is one vector read.  LDS row cb*16 + j holds
+// tile column tile_col<true>(cb, j).
+template <int KBLK>
+struct MmaBf16Base {
+  static constexpr bool kPaired = true;
+  static __host__ __device__ int mb_pad(int MB) { return (MB + 1) & ~1; }
+  static __host__ __device__ int ws(int KB, int MB) { return KB * KBLK + 8; }
+  static __host__ __device__ int tile_elems(int KB, int MB) {
+    return mb_pad(MB) * 16 * ws(KB, MB);
+  }
+  // zero the padded tile, then transpose the hb diagonal (K x M) blocks: a
+  // thread gathers 8 consecutive k of one column (loads coalesce across threads
+  // along the columns) and writes them as one 16-byte LDS vector.  No divisions.
+  static __device__ void stage(const bf16_t *__restrict__ w, bf16_t *tile,
+                               const MmGeom &g) {
+    const int wsv = ws(g.KB, g.MB);
+    const int total8 = (mb_pad(g.MB) * 16 * wsv) >> 3;   // wsv is a multiple of 8
+    for (int i = threadIdx.x; i < total8; i += kBlock)
+      reinterpret_cast<uint4 *>(tile)[i] = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+    const int tx = threadIdx.x & (kWave - 1), ty = threadIdx.x / kWave;
+    for (int h = 0; h < g.hb; ++h) {
+      const bf16_t *wh = w + (int64_t)h * g.K * g.M;
+      for (int kc = ty * 8; kc < g.K; kc += (kBlock / kWave) * 8)
+        for (int m = tx; m < g.M; m += kWave) {
+          uint32_t v[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q)
+            v[q] = kc + q < g.K ? (uint32_t)wh[(int64_t)(kc + q) * g.M + m] : 0u;
+          const int c = h * g.M + m;                       // tile column
+          const int lrow = ((c >> 5) * 2 + (c & 1)) * 16 + ((c & 31) >> 1);
+          bf16_t *d = tile + lrow * wsv + h * g.K + kc;
+          if (((h * g.K + kc) & 7) == 0) {
+            uint4 o;
+            o.x = v[0] | (v[1] << 16);
+            o.y = v[2] | (v[3] << 16);
+            o.z = v[4] | (v[5] << 16);
+            o.w = v[6] | (v[7] << 16);
+            *reinterpret_cast<uint4 *>(d) = o;
+          } else {
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+              if (kc + q < g.K) d[q] = (bf16_t)v[q];
+          }
+        }
+    }
+  }
+};
+
 template <>
-struct MmTraits<bf16_t> {
-  static constexpr int kColGroup = 8;
-  static __host__ __device__ int w_stride(int kb, int mb) { return kb * 32 + 8; }
-  static __host__ __device__ size_t lds_bytes(int heads, int kb, int mb) {
-    return (size_t)heads * mb * 16 * w_stride(kb, mb) * sizeof(bf16_t);
+struct Mma<bf16_t, 32> : MmaBf16Base<32> {
+  typedef uint4 frag_t;
+  static __device__ __forceinline__ frag_t zero() { return make_uint4(0, 0, 0, 0); }
+  static __device__ __forceinline__ frag_t load(const bf16_t *p) {
+    return *reinterpret_cast<const uint4 *>(p);
+  }
+  static __device__ __forceinline__ int k_of_lane(int lk) { return lk * 8; }
+  static __device__ __forceinline__ floatx4 mma(floatx4 acc, const bf16_t *tile, int wsv,
+                                                int kb, int cb, int lr, int lk,
+                                                const frag_t &x) {
+    const uint4 w = *reinterpret_cast<const uint4 *>(tile + (cb * 16 + lr) * wsv +
+                                                     kb * 32 + lk * 8);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x),
+                                                   __builtin_bit_cast(bf16x8, w),
+                                                   acc, 0, 0, 0);
+  }
+};
+
+template <>
+struct Mma<bf16_t, 16> : MmaBf16Base<16> {
+  typedef uint2 frag_t;
+  static __device__ __forceinline__ frag_t zero() { return make_uint2(0, 0); }
+  static __device__ __forceinline__ frag_t load(const bf16_t *p) {
+    return *reinterpret_cast<const uint2 *>(p);
+  }
+  static __device__ __forceinline__ int k_of_lane(int lk) { return lk * 4; }
+  static __device__ __forceinline__ floatx4 mma(floatx4 acc, const bf16_t *tile, int wsv,
+                                                int kb, int cb, int lr, int lk,
+                                                const frag_t &x) {
+    const uint2 w = *reinterpret_cast<const uint2 *>(tile + (cb * 16 + lr) * wsv +
+                                                     kb * 16 + lk * 4);
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(shortx4, x),
+                                                     __builtin_bit_cast(shortx4, w),
+                                                     acc, 0, 0, 0);
   }
 };
 
@@ -91,76 +252,86 @@ __device__ __forceinline__ bool locate_chunk(const int32_t *__restrict__ tp,
   return true;
 }
 
-// ---- fp32 ----------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void segment_mm_f32_kernel(
-    const int32_t *__restrict__ tp, int n_types, const float *__restrict__ X,
-    const float *__restrict__ W, float *__restrict__ Y, int heads, int K, int M,
-    int KB, int MB, int chunk_rows) {
-  typedef MmTraits<float> Tr;
-  extern __shared__ __attribute__((aligned(16))) float ldsw[];
+// CG = 16-column blocks accumulated per pass (compile time, so accumulators
+// stay in registers); passes repeat when the tile is wider.
+template <typename T, int KBLK, int CG>
+__global__ __launch_bounds__(kBlock) void segment_mm_kernel(
+    const int32_t *__restrict__ tp, const T *__restrict__ X,
+    const T *__restrict__ W, T *__restrict__ Y, MmGeom g) {
+  typedef Mma<T, KBLK> MM;
+  typedef typename MM::frag_t frag_t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T *tile = reinterpret_cast<T *>(lds_raw);
   int type, row0, row1;
-  if (!locate_chunk(tp, n_types, chunk_rows, type, row0, row1)) return;
-
-  const int ws = Tr::w_stride(KB, MB);
-  const int kpad = KB * 16, mpad = MB * 16;
-  // weights of this type, all heads: ldsw[h][k][m], zero padded
-  for (int i = threadIdx.x; i < heads * kpad * mpad; i += kBlock) {
-    const int m = i % mpad;
-    const int k = (i / mpad) % kpad;
-    const int h = i / (mpad * kpad);
-    float v = 0.0f;
-    if (k < K && m < M) v = W[(((int64_t)type * heads + h) * K + k) * M + m];
-    ldsw[(h * kpad + k) * ws + m] = v;
-  }
+  if (!locate_chunk(tp, g.n_types, g.chunk_rows, type, row0, row1)) return;
+  MM::stage(W + (int64_t)type * g.w_type_stride, tile, g);
   __syncthreads();
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  const int lr = lane & 15;   // row inside the tile / column inside a block
-  const int lk = lane >> 4;   // k slot (0..3)
-  const int64_t ldx = (int64_t)heads * K, ldy = (int64_t)heads * M;
-  const bool vec_store = (M & 3) == 0;
+  const int lr = lane & 15;   // X row inside the tile (loads) / column (results)
+  const int lk = lane >> 4;   // k slot (loads) / row quad (results)
+  const int wsv = MM::ws(g.KB, g.MB);
+  const int klane = MM::k_of_lane(lk);
+  const int mb_pad = MM::mb_pad(g.MB);
 
   for (int tile0 = row0 + wave * kTileRows; tile0 < row1; tile0 += kTileBlock) {
-    const int row = tile0 + lr;
-    const bool live = row < row1;
-    for (int h = 0; h < heads; ++h) {
-      const float *xrow = X + (int64_t)row * ldx + (int64_t)h * K;
-      const float *wh = ldsw + h * kpad * ws;
-      for (int cg = 0; cg < MB; cg += Tr::kColGroup) {
-        floatx4 acc[Tr::kColGroup];
+    const T *xrow = X + (int64_t)(tile0 + lr) * g.ldx;
+    const bool xlive = tile0 + lr < row1;
+    for (int cg = 0; cg < mb_pad; cg += CG) {
+      floatx4 acc[CG];
 #pragma unroll
-        for (int cb = 0; cb < Tr::kColGroup; ++cb) acc[cb] = floatx4{0, 0, 0, 0};
-        for (int kb = 0; kb < KB; ++kb) {
-          const int k0 = kb * 16 + lk * 4;
-          float4 xa = make_float4(0, 0, 0, 0);
-          if (live && k0 < K) xa = *reinterpret_cast<const float4 *>(xrow + k0);
-          const float xv[4] = {xa.x, xa.y, xa.z, xa.w};
+      for (int cb = 0; cb < CG; ++cb) acc[cb] = floatx4{0, 0, 0, 0};
+      // k blocks that meet a non-zero part of these columns (heads on the
+      // diagonal); everything when there is one head
+      int kb_lo = 0, kb_hi = g.KB - 1;
+      if (g.hb > 1) {
+        const int c_lo = cg * 16, c_hi = min((cg + CG) * 16, g.Mt) - 1;
+        kb_lo = ((c_lo / g.M) * g.K) / KBLK;
+        kb_hi = min(((c_hi / g.M + 1) * g.K - 1) / KBLK, g.KB - 1);
+      }
+      for (int kc = kb_lo; kc <= kb_hi; kc += kMaxFrags) {
+        frag_t xa[kMaxFrags];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float *wk = wh + (k0 + q) * ws + lr;
+        for (int f = 0; f < kMaxFrags; ++f) {
+          const int k0 = (kc + f) * KBLK + klane;
+          xa[f] = MM::zero();
+          if (xlive && kc + f <= kb_hi && k0 < g.Kt) xa[f] = MM::load(xrow + k0);
+        }
 #pragma unroll
-            for (int cb = 0; cb < Tr::kColGroup; ++cb) {
-              if (cg + cb < MB)
-                acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                    wk[(cg + cb) * 16], xv[q], acc[cb], 0, 0, 0);
-            }
+        for (int f = 0; f < kMaxFrags; ++f) {
+          if (kc + f <= kb_hi) {
+#pragma unroll
+            for (int cb = 0; cb < CG; ++cb)
+              if (cg + cb < mb_pad)
+                acc[cb] = MM::mma(acc[cb], tile, wsv, kc + f, cg + cb, lr, lk, xa[f]);
           }
         }
-        if (live) {
-          float *yrow = Y + (int64_t)row * ldy + (int64_t)h * M;
+      }
+      // lane holds rows tile0 + 4*lk + r, column lr of every block
 #pragma unroll
-          for (int cb = 0; cb < Tr::kColGroup; ++cb) {
-            const int m0 = (cg + cb) * 16 + lk * 4;
-            if (cg + cb < MB && m0 < M) {
-              if (vec_store) {
-                *reinterpret_cast<float4 *>(yrow + m0) =
-                    make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
+      for (int r = 0; r < 4; ++r) {
+        const int row = tile0 + lk * 4 + r;
+        if (row < row1) {
+          T *yrow = Y + (int64_t)row * g.ldy;
+          if (MM::kPaired) {
+#pragma unroll
+            for (int cb = 0; cb < CG; cb += 2) {
+              const int m = tile_col<true>(cg + cb, lr);   // even column
+              if (m + 1 < g.Mt && (g.Mt & 1) == 0) {
+                *reinterpret_cast<uint32_t *>(yrow + m) =
+                    pack_bf16(acc[cb][r], acc[cb + 1 < CG ? cb + 1 : cb][r]);
               } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                  if (m0 + r < M) yrow[m0 + r] = acc[cb][r];
+                if (m < g.Mt) yrow[m] = (T)f32_to_bf16_bits(acc[cb][r]);
+                if (m + 1 < g.Mt && cb + 1 < CG)
+                  yrow[m + 1] = (T)f32_to_bf16_bits(acc[cb + 1][r]);
               }
+            }
+          } else {
+#pragma unroll
+            for (int cb = 0; cb < CG; ++cb) {
+              const int m = (cg + cb) * 16 + lr;
+              if (m < g.Mt) yrow[m] = acc[cb][r];
             }
           }
         }
@@ -169,80 +340,138 @@ __global__ __launch_bounds__(kBlock) void segment_mm_f32_kernel(
   }
 }
 
-// ---- bf16 ----------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void segment_mm_bf16_kernel(
-    const int32_t *__restrict__ tp, int n_types, const bf16_t *__restrict__ X,
-    const bf16_t *__restrict__ W, bf16_t *__restrict__ Y, int heads, int K, int M,
-    int KB, int MB, int chunk_rows) {
-  typedef MmTraits<bf16_t> Tr;
-  extern __shared__ __attribute__((aligned(16))) float ldsw_raw[];
-  bf16_t *ldsw = reinterpret_cast<bf16_t *>(ldsw_raw);
-  int type, row0, row1;
-  if (!locate_chunk(tp, n_types, chunk_rows, type, row0, row1)) return;
+// ---- exact-shape kernel ------------------------------------------------------
+// NF = k blocks and CG = 16-column blocks of the tile, both compile-time (the
+// tile is zero padded up to them), so the LDS layout, every LDS / global offset
+// and the accumulator set are static and the loop body is straight-line code:
+// NF wide loads, NF*CG MFMAs, 4*CG coalesced stores.
+template <typename T, int KBLK, int NF, int CG>
+struct Tight;
 
-  const int ws = Tr::w_stride(KB, MB);
-  const int kpad = KB * 32, mpad = MB * 16;
-  // weights of this type, all heads, transposed: ldsw[h][m][k], zero padded
-  for (int i = threadIdx.x; i < heads * kpad * mpad; i += kBlock) {
-    const int m = i % mpad;
-    const int k = (i / mpad) % kpad;
-    const int h = i / (mpad * kpad);
-    bf16_t v = 0;
-    if (k < K && m < M) v = W[(((int64_t)type * heads + h) * K + k) * M + m];
-    ldsw[(h * mpad + m) * ws + k] = v;
+template <int NF, int CG>
+struct Tight<float, 16, NF, CG> {
+  static constexpr int kWs = CG * 16 + 4;
+  static constexpr int kTileElems = NF * 16 * kWs;
+  static __device__ __forceinline__ floatx4 mma(floatx4 acc, const float *wl, int f,
+                                                int cb, const float4 &x) {
+    const float *w = wl + f * 16 * kWs + cb * 16;   // wl = tile + lk*4*kWs + lr
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x.x, w[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x.y, w[kWs], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x.z, w[2 * kWs], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x.w, w[3 * kWs], acc, 0, 0, 0);
+    return acc;
   }
+  static __device__ __forceinline__ const float *lane_base(const float *tile, int lr, int lk) {
+    return tile + lk * 4 * kWs + lr;
+  }
+};
+
+template <int NF, int CG>
+struct Tight<bf16_t, 32, NF, CG> {
+  static constexpr int kWs = NF * 32 + 8;
+  static constexpr int kTileElems = CG * 16 * kWs;
+  static __device__ __forceinline__ floatx4 mma(floatx4 acc, const bf16_t *wl, int f,
+                                                int cb, const uint4 &x) {
+    const uint4 w = *reinterpret_cast<const uint4 *>(wl + cb * 16 * kWs + f * 32);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x),
+                                                   __builtin_bit_cast(bf16x8, w),
+                                                   acc, 0, 0, 0);
+  }
+  static __device__ __forceinline__ const bf16_t *lane_base(const bf16_t *tile, int lr, int lk) {
+    return tile + lr * kWs + lk * 8;   // wl = tile + lr*kWs + lk*8
+  }
+};
+
+template <typename T, int KBLK, int NF, int CG>
+__global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
+    const int32_t *__restrict__ tp, const T *__restrict__ X,
+    const T *__restrict__ W, T *__restrict__ Y, MmGeom g) {
+  typedef Mma<T, KBLK> MM;
+  typedef Tight<T, KBLK, NF, CG> TT;
+  typedef typename MM::frag_t frag_t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T *tile = reinterpret_cast<T *>(lds_raw);
+  int type, row0, row1;
+  if (!locate_chunk(tp, g.n_types, g.chunk_rows, type, row0, row1)) return;
+  MM::stage(W + (int64_t)type * g.w_type_stride, tile, g);   // g.KB == NF, g.MB == CG
   __syncthreads();
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int lr = lane & 15;
   const int lk = lane >> 4;
-  const int64_t ldx = (int64_t)heads * K, ldy = (int64_t)heads * M;
-  const bool vec_store = (M & 3) == 0;
+  const int klane = MM::k_of_lane(lk);
+  const T *wl = TT::lane_base(tile, lr, lk);
 
-  for (int tile0 = row0 + wave * kTileRows; tile0 < row1; tile0 += kTileBlock) {
-    const int row = tile0 + lr;
-    const bool live = row < row1;
-    for (int h = 0; h < heads; ++h) {
-      const bf16_t *xrow = X + (int64_t)row * ldx + (int64_t)h * K;
-      const bf16_t *wh = ldsw + h * mpad * ws;
-      for (int cg = 0; cg < MB; cg += Tr::kColGroup) {
-        floatx4 acc[Tr::kColGroup];
+  // k fragments of this lane that lie inside the row
+  unsigned kmask = 0;
 #pragma unroll
-        for (int cb = 0; cb < Tr::kColGroup; ++cb) acc[cb] = floatx4{0, 0, 0, 0};
-        for (int kb = 0; kb < KB; ++kb) {
-          const int k0 = kb * 32 + lk * 8;
-          uint4 xa = make_uint4(0, 0, 0, 0);
-          if (live && k0 < K) xa = *reinterpret_cast<const uint4 *>(xrow + k0);
-          const bf16x8 xv = __builtin_bit_cast(bf16x8, xa);
+  for (int f = 0; f < NF; ++f)
+    if (f * KBLK + klane < g.Kt) kmask |= 1u << f;
+  const bool full_cols = g.Mt == CG * 16;
+  const bool pack_ok = (g.Mt & 1) == 0 && (g.ldy & 1) == 0;
+
+  const T *xp = X + (int64_t)(row0 + wave * kTileRows + lr) * g.ldx + klane;
+  T *yp = Y + (int64_t)(row0 + wave * kTileRows + lk * 4) * g.ldy +
+          (MM::kPaired ? 2 * lr : lr);
+  const int64_t xstep = (int64_t)kTileBlock * g.ldx, ystep = (int64_t)kTileBlock * g.ldy;
+
+  // fragments of the next tile are requested before the current tile's MFMAs
+  frag_t xn[NF];
+  {
+    const bool xlive = row0 + wave * kTileRows + lr < row1;
 #pragma unroll
-          for (int cb = 0; cb < Tr::kColGroup; ++cb) {
-            if (cg + cb < MB) {
-              const uint4 wa = *reinterpret_cast<const uint4 *>(
-                  wh + ((cg + cb) * 16 + lr) * ws + k0);
-              acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  __builtin_bit_cast(bf16x8, wa), xv, acc[cb], 0, 0, 0);
+    for (int f = 0; f < NF; ++f) {
+      xn[f] = MM::zero();
+      if (xlive && (kmask >> f & 1)) xn[f] = MM::load(xp + f * KBLK);
+    }
+  }
+  for (int tile0 = row0 + wave * kTileRows; tile0 < row1;
+       tile0 += kTileBlock, yp += ystep) {
+    // With many weight fragments the compiler would otherwise keep them all in
+    // registers across tiles (one wave per SIMD); re-reading them from LDS per
+    // tile is cheap, so forbid hoisting past this point.
+    if (NF * CG * (int)(sizeof(frag_t) / 4) > 32) asm volatile("" ::: "memory");
+    frag_t xa[NF];
+#pragma unroll
+    for (int f = 0; f < NF; ++f) xa[f] = xn[f];
+    xp += xstep;
+    const bool xlive = tile0 + kTileBlock + lr < row1;
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      xn[f] = MM::zero();
+      if (xlive && (kmask >> f & 1)) xn[f] = MM::load(xp + f * KBLK);
+    }
+    floatx4 acc[CG];
+#pragma unroll
+    for (int cb = 0; cb < CG; ++cb) acc[cb] = floatx4{0, 0, 0, 0};
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+#pragma unroll
+      for (int cb = 0; cb < CG; ++cb)
+        acc[cb] = TT::mma(acc[cb], wl, f, cb, xa[f]);
+    }
+    // lane holds rows tile0 + 4*lk + r, lane column lr of every column block
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (tile0 + lk * 4 + r < row1) {
+        T *yrow = yp + (int64_t)r * g.ldy;
+        if (MM::kPaired) {
+#pragma unroll
+          for (int cb = 0; cb < CG; cb += 2) {
+            const int m = (cb >> 1) * 32 + 2 * lr;
+            if (pack_ok && (full_cols || m + 1 < g.Mt)) {
+              *reinterpret_cast<uint32_t *>(yrow + (cb >> 1) * 32) =
+                  pack_bf16(acc[cb][r], acc[cb + 1][r]);
+            } else {
+              if (m < g.Mt) yrow[(cb >> 1) * 32] = (T)f32_to_bf16_bits(acc[cb][r]);
+              if (m + 1 < g.Mt) yrow[(cb >> 1) * 32 + 1] = (T)f32_to_bf16_bits(acc[cb + 1][r]);
             }
           }
-        }
-        if (live) {
-          bf16_t *yrow = Y + (int64_t)row * ldy + (int64_t)h * M;
+        } else {
 #pragma unroll
-          for (int cb = 0; cb < Tr::kColGroup; ++cb) {
-            const int m0 = (cg + cb) * 16 + lk * 4;
-            if (cg + cb < MB && m0 < M) {
-              if (vec_store) {
-                uint2 o;
-                o.x = pack_bf16(acc[cb][0], acc[cb][1]);
-                o.y = pack_bf16(acc[cb][2], acc[cb][3]);
-                *reinterpret_cast<uint2 *>(yrow + m0) = o;
-              } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                  if (m0 + r < M) yrow[m0 + r] = (bf16_t)f32_to_bf16_bits(acc[cb][r]);
-              }
-            }
-          }
+          for (int cb = 0; cb < CG; ++cb)
+            if (full_cols || cb * 16 + lr < g.Mt) yrow[cb * 16] = acc[cb][r];
         }
       }
     }
@@ -282,6 +511,123 @@ __global__ __launch_bounds__(kBlock) void segment_mm_scalar_kernel(
   stf(Y + i, s);
 }
 
+template <typename T, int KBLK, int CG>
+void launch_cg(const int32_t *tp, const T *X, const T *W, T *Y, const MmGeom &g,
+               int64_t grid, size_t lds, hipStream_t s) {
+  hipLaunchKernelGGL((segment_mm_kernel<T, KBLK, CG>), dim3((unsigned)grid),
+                     dim3(kBlock), lds, s, tp, X, W, Y, g);
+}
+
+template <typename T, int KBLK, int NF, int CG>
+int launch_tight(const int32_t *tp, const T *X, const T *W, T *Y, MmGeom g,
+                 int64_t grid, hipStream_t s) {
+  typedef Tight<T, KBLK, NF, CG> TT;
+  const size_t lds = (size_t)TT::kTileElems * sizeof(T);
+  if (!allow_lds((const void *)segment_mm_tight_kernel<T, KBLK, NF, CG>, lds))
+    return GA_EUNSUPPORTED;
+  g.KB = NF;   // the tile is padded to the compile-time shape
+  g.MB = CG;
+  hipLaunchKernelGGL((segment_mm_tight_kernel<T, KBLK, NF, CG>),
+                     dim3((unsigned)grid), dim3(kBlock), lds, s, tp, X, W, Y, g);
+  return launch_status();
+}
+
+template <typename T, int KBLK, int NF>
+int pick_tight_cg(int cg, const int32_t *tp, const T *X, const T *W, T *Y,
+                  const MmGeom &g, int64_t grid, hipStream_t s) {
+  switch (cg) {
+    case 1: return launch_tight<T, KBLK, NF, Mma<T, KBLK>::kPaired ? 2 : 1>(tp, X, W, Y, g, grid, s);
+    case 2: return launch_tight<T, KBLK, NF, 2>(tp, X, W, Y, g, grid, s);
+    case 4: return launch_tight<T, KBLK, NF, 4>(tp, X, W, Y, g, grid, s);
+    default: return launch_tight<T, KBLK, NF, 8>(tp, X, W, Y, g, grid, s);
+  }
+}
+
+template <typename T, int KBLK>
+int pick_tight(int nf, int cg, const int32_t *tp, const T *X, const T *W, T *Y,
+               const MmGeom &g, int64_t grid, hipStream_t s) {
+  switch (nf) {
+    case 1: return pick_tight_cg<T, KBLK, 1>(cg, tp, X, W, Y, g, grid, s);
+    case 2: return pick_tight_cg<T, KBLK, 2>(cg, tp, X, W, Y, g, grid, s);
+    case 4: return pick_tight_cg<T, KBLK, 4>(cg, tp, X, W, Y, g, grid, s);
+    default: return pick_tight_cg<T, KBLK, 8>(cg, tp, X, W, Y, g, grid, s);
+  }
+}
+
+inline int pow2_ceil_int(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+// One launch for `hb` folded heads starting at head h0.
+template <typename T, int KBLK>
+int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
+                int64_t rows, int heads, int K, int M, int h0, int hb,
+                hipStream_t s) {
+  typedef Mma<T, KBLK> MM;
+  MmGeom g;
+  g.n_types = n_types;
+  g.K = K; g.M = M; g.hb = hb;
+  g.Kt = hb * K; g.Mt = hb * M;
+  g.KB = (g.Kt + KBLK - 1) / KBLK;
+  g.MB = (g.Mt + 15) / 16;
+  g.ldx = (int64_t)heads * K;
+  g.ldy = (int64_t)heads * M;
+  g.w_type_stride = (int64_t)heads * K * M;
+  // rows per workgroup: a multiple of the 64-row step, large enough to
+  // amortise the weight staging, small enough to keep every CU busy
+  int64_t steps = rows / (kTileBlock * 2048);
+  if (steps < 1) steps = 1;
+  if (steps > 16) steps = 16;
+  g.chunk_rows = (int)steps * kTileBlock;
+  const int64_t grid = (rows + g.chunk_rows - 1) / g.chunk_rows + n_types;
+  if (grid > 0x7fffffff) return GA_EUNSUPPORTED;
+  const T *Xh = X + (int64_t)h0 * K;
+  const T *Wh = W + (int64_t)h0 * K * M;
+  T *Yh = Y + (int64_t)h0 * M;
+  if (KBLK != 16 || sizeof(T) == 4) {   // exact-shape kernels: fp32 and bf16 x32
+    if (g.KB <= 8 && g.MB <= 8) {
+      const int rc = pick_tight<T, (sizeof(T) == 4 ? 16 : 32)>(
+          pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), tp, Xh, Wh, Yh, g, grid, s);
+      if (rc != GA_EUNSUPPORTED) return rc;
+    }
+  }
+  const size_t lds = (size_t)MM::tile_elems(g.KB, g.MB) * sizeof(T);
+  if (lds > (size_t)kMaxLds) return GA_EUNSUPPORTED;
+  const int mbp = MM::mb_pad(g.MB);
+  if (MM::kPaired) {
+    if (mbp <= 2) launch_cg<T, KBLK, 2>(tp, Xh, Wh, Yh, g, grid, lds, s);
+    else if (mbp <= 4) launch_cg<T, KBLK, 4>(tp, Xh, Wh, Yh, g, grid, lds, s);
+    else launch_cg<T, KBLK, 8>(tp, Xh, Wh, Yh, g, grid, lds, s);
+  } else {
+    if (mbp <= 1) launch_cg<T, KBLK, 1>(tp, Xh, Wh, Yh, g, grid, lds, s);
+    else if (mbp <= 2) launch_cg<T, KBLK, 2>(tp, Xh, Wh, Yh, g, grid, lds, s);
+    else launch_cg<T, KBLK, 4>(tp, Xh, Wh, Yh, g, grid, lds, s);
+  }
+  return launch_status();
+}
+
+template <typename T, int KBLK>
+int launch_mfma(const int32_t *tp, int n_types, const void *X, const void *W,
+                void *Y, int64_t rows, int heads, int K, int M, hipStream_t s) {
+  // all heads folded into one block-diagonal tile when that fits the LDS and
+  // the fragment budget; otherwise one launch per head
+  if (heads > 1) {
+    int rc = GA_EUNSUPPORTED;
+    if ((int64_t)heads * K <= kMaxFrags * KBLK)
+      rc = launch_fold<T, KBLK>(tp, n_types, (const T *)X, (const T *)W, (T *)Y,
+                                rows, heads, K, M, 0, heads, s);
+    if (rc != GA_EUNSUPPORTED) return rc;
+  }
+  for (int h = 0; h < heads; ++h) {
+    const int rc = launch_fold<T, KBLK>(tp, n_types, (const T *)X, (const T *)W,
+                                        (T *)Y, rows, heads, K, M, h, 1, s);
+    if (rc != GA_OK) return rc;
+  }
+  return GA_OK;
+}
+
 }  // namespace
 }  // namespace ga
 
@@ -301,34 +647,21 @@ extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
   if (!aligned(X, esz) || !aligned(W, esz) || !aligned(Y, esz)) return GA_EALIGN;
   hipStream_t s = (hipStream_t)stream;
 
-  const int kblk = dtype == GA_F32 ? 16 : 32;
-  const int vec = dtype == GA_F32 ? 4 : 8;
-  const int KB = (int)((K + kblk - 1) / kblk), MB = (int)((M + 15) / 16);
-  const size_t lds = dtype == GA_F32 ? MmTraits<float>::lds_bytes((int)heads, KB, MB)
-                                     : MmTraits<bf16_t>::lds_bytes((int)heads, KB, MB);
-  const bool mfma_ok = K % vec == 0 && aligned(X, 16) && aligned(Y, 16) &&
-                       lds <= (size_t)kMaxLds;
-  if (mfma_ok) {
-    // rows per workgroup: a multiple of the 64-row step, large enough to
-    // amortise the weight load, small enough to keep every CU busy
-    int64_t steps = rows / (kTileBlock * 1024);
-    if (steps < 1) steps = 1;
-    if (steps > 16) steps = 16;
-    const int chunk_rows = (int)steps * kTileBlock;
-    const int64_t grid = (rows + chunk_rows - 1) / chunk_rows + n_types;
-    if (grid > 0x7fffffff) return GA_EUNSUPPORTED;
-    if (dtype == GA_F32)
-      hipLaunchKernelGGL(segment_mm_f32_kernel, dim3((unsigned)grid), dim3(kBlock),
-                         lds, s, type_pointer, (int)n_types, (const float *)X,
-                         (const float *)W, (float *)Y, (int)heads, (int)K, (int)M,
-                         KB, MB, chunk_rows);
-    else
-      hipLaunchKernelGGL(segment_mm_bf16_kernel, dim3((unsigned)grid), dim3(kBlock),
-                         lds, s, type_pointer, (int)n_types, (const bf16_t *)X,
-                         (const bf16_t *)W, (bf16_t *)Y, (int)heads, (int)K, (int)M,
-                         KB, MB, chunk_rows);
-    return launch_status();
+  int rc = GA_EUNSUPPORTED;
+  if (aligned(X, 16) && aligned(Y, 16)) {
+    if (dtype == GA_F32 && K % 4 == 0)
+      rc = launch_mfma<float, 16>(type_pointer, (int)n_types, X, W, Y, rows,
+                                  (int)heads, (int)K, (int)M, s);
+    else if (dtype == GA_BF16 && K % 8 == 0)
+      rc = launch_mfma<bf16_t, 32>(type_pointer, (int)n_types, X, W, Y, rows,
+                                   (int)heads, (int)K, (int)M, s);
+    else if (dtype == GA_BF16 && K % 4 == 0)
+      rc = launch_mfma<bf16_t, 16>(type_pointer, (int)n_types, X, W, Y, rows,
+                                   (int)heads, (int)K, (int)M, s);
   }
+  if (rc != GA_EUNSUPPORTED) return rc;
+
+  // shapes the MFMA path does not take (odd K, weights beyond the LDS budget)
   const int64_t total = rows * heads * M;
   const int64_t blocks = (total + kBlock - 1) / kBlock;
   if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
