@@ -73,3 +73,38 @@ def rgcn_layer(g: DGLGraph, h, weight, norm):
     msg = ops.SegmentMMEdge(hs, weight, g)
     msg = msg * norm.to(msg.dtype)
     return ops.SpMMEdge(msg, [1], False, None, g)
+
+
+def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
+              relation_att, relation_msg, relation_pri, skip, heads: int = 1):
+    """examples/HGT/HGT.py:28-60 as the operator sequence of its optimised plan,
+    generalised from one head to ``heads`` heads of width D = hidden / heads:
+
+      K, V, Q   = SegmentMMNode(h, W_k | W_v | W_q)            per node type
+      k_e, v_e  = BroadcastSrcNode(K | V);  q_e = BroadcastDstNode(Q)
+      k_e, v_e  = SegmentMMEdge(k_e, relation_att | relation_msg)   per edge type,
+                                                         one (D x D) block per head
+      attn      = sum_D(k_e * q_e) * BroadcastEdgeType(relation_pri) / sqrt(D)
+      t         = SpMMEdge(SegmentSoftmax(attn) * v_e)
+      out       = SegmentMMNode(t, W_a) * sigmoid(BroadcastNodeType(skip))
+
+    k/q/v/a_weight: (T_n, hidden, hidden); relation_att / relation_msg:
+    (T_e, heads, D, D); relation_pri: (T_e, heads); skip: (T_n,).
+    """
+    n, hidden = h.shape
+    d = hidden // heads
+    e = g.num_edges
+    k = ops.SegmentMMNode(h, k_weight, g)
+    v = ops.SegmentMMNode(h, v_weight, g)
+    q = ops.SegmentMMNode(h, q_weight, g)
+    k_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(k, g), relation_att, g)
+    v_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(v, g), relation_msg, g)
+    q_e = ops.BroadcastDstNode(q, g)
+    attn = (k_e.view(e, heads, d).float() * q_e.view(e, heads, d).float()).sum(-1)
+    attn = attn * ops.BroadcastEdgeType(relation_pri.float(), g) / (d ** 0.5)
+    a = ops.SegmentSoftmax(attn.contiguous(), 1, None, g)          # (E, heads) fp32
+    m = (v_e.view(e, heads, d).float() * a.unsqueeze(-1)).to(h.dtype).view(e, hidden)
+    t = ops.SpMMEdge(m, [1], False, None, g)
+    alpha = torch.sigmoid(ops.BroadcastNodeType(skip.float().unsqueeze(1), g))
+    out = ops.SegmentMMNode(t, a_weight, g)
+    return (out.float() * alpha).to(h.dtype)

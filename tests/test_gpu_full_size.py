@@ -1,0 +1,145 @@
+"""Parity at the benchmark configurations' full sizes.
+
+Configs 2-4 are small enough for the C oracle to evaluate completely; config 5
+(64 M edges x 256 features) is checked on every row of a seeded sample (the
+oracle runs on the sub-adjacency of the sampled destinations, including the
+highest-degree row) and through size-independent properties: the column sums
+of an SpMM equal the sums of its messages, and every softmax segment sums to 1.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from graphiler_amd import datasets, layers, ops, prepare_graph
+from helpers import TOL_BF16, TOL_F32, assert_close, to_bf16_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(a, device, bf16=False):
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    return t.to(torch.bfloat16) if bf16 else t
+
+
+def _host(g):
+    return (g.in_pointer.cpu().numpy(), g.in_node_indices.cpu().numpy(),
+            g.in_edge_indices.cpu().numpy())
+
+
+def test_config2_gat_full(device):
+    wl = datasets.gat_rmat()                     # N=232,965  E=11.6 M
+    n, e = wl.num_nodes, wl.num_edges
+    g = prepare_graph(wl.src, wl.dst, n, device=device)
+    ptr, nbr, eid = _host(g)
+    assert g.in_eid_is_identity and np.array_equal(eid, np.arange(e, dtype=np.int32))
+    rng = np.random.default_rng(1)
+    z = rng.standard_normal((n, 64), dtype=np.float32)
+    el = rng.standard_normal((n, 1), dtype=np.float32)
+    er = rng.standard_normal((n, 1), dtype=np.float32)
+    dz, dl, dr = _t(z, device), _t(el, device), _t(er, device)
+    ref = oracle.gat_aggregate(ptr, nbr, el, er, z, heads=1, slope=0.2)
+    assert_close(ops.gat_aggregate(dl, dr, dz, g, 0.2).cpu().numpy(), ref, TOL_F32,
+                 "config 2 fused GAT")
+    logits = ops.gsddmm_u_add_v_mul_alpha(dl, dr, 1, g)
+    assert np.array_equal(logits.cpu().numpy(),
+                          oracle.sddmm_u_add_v(wl.src, wl.dst, el, er))
+    att = ops.SegmentSoftmax(torch.nn.functional.leaky_relu(logits, 0.2), 1, None, g)
+    out = ops.gspmm_src_mul_e_sum(dz, att, [1], False, None, g)
+    assert_close(out.cpu().numpy(), ref, TOL_F32, "config 2 four-operator plan")
+    # max over in-edges, bit-exact (values are copies)
+    got = ops.spmm(g, "copy_u", "max", dz).cpu().numpy()
+    assert np.array_equal(got, oracle.spmm(ptr, nbr, eid, z, op="copy_u", reduce="max"))
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_config3_rgcn_full(device, bf16):
+    wl = datasets.rgcn_zipf()                    # N=100k  E=1M  R=60
+    n = wl.num_nodes
+    g = prepare_graph(wl.src, wl.dst, n, device=device, etype_of=wl.etype,
+                      num_etypes=60)
+    ptr, nbr, eid = _host(g)
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((n, 16), dtype=np.float32)
+    w1 = datasets.glorot(rng, (60, 16, 64))
+    if bf16:
+        x, w1 = to_bf16_f32(x), to_bf16_f32(w1)
+    deg = np.maximum(np.bincount(wl.dst, minlength=n), 1)
+    norm = (1.0 / deg[wl.dst]).astype(np.float32)[:, None]
+    got = layers.rgcn_layer(g, _t(x, device, bf16), _t(w1, device, bf16), _t(norm, device))
+    etp = oracle.type_pointer(wl.etype, 60)
+    msg = oracle.segment_mm(etp, oracle.gather_rows(wl.src, x), w1) * norm
+    ref = oracle.spmm(ptr, nbr, eid, msg.astype(np.float32), op="copy_e")
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else 2 * TOL_F32,
+                 "config 3 RGCN layer")
+
+
+def test_config4_hgt_operators_full(device):
+    wl = datasets.hgt_hetero()                   # N=100k  E=2M  8 heads x 16
+    n, e, heads, d = wl.num_nodes, wl.num_edges, 8, 16
+    g = prepare_graph(wl.src, wl.dst, n, device=device, ntype_of=wl.ntype,
+                      num_ntypes=4, etype_of=wl.etype, num_etypes=10)
+    ptr, nbr, eid = _host(g)
+    rng = np.random.default_rng(3)
+    h = to_bf16_f32(rng.standard_normal((n, 128), dtype=np.float32))
+    wq = to_bf16_f32(datasets.glorot(rng, (4, 128, 128)))
+    q = ops.SegmentMMNode(_t(h, device, True), _t(wq, device, True), g)
+    q_ref = oracle.segment_mm(oracle.type_pointer(wl.ntype, 4), h, wq)
+    assert_close(q.float().cpu().numpy(), q_ref, TOL_BF16, "config 4 Q projection")
+    ke = to_bf16_f32(rng.standard_normal((e, 128), dtype=np.float32))
+    ratt = to_bf16_f32(datasets.glorot(rng, (10, heads, d, d)))
+    got = ops.SegmentMMEdge(_t(ke, device, True), _t(ratt, device, True), g)
+    ref = oracle.segment_mm(oracle.type_pointer(wl.etype, 10), ke, ratt, heads=heads)
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16, "config 4 relation transform")
+    k3 = h.reshape(n, heads, d)
+    dot = ops.gsddmm_u_dot_v(_t(k3, device, True), _t(k3, device, True), g)
+    assert_close(dot.cpu().numpy(), oracle.sddmm_u_dot_v(wl.src, wl.dst, k3, k3),
+                 TOL_F32, "config 4 u_dot_v")
+    logits = (rng.standard_normal((e, heads)) * 3).astype(np.float32)
+    att = ops.SegmentSoftmax(_t(logits, device), 1, None, g)
+    att_ref = oracle.segment_softmax(ptr, eid, logits)
+    assert_close(att.cpu().numpy(), att_ref, TOL_F32, "config 4 softmax")
+    out = ops.gspmm_src_mul_e_sum(_t(h, device, True), att, [1], False, None, g)
+    ref = oracle.spmm(ptr, nbr, eid, h, att_ref, op="u_mul_e", heads=heads)
+    assert_close(out.float().cpu().numpy(), ref, TOL_BF16, "config 4 u_mul_e")
+
+
+@pytest.mark.timeout(400)
+def test_config5_large_gat_sampled_and_properties(device):
+    wl = datasets.gat_rmat_large()               # N=2,449,029  E=64,308,169
+    n, e, heads, d = wl.num_nodes, wl.num_edges, 4, 64
+    assert e == 61_859_140 + n
+    deg = np.bincount(wl.dst, minlength=n)
+    assert deg.max() > 10_000, "config 5 must exercise long segments"
+    g = prepare_graph(wl.src, wl.dst, n, device=device)
+    ptr = g.in_pointer.cpu().numpy()
+    # index work is bit-exact: pointer = running sum of in-degrees, rows sorted
+    assert np.array_equal(np.diff(ptr), deg)
+    assert np.array_equal(g.in_node_indices.cpu().numpy(), wl.src.astype(np.int32))
+    rows_dev = g.in_row_of_slot
+    assert torch.equal(rows_dev.long(), _t(wl.dst, device))
+    rng = np.random.default_rng(4)
+    z = to_bf16_f32(rng.standard_normal((n, heads * d), dtype=np.float32))
+    el = rng.standard_normal((n, heads), dtype=np.float32)
+    er = rng.standard_normal((n, heads), dtype=np.float32)
+    dz, dl, dr = _t(z, device, True), _t(el, device), _t(er, device)
+    out = ops.gat_aggregate(dl, dr, dz, g, 0.2).float().cpu().numpy()
+    # oracle on the sub-adjacency of sampled destinations (+ the heaviest rows)
+    sample = np.unique(np.concatenate([rng.integers(0, n, 3000),
+                                       np.argsort(deg)[-3:], [0, n - 1]]))
+    sub_ptr = np.concatenate([[0], np.cumsum(deg[sample])]).astype(np.int32)
+    sub_nbr = np.concatenate([wl.src[ptr[v]:ptr[v + 1]] for v in sample]).astype(np.int32)
+    ref = oracle.gat_aggregate(sub_ptr, sub_nbr, el, er[sample], z, heads=heads, slope=0.2)
+    assert_close(out[sample], ref, TOL_BF16, "config 5 fused GAT (sampled rows)")
+    assert not out[deg == 0].any()
+    # properties over ALL rows: softmax segments sum to one; SpMM column sums
+    logits = ops.gsddmm_u_add_v_mul_alpha(dl, dr, 1, g)
+    att = ops.SegmentSoftmax(logits, 1, None, g)
+    sums = ops.SpMMEdge(att, [1], False, None, g).cpu().numpy()
+    assert np.abs(sums[deg > 0] - 1.0).max() < 1e-4
+    assert not sums[deg == 0].any()
+    x32 = torch.randn(n, 16, device=device)
+    col = ops.SpMMSrc(x32, [1], False, None, g).double().sum(0).cpu().numpy()
+    want = (x32.double() * _t(np.bincount(wl.src, minlength=n).astype(np.float64),
+                              device)[:, None]).sum(0).cpu().numpy()
+    np.testing.assert_allclose(col, want, rtol=1e-6, atol=1e-3 * np.abs(want).max())
