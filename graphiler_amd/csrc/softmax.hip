@@ -1,146 +1,391 @@
 // Edge segment softmax for gfx950 (any number of heads), fp32.
 //
-// A segment is the run of (slot, head) elements of one destination row, n =
-// degree * heads values that are contiguous in memory when edge ids are slot
-// numbers.  Power-of-two head counts (<= 64) take three size classes, each with
-// its own launch so that no lane group idles behind a long row:
-//   small   n <= 4*S      a group of S adjacent lanes per row (S from the mean
-//                         segment size), every element held in a register;
-//   medium  n <= 1024     one wavefront per row, 16 elements per lane in
-//                         registers.  Waves are not launched per row but per
-//                         chunk of 1024 elements: a wave scans the rows that
-//                         START in its chunk and takes the medium ones;
-//   long    n  > 1024     cut at multiples of 1024/heads slots, one workgroup
-//                         per chunk: pass A writes per-chunk (max, sum-exp) per
-//                         head to the workspace, pass B merges them in chunk
-//                         order and normalises.
-// Every segment is read once (small, medium) or twice (long).  Other head
-// counts use a generic lane-group kernel that runs the heads one after the
-// other.  No atomics; the order of every reduction is fixed by the sizes.
+// Power-of-two head counts (<= 64) run a chunked, load-balanced scheme: the
+// (slot, head) elements are cut into chunks of 1024 elements, one wavefront per
+// chunk whatever the degree distribution.  Lane = (slot group g, head h); a lane
+// owns 16 consecutive slots of its head, so
+//   1. segments that lie inside one lane are reduced sequentially in registers;
+//   2. segments shared by neighbouring lanes are combined with two segmented
+//      shuffle scans over the lanes of a head (rows are sorted, so equal keys at
+//      distance d imply equal keys in between);
+//   3. rows that lie inside the chunk are normalised and written at once: their
+//      logits are read exactly once;
+//   4. the (at most two) rows a chunk shares with its neighbours leave their
+//      per-head (max, sum-exp) in the workspace; a second launch merges the
+//      partials of such a row in chunk order and writes its elements.
+// Other head counts use a lane-group kernel that runs the heads one after the
+// other, with chunked two-pass handling of rows longer than 1024 slots.
+// No atomics; the order of every reduction is fixed by the graph and sizes.
 #include "common.h"
 
 namespace ga {
 namespace {
 
-constexpr int kSmallCache = 4;     // elements per lane, small rows
-constexpr int kMediumCache = 16;   // elements per lane, medium rows
-constexpr int kMediumMax = kWave * kMediumCache;   // 1024 elements
-constexpr int kChunkElems = 1024;  // elements scanned per medium-kernel wave
-constexpr int kLongRow = 1024;     // generic path: slots per long-row chunk
+constexpr int kT = 16;                    // slots per lane
+constexpr int kChunkElems = kWave * kT;   // 1024 elements per wavefront
+constexpr int kLongRow = 1024;            // generic path: slots per long-row chunk
 
-__device__ __forceinline__ int64_t elem_offset(const int32_t *__restrict__ eid,
-                                               int64_t start, int64_t q,
-                                               int head_shift) {
-  const int64_t slot = start + (q >> head_shift);
-  const int64_t e = eid ? (int64_t)eid[slot] : slot;
-  return (e << head_shift) + (q & ((1 << head_shift) - 1));
+// exp(x) as exp2(x * log2 e) with the rounding error of the product fed back
+// (x*log2e = t + r, exp2(t + r) ~ exp2(t) * (1 + r ln 2)): about 2 ulp, six
+// instructions instead of the library routine's thirty.
+__device__ __forceinline__ float exp_fast(float x) {
+  const float t = x * 1.44269502162933349609375f;
+  const float r = fmaf(x, 1.44269502162933349609375f, -t) + x * 1.925963033e-8f;
+  return __builtin_amdgcn_exp2f(t) * fmaf(r, 0.693147182464599609375f, 1.0f);
 }
 
-// ---- small rows -----------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void softmax_small_kernel(
-    const int32_t *__restrict__ pointer, const int32_t *__restrict__ eid,
-    const float *__restrict__ x, float *__restrict__ y, int64_t n_rows,
-    int head_shift, int s_shift) {
-  const int S = 1 << s_shift;
-  const int H = 1 << head_shift;
-  const int lane = threadIdx.x & (S - 1);
-  const int64_t row = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> s_shift;
-  int64_t start = 0, n = 0;
-  if (row < n_rows) {
-    start = pointer[row];
-    n = (int64_t)(pointer[row + 1] - start) << head_shift;
-    if (n > (int64_t)kSmallCache * S) n = 0;   // another class owns this row
-  }
-  float c[kSmallCache];
-  int64_t off[kSmallCache];
-  float m = -INFINITY;
-#pragma unroll
-  for (int t = 0; t < kSmallCache; ++t) {
-    const int64_t q = lane + (int64_t)t * S;   // lane keeps one head: S % H == 0
-    c[t] = -INFINITY;
-    off[t] = -1;
-    if (q < n) {
-      off[t] = elem_offset(eid, start, q, head_shift);
-      c[t] = x[off[t]];
-      m = fmaxf(m, c[t]);
-    }
-  }
-  for (int o = S >> 1; o >= H; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-  float l = 0.0f;
-#pragma unroll
-  for (int t = 0; t < kSmallCache; ++t) {
-    c[t] = off[t] >= 0 ? expf(c[t] - m) : 0.0f;
-    l += c[t];
-  }
-  for (int o = S >> 1; o >= H; o >>= 1) l += __shfl_xor(l, o);
-#pragma unroll
-  for (int t = 0; t < kSmallCache; ++t)
-    if (off[t] >= 0) y[off[t]] = c[t] / l;
+// Per-chunk partial statistics: [chunk][A|B][head][max, sum].  A = the chunk's
+// first row when it began in an earlier chunk; B = its last row when that row
+// started inside the chunk and continues in the next one.
+__device__ __forceinline__ float *stat_ptr(float *stats, int64_t chunk, int which,
+                                           int H, int h) {
+  return stats + ((chunk * 2 + which) * H + h) * 2;
 }
 
-// ---- medium rows ----------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void softmax_medium_kernel(
-    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
-    const int32_t *__restrict__ eid, const float *__restrict__ x,
-    float *__restrict__ y, int64_t n_rows, int64_t n_edges, int head_shift,
-    int small_max) {
-  const int H = 1 << head_shift;
-  const int lane = threadIdx.x & (kWave - 1);
+struct ChunkInfo {
+  int64_t c0, c1;       // slot range of the chunk
+  int row_first, row_last;
+  bool began_before;    // first row started in an earlier chunk
+  bool continues;       // last row goes on in the next chunk
+};
+
+__device__ __forceinline__ bool chunk_info(const int32_t *__restrict__ row_of_slot,
+                                           int64_t n_edges, int head_shift,
+                                           ChunkInfo &ci) {
   const int64_t chunk = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
   const int chunk_slots = kChunkElems >> head_shift;
-  const int64_t c0 = chunk * chunk_slots;
-  if (c0 >= n_edges) return;                       // whole wave
-  const int64_t c1 = min(c0 + (int64_t)chunk_slots, n_edges);
-  // first row that starts inside [c0, c1)
-  int64_t r0 = row_of_slot[c0];
-  if ((int64_t)pointer[r0] < c0) ++r0;
-  for (;; r0 += kWave) {
-    const int64_t r = r0 + lane;
-    int64_t start = n_edges, end = n_edges;
-    if (r < n_rows) {
-      start = pointer[r];
-      end = pointer[r + 1];
-    }
-    const bool starts_here = r < n_rows && start < c1;
-    const int64_t n = (end - start) << head_shift;
-    uint64_t todo = __ballot(starts_here && n > small_max && n <= kMediumMax);
-    while (todo) {
-      const int src = __ffsll((unsigned long long)todo) - 1;
-      todo &= todo - 1;
-      const int64_t rs = __shfl(start, src);
-      const int64_t rn = __shfl(n, src);
-      float c[kMediumCache];
-      int64_t off[kMediumCache];
-      float m = -INFINITY;
+  ci.c0 = chunk * chunk_slots;
+  if (ci.c0 >= n_edges) return false;
+  ci.c1 = min(ci.c0 + (int64_t)chunk_slots, n_edges);
+  ci.row_first = row_of_slot[ci.c0];
+  ci.row_last = row_of_slot[ci.c1 - 1];
+  ci.began_before = ci.c0 > 0 && row_of_slot[ci.c0 - 1] == ci.row_first;
+  ci.continues = ci.c1 < n_edges && row_of_slot[ci.c1] == ci.row_last;
+  return true;
+}
+
+// Segmented scans over the lanes of one head (lanes at distance `step`
+// multiples).  Keys ascend with the lane, so a match at distance d means every
+// lane in between holds that key only.
+template <bool IS_MAX>
+__device__ __forceinline__ float scan_up(float v, int key, int lane, int step) {
+  for (int off = step; off < kWave; off <<= 1) {
+    const int pk = __shfl_up(key, off);
+    const bool hit = lane >= off && pk == key;
+    if (!__ballot(hit)) break;   // no match at this distance: none further away
+    const float pv = __shfl_up(v, off);
+    if (hit) v = IS_MAX ? fmaxf(v, pv) : v + pv;
+  }
+  return v;
+}
+template <bool IS_MAX>
+__device__ __forceinline__ float scan_down(float v, int key, int lane, int step) {
+  for (int off = step; off < kWave; off <<= 1) {
+    const int nk = __shfl_down(key, off);
+    const bool hit = lane + off < kWave && nk == key;
+    if (!__ballot(hit)) break;
+    const float nv = __shfl_down(v, off);
+    if (hit) v = IS_MAX ? fmaxf(v, nv) : v + nv;
+  }
+  return v;
+}
+
+// Totals of a lane's first and last segment over the whole chunk, from the
+// lane-local values vf (first segment) and vl (last segment).
+template <bool IS_MAX>
+__device__ __forceinline__ void chunk_totals(float vf, float vl, int kf, int kl,
+                                             int lane, int H, float &tf, float &tl) {
+  const float P = scan_up<IS_MAX>(vl, kl, lane, H);     // lanes <= me, key kl
+  const float S = scan_down<IS_MAX>(vf, kf, lane, H);   // lanes >= me, key kf
+  const int pk = __shfl_up(kl, H);
+  const float pP = __shfl_up(P, H);
+  const int nk = __shfl_down(kf, H);
+  const float nS = __shfl_down(S, H);
+  const float none = IS_MAX ? -INFINITY : 0.0f;
+  const float prev = (lane >= H && pk == kf) ? pP : none;
+  const float next = (lane + H < kWave && nk == kl) ? nS : none;
+  tf = IS_MAX ? fmaxf(S, prev) : S + prev;
+  tl = IS_MAX ? fmaxf(P, next) : P + next;
+}
+
+// Pass 1: one wavefront per chunk.  DIRECT: edge ids are slot numbers, so the
+// chunk is one contiguous piece of x / y; it is moved with fully coalesced
+// 16-byte accesses and re-distributed to the owning lanes through a padded,
+// wave-private LDS tile.  Otherwise every element is gathered through eid.
+// FULL: the chunk holds all 1024 elements (every chunk but the last), so no
+// element needs a validity test.
+template <bool DIRECT, bool FULL>
+__device__ __forceinline__ void softmax_chunk_body(
+    const int32_t *__restrict__ row_of_slot, const int32_t *__restrict__ eid,
+    const float *__restrict__ x, float *__restrict__ y, float *__restrict__ stats,
+    int64_t n_edges, int head_shift, int64_t chunk_id, int64_t c0, int64_t c1,
+    float (*lds_v)[kChunkElems + kChunkElems / kT]) {
+  const int H = 1 << head_shift;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int g = lane >> head_shift, h = lane & (H - 1);
+  const int64_t s0 = c0 + (int64_t)g * kT;   // first slot of this lane
+
+  int key[kT];
+  int64_t off[kT];
+  float v[kT];
+  const int64_t base_elem = c0 << head_shift;
+  const int n_elem = (int)((c1 - c0) << head_shift);
+  // LDS word of element q = (i*64 + lane)*4 + c of the chunk, as seen by the
+  // lane that loads / stores it from global memory
+  int lds_at[kChunkElems / (kWave * 4)][4];
+  if (DIRECT) {
 #pragma unroll
-      for (int t = 0; t < kMediumCache; ++t) {
-        const int64_t q = lane + (int64_t)t * kWave;
-        c[t] = -INFINITY;
-        off[t] = -1;
-        if (q < rn) {
-          off[t] = elem_offset(eid, rs, q, head_shift);
-          c[t] = x[off[t]];
-          m = fmaxf(m, c[t]);
-        }
+    for (int i = 0; i < kChunkElems / (kWave * 4); ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int q = (i * kWave + lane) * 4 + c;
+        const int slot = q >> head_shift, hd = q & (H - 1);
+        lds_at[i][c] = (((slot >> 4) << head_shift) + hd) * (kT + 1) + (slot & 15);
       }
-      for (int o = kWave >> 1; o >= H; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-      float l = 0.0f;
+    float *tv = lds_v[wave];
+    int *tk = reinterpret_cast<int *>(lds_v[wave]);
+    const int n_slots = (int)(c1 - c0);
+    // all global loads first (keys and logits), then the two redistributions
+    int4 kk[kChunkElems / (kWave * 4)];
+    float4 xv[kChunkElems / (kWave * 4)];
 #pragma unroll
-      for (int t = 0; t < kMediumCache; ++t) {
-        c[t] = off[t] >= 0 ? expf(c[t] - m) : 0.0f;
-        l += c[t];
+    for (int i = 0; i < kChunkElems / (kWave * 4); ++i) {
+      const int q = (i * kWave + lane) * 4;
+      kk[i] = make_int4(-1, -1, -1, -1);
+      if (FULL ? q < n_slots : q + 3 < n_slots) {
+        kk[i] = *reinterpret_cast<const int4 *>(row_of_slot + c0 + q);
+      } else if (!FULL && q < n_slots) {
+        kk[i].x = row_of_slot[c0 + q];
+        if (q + 1 < n_slots) kk[i].y = row_of_slot[c0 + q + 1];
+        if (q + 2 < n_slots) kk[i].z = row_of_slot[c0 + q + 2];
       }
-      for (int o = kWave >> 1; o >= H; o >>= 1) l += __shfl_xor(l, o);
-#pragma unroll
-      for (int t = 0; t < kMediumCache; ++t)
-        if (off[t] >= 0) y[off[t]] = c[t] / l;
+      xv[i] = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+      if (FULL || q + 3 < n_elem) {
+        xv[i] = *reinterpret_cast<const float4 *>(x + base_elem + q);
+      } else if (q < n_elem) {
+        xv[i].x = x[base_elem + q];
+        if (q + 1 < n_elem) xv[i].y = x[base_elem + q + 1];
+        if (q + 2 < n_elem) xv[i].z = x[base_elem + q + 2];
+      }
     }
-    // stop once a lane's row starts at or beyond the chunk end (rows ascend)
-    if (__ballot(!starts_here)) break;
+#pragma unroll
+    for (int i = 0; i < kChunkElems / (kWave * 4); ++i) {
+      const int q = (i * kWave + lane) * 4;
+      if (q < n_slots) {          // keys: one per slot, word slot + slot/16
+        const int w = q + (q >> 4);
+        tk[w] = kk[i].x; tk[w + 1] = kk[i].y; tk[w + 2] = kk[i].z; tk[w + 3] = kk[i].w;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int j = 0; j < kT; ++j)
+      key[j] = (FULL || s0 + j < c1) ? tk[g * (kT + 1) + j] : -1;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < kChunkElems / (kWave * 4); ++i) {
+      tv[lds_at[i][0]] = xv[i].x; tv[lds_at[i][1]] = xv[i].y;
+      tv[lds_at[i][2]] = xv[i].z; tv[lds_at[i][3]] = xv[i].w;
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int j = 0; j < kT; ++j) {
+      v[j] = (FULL || key[j] >= 0) ? tv[lane * (kT + 1) + j] : -INFINITY;
+      off[j] = 0;
+    }
+    __builtin_amdgcn_wave_barrier();
+  } else {
+#pragma unroll
+    for (int j = 0; j < kT; ++j) {
+      const int64_t slot = s0 + j;
+      const bool valid = FULL || slot < c1;
+      key[j] = valid ? row_of_slot[slot] : -1;
+      const int64_t e = (valid && eid) ? (int64_t)eid[slot] : slot;
+      off[j] = (e << head_shift) + h;
+      v[j] = valid ? x[off[j]] : -INFINITY;
+    }
+  }
+  // which rows does the chunk share with its neighbours?  (needed last)
+  ChunkInfo ci;
+  chunk_info(row_of_slot, n_edges, head_shift, ci);
+  // ---- maxima ------------------------------------------------------------
+  float m[kT];
+  m[0] = v[0];
+#pragma unroll
+  for (int j = 1; j < kT; ++j)
+    m[j] = key[j] == key[j - 1] ? fmaxf(m[j - 1], v[j]) : v[j];
+#pragma unroll
+  for (int j = kT - 2; j >= 0; --j)
+    if (key[j] == key[j + 1]) m[j] = m[j + 1];
+  const int kf = key[0], kl = key[kT - 1];
+  float mf, ml;
+  chunk_totals<true>(m[0], m[kT - 1], kf, kl, lane, H, mf, ml);
+#pragma unroll
+  for (int j = 0; j < kT; ++j) m[j] = key[j] == kf ? mf : (key[j] == kl ? ml : m[j]);
+  // ---- sums of exponentials ------------------------------------------------
+  float p[kT], l[kT];
+#pragma unroll
+  for (int j = 0; j < kT; ++j)
+    p[j] = (FULL || key[j] >= 0) ? exp_fast(v[j] - m[j]) : 0.0f;
+  l[0] = p[0];
+#pragma unroll
+  for (int j = 1; j < kT; ++j) l[j] = key[j] == key[j - 1] ? l[j - 1] + p[j] : p[j];
+#pragma unroll
+  for (int j = kT - 2; j >= 0; --j)
+    if (key[j] == key[j + 1]) l[j] = l[j + 1];
+  float lf, ll;
+  chunk_totals<false>(l[0], l[kT - 1], kf, kl, lane, H, lf, ll);
+  // ---- rows inside the chunk: done; boundary rows: leave their statistics --
+  // (pass 2 rewrites every element of a boundary row, so DIRECT stores all)
+  const float rf = __builtin_amdgcn_rcpf(lf), rl = __builtin_amdgcn_rcpf(ll);
+  if (DIRECT) {
+    float *tv = lds_v[wave];
+#pragma unroll
+    for (int j = 0; j < kT; ++j) {
+      const float rt = key[j] == kf ? rf : (key[j] == kl ? rl : __builtin_amdgcn_rcpf(l[j]));
+      tv[lane * (kT + 1) + j] = p[j] * rt;
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < kChunkElems / (kWave * 4); ++i) {
+      const int q = (i * kWave + lane) * 4;
+      const float4 o = make_float4(tv[lds_at[i][0]], tv[lds_at[i][1]],
+                                   tv[lds_at[i][2]], tv[lds_at[i][3]]);
+      if (FULL || q + 3 < n_elem) {
+        *reinterpret_cast<float4 *>(y + base_elem + q) = o;
+      } else if (q < n_elem) {
+        y[base_elem + q] = o.x;
+        if (q + 1 < n_elem) y[base_elem + q + 1] = o.y;
+        if (q + 2 < n_elem) y[base_elem + q + 2] = o.z;
+      }
+    }
+  } else {
+    const int skip_a = ci.began_before ? ci.row_first : -2;
+    const int skip_b = ci.continues ? ci.row_last : -2;
+#pragma unroll
+    for (int j = 0; j < kT; ++j) {
+      const float rt = key[j] == kf ? rf : (key[j] == kl ? rl : __builtin_amdgcn_rcpf(l[j]));
+      if ((FULL || key[j] >= 0) && key[j] != skip_a && key[j] != skip_b)
+        y[off[j]] = p[j] * rt;
+    }
+  }
+  const int64_t chunk = chunk_id;
+  if (ci.began_before && g == 0) {           // lanes 0..H-1 start with row_first
+    float *st = stat_ptr(stats, chunk, 0, H, h);
+    st[0] = mf;
+    st[1] = lf;
+  }
+  if (ci.continues && !(ci.began_before && ci.row_first == ci.row_last) &&
+      g == (kWave >> head_shift) - 1) {      // a continuing chunk is full
+    float *st = stat_ptr(stats, chunk, 1, H, h);
+    st[0] = ml;
+    st[1] = ll;
   }
 }
 
-// ---- long rows -------------------------------------------------------------
+template <bool DIRECT>
+__global__ __launch_bounds__(kBlock) void softmax_chunks_kernel(
+    const int32_t *__restrict__ row_of_slot, const int32_t *__restrict__ eid,
+    const float *__restrict__ x, float *__restrict__ y, float *__restrict__ stats,
+    int64_t n_edges, int head_shift) {
+  // per wave: one tile of 1024 words (+ one pad word per 16), used in turn for
+  // the keys, the logits and the results
+  __shared__ float lds_v[kBlock / kWave][kChunkElems + kChunkElems / kT];
+  const int chunk_slots = kChunkElems >> head_shift;
+  const int64_t chunk_id = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const int64_t c0 = chunk_id * chunk_slots;
+  if (c0 >= n_edges) return;                                        // whole wave
+  const int64_t c1 = min(c0 + (int64_t)chunk_slots, n_edges);
+  if (c1 - c0 == chunk_slots)
+    softmax_chunk_body<DIRECT, true>(row_of_slot, eid, x, y, stats, n_edges,
+                                     head_shift, chunk_id, c0, c1, lds_v);
+  else
+    softmax_chunk_body<DIRECT, false>(row_of_slot, eid, x, y, stats, n_edges,
+                                      head_shift, chunk_id, c0, c1, lds_v);
+}
+
+// Pass 2: the rows a chunk shares with its neighbours (A = first row, begun in
+// an earlier chunk; B = last row, started here and continuing).  Both rows are
+// handled side by side so their dependent loads overlap.
+__global__ __launch_bounds__(kBlock) void softmax_boundary_kernel(
+    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
+    const int32_t *__restrict__ eid, const float *__restrict__ x,
+    float *__restrict__ y, float *__restrict__ stats, int64_t n_edges,
+    int head_shift) {
+  ChunkInfo ci;
+  if (!chunk_info(row_of_slot, n_edges, head_shift, ci)) return;
+  const bool has_b = ci.continues && !(ci.began_before && ci.row_first == ci.row_last);
+  if (!ci.began_before && !has_b) return;
+  const int H = 1 << head_shift;
+  const int G = kWave >> head_shift;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int g = lane >> head_shift, h = lane & (H - 1);
+  const int cs_shift = 10 - head_shift;       // chunk_slots = 1024 >> head_shift
+
+  int64_t s[2] = {0, 0}, e[2] = {0, 0};
+  if (ci.began_before) { s[0] = pointer[ci.row_first]; e[0] = pointer[ci.row_first + 1]; }
+  if (has_b) { s[1] = pointer[ci.row_last]; e[1] = pointer[ci.row_last + 1]; }
+  int64_t lo[2], hi[2], o0[2];
+  float x0[2];
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {            // first element of each row, early
+    lo[w] = max(s[w], ci.c0);
+    hi[w] = min(e[w], ci.c1);
+    o0[w] = -1;
+    x0[w] = 0.0f;
+    if (lo[w] + g < hi[w]) {
+      const int64_t slot = lo[w] + g;
+      const int64_t ed = eid ? (int64_t)eid[slot] : slot;
+      o0[w] = (ed << head_shift) + h;
+      x0[w] = x[o0[w]];
+    }
+  }
+  float m[2], rcp_l[2];
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    // merge the row's partials (B of its first chunk, then A's): the lanes of
+    // a head split the chunk list, then combine with a fixed shuffle tree
+    const int64_t k_lo = s[w] >> cs_shift, k_hi = (e[w] - 1) >> cs_shift;
+    float mm = -INFINITY;
+    if (e[w] > s[w])
+      for (int64_t c = k_lo + g; c <= k_hi; c += G)
+        mm = fmaxf(mm, stat_ptr(stats, c, c == k_lo ? 1 : 0, H, h)[0]);
+    for (int o = kWave >> 1; o >= H; o >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o));
+    float l = 0.0f;
+    if (e[w] > s[w])
+      for (int64_t c = k_lo + g; c <= k_hi; c += G) {
+        const float *st = stat_ptr(stats, c, c == k_lo ? 1 : 0, H, h);
+        l += st[1] * exp_fast(st[0] - mm);
+      }
+    for (int o = kWave >> 1; o >= H; o >>= 1) l += __shfl_xor(l, o);
+    m[w] = mm;
+    rcp_l[w] = __builtin_amdgcn_rcpf(l);
+  }
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    if (o0[w] >= 0) y[o0[w]] = exp_fast(x0[w] - m[w]) * rcp_l[w];
+    // the rest of the row's slots in this chunk, eight loads in flight
+    for (int64_t base = lo[w] + g + G; base < hi[w]; base += 8 * (int64_t)G) {
+      int64_t o[8];
+      float xv[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const int64_t slot = base + (int64_t)t * G;
+        o[t] = -1;
+        xv[t] = 0.0f;
+        if (slot < hi[w]) {
+          const int64_t ed = eid ? (int64_t)eid[slot] : slot;
+          o[t] = (ed << head_shift) + h;
+          xv[t] = x[o[t]];
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 8; ++t)
+        if (o[t] >= 0) y[o[t]] = exp_fast(xv[t] - m[w]) * rcp_l[w];
+    }
+  }
+}
+
 // Chunk c of L slots belongs to the long row that contains slot c*L; the first
 // chunk of a row also takes the row's slots before its first multiple of L.
 __device__ __forceinline__ bool long_chunk(const int32_t *pointer,
@@ -157,78 +402,6 @@ __device__ __forceinline__ bool long_chunk(const int32_t *pointer,
   lo = c == c_first ? start : c * L;
   hi = min(end, (c + 1) * (int64_t)L);
   return true;
-}
-
-// reduce over the lanes of the workgroup that share (tid & (H-1))
-template <bool IS_MAX>
-__device__ __forceinline__ float block_reduce_heads(float v, int H, float *lds) {
-  for (int o = kWave >> 1; o >= H; o >>= 1) {
-    const float other = __shfl_xor(v, o);
-    v = IS_MAX ? fmaxf(v, other) : v + other;
-  }
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  __syncthreads();   // lds may still be read from the previous reduction
-  if (lane < H) lds[wave * kWave + lane] = v;
-  __syncthreads();
-  const int h = lane & (H - 1);
-  float r = lds[h];
-  for (int w = 1; w < kBlock / kWave; ++w)
-    r = IS_MAX ? fmaxf(r, lds[w * kWave + h]) : r + lds[w * kWave + h];
-  return r;
-}
-
-// power-of-two heads: all heads of the chunk at once, read once
-__global__ __launch_bounds__(kBlock) void softmax_long_stats_kernel(
-    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
-    const int32_t *__restrict__ eid, const float *__restrict__ x,
-    float *__restrict__ stats, int head_shift, int L, int long_min_deg) {
-  __shared__ float lds[kBlock];
-  int64_t lo, hi, c_first, c_last;
-  if (!long_chunk(pointer, row_of_slot, L, long_min_deg, lo, hi, c_first, c_last))
-    return;
-  const int H = 1 << head_shift;
-  const int64_t n = (hi - lo) << head_shift;    // < 2 * 1024 elements
-  float c[8];
-  float m = -INFINITY;
-#pragma unroll
-  for (int t = 0; t < 8; ++t) {
-    const int64_t q = threadIdx.x + (int64_t)t * kBlock;
-    c[t] = q < n ? x[elem_offset(eid, lo, q, head_shift)] : -INFINITY;
-    m = fmaxf(m, c[t]);
-  }
-  m = block_reduce_heads<true>(m, H, lds);
-  float l = 0.0f;
-#pragma unroll
-  for (int t = 0; t < 8; ++t) l += expf(c[t] - m);   // exp(-inf) == 0
-  l = block_reduce_heads<false>(l, H, lds);
-  if (threadIdx.x < H) {
-    stats[((int64_t)blockIdx.x * H + threadIdx.x) * 2] = m;
-    stats[((int64_t)blockIdx.x * H + threadIdx.x) * 2 + 1] = l;
-  }
-}
-
-__global__ __launch_bounds__(kBlock) void softmax_long_write_kernel(
-    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
-    const int32_t *__restrict__ eid, const float *__restrict__ x,
-    const float *__restrict__ stats, float *__restrict__ y, int head_shift, int L,
-    int long_min_deg) {
-  int64_t lo, hi, c_first, c_last;
-  if (!long_chunk(pointer, row_of_slot, L, long_min_deg, lo, hi, c_first, c_last))
-    return;
-  const int H = 1 << head_shift;
-  const int h = threadIdx.x & (H - 1);
-  // merge the row's chunk statistics in chunk order (every lane, its own head)
-  float m = -INFINITY;
-  for (int64_t c = c_first; c <= c_last; ++c)
-    m = fmaxf(m, stats[(c * H + h) * 2]);
-  float l = 0.0f;
-  for (int64_t c = c_first; c <= c_last; ++c)
-    l += stats[(c * H + h) * 2 + 1] * expf(stats[(c * H + h) * 2] - m);
-  const int64_t n = (hi - lo) << head_shift;
-  for (int64_t q = threadIdx.x; q < n; q += kBlock) {
-    const int64_t o = elem_offset(eid, lo, q, head_shift);
-    y[o] = expf(x[o] - m) / l;
-  }
 }
 
 // ---- any head count ---------------------------------------------------------
@@ -335,10 +508,6 @@ __global__ __launch_bounds__(kBlock) void softmax_long_write_generic_kernel(
 inline bool pow2_heads(int64_t heads) {
   return (heads & (heads - 1)) == 0 && heads <= kWave;
 }
-// slots per long-row chunk
-inline int long_chunk_slots(int64_t heads) {
-  return pow2_heads(heads) ? (int)(kMediumMax / heads) : kLongRow;
-}
 
 }  // namespace
 }  // namespace ga
@@ -347,10 +516,14 @@ extern "C" {
 
 size_t ga_softmax_workspace_bytes(int64_t n_edges, int64_t heads) {
   if (n_edges <= 0 || heads <= 0) return 0;
-  // (max, sum-exp) per head for every chunk of a long row
-  const int64_t L = ga::long_chunk_slots(heads);
-  if (n_edges <= L) return 0;
-  const int64_t chunks = (n_edges + L - 1) / L;
+  if (ga::pow2_heads(heads)) {
+    // two partial (max, sum) pairs per head for every 1024-element chunk
+    const int64_t chunk_slots = ga::kChunkElems / heads;
+    const int64_t chunks = (n_edges + chunk_slots - 1) / chunk_slots;
+    return (size_t)chunks * 2 * (size_t)heads * 2 * sizeof(float);
+  }
+  if (n_edges <= ga::kLongRow) return 0;
+  const int64_t chunks = (n_edges + ga::kLongRow - 1) / ga::kLongRow;
   return (size_t)chunks * (size_t)heads * 2 * sizeof(float);
 }
 
@@ -371,46 +544,30 @@ int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
     return GA_EWORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   float *stats = (float *)workspace;
-  const int L = long_chunk_slots(heads);
-  const int64_t lchunks = (n_edges + L - 1) / L;
-  if (lchunks > 0x7fffffff) return GA_EUNSUPPORTED;
 
   if (pow2_heads(heads)) {
     const int head_shift = ilog2_floor((uint64_t)heads);
-    // lanes per small row: the register cache covers the mean segment
-    const int64_t avg = (n_edges * heads + n_rows - 1) / n_rows;
-    int s_shift = ilog2_ceil((uint64_t)((avg + kSmallCache - 1) / kSmallCache));
-    // at least 16 lanes: medium rows then have > 64 elements, so a wave of the
-    // medium kernel (one per 1024 elements) never meets more than 16 of them
-    if (s_shift < 4) s_shift = 4;
-    if (s_shift > 6) s_shift = 6;
-    if (s_shift < head_shift) s_shift = head_shift;
-    const int small_max = kSmallCache << s_shift;
-    const int64_t per_block = kBlock >> s_shift;
-    const int64_t blocks = (n_rows + per_block - 1) / per_block;
+    const int64_t chunk_slots = kChunkElems >> head_shift;
+    const int64_t chunks = (n_edges + chunk_slots - 1) / chunk_slots;
+    const int64_t blocks = (chunks + kBlock / kWave - 1) / (kBlock / kWave);
     if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-    hipLaunchKernelGGL(softmax_small_kernel, dim3((unsigned)blocks), dim3(kBlock),
-                       0, s, pointer, eid, x, y, n_rows, head_shift, s_shift);
-    if (small_max < kMediumMax) {
-      const int64_t chunk_slots = kChunkElems >> head_shift;
-      const int64_t chunks = (n_edges + chunk_slots - 1) / chunk_slots;
-      const int64_t mblocks = (chunks + kBlock / kWave - 1) / (kBlock / kWave);
-      hipLaunchKernelGGL(softmax_medium_kernel, dim3((unsigned)mblocks),
-                         dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, y,
-                         n_rows, n_edges, head_shift, small_max);
-    }
-    if (n_edges > L) {
-      const int long_min_deg = L + 1;   // n > 1024 elements
-      hipLaunchKernelGGL(softmax_long_stats_kernel, dim3((unsigned)lchunks),
-                         dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, stats,
-                         head_shift, L, long_min_deg);
-      hipLaunchKernelGGL(softmax_long_write_kernel, dim3((unsigned)lchunks),
-                         dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, stats,
-                         y, head_shift, L, long_min_deg);
-    }
+    if (!eid && aligned(x, 16) && aligned(y, 16) && aligned(row_of_slot, 16))
+      hipLaunchKernelGGL(softmax_chunks_kernel<true>, dim3((unsigned)blocks),
+                         dim3(kBlock), 0, s, row_of_slot, eid, x, y, stats,
+                         n_edges, head_shift);
+    else
+      hipLaunchKernelGGL(softmax_chunks_kernel<false>, dim3((unsigned)blocks),
+                         dim3(kBlock), 0, s, row_of_slot, eid, x, y, stats,
+                         n_edges, head_shift);
+    if (chunks > 1)
+      hipLaunchKernelGGL(softmax_boundary_kernel, dim3((unsigned)blocks),
+                         dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, y, stats,
+                         n_edges, head_shift);
     return launch_status();
   }
 
+  const int64_t lchunks = (n_edges + kLongRow - 1) / kLongRow;
+  if (lchunks > 0x7fffffff) return GA_EUNSUPPORTED;
   const int64_t avg = (n_edges + n_rows - 1) / n_rows;
   int s_shift = ilog2_ceil((uint64_t)(avg < 1 ? 1 : avg));
   if (s_shift < 2) s_shift = 2;
