@@ -39,6 +39,8 @@ SIGNATURES = {
     "ga_segment_mm": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                              _int, _vp]),
     "ga_gather_rows": (_int, [_vp, _int, _vp, _vp, _i64, _i64, _vp]),
+    "ga_linear_attn": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+                              _i64, _vp]),
     "ga_gat_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "ga_gat_aggregate": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
                                 _i64, _i64, ctypes.c_float, _int, _vp, _sz,

@@ -327,3 +327,33 @@ def gat_aggregate(el, er, z, graph: DGLGraph, negative_slope: float = 0.01):
         feat // heads, float(negative_slope), dt, ws.data_ptr(), ws.numel(),
         _stream(out)), "ga_gat_aggregate")
     return out
+
+
+# ------------------------------------------------------ dense projection ----
+def linear_attn(x, weight, a_l=None, a_r=None):
+    """z = x @ weight and, when a_l / a_r (heads, D) are given, the GAT attention
+    terms el = <z_h, a_l[h]>, er = <z_h, a_r[h]> from the same kernel (fp32).
+    Returns z or (z, el, er).  A head width other than 16/32/64 raises
+    GraphilerError with GA_EUNSUPPORTED."""
+    _check_input(x, "x")
+    _check_input(weight, "weight")
+    if x.dtype != torch.float32 or weight.dtype != torch.float32:
+        raise RuntimeError("linear_attn is float32 only")
+    rows, K = int(x.shape[0]), int(x.shape[1])
+    if int(weight.shape[0]) != K:
+        raise RuntimeError("weight must be (K, M)")
+    M = int(weight.shape[1])
+    z = torch.empty((rows, M), dtype=x.dtype, device=x.device)
+    heads, el, er = 1, None, None
+    if a_l is not None:
+        _check_input(a_l, "a_l")
+        _check_input(a_r, "a_r")
+        heads = int(a_l.shape[0])
+        if a_l.numel() != M or a_r.numel() != M:
+            raise RuntimeError("a_l and a_r must be (heads, M / heads)")
+        el = torch.empty((rows, heads), dtype=x.dtype, device=x.device)
+        er = torch.empty((rows, heads), dtype=x.dtype, device=x.device)
+    capi.check(capi.load().ga_linear_attn(
+        x.data_ptr(), weight.data_ptr(), _ptr(a_l), _ptr(a_r), z.data_ptr(),
+        _ptr(el), _ptr(er), rows, K, M, heads, _stream(x)), "ga_linear_attn")
+    return z if a_l is None else (z, el, er)

@@ -164,6 +164,23 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
                      void *workspace, size_t workspace_bytes,
                      ga_stream_t stream);
 
+/* ------------------------------------------- dense projection (fp32) ------
+ * Z = X @ W and, optionally, the per-head attention terms of a GAT layer
+ * el[n, h] = <Z[n, h, :], a_l[h, :]>, er likewise, in the same kernel.
+ * Replaces the dense operators in front of the graph chain in the reference's
+ * GAT plan: mm(h, fc_weight) and the two halves of mm(z2, attn_weight)
+ * (examples/GAT/GAT.py:25-29 after the split and reorder passes,
+ * src/optimizer/split.cpp:5-34); with el == er == NULL it is the plain node
+ * projection of examples/GCN/GCN.py:39.  X (rows, K), W (K, M), Z (rows, M),
+ * a_l / a_r (heads, M/heads), el / er (rows, heads), all fp32.
+ * GA_EUNSUPPORTED when the attention terms are requested with M/heads not in
+ * {16, 32, 64}.
+ */
+int ga_linear_attn(const float *X, const float *W, const float *a_l,
+                   const float *a_r, float *Z, float *el, float *er,
+                   int64_t rows, int64_t K, int64_t M, int64_t heads,
+                   ga_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -312,3 +312,30 @@ def test_segment_mm_ops_and_rgcn_layer(device):
     with pytest.raises(RuntimeError, match="type pointer"):
         g2 = prepare_graph(wl.src, wl.dst, wl.num_nodes, device=device)
         ops.SegmentMMEdge(_dev(h[:1], device), _dev(W, device), g2)
+
+
+@pytest.mark.parametrize("rows,K,M,heads", [(1000, 602, 64, 1), (333, 77, 64, 2),
+                                            (777, 64, 64, 4),
+                                            (300, 100, 256, 4), (5000, 16, 32, 2),
+                                            (50, 8, 16, 1), (1, 4, 64, 1)])
+def test_linear_attn(device, rows, K, M, heads):
+    rng = np.random.default_rng(K + M)
+    x = rng.standard_normal((rows, K), dtype=np.float32)
+    w = datasets.glorot(rng, (K, M))
+    a = rng.standard_normal((2, heads, M // heads), dtype=np.float32)
+    z, el, er = ops.linear_attn(_dev(x, device), _dev(w, device), _dev(a[0], device),
+                                _dev(a[1], device))
+    zr = x.astype(np.float64) @ w.astype(np.float64)
+    assert_close(z.cpu().numpy(), zr, TOL_F32, "linear z")
+    zh = zr.reshape(rows, heads, -1)
+    assert_close(el.cpu().numpy(), (zh * a[0]).sum(-1), 2 * TOL_F32, "linear el")
+    assert_close(er.cpu().numpy(), (zh * a[1]).sum(-1), 2 * TOL_F32, "linear er")
+    z2 = ops.linear_attn(_dev(x, device), _dev(w, device))
+    assert np.array_equal(z2.cpu().numpy(), z.cpu().numpy())
+
+
+def test_linear_attn_unsupported_shapes(device):
+    x = torch.ones(8, 8, device=device)          # head width 8
+    with pytest.raises(capi.GraphilerError):
+        ops.linear_attn(x, torch.ones(8, 16, device=device),
+                        torch.ones(2, 8, device=device), torch.ones(2, 8, device=device))
