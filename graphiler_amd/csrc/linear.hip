@@ -5,14 +5,19 @@
 // examples/GAT/GAT.py:25-29 after the split / reorder passes) as one kernel, so
 // Z is written once and never re-read for the attention terms.
 //
-// Tall-skinny GEMM on v_mfma_f32_16x16x4_f32: a workgroup (4 waves) owns 256
-// rows, each wave 64 rows (4 tiles of 16) x 64 columns per pass; W is streamed
-// through LDS in double-buffered slices of 64 k, X fragments go global ->
-// registers (one 16-byte load per lane covers 16 k of a row, the k order inside
-// a block being permuted identically for X and W).  Per slice and wave:
-// 16 X loads, 64 LDS reads, 256 MFMAs.  Accumulators come out as D[row][col]
-// with 16 adjacent lanes on 16 adjacent columns: Z stores coalesce, and the
-// per-head dot products need one 16-lane shuffle tree per row and head.
+// Tall-skinny GEMM on v_mfma_f32_16x16x4_f32: a workgroup (4 waves) owns 128
+// rows, each wave 32 rows (2 tiles of 16) x 64 columns per pass.  Both operands
+// go global -> registers -> LDS in slices of 32 k: the MFMA operand layout puts
+// the 16 rows of a tile on 16 adjacent lanes, so loading X straight into that
+// layout makes every lane its own cache access (the address unit then bounds
+// the kernel at well under half the MFMA rate); staged through LDS, adjacent
+// lanes read adjacent addresses of a row and the layout change costs one
+// 16-byte LDS read per lane and 16 k.  Two register sets hold the slices one
+// and two ahead of the one being multiplied, two LDS buffers the current and
+// the next slice, so a slice costs one barrier and its global loads have two
+// slices of MFMAs to arrive.  Accumulators come out as D[row][col] with 16
+// adjacent lanes on 16 adjacent columns: Z stores coalesce, and the per-head
+// dot products need one 16-lane DPP sum per row and head.
 #include "common.h"
 
 namespace ga {
@@ -20,51 +25,114 @@ namespace {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kRT = 4;                                   // 16-row tiles per wave
-constexpr int kWaveRows = kRT * 16;                      // 64
-constexpr int kWgRows = kWaveRows * (kBlock / kWave);    // 256
+constexpr int kRT = 2;                                   // 16-row tiles per wave
+constexpr int kWaveRows = kRT * 16;                      // 32
+constexpr int kWgRows = kWaveRows * (kBlock / kWave);    // 128
 constexpr int kCB = 4;                                   // 16-column blocks per pass
 constexpr int kPassCols = kCB * 16;                      // 64
-constexpr int kSliceK = 64;                              // k per LDS slice
-constexpr int kWs = kPassCols + 4;                       // padded LDS row stride
+constexpr int kSliceK = 32;                              // k per LDS slice
+constexpr int kXs = kSliceK + 4;                         // LDS row stride of the X tile
+constexpr int kWs = kPassCols + 4;                       // LDS row stride of the W tile
+
+// Sum over the 16 lanes of a DPP row (lanes 16j..16j+15), result in every lane:
+// swaps inside quads, then the half-row and row mirrors; all VALU, no LDS.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));  // row_mirror
+  return v;
+}
+
+template <int VK> struct XVec;
+template <> struct XVec<4> { using type = float4; };
+template <> struct XVec<2> { using type = float2; };
+template <> struct XVec<1> { using type = float; };
 
 // HAS_ATTN: also produce el / er; requires heads to tile a pass exactly
 // (dph = M / heads in {16, 32, 64}).
-// VK = widest aligned vector (floats) a lane may use for its four k values:
-// 4 when K % 4 == 0, 2 when K % 2 == 0, else 1.
+// VK = widest aligned vector (floats) of a row of X: 4 when K % 4 == 0, 2 when
+// K % 2 == 0, else 1.  K % VK == 0, so such a vector lies wholly inside or
+// wholly outside a row: ragged edges clamp the address at fetch time (a valid
+// one, the row's last vector) and zero by select at commit time, where the
+// value is consumed anyway; no lane is ever predicated off in the k loop.
 template <bool HAS_ATTN, int VK>
 __global__ __launch_bounds__(kBlock) void linear_attn_kernel(
     const float *__restrict__ X, const float *__restrict__ W,
     const float *__restrict__ a_l, const float *__restrict__ a_r,
     float *__restrict__ Z, float *__restrict__ el, float *__restrict__ er,
     int64_t rows, int K, int M, int heads) {
-  __shared__ __attribute__((aligned(16))) float wt[2][kSliceK * kWs];
+  using xvec_t = typename XVec<VK>::type;
+  __shared__ __attribute__((aligned(16))) float xs[2][kWgRows * kXs];
+  __shared__ __attribute__((aligned(16))) float ws[2][kSliceK * kWs];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int lr = lane & 15, lk = lane >> 4;
   const int col0 = blockIdx.y * kPassCols;               // first column of the pass
-  const int64_t wrow0 = (int64_t)blockIdx.x * kWgRows + wave * kWaveRows;
+  const int64_t wg_row0 = (int64_t)blockIdx.x * kWgRows;
+  const int64_t wrow0 = wg_row0 + wave * kWaveRows;
   const bool vec_w = (M & 3) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0;
+  const int n_slices = (K + kSliceK - 1) / kSliceK;
 
-  // slice sl (k in [sl*64, sl*64+64)) of W[:, col0:col0+64] -> wt[buf], zero padded
-  auto stage = [&](int sl, int buf) {
-    const int k0 = sl * kSliceK;
-    for (int i = threadIdx.x; i < kSliceK * (kPassCols / 4); i += kBlock) {
-      const int k = i >> 4, c4 = (i & 15) * 4;
-      const int kk = k0 + k, cc = col0 + c4;
-      float4 v = make_float4(0, 0, 0, 0);
-      if (kk < K) {
-        const float *src = W + (int64_t)kk * M + cc;
-        if (vec_w && cc + 3 < M) {
-          v = *reinterpret_cast<const float4 *>(src);
-        } else {
-          if (cc < M) v.x = src[0];
-          if (cc + 1 < M) v.y = src[1];
-          if (cc + 2 < M) v.z = src[2];
-          if (cc + 3 < M) v.w = src[3];
-        }
+  // X slice: 128 rows x 32 k in vectors of VK floats, kVpr per row; thread i
+  // owns vectors i, i + 256, ...: a wave instruction reads 64 * VK * 4
+  // contiguous-by-row bytes (8 * VK rows of 128 bytes).  Slices past the last
+  // are fetched too (from the clamped address) and never multiplied.
+  constexpr int kVpr = kSliceK / VK;                     // vectors per row and slice
+  constexpr int kXPieces = kWgRows * kVpr / kBlock;      // 4 / 8 / 16 per thread
+  constexpr int kRowStep = kBlock / kVpr;                // rows between a thread's vectors
+  constexpr int kWPieces = kSliceK * (kPassCols / 4) / kBlock;  // float4 of W: 2
+  struct Stage {
+    xvec_t x[kXPieces];
+    float4 w[kWPieces];
+  };
+  const int xr = threadIdx.x / kVpr, xc = (threadIdx.x % kVpr) * VK;
+  const float *xbase[kXPieces];
+#pragma unroll
+  for (int j = 0; j < kXPieces; ++j)
+    xbase[j] = X + min(wg_row0 + xr + j * kRowStep, rows - 1) * K;
+  const bool w_cols_plain = vec_w && col0 + kPassCols <= M;     // uniform
+
+  auto fetch = [&](int sl, Stage &st) {
+    const int kc = min(sl * kSliceK + xc, K - VK);
+#pragma unroll
+    for (int j = 0; j < kXPieces; ++j)
+      st.x[j] = *reinterpret_cast<const xvec_t *>(xbase[j] + kc);
+#pragma unroll
+    for (int j = 0; j < kWPieces; ++j) {
+      const int i = threadIdx.x + j * kBlock;
+      const int kk = min(sl * kSliceK + (i >> 4), K - 1), cc = col0 + (i & 15) * 4;
+      const float *src = W + (int64_t)kk * M;
+      if (w_cols_plain) {
+        st.w[j] = *reinterpret_cast<const float4 *>(src + cc);
+      } else {
+        st.w[j].x = src[min(cc, M - 1)];
+        st.w[j].y = src[min(cc + 1, M - 1)];
+        st.w[j].z = src[min(cc + 2, M - 1)];
+        st.w[j].w = src[min(cc + 3, M - 1)];
       }
-      *reinterpret_cast<float4 *>(&wt[buf][k * kWs + c4]) = v;
+    }
+  };
+  auto commit = [&](int sl, const Stage &st) {
+    const int buf = sl & 1;
+    const bool xin = sl * kSliceK + xc < K;
+#pragma unroll
+    for (int j = 0; j < kXPieces; ++j) {
+      xvec_t v = st.x[j];
+      if (!xin) v = xvec_t{};
+      *reinterpret_cast<xvec_t *>(&xs[buf][(xr + j * kRowStep) * kXs + xc]) = v;
+    }
+#pragma unroll
+    for (int j = 0; j < kWPieces; ++j) {
+      const int i = threadIdx.x + j * kBlock;
+      const int cc = col0 + (i & 15) * 4;
+      const bool kin = sl * kSliceK + (i >> 4) < K;
+      float4 v = st.w[j];
+      v.x = kin && cc < M ? v.x : 0.0f;
+      v.y = kin && cc + 1 < M ? v.y : 0.0f;
+      v.z = kin && cc + 2 < M ? v.z : 0.0f;
+      v.w = kin && cc + 3 < M ? v.w : 0.0f;
+      *reinterpret_cast<float4 *>(&ws[buf][(i >> 4) * kWs + (i & 15) * 4]) = v;
     }
   };
 
@@ -74,76 +142,73 @@ __global__ __launch_bounds__(kBlock) void linear_attn_kernel(
 #pragma unroll
     for (int cb = 0; cb < kCB; ++cb) acc[t][cb] = floatx4{0, 0, 0, 0};
 
-  const float *xrow[kRT];
-  bool xlive[kRT];
+  // MFMA operands of the lane: X[row lr of tile t][k = kb*16 + lk*4 + q] against
+  // W[k = kb*16 + lk*4 + q][column cb*16 + lr], q = 0..3 (the k order inside a
+  // block of 16 is permuted identically for both operands)
+  const int xl_ofs = (wave * kWaveRows + lr) * kXs + lk * 4;
+  const int wl_ofs = lk * 4 * kWs + lr;
+  struct Frag {
+    float4 x[kRT];
+    float w[4][kCB];
+  };
+  auto read_frag = [&](int buf, int kb, Frag &f) {
+    const float *xl = &xs[buf][xl_ofs + kb * 16];
+    const float *wl = &ws[buf][wl_ofs + kb * 16 * kWs];
 #pragma unroll
-  for (int t = 0; t < kRT; ++t) {
-    const int64_t r = wrow0 + t * 16 + lr;
-    xlive[t] = r < rows;
-    xrow[t] = X + (xlive[t] ? r : 0) * (int64_t)K + lk * 4;
-  }
-
-  // X fragments of k block kb (16 k): the lane's four values of each row tile
-  auto load_frags = [&](int kofs, float4 (&xa)[kRT]) {
+    for (int t = 0; t < kRT; ++t) f.x[t] = *reinterpret_cast<const float4 *>(xl + t * 16 * kXs);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int cb = 0; cb < kCB; ++cb) f.w[q][cb] = wl[q * kWs + cb * 16];
+  };
+  auto mma = [&](const Frag &f) {
 #pragma unroll
     for (int t = 0; t < kRT; ++t) {
-      xa[t] = make_float4(0, 0, 0, 0);
-      const int k0 = kofs + lk * 4;
-      const float *px = xrow[t] + kofs;
-      if (xlive[t] && k0 < K) {
-        if (VK == 4) {
-          xa[t] = *reinterpret_cast<const float4 *>(px);
-        } else if (VK == 2) {
-          const float2 lo = *reinterpret_cast<const float2 *>(px);
-          xa[t].x = lo.x; xa[t].y = lo.y;
-          if (k0 + 2 < K) {
-            const float2 hi = *reinterpret_cast<const float2 *>(px + 2);
-            xa[t].z = hi.x; xa[t].w = hi.y;
-          }
-        } else {
-          xa[t].x = px[0];
-          if (k0 + 1 < K) xa[t].y = px[1];
-          if (k0 + 2 < K) xa[t].z = px[2];
-          if (k0 + 3 < K) xa[t].w = px[3];
-        }
-      }
-    }
-  };
-
-  const int n_slices = (K + kSliceK - 1) / kSliceK;
-  stage(0, 0);
-  float4 xn[kRT];
-  load_frags(0, xn);                                     // software pipeline: the
-  __syncthreads();                                       // next block's X is in
-  for (int sl = 0; sl < n_slices; ++sl) {                // flight during the MFMAs
-    const int buf = sl & 1;
-    if (sl + 1 < n_slices) stage(sl + 1, buf ^ 1);       // other buffer: free since
-    const float *wl = &wt[buf][lk * 4 * kWs + lr];       // the barrier of slice sl-1
-#pragma unroll
-    for (int kb = 0; kb < kSliceK / 16; ++kb) {
-      const int kofs = sl * kSliceK + kb * 16;
-      float4 xa[kRT];
-#pragma unroll
-      for (int t = 0; t < kRT; ++t) xa[t] = xn[t];
-      load_frags(kofs + 16, xn);                         // zero beyond K
-      float wv[4][kCB];
+      const float xv[4] = {f.x[t].x, f.x[t].y, f.x[t].z, f.x[t].w};
 #pragma unroll
       for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int cb = 0; cb < kCB; ++cb) wv[q][cb] = wl[(kb * 16 + q) * kWs + cb * 16];
-#pragma unroll
-      for (int t = 0; t < kRT; ++t) {
-        const float xv[4] = {xa[t].x, xa[t].y, xa[t].z, xa[t].w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-          for (int cb = 0; cb < kCB; ++cb)
-            acc[t][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[q], wv[q][cb],
-                                                              acc[t][cb], 0, 0, 0);
-      }
+        for (int cb = 0; cb < kCB; ++cb)
+          acc[t][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[q], f.w[q][cb], acc[t][cb], 0, 0, 0);
     }
+  };
+  // One slice.  Waves of one SIMD run this loop in step with each other, so a
+  // stall is not covered by another wave's MFMAs: each wave hides its own.  The
+  // fragments of a block are read from LDS while the block before it multiplies;
+  // the next slice's registers go to the other LDS buffer (last read a slice ago,
+  // before that slice's barrier) and the slice three ahead is fetched into the
+  // registers just freed, all under the first block's MFMAs.
+  Frag f0, f1;
+  auto step = [&](int sl, Stage &next) {
+    read_frag(sl & 1, 1, f1);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(f0);
+    commit(sl + 1, next);
+    fetch(sl + 3, next);
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
+    read_frag((sl + 1) & 1, 0, f0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(f1);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  Stage sa, sb;                                          // even / odd slices
+  fetch(0, sa);
+  fetch(1, sb);
+  commit(0, sa);
+  fetch(2, sa);
+  __syncthreads();
+  read_frag(0, 0, f0);
+  // slices in pairs (the register sets alternate), an odd last one on its own:
+  // a conditional second half inside the loop would make the allocator copy
+  // the accumulators around on every trip
+  int sl = 0;
+  for (; sl + 1 < n_slices; sl += 2) {
+    step(sl, sb);
+    step(sl + 1, sa);
   }
+  if (sl < n_slices) step(sl, sb);
 
   // epilogue: lane holds rows wrow0 + t*16 + 4*lk + r, column col0 + cb*16 + lr
   float al[kCB], ar[kCB];
@@ -184,11 +249,7 @@ __global__ __launch_bounds__(kBlock) void linear_attn_kernel(
 #pragma unroll
         for (int cb = 0; cb < kCB; ++cb) {
           if (cb % bph == 0) {                           // first block of a head
-            float sl_ = pl[cb], sr_ = pr[cb];
-            for (int o = 8; o > 0; o >>= 1) {
-              sl_ += __shfl_xor(sl_, o);
-              sr_ += __shfl_xor(sr_, o);
-            }
+            const float sl_ = row16_sum(pl[cb]), sr_ = row16_sum(pr[cb]);
             const int head = (col0 + cb * 16) / dph;
             if (live && lr == 0 && head < heads) {
               el[row * heads + head] = sl_;
