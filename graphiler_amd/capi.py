@@ -29,6 +29,9 @@ SIGNATURES = {
     "ga_spmm_workspace_bytes": (_sz, [_i64, _i64]),
     "ga_spmm_csr": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                            _i64, _int, _int, _int, _vp, _sz, _vp]),
+    "ga_spmm_arg_workspace_bytes": (_sz, [_i64, _i64]),
+    "ga_spmm_csr_arg": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+                               _i64, _i64, _int, _int, _int, _vp, _sz, _vp]),
     "ga_sddmm_u_add_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _int,
                                 _vp]),
     "ga_sddmm_u_dot_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64,

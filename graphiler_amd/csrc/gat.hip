@@ -56,6 +56,14 @@ struct GatPolicy {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) o[v] = 0.0f;
   }
+  static __device__ __forceinline__ void emit(const Args &, out_t *out, int64_t row, int feat,
+                                              int f0, const float (&st)[kState]) {
+    emit_row<GatPolicy>(out, row, feat, f0, st);
+  }
+  static __device__ __forceinline__ void emit_empty(const Args &, out_t *out, int64_t row,
+                                                    int feat, int f0) {
+    emit_empty_row<GatPolicy>(out, row, feat, f0);
+  }
 
   template <class Close>
   static __device__ __forceinline__ void walk(const Args &A,

@@ -21,6 +21,10 @@
 //   merge(dst, src)             dst <- dst (+) src, dst precedes src in slot order
 //   finish(st, o)               state -> VEC output features
 //   empty_row(o)                output of a row without edges
+//   emit(args, out, row, feat, f0, st) / emit_empty(args, out, row, feat, f0)
+//                               write a finished / an edgeless row's tile; the
+//                               usual ones are emit_row / emit_empty_row below,
+//                               a policy with further outputs writes them here
 #pragma once
 
 #include "common.h"
@@ -49,13 +53,27 @@ struct RunFlags {
 };
 
 template <class Policy>
+__device__ __forceinline__ void emit_row(typename Policy::out_t *out, int64_t row, int feat,
+                                         int f0, const float (&st)[Policy::kState]) {
+  float o[Policy::kVec];
+  Policy::finish(st, o);
+  Frag<typename Policy::out_t, Policy::kVec>::store(out + row * feat + f0, o);
+}
+template <class Policy>
+__device__ __forceinline__ void emit_empty_row(typename Policy::out_t *out, int64_t row,
+                                               int feat, int f0) {
+  float o[Policy::kVec];
+  Policy::empty_row(o);
+  Frag<typename Policy::out_t, Policy::kVec>::store(out + row * feat + f0, o);
+}
+
+template <class Policy>
 __global__ __launch_bounds__(kBlock) void runs_kernel(
     typename Policy::Args args, const int32_t *__restrict__ row_of_slot,
     typename Policy::out_t *__restrict__ out, float *__restrict__ partial,
     RunGeom geo) {
   constexpr int VEC = Policy::kVec;
   constexpr int SF = Policy::kState;
-  typedef Frag<typename Policy::out_t, VEC> OutIO;
   // LDS: [run in block][A|B][lane in group][SF]
   extern __shared__ float lds_state[];
   __shared__ RunFlags flags[kBlock];
@@ -93,9 +111,7 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
 #pragma unroll
         for (int i = 0; i < SF; ++i) my_a[i] = st[i];
       } else {
-        float o[VEC];
-        Policy::finish(st, o);
-        OutIO::store(out + (int64_t)cur * geo.feat + f0, o);
+        Policy::emit(args, out, cur, geo.feat, f0, st);
       }
       first_seg = false;
     };
@@ -115,9 +131,7 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
 #pragma unroll
       for (int i = 0; i < SF; ++i) my_b[i] = st[i];
     } else {
-      float o[VEC];
-      Policy::finish(st, o);
-      OutIO::store(out + (int64_t)cur * geo.feat + f0, o);
+      Policy::emit(args, out, cur, geo.feat, f0, st);
     }
   }
   if (lane == 0) {
@@ -156,9 +170,7 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
   if (has_a && !a_open) {            // a row ends in my run
     float acc[SF];
     if (chain_into(grp, acc)) {
-      float o[VEC];
-      Policy::finish(acc, o);
-      OutIO::store(out + (int64_t)row_a * geo.feat + f0, o);
+      Policy::emit(args, out, row_a, geo.feat, f0, acc);
     } else {                         // began before this workgroup: slot 0
       float *p = gp + (int64_t)flane * SF;
 #pragma unroll
@@ -186,18 +198,17 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
 // blocks: one lane group per row, rows without edges get Policy::empty_row.
 template <class Policy>
 __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
-    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
+    typename Policy::Args args, const int32_t *__restrict__ pointer,
+    const int32_t *__restrict__ row_of_slot,
     const float *__restrict__ partial, typename Policy::out_t *__restrict__ out,
     RunGeom geo, int64_t n_wg, int fix_blocks) {
   constexpr int VEC = Policy::kVec;
   constexpr int SF = Policy::kState;
-  typedef Frag<typename Policy::out_t, VEC> OutIO;
   const int tpr = 1 << geo.tpr_shift;
   const int G = kBlock >> geo.tpr_shift;
   const int flane = (int)blockIdx.y * tpr + (threadIdx.x & (tpr - 1));
   const int f0 = flane * VEC;
   if (f0 >= geo.feat) return;
-  float o[VEC];
   if ((int)blockIdx.x < fix_blocks) {
     const int64_t q = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> geo.tpr_shift;
     if (q >= n_wg) return;
@@ -214,15 +225,13 @@ __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
     for (int i = 0; i < SF; ++i) acc[i] = p[i];
     for (int64_t w = q_lo + 1; w <= q; ++w)
       Policy::merge(acc, partial + ((w * 2) * geo.lanes_total + flane) * SF);
-    Policy::finish(acc, o);
-    OutIO::store(out + (int64_t)row * geo.feat + f0, o);
+    Policy::emit(args, out, row, geo.feat, f0, acc);
     (void)G;
   } else {
     const int64_t row =
         ((int64_t)(blockIdx.x - fix_blocks) * kBlock + threadIdx.x) >> geo.tpr_shift;
     if (row >= geo.n_rows || pointer[row] != pointer[row + 1]) return;
-    Policy::empty_row(o);
-    OutIO::store(out + row * geo.feat + f0, o);
+    Policy::emit_empty(args, out, row, geo.feat, f0);
   }
 }
 
@@ -270,7 +279,7 @@ int launch_runs(typename Policy::Args args, const int32_t *pointer,
   if (fix_blocks + fill_blocks > 0)
     hipLaunchKernelGGL((runs_fixup_kernel<Policy>),
                        dim3((unsigned)(fix_blocks + fill_blocks), ftiles),
-                       dim3(kBlock), 0, stream, pointer, row_of_slot, partial,
+                       dim3(kBlock), 0, stream, args, pointer, row_of_slot, partial,
                        (out_t *)out, geo, n_wg, (int)fix_blocks);
   return launch_status();
 }

@@ -58,6 +58,14 @@ struct SpmmPolicy {
     for (int v = 0; v < VEC; ++v) o[v] = st[v];
   }
   static __device__ __forceinline__ void empty_row(float (&o)[VEC]) { init(o); }
+  static __device__ __forceinline__ void emit(const Args &, out_t *out, int64_t row, int feat,
+                                              int f0, const float (&st)[kState]) {
+    emit_row<SpmmPolicy>(out, row, feat, f0, st);
+  }
+  static __device__ __forceinline__ void emit_empty(const Args &, out_t *out, int64_t row,
+                                                    int feat, int f0) {
+    emit_empty_row<SpmmPolicy>(out, row, feat, f0);
+  }
 
   template <class Close>
   static __device__ __forceinline__ void walk(const Args &A,
@@ -112,6 +120,152 @@ int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
   typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, feat,
                         partial, stream);
+}
+
+// max / min with the position of the extremum (the reference's generic kernel,
+// spmm.cuh:30-71 with functor.cuh:148-213): beside each running extremum the
+// state keeps the SLOT that produced it, so "first extremum in slot order wins"
+// survives every merge (a later partial replaces an earlier one only when
+// strictly better) and the ids are looked up once, when the row is written:
+// arg_u = neighbour id of that slot (operators that read u), arg_e = its edge id
+// (operators that read edge data).  Rows whose extremum was never replaced
+// (no edges, or only NaN / infinities of the wrong sign) report 0, as the
+// reference's zero-initialised locals do.
+template <typename T, int VEC, int RED, bool HASW>
+struct SpmmArgPolicy {
+  typedef T out_t;
+  static constexpr int kVec = VEC;
+  static constexpr int kState = 2 * VEC;
+  struct Args {
+    const int32_t *gidx;  // row of `u` gathered per slot; nullptr: the slot index
+    const int32_t *eid;   // edge id per slot; nullptr: the slot index
+    const int32_t *nbr;   // neighbour id per slot (for arg_u)
+    const T *u;
+    const float *w;
+    int32_t *arg_u;       // nullptr: not wanted
+    int32_t *arg_e;
+    int heads;
+    int dph;
+  };
+  static __device__ __forceinline__ void init(float (&st)[2 * VEC]) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      st[v] = red_init<RED>();
+      st[VEC + v] = __int_as_float(-1);
+    }
+  }
+  static __device__ __forceinline__ bool better(float acc, float m) {
+    return RED == GA_MAX ? acc < m : acc > m;
+  }
+  static __device__ __forceinline__ void merge(float (&dst)[2 * VEC], const float *src) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v)
+      if (better(dst[v], src[v])) {
+        dst[v] = src[v];
+        dst[VEC + v] = src[VEC + v];
+      }
+  }
+  static __device__ __forceinline__ void finish(const float (&st)[2 * VEC], float (&o)[VEC]) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o[v] = st[v];
+  }
+  static __device__ __forceinline__ void empty_row(float (&o)[VEC]) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o[v] = red_init<RED>();
+  }
+  static __device__ __forceinline__ void emit(const Args &A, out_t *out, int64_t row, int feat,
+                                              int f0, const float (&st)[2 * VEC]) {
+    emit_row<SpmmArgPolicy>(out, row, feat, f0, st);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      if (f0 + v >= feat) break;
+      const int slot = __float_as_int(st[VEC + v]);
+      if (A.arg_u) A.arg_u[row * feat + f0 + v] = slot < 0 ? 0 : A.nbr[slot];
+      if (A.arg_e) A.arg_e[row * feat + f0 + v] = slot < 0 ? 0 : (A.eid ? A.eid[slot] : slot);
+    }
+  }
+  static __device__ __forceinline__ void emit_empty(const Args &A, out_t *out, int64_t row,
+                                                    int feat, int f0) {
+    emit_empty_row<SpmmArgPolicy>(out, row, feat, f0);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      if (f0 + v >= feat) break;
+      if (A.arg_u) A.arg_u[row * feat + f0 + v] = 0;
+      if (A.arg_e) A.arg_e[row * feat + f0 + v] = 0;
+    }
+  }
+
+  template <class Close>
+  static __device__ __forceinline__ void walk(const Args &A,
+                                              const int32_t *__restrict__ row_of_slot,
+                                              int64_t a, int64_t b, int f0, int feat,
+                                              float (&st)[2 * VEC], int &cur,
+                                              Close &&close_segment) {
+    typedef Frag<T, VEC> IO;
+    const int h = HASW ? f0 / A.dph : 0;
+    for (int64_t j = a; j < b; j += kUnroll) {
+      int r[kUnroll];
+      int64_t g[kUnroll];
+      float ww[kUnroll];
+      typename IO::raw_t x[kUnroll];
+#pragma unroll
+      for (int t = 0; t < kUnroll; ++t) {
+        const int64_t jj = j + t < b ? j + t : b - 1;
+        r[t] = row_of_slot[jj];
+        g[t] = A.gidx ? (int64_t)A.gidx[jj] : jj;
+        if (HASW) {
+          const int64_t e = A.eid ? (int64_t)A.eid[jj] : jj;
+          ww[t] = A.w[e * A.heads + h];
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < kUnroll; ++t) x[t] = IO::load(A.u + g[t] * feat + f0);
+#pragma unroll
+      for (int t = 0; t < kUnroll; ++t) {
+        if (j + t < b) {
+          if (r[t] != cur) {
+            close_segment();
+            cur = r[t];
+            init(st);
+          }
+          float xf[VEC];
+          IO::widen(x[t], xf);
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const float m = HASW ? xf[v] * ww[t] : xf[v];
+            if (better(st[v], m)) {
+              st[v] = m;
+              st[VEC + v] = __int_as_float((int)(j + t));
+            }
+          }
+        }
+      }
+    }
+  }
+};
+
+template <typename T, int VEC>
+int launch_spmm_arg(int reduce, bool hasw, const int32_t *pointer,
+                    const int32_t *row_of_slot, const int32_t *gidx,
+                    const int32_t *eid, const int32_t *nbr, const void *u,
+                    const float *w, void *out, int32_t *arg_u, int32_t *arg_e,
+                    int64_t n_rows, int64_t n_edges, int feat, int heads,
+                    float *partial, hipStream_t stream) {
+#define GA_SPMM_ARG(RED, HASW)                                                     \
+  do {                                                                             \
+    typedef SpmmArgPolicy<T, VEC, RED, HASW> P;                                    \
+    typename P::Args args{gidx, eid, nbr, (const T *)u, w, arg_u, arg_e, heads,    \
+                          feat / heads};                                           \
+    return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, feat,  \
+                          partial, stream);                                        \
+  } while (0)
+  if (reduce == GA_MAX) {
+    if (hasw) GA_SPMM_ARG(GA_MAX, true);
+    GA_SPMM_ARG(GA_MAX, false);
+  }
+  if (hasw) GA_SPMM_ARG(GA_MIN, true);
+  GA_SPMM_ARG(GA_MIN, false);
+#undef GA_SPMM_ARG
 }
 
 template <typename T, int VEC, int RED>
@@ -234,6 +388,66 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
   return ga::pick_red<ga::bf16_t, 1>(reduce, hasw, pointer, row_of_slot, gidx,
                                      eid, u, w, out, n_rows, n_edges, (int)feat,
                                      (int)heads, partial, s);
+}
+
+size_t ga_spmm_arg_workspace_bytes(int64_t n_edges, int64_t feat) {
+  return ga::runs_workspace_bytes(n_edges, feat, 2);
+}
+
+int ga_spmm_csr_arg(const int32_t *pointer, const int32_t *row_of_slot,
+                    const int32_t *nbr, const int32_t *eid, const void *u,
+                    const float *w, void *out, int32_t *arg_u, int32_t *arg_e,
+                    int64_t n_rows, int64_t n_edges, int64_t feat, int64_t heads,
+                    int op, int reduce, int dtype, void *workspace,
+                    size_t workspace_bytes, ga_stream_t stream) {
+  if (n_rows < 0 || n_edges < 0 || feat <= 0 || heads <= 0 || feat % heads)
+    return GA_EINVAL;
+  if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || feat > 0x7fffffff)
+    return GA_EINVAL;
+  if (op < GA_COPY_U || op > GA_U_MUL_E) return GA_EINVAL;
+  if (reduce != GA_MAX && reduce != GA_MIN) return GA_EINVAL;   // sum has no position
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  // arg_u exists for operators that read u, arg_e for those that read edge data
+  if (op == GA_COPY_E && arg_u) return GA_EINVAL;
+  if (op == GA_COPY_U && arg_e) return GA_EINVAL;
+  if (n_rows == 0) return GA_OK;
+  if (!pointer || !out) return GA_EINVAL;
+  if (n_edges > 0) {
+    if (!row_of_slot || !u) return GA_EINVAL;
+    if (op != GA_COPY_E && !nbr) return GA_EINVAL;
+    if (op == GA_U_MUL_E && !w) return GA_EINVAL;
+    if (ga_spmm_arg_workspace_bytes(n_edges, feat) > workspace_bytes || !workspace)
+      return GA_EWORKSPACE;
+    if (!ga::aligned(workspace, 16)) return GA_EWORKSPACE;
+  }
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!ga::aligned(out, esz) || (u && !ga::aligned(u, esz)) ||
+      (w && !ga::aligned(w, 4)) || (arg_u && !ga::aligned(arg_u, 4)) ||
+      (arg_e && !ga::aligned(arg_e, 4)))
+    return GA_EALIGN;
+
+  const bool hasw = op == GA_U_MUL_E;
+  const int32_t *gidx = op == GA_COPY_E ? eid : nbr;
+  const int64_t dph = feat / heads;
+  const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
+  hipStream_t s = (hipStream_t)stream;
+  float *partial = (float *)workspace;
+  if (dtype == GA_F32) {
+    if (vec_ok && feat % 4 == 0 && (!hasw || dph % 4 == 0))
+      return ga::launch_spmm_arg<float, 4>(reduce, hasw, pointer, row_of_slot, gidx, eid,
+                                           nbr, u, w, out, arg_u, arg_e, n_rows, n_edges,
+                                           (int)feat, (int)heads, partial, s);
+    return ga::launch_spmm_arg<float, 1>(reduce, hasw, pointer, row_of_slot, gidx, eid, nbr,
+                                         u, w, out, arg_u, arg_e, n_rows, n_edges,
+                                         (int)feat, (int)heads, partial, s);
+  }
+  if (vec_ok && feat % 8 == 0 && (!hasw || dph % 8 == 0))
+    return ga::launch_spmm_arg<ga::bf16_t, 8>(reduce, hasw, pointer, row_of_slot, gidx, eid,
+                                              nbr, u, w, out, arg_u, arg_e, n_rows, n_edges,
+                                              (int)feat, (int)heads, partial, s);
+  return ga::launch_spmm_arg<ga::bf16_t, 1>(reduce, hasw, pointer, row_of_slot, gidx, eid,
+                                            nbr, u, w, out, arg_u, arg_e, n_rows, n_edges,
+                                            (int)feat, (int)heads, partial, s);
 }
 
 }  // extern "C"

@@ -17,9 +17,11 @@ from __future__ import annotations
 
 from typing import Optional, Sequence
 
+import numpy as np
 import torch
 
 from . import capi
+from .bcast import calc_bcast_off
 from .graph import DGLGraph
 
 _DTYPES = {torch.float32: capi.GA_F32, torch.bfloat16: capi.GA_BF16}
@@ -61,11 +63,15 @@ def _out_shape(rows: int, x: torch.Tensor):
 
 # ----------------------------------------------------------------- SpMM ----
 def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
-         w: Optional[torch.Tensor] = None, reverse: bool = False) -> torch.Tensor:
+         w: Optional[torch.Tensor] = None, reverse: bool = False,
+         return_arg: bool = False):
     """Generalised SpMM over the in-adjacency (``reverse``: the out-adjacency).
 
     op: "copy_u" (u is (N, ...)), "copy_e" (u is (E, ...)), "u_mul_e"
     (w is (E,), (E, 1) or (E, H) fp32).  reduce: "sum" | "max" | "min".
+    ``return_arg`` (max / min only): also return ``(arg_u, arg_e)``, the int32
+    neighbour id and edge id that supplied each output element (spmm.cuh:30-71);
+    the one the operator has no use for is None.
     """
     _check_input(u, "features")
     dt = _feat_dtype(u, "features")
@@ -88,11 +94,36 @@ def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
         heads = get_feat_dim(w)
         if feat % heads:
             raise RuntimeError("feature width is not a multiple of the heads")
+        if w.dim() == u.dim() and u.dim() >= 3:
+            # shaped operands, e.g. (N, H, D) * (E, H, 1): accept exactly the
+            # broadcasts that are "one weight per head" (bcast.cc:19-71 tables)
+            b = calc_bcast_off("mul", tuple(u.shape), tuple(w.shape))
+            per_head = np.arange(feat, dtype=np.int64) // (feat // heads)
+            if b.out_len != feat or not np.array_equal(b.lhs_offset, np.arange(feat)) \
+                    or not np.array_equal(b.rhs_offset, per_head):
+                raise RuntimeError("unsupported broadcast between features "
+                                   f"{tuple(u.shape)} and edge weights {tuple(w.shape)}")
     n_src = g.num_edges if op == "copy_e" else g.num_nodes
     if u.shape[0] != n_src:
         raise RuntimeError("features have the wrong number of rows")
     out = torch.empty(_out_shape(g.num_nodes, u), dtype=u.dtype, device=u.device)
     lib = capi.load()
+    if return_arg:
+        if reduce not in ("max", "min"):
+            raise RuntimeError("return_arg needs the max or the min reducer")
+        arg_u = arg_e = None
+        if op != "copy_e":
+            arg_u = torch.empty(out.shape, dtype=torch.int32, device=u.device)
+        if op != "copy_u":
+            arg_e = torch.empty(out.shape, dtype=torch.int32, device=u.device)
+        ws = g.workspace(lib.ga_spmm_arg_workspace_bytes(g.num_edges, feat))
+        capi.check(lib.ga_spmm_csr_arg(
+            pointer.data_ptr(), rows.data_ptr(), nbr.data_ptr(),
+            None if ident else eid.data_ptr(), u.data_ptr(), _ptr(w),
+            out.data_ptr(), _ptr(arg_u), _ptr(arg_e), g.num_nodes, g.num_edges,
+            feat, heads, code, _REDUCE[reduce], dt, ws.data_ptr(), ws.numel(),
+            _stream(u)), "ga_spmm_csr_arg")
+        return out, arg_u, arg_e
     ws_bytes = lib.ga_spmm_workspace_bytes(g.num_edges, feat)
     ws = g.workspace(ws_bytes)
     capi.check(lib.ga_spmm_csr(

@@ -83,6 +83,26 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
                 int64_t feat, int64_t heads, int op, int reduce, int dtype,
                 void *workspace, size_t workspace_bytes, ga_stream_t stream);
 
+/* SpMM with max / min and the position of each extremum: the arg_u / arg_e
+ * outputs of the reference's generic kernel (SpMMCsrKernel, spmm.cuh:30-71,
+ * reducers functor.cuh:148-213: strict comparison, so the first extremum in
+ * adjacency order wins; the locals start at 0, so a row whose extremum is never
+ * replaced - no edges, only NaN - reports 0).
+ *   arg_u  (n_rows, feat) int32 or NULL: neighbour id that supplied out[v, f];
+ *          COPY_U and U_MUL_E only (operators that read u)
+ *   arg_e  (n_rows, feat) int32 or NULL: edge id that supplied out[v, f];
+ *          COPY_E and U_MUL_E only (operators that read edge data)
+ *   reduce GA_MAX or GA_MIN; everything else as ga_spmm_csr
+ *   workspace  ga_spmm_arg_workspace_bytes() bytes, 16-byte aligned
+ */
+size_t ga_spmm_arg_workspace_bytes(int64_t n_edges, int64_t feat);
+int ga_spmm_csr_arg(const int32_t *pointer, const int32_t *row_of_slot,
+                    const int32_t *nbr, const int32_t *eid, const void *u,
+                    const float *w, void *out, int32_t *arg_u, int32_t *arg_e,
+                    int64_t n_rows, int64_t n_edges, int64_t feat, int64_t heads,
+                    int op, int reduce, int dtype, void *workspace,
+                    size_t workspace_bytes, ga_stream_t stream);
+
 /* ------------------------------------------------------------------ SDDMM --
  * out[i, k] = u[lhs[i], k] + v[rhs[i], k], fp32 output (E, feat).
  * Replaces SDDMMCoo_u_add_v_mul_alpha (sddmm.cu:118-129, kernel

@@ -90,6 +90,24 @@ def test_spmm_u_mul_e_sum_f32(graph, device, feat, heads, reverse):
     assert_close(got, ref, TOL_F32, f"u_mul_e {name} F={feat} H={heads}")
 
 
+def test_spmm_u_mul_e_shaped_operands(graph, device):
+    """(N, H, D) features with (E, H, 1) weights: the per-head broadcast of the
+    reference's shape tables; any other broadcast is rejected."""
+    name, g, arr = graph
+    rng = np.random.default_rng(11)
+    e = arr.COO_src.shape[0]
+    x = rng.standard_normal((arr.num_nodes, 4, 8), dtype=np.float32)
+    w = rng.standard_normal((e, 4, 1), dtype=np.float32)
+    got = ops.gspmm_src_mul_e_sum(_dev(x, device), _dev(w, device), [1], False, None, g)
+    assert tuple(got.shape) == (arr.num_nodes, 4, 8)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      x.reshape(arr.num_nodes, 32), w.reshape(e, 4), op="u_mul_e", heads=4)
+    assert_close(got.cpu().numpy().reshape(arr.num_nodes, 32), ref, TOL_F32, f"shaped {name}")
+    bad = rng.standard_normal((e, 1, 8), dtype=np.float32)      # per-feature, not per-head
+    with pytest.raises(RuntimeError, match="unsupported broadcast"):
+        ops.gspmm_src_mul_e_sum(_dev(x, device), _dev(bad, device), [1], False, None, g)
+
+
 @pytest.mark.parametrize("reduce", ["max", "min"])
 @pytest.mark.parametrize("op,feat,heads", [("copy_u", 64, 1), ("copy_u", 7, 1),
                                            ("copy_e", 32, 1),
@@ -107,6 +125,45 @@ def test_spmm_max_min_f32(graph, device, reduce, op, feat, heads):
                       x, w, op=op, reduce=reduce, heads=heads)
     # a max / min of fp32 products is exact: compare bit for bit
     assert np.array_equal(got, ref), f"{op} {reduce} {name}"
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+@pytest.mark.parametrize("op,feat,heads,bf16", [("copy_u", 64, 1, False), ("copy_u", 5, 1, False),
+                                                ("copy_e", 16, 1, False), ("u_mul_e", 32, 4, False),
+                                                ("u_mul_e", 6, 2, False), ("copy_u", 64, 1, True)])
+def test_spmm_arg_outputs_bit_exact(graph, device, reduce, op, feat, heads, bf16):
+    """Positions of the extrema: small-integer data (exact products, many ties)
+    so that "first extremum in adjacency order wins" decides most elements."""
+    name, g, arr = graph
+    rng = np.random.default_rng(feat + heads)
+    e = arr.COO_src.shape[0]
+    rows = e if op == "copy_e" else arr.num_nodes
+    x = rng.integers(-3, 4, size=(rows, feat)).astype(np.float32)
+    w = rng.integers(-2, 3, size=(e, heads)).astype(np.float32) if op == "u_mul_e" else None
+    out, arg_u, arg_e = ops.spmm(g, op, reduce, _dev(x, device, bf16),
+                                 None if w is None else _dev(w, device), return_arg=True)
+    ref, ref_u, ref_e = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                                    x, w, op=op, reduce=reduce, heads=heads, want_arg=True)
+    np.testing.assert_array_equal(out.float().cpu().numpy(), ref, err_msg=f"{name} values")
+    assert (arg_u is None) == (op == "copy_e") and (arg_e is None) == (op == "copy_u")
+    if arg_u is not None:
+        assert arg_u.dtype == torch.int32
+        np.testing.assert_array_equal(arg_u.cpu().numpy(), ref_u, err_msg=f"{name} arg_u")
+    if arg_e is not None:
+        np.testing.assert_array_equal(arg_e.cpu().numpy(), ref_e, err_msg=f"{name} arg_e")
+
+
+def test_spmm_arg_rejects_sum(graph, device):
+    name, g, arr = graph
+    x = torch.zeros((arr.num_nodes, 4), device=device)
+    with pytest.raises(RuntimeError, match="max or the min"):
+        ops.spmm(g, "copy_u", "sum", x, return_arg=True)
+    lib = capi.load()
+    rc = lib.ga_spmm_csr_arg(g.in_pointer.data_ptr(), g.in_row_of_slot.data_ptr(),
+                             g.in_node_indices.data_ptr(), None, x.data_ptr(), None,
+                             x.data_ptr(), None, None, arr.num_nodes, g.num_edges, 4, 1,
+                             capi.GA_COPY_U, capi.GA_SUM, capi.GA_F32, None, 0, None)
+    assert rc == capi.GA_EINVAL
 
 
 @pytest.mark.parametrize("feat,heads", [(64, 1), (128, 8), (256, 4), (24, 3),

@@ -128,3 +128,58 @@ def test_debug_graphs_match_fixture_file():
     assert arr.in_pointer.tolist() == [0, 1, 3, 6]
     assert arr.in_node_indices.tolist() == [0, 0, 1, 0, 1, 2]
     assert arr.in_edge_indices.tolist() == [0, 1, 3, 2, 4, 5]
+
+
+# ---- broadcast tables (bcast.cc) ------------------------------------------------
+
+def test_bcast_header_example():
+    """The worked example in the reference's bcast.h:24-35: feature shapes (1, 3)
+    and (5, 1) give a (5, 3) output and these two offset lists."""
+    from graphiler_amd.bcast import calc_bcast_off
+    b = calc_bcast_off("add", (7, 1, 3), (7, 5, 1))
+    assert b.use_bcast and (b.lhs_len, b.rhs_len, b.out_len, b.reduce_size) == (3, 5, 15, 1)
+    assert b.lhs_offset.tolist() == [0, 1, 2] * 5
+    assert b.rhs_offset.tolist() == [0, 0, 0, 1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4]
+
+
+def test_bcast_matches_numpy_broadcasting():
+    """Gathering through the tables must reproduce numpy's own broadcasting of
+    the per-row feature blocks (any mistake in stride or dimension order fails)."""
+    from graphiler_amd.bcast import calc_bcast_off
+    rng = np.random.default_rng(5)
+    cases = [((4, 3), (4, 1)), ((4, 1), (4, 6)), ((4, 2, 1, 5), (4, 1, 3, 5)),
+             ((4, 3, 5), (4, 5)), ((4, 5), (4, 2, 1)), ((4, 8, 16), (4, 8, 1)),
+             ((4, 2, 3, 4), (4, 3, 1))]
+    for ls, rs in cases:
+        lhs, rhs = rng.standard_normal(ls), rng.standard_normal(rs)
+        b = calc_bcast_off("mul", ls, rs)
+        assert b.use_bcast
+        for row in range(ls[0]):
+            want = (lhs[row] * rhs[row]).reshape(-1)
+            got = lhs[row].reshape(-1)[b.lhs_offset] * rhs[row].reshape(-1)[b.rhs_offset]
+            assert b.out_len == want.size
+            np.testing.assert_array_equal(got, want)
+
+
+def test_bcast_dot_and_plain_shapes():
+    from graphiler_amd.bcast import calc_bcast_off, use_bcast
+    # same shapes: no table, lengths only
+    b = calc_bcast_off("add", (9, 8, 16), (9, 8, 16))
+    assert not b.use_bcast and b.out_len == 128 and b.reduce_size == 1
+    assert b.lhs_offset.tolist() == [0] and b.rhs_offset.tolist() == [0]
+    # dot over the last dimension, heads kept (HGT's u_dot_v: (E, 8, 16) -> (E, 8))
+    b = calc_bcast_off("dot", (9, 8, 16), (9, 8, 16))
+    assert not b.use_bcast and b.out_len == 8 and b.reduce_size == 16
+    # copies never broadcast and take the length of the copied side
+    assert not use_bcast("copy_lhs", (3, 4), (3, 7, 2))
+    assert calc_bcast_off("copy_rhs", (3, 4), (3, 7, 2)).out_len == 14
+    # broadcast dot: (E, 1, 16) . (E, 8, 16) -> 8 outputs of 16-vectors; offsets
+    # count vectors, not elements
+    b = calc_bcast_off("dot", (9, 1, 16), (9, 8, 16))
+    assert b.use_bcast and b.reduce_size == 16 and b.out_len == 8
+    assert b.lhs_offset.tolist() == [0] * 8 and b.rhs_offset.tolist() == list(range(8))
+    rng = np.random.default_rng(6)
+    u, v = rng.standard_normal((1, 16)), rng.standard_normal((8, 16))
+    got = [(u.reshape(-1, 16)[b.lhs_offset[k]] * v.reshape(-1, 16)[b.rhs_offset[k]]).sum()
+           for k in range(b.out_len)]
+    np.testing.assert_allclose(got, (u * v).sum(-1))
