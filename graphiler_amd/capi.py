@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libgraphiler_hip.so")
 GA_OK = 0
 GA_EINVAL, GA_EUNSUPPORTED, GA_EWORKSPACE, GA_EALIGN = -1, -2, -3, -4
 GA_F32, GA_BF16 = 0, 1
-GA_COPY_U, GA_COPY_E, GA_U_MUL_E = 0, 1, 2
+GA_COPY_U, GA_COPY_E, GA_U_MUL_E, GA_U_ADD_E, GA_U_SUB_E, GA_U_DIV_E = 0, 1, 2, 3, 4, 5
 GA_SUM, GA_MAX, GA_MIN = 0, 1, 2
 
 _vp, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t

@@ -30,9 +30,21 @@ __device__ __forceinline__ float red_apply(float acc, float m) {
   return acc > m ? m : acc;
 }
 
+// Binary operator between the gathered feature and the edge datum
+// (functor.cuh:19-100): 0 = none (copy), else GA_U_MUL_E .. GA_U_DIV_E.
+template <int BOP>
+__device__ __forceinline__ float bin_apply(float x, float w) {
+  if (BOP == GA_U_MUL_E) return x * w;
+  if (BOP == GA_U_ADD_E) return x + w;
+  if (BOP == GA_U_SUB_E) return x - w;
+  if (BOP == GA_U_DIV_E) return x / w;
+  return x;
+}
+
 // Row-reduction policy of the SpMM: the state is the VEC running reductions.
-template <typename T, int VEC, int RED, bool HASW>
+template <typename T, int VEC, int RED, int BOP>
 struct SpmmPolicy {
+  static constexpr bool HASW = BOP != 0;
   typedef T out_t;
   static constexpr int kVec = VEC;
   static constexpr int kState = VEC;
@@ -104,19 +116,19 @@ struct SpmmPolicy {
           IO::widen(x[t], xf);
 #pragma unroll
           for (int v = 0; v < VEC; ++v)
-            st[v] = red_apply<RED>(st[v], HASW ? xf[v] * ww[t] : xf[v]);
+            st[v] = red_apply<RED>(st[v], bin_apply<BOP>(xf[v], ww[t]));
         }
       }
     }
   }
 };
 
-template <typename T, int VEC, int RED, bool HASW>
+template <typename T, int VEC, int RED, int BOP>
 int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
                 const int32_t *gidx, const int32_t *eid, const void *u,
                 const float *w, void *out, int64_t n_rows, int64_t n_edges,
                 int feat, int heads, float *partial, hipStream_t stream) {
-  typedef SpmmPolicy<T, VEC, RED, HASW> P;
+  typedef SpmmPolicy<T, VEC, RED, BOP> P;
   typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, feat,
                         partial, stream);
@@ -131,8 +143,9 @@ int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
 // (operators that read edge data).  Rows whose extremum was never replaced
 // (no edges, or only NaN / infinities of the wrong sign) report 0, as the
 // reference's zero-initialised locals do.
-template <typename T, int VEC, int RED, bool HASW>
+template <typename T, int VEC, int RED, int BOP>
 struct SpmmArgPolicy {
+  static constexpr bool HASW = BOP != 0;
   typedef T out_t;
   static constexpr int kVec = VEC;
   static constexpr int kState = 2 * VEC;
@@ -232,7 +245,7 @@ struct SpmmArgPolicy {
           IO::widen(x[t], xf);
 #pragma unroll
           for (int v = 0; v < VEC; ++v) {
-            const float m = HASW ? xf[v] * ww[t] : xf[v];
+            const float m = bin_apply<BOP>(xf[v], ww[t]);
             if (better(st[v], m)) {
               st[v] = m;
               st[VEC + v] = __int_as_float((int)(j + t));
@@ -245,59 +258,69 @@ struct SpmmArgPolicy {
 };
 
 template <typename T, int VEC>
-int launch_spmm_arg(int reduce, bool hasw, const int32_t *pointer,
+int launch_spmm_arg(int reduce, int bop, const int32_t *pointer,
                     const int32_t *row_of_slot, const int32_t *gidx,
                     const int32_t *eid, const int32_t *nbr, const void *u,
                     const float *w, void *out, int32_t *arg_u, int32_t *arg_e,
                     int64_t n_rows, int64_t n_edges, int feat, int heads,
                     float *partial, hipStream_t stream) {
-#define GA_SPMM_ARG(RED, HASW)                                                     \
+#define GA_SPMM_ARG(RED, B)                                                        \
   do {                                                                             \
-    typedef SpmmArgPolicy<T, VEC, RED, HASW> P;                                    \
+    typedef SpmmArgPolicy<T, VEC, RED, B> P;                                       \
     typename P::Args args{gidx, eid, nbr, (const T *)u, w, arg_u, arg_e, heads,    \
                           feat / heads};                                           \
     return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, feat,  \
                           partial, stream);                                        \
   } while (0)
-  if (reduce == GA_MAX) {
-    if (hasw) GA_SPMM_ARG(GA_MAX, true);
-    GA_SPMM_ARG(GA_MAX, false);
+#define GA_SPMM_ARG_RED(RED)                                                       \
+  switch (bop) {                                                                   \
+    case GA_U_MUL_E: GA_SPMM_ARG(RED, GA_U_MUL_E);                                 \
+    case GA_U_ADD_E: GA_SPMM_ARG(RED, GA_U_ADD_E);                                 \
+    case GA_U_SUB_E: GA_SPMM_ARG(RED, GA_U_SUB_E);                                 \
+    case GA_U_DIV_E: GA_SPMM_ARG(RED, GA_U_DIV_E);                                 \
+    default: GA_SPMM_ARG(RED, 0);                                                  \
   }
-  if (hasw) GA_SPMM_ARG(GA_MIN, true);
-  GA_SPMM_ARG(GA_MIN, false);
+  if (reduce == GA_MAX) GA_SPMM_ARG_RED(GA_MAX)
+  GA_SPMM_ARG_RED(GA_MIN)
+#undef GA_SPMM_ARG_RED
 #undef GA_SPMM_ARG
 }
 
 template <typename T, int VEC, int RED>
-int pick_w(bool hasw, const int32_t *pointer, const int32_t *row_of_slot,
+int pick_w(int bop, const int32_t *pointer, const int32_t *row_of_slot,
            const int32_t *gidx, const int32_t *eid, const void *u,
            const float *w, void *out, int64_t n_rows, int64_t n_edges, int feat,
            int heads, float *partial, hipStream_t stream) {
-  return hasw ? launch_spmm<T, VEC, RED, true>(pointer, row_of_slot, gidx, eid,
-                                                u, w, out, n_rows, n_edges, feat,
-                                                heads, partial, stream)
-              : launch_spmm<T, VEC, RED, false>(pointer, row_of_slot, gidx, eid,
-                                                 u, w, out, n_rows, n_edges,
-                                                 feat, heads, partial, stream);
+#define GA_SPMM_BOP(B)                                                             \
+  return launch_spmm<T, VEC, RED, B>(pointer, row_of_slot, gidx, eid, u, w, out,   \
+                                     n_rows, n_edges, feat, heads, partial, stream)
+  switch (bop) {
+    case GA_U_MUL_E: GA_SPMM_BOP(GA_U_MUL_E);
+    case GA_U_ADD_E: GA_SPMM_BOP(GA_U_ADD_E);
+    case GA_U_SUB_E: GA_SPMM_BOP(GA_U_SUB_E);
+    case GA_U_DIV_E: GA_SPMM_BOP(GA_U_DIV_E);
+    default: GA_SPMM_BOP(0);
+  }
+#undef GA_SPMM_BOP
 }
 
 template <typename T, int VEC>
-int pick_red(int reduce, bool hasw, const int32_t *pointer,
+int pick_red(int reduce, int bop, const int32_t *pointer,
              const int32_t *row_of_slot, const int32_t *gidx,
              const int32_t *eid, const void *u, const float *w, void *out,
              int64_t n_rows, int64_t n_edges, int feat, int heads,
              float *partial, hipStream_t stream) {
   switch (reduce) {
     case GA_SUM:
-      return pick_w<T, VEC, GA_SUM>(hasw, pointer, row_of_slot, gidx, eid, u, w,
+      return pick_w<T, VEC, GA_SUM>(bop, pointer, row_of_slot, gidx, eid, u, w,
                                     out, n_rows, n_edges, feat, heads, partial,
                                     stream);
     case GA_MAX:
-      return pick_w<T, VEC, GA_MAX>(hasw, pointer, row_of_slot, gidx, eid, u, w,
+      return pick_w<T, VEC, GA_MAX>(bop, pointer, row_of_slot, gidx, eid, u, w,
                                     out, n_rows, n_edges, feat, heads, partial,
                                     stream);
     default:
-      return pick_w<T, VEC, GA_MIN>(hasw, pointer, row_of_slot, gidx, eid, u, w,
+      return pick_w<T, VEC, GA_MIN>(bop, pointer, row_of_slot, gidx, eid, u, w,
                                     out, n_rows, n_edges, feat, heads, partial,
                                     stream);
   }
@@ -348,7 +371,7 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
     return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || feat > 0x7fffffff)
     return GA_EINVAL;
-  if (op < GA_COPY_U || op > GA_U_MUL_E || reduce < GA_SUM || reduce > GA_MIN)
+  if (op < GA_COPY_U || op > GA_U_DIV_E || reduce < GA_SUM || reduce > GA_MIN)
     return GA_EINVAL;
   if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
   if (n_rows == 0) return GA_OK;
@@ -356,7 +379,7 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
   if (n_edges > 0) {
     if (!row_of_slot || !u) return GA_EINVAL;
     if (op != GA_COPY_E && !nbr) return GA_EINVAL;
-    if (op == GA_U_MUL_E && !w) return GA_EINVAL;
+    if (op >= GA_U_MUL_E && !w) return GA_EINVAL;
     if (ga_spmm_workspace_bytes(n_edges, feat) > workspace_bytes || !workspace)
       return GA_EWORKSPACE;
     if (!ga::aligned(workspace, 16)) return GA_EWORKSPACE;
@@ -366,7 +389,8 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
       (w && !ga::aligned(w, 4)))
     return GA_EALIGN;
 
-  const bool hasw = op == GA_U_MUL_E;
+  const bool hasw = op >= GA_U_MUL_E;
+  const int bop = hasw ? op : 0;
   const int32_t *gidx = op == GA_COPY_E ? eid : nbr;
   const int64_t dph = feat / heads;
   const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
@@ -374,18 +398,18 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
   float *partial = (float *)workspace;
   if (dtype == GA_F32) {
     if (vec_ok && feat % 4 == 0 && (!hasw || dph % 4 == 0))
-      return ga::pick_red<float, 4>(reduce, hasw, pointer, row_of_slot, gidx,
+      return ga::pick_red<float, 4>(reduce, bop, pointer, row_of_slot, gidx,
                                     eid, u, w, out, n_rows, n_edges, (int)feat,
                                     (int)heads, partial, s);
-    return ga::pick_red<float, 1>(reduce, hasw, pointer, row_of_slot, gidx, eid,
+    return ga::pick_red<float, 1>(reduce, bop, pointer, row_of_slot, gidx, eid,
                                   u, w, out, n_rows, n_edges, (int)feat,
                                   (int)heads, partial, s);
   }
   if (vec_ok && feat % 8 == 0 && (!hasw || dph % 8 == 0))
-    return ga::pick_red<ga::bf16_t, 8>(reduce, hasw, pointer, row_of_slot, gidx,
+    return ga::pick_red<ga::bf16_t, 8>(reduce, bop, pointer, row_of_slot, gidx,
                                        eid, u, w, out, n_rows, n_edges,
                                        (int)feat, (int)heads, partial, s);
-  return ga::pick_red<ga::bf16_t, 1>(reduce, hasw, pointer, row_of_slot, gidx,
+  return ga::pick_red<ga::bf16_t, 1>(reduce, bop, pointer, row_of_slot, gidx,
                                      eid, u, w, out, n_rows, n_edges, (int)feat,
                                      (int)heads, partial, s);
 }
@@ -404,7 +428,7 @@ int ga_spmm_csr_arg(const int32_t *pointer, const int32_t *row_of_slot,
     return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || feat > 0x7fffffff)
     return GA_EINVAL;
-  if (op < GA_COPY_U || op > GA_U_MUL_E) return GA_EINVAL;
+  if (op < GA_COPY_U || op > GA_U_DIV_E) return GA_EINVAL;
   if (reduce != GA_MAX && reduce != GA_MIN) return GA_EINVAL;   // sum has no position
   if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
   // arg_u exists for operators that read u, arg_e for those that read edge data
@@ -415,7 +439,7 @@ int ga_spmm_csr_arg(const int32_t *pointer, const int32_t *row_of_slot,
   if (n_edges > 0) {
     if (!row_of_slot || !u) return GA_EINVAL;
     if (op != GA_COPY_E && !nbr) return GA_EINVAL;
-    if (op == GA_U_MUL_E && !w) return GA_EINVAL;
+    if (op >= GA_U_MUL_E && !w) return GA_EINVAL;
     if (ga_spmm_arg_workspace_bytes(n_edges, feat) > workspace_bytes || !workspace)
       return GA_EWORKSPACE;
     if (!ga::aligned(workspace, 16)) return GA_EWORKSPACE;
@@ -426,7 +450,8 @@ int ga_spmm_csr_arg(const int32_t *pointer, const int32_t *row_of_slot,
       (arg_e && !ga::aligned(arg_e, 4)))
     return GA_EALIGN;
 
-  const bool hasw = op == GA_U_MUL_E;
+  const bool hasw = op >= GA_U_MUL_E;
+  const int bop = hasw ? op : 0;
   const int32_t *gidx = op == GA_COPY_E ? eid : nbr;
   const int64_t dph = feat / heads;
   const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
@@ -434,18 +459,18 @@ int ga_spmm_csr_arg(const int32_t *pointer, const int32_t *row_of_slot,
   float *partial = (float *)workspace;
   if (dtype == GA_F32) {
     if (vec_ok && feat % 4 == 0 && (!hasw || dph % 4 == 0))
-      return ga::launch_spmm_arg<float, 4>(reduce, hasw, pointer, row_of_slot, gidx, eid,
+      return ga::launch_spmm_arg<float, 4>(reduce, bop, pointer, row_of_slot, gidx, eid,
                                            nbr, u, w, out, arg_u, arg_e, n_rows, n_edges,
                                            (int)feat, (int)heads, partial, s);
-    return ga::launch_spmm_arg<float, 1>(reduce, hasw, pointer, row_of_slot, gidx, eid, nbr,
+    return ga::launch_spmm_arg<float, 1>(reduce, bop, pointer, row_of_slot, gidx, eid, nbr,
                                          u, w, out, arg_u, arg_e, n_rows, n_edges,
                                          (int)feat, (int)heads, partial, s);
   }
   if (vec_ok && feat % 8 == 0 && (!hasw || dph % 8 == 0))
-    return ga::launch_spmm_arg<ga::bf16_t, 8>(reduce, hasw, pointer, row_of_slot, gidx, eid,
+    return ga::launch_spmm_arg<ga::bf16_t, 8>(reduce, bop, pointer, row_of_slot, gidx, eid,
                                               nbr, u, w, out, arg_u, arg_e, n_rows, n_edges,
                                               (int)feat, (int)heads, partial, s);
-  return ga::launch_spmm_arg<ga::bf16_t, 1>(reduce, hasw, pointer, row_of_slot, gidx, eid,
+  return ga::launch_spmm_arg<ga::bf16_t, 1>(reduce, bop, pointer, row_of_slot, gidx, eid,
                                             nbr, u, w, out, arg_u, arg_e, n_rows, n_edges,
                                             (int)feat, (int)heads, partial, s);
 }

@@ -173,7 +173,7 @@ torch::Tensor spmm(const GraphPtr &g, int op, int reduce, const torch::Tensor &u
   const torch::Tensor &eid = reverse ? g->out_edge_indices : g->in_edge_indices;
   const int64_t feat = feat_dim(u);
   int64_t heads = 1;
-  if (op == GA_U_MUL_E) {
+  if (op >= GA_U_MUL_E) {
     TORCH_CHECK(w.has_value(), "edge weights are required");
     check_input(w.value(), "edge weights");
     TORCH_CHECK(w.value().scalar_type() == at::kFloat, "edge weights must be float32");
@@ -228,7 +228,8 @@ torch::Tensor dst_mul_e_sum(torch::Tensor ufeature, torch::Tensor efeature,
 torch::Tensor gspmm(torch::Tensor ufeature, at::optional<torch::Tensor> efeature,
                     std::string op, std::string reduce, const GraphPtr &graph) {
   int o = op == "copy_u" ? GA_COPY_U : op == "copy_e" ? GA_COPY_E
-          : op == "u_mul_e" ? GA_U_MUL_E : -1;
+          : op == "u_mul_e" ? GA_U_MUL_E : op == "u_add_e" ? GA_U_ADD_E
+          : op == "u_sub_e" ? GA_U_SUB_E : op == "u_div_e" ? GA_U_DIV_E : -1;
   int r = reduce == "sum" ? GA_SUM : reduce == "max" ? GA_MAX
           : reduce == "min" ? GA_MIN : -1;
   TORCH_CHECK(o >= 0, "Unsupported SpMM binary operator: ", op);

@@ -67,8 +67,9 @@ def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
          return_arg: bool = False):
     """Generalised SpMM over the in-adjacency (``reverse``: the out-adjacency).
 
-    op: "copy_u" (u is (N, ...)), "copy_e" (u is (E, ...)), "u_mul_e"
-    (w is (E,), (E, 1) or (E, H) fp32).  reduce: "sum" | "max" | "min".
+    op: "copy_u" (u is (N, ...)), "copy_e" (u is (E, ...)), "u_mul_e" /
+    "u_add_e" / "u_sub_e" / "u_div_e" (functor.cuh:19-72; w is (E,), (E, 1) or
+    (E, H) fp32).  reduce: "sum" | "max" | "min".
     ``return_arg`` (max / min only): also return ``(arg_u, arg_e)``, the int32
     neighbour id and edge id that supplied each output element (spmm.cuh:30-71);
     the one the operator has no use for is None.
@@ -84,8 +85,9 @@ def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
     feat = get_feat_dim(u)
     heads = 1
     code = {"copy_u": capi.GA_COPY_U, "copy_e": capi.GA_COPY_E,
-            "u_mul_e": capi.GA_U_MUL_E}[op]
-    if op == "u_mul_e":
+            "u_mul_e": capi.GA_U_MUL_E, "u_add_e": capi.GA_U_ADD_E,
+            "u_sub_e": capi.GA_U_SUB_E, "u_div_e": capi.GA_U_DIV_E}[op]
+    if code >= capi.GA_U_MUL_E:
         _check_input(w, "edge weights")
         if w.dtype != torch.float32:
             raise RuntimeError("edge weights must be float32")

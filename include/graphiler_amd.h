@@ -41,7 +41,10 @@ typedef void *ga_stream_t;
 
 enum ga_dtype { GA_F32 = 0, GA_BF16 = 1 };
 /* message = u[nbr] | e[eid] | u[nbr] * w[eid]   (functor.cuh:18-121)         */
-enum ga_spmm_op { GA_COPY_U = 0, GA_COPY_E = 1, GA_U_MUL_E = 2 };
+enum ga_spmm_op {
+  GA_COPY_U = 0, GA_COPY_E = 1,
+  GA_U_MUL_E = 2, GA_U_ADD_E = 3, GA_U_SUB_E = 4, GA_U_DIV_E = 5 /* u[src] (op) w[edge] */
+};
 /* functor.cuh:125-213: sum starts at 0, max at -inf, min at +inf             */
 enum ga_reduce { GA_SUM = 0, GA_MAX = 1, GA_MIN = 2 };
 
@@ -65,13 +68,14 @@ int ga_csr_row_ids(const int32_t *pointer, int64_t n_rows, int64_t n_edges,
  * Replaces SpMMSrc (spmm.cu:375-389; op GA_COPY_U, gather by nbr),
  * SpMMEdge (spmm.cu:359-373; op GA_COPY_E, gather rows of the (E, feat) matrix
  * `u` by eid), src_mul_e_sum / dst_mul_e_sum (spmm.cu:286-356; op GA_U_MUL_E,
- * pass the in- or the out-adjacency) and the generic SpMMCsrKernel with the
- * Max / Min reducers (spmm.cuh:30-71).
+ * pass the in- or the out-adjacency) and the generic SpMMCsrKernel with its
+ * add / sub / mul / div binary operators (functor.cuh:19-72; GA_U_ADD_E ..
+ * GA_U_DIV_E, w per head like U_MUL_E) and Max / Min reducers (spmm.cuh:30-71).
  *   pointer      (n_rows+1) int32     nbr (n_edges) int32, unused for COPY_E
  *   row_of_slot  (n_edges)  int32     from ga_csr_row_ids
  *   eid          (n_edges)  int32 or NULL when eid[i] == i
  *   u            (n_src, feat)  or (n_edges, feat) for COPY_E, `dtype`
- *   w            (n_edges, heads) fp32, U_MUL_E only; feat % heads == 0
+ *   w            (n_edges, heads) fp32, the U_*_E operators only; feat % heads == 0
  *   out          (n_rows, feat) `dtype`; every row is written (rows without
  *                edges get 0, -inf or +inf by reducer)
  *   workspace    ga_spmm_workspace_bytes() bytes, 16-byte aligned

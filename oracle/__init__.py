@@ -21,7 +21,8 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 OP_COPY_U, OP_COPY_E, OP_U_MUL_E = 0, 1, 2
 RED_SUM, RED_MAX, RED_MIN = 0, 1, 2
-_OPS = {"copy_u": OP_COPY_U, "copy_e": OP_COPY_E, "u_mul_e": OP_U_MUL_E}
+_OPS = {"copy_u": OP_COPY_U, "copy_e": OP_COPY_E, "u_mul_e": OP_U_MUL_E,
+        "u_add_e": 3, "u_sub_e": 4, "u_div_e": 5}
 _REDS = {"sum": RED_SUM, "max": RED_MAX, "min": RED_MIN}
 
 

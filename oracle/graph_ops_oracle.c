@@ -36,7 +36,10 @@
 #define ORC_OK 0
 #define ORC_EINVAL (-1)
 
-enum { ORC_OP_COPY_U = 0, ORC_OP_COPY_E = 1, ORC_OP_U_MUL_E = 2 };
+enum {
+  ORC_OP_COPY_U = 0, ORC_OP_COPY_E = 1, ORC_OP_U_MUL_E = 2,
+  ORC_OP_U_ADD_E = 3, ORC_OP_U_SUB_E = 4, ORC_OP_U_DIV_E = 5 /* functor.cuh:19-72 */
+};
 enum { ORC_RED_SUM = 0, ORC_RED_MAX = 1, ORC_RED_MIN = 2 };
 
 int orc_num_threads(void) {
@@ -127,7 +130,7 @@ int orc_spmm(int64_t n_rows, const int32_t *ptr, const int32_t *nbr,
              int32_t *arg_u, int32_t *arg_e, int64_t feat, int64_t heads,
              int op, int reduce) {
   if (feat <= 0 || heads <= 0 || feat % heads) return ORC_EINVAL;
-  if (op < 0 || op > 2 || reduce < 0 || reduce > 2) return ORC_EINVAL;
+  if (op < 0 || op > 5 || reduce < 0 || reduce > 2) return ORC_EINVAL;
   const int64_t dph = feat / heads;
 #pragma omp parallel
   {
@@ -151,8 +154,14 @@ int orc_spmm(int64_t n_rows, const int32_t *ptr, const int32_t *nbr,
             m = u[c * feat + f];
           else if (op == ORC_OP_COPY_E)
             m = u[e * feat + f];
-          else /* one fp32 product, as the device computes it */
+          else if (op == ORC_OP_U_MUL_E)
             m = (double)u[c * feat + f] * (double)w[e * heads + f / dph];
+          else if (op == ORC_OP_U_ADD_E)
+            m = (double)u[c * feat + f] + (double)w[e * heads + f / dph];
+          else if (op == ORC_OP_U_SUB_E)
+            m = (double)u[c * feat + f] - (double)w[e * heads + f / dph];
+          else
+            m = (double)u[c * feat + f] / (double)w[e * heads + f / dph];
           if (reduce == ORC_RED_SUM) {
             acc[f] += m;
           } else if ((reduce == ORC_RED_MAX && acc[f] < m) ||

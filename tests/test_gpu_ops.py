@@ -90,6 +90,26 @@ def test_spmm_u_mul_e_sum_f32(graph, device, feat, heads, reverse):
     assert_close(got, ref, TOL_F32, f"u_mul_e {name} F={feat} H={heads}")
 
 
+@pytest.mark.parametrize("op", ["u_add_e", "u_sub_e", "u_div_e"])
+@pytest.mark.parametrize("reduce", ["sum", "max", "min"])
+@pytest.mark.parametrize("feat,heads,bf16", [(64, 4, False), (6, 2, False), (64, 1, True)])
+def test_spmm_add_sub_div(graph, device, op, reduce, feat, heads, bf16):
+    name, g, arr = graph
+    rng = np.random.default_rng(feat + 3 * heads)
+    e = arr.COO_src.shape[0]
+    x = rng.standard_normal((arr.num_nodes, feat), dtype=np.float32)
+    w = (rng.uniform(0.5, 2.0, (e, heads)) * rng.choice([-1, 1], (e, heads))).astype(np.float32)
+    if bf16:
+        x = to_bf16_f32(x)
+    got = ops.spmm(g, op, reduce, _dev(x, device, bf16), _dev(w, device)).float().cpu().numpy()
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices, x, w,
+                      op=op, reduce=reduce, heads=heads)
+    finite = np.isfinite(ref)
+    assert np.array_equal(np.isfinite(got), finite), f"{name}: empty rows differ"
+    assert_close(np.where(finite, got, 0), np.where(finite, ref, 0),
+                 TOL_BF16 if bf16 else TOL_F32, f"{op} {reduce} {name}")
+
+
 def test_spmm_u_mul_e_shaped_operands(graph, device):
     """(N, H, D) features with (E, H, 1) weights: the per-head broadcast of the
     reference's shape tables; any other broadcast is rejected."""

@@ -199,6 +199,37 @@ def test_spmm_max_min_against_reduceat_and_ties():
 
 
 # ----------------------------------------------------------------- SDDMM ----
+def test_spmm_add_sub_div_against_scatter_and_reduceat():
+    """The other binary operators of the generic kernel (functor.cuh:19-72):
+    sum against np.add.at on explicitly formed messages (operand order and the
+    per-head broadcast of w matter for sub / div), max against reduceat."""
+    rng = np.random.default_rng(15)
+    n, s, d, ptr, nbr, eid = _graph(rng, "skewed")
+    e, H, D = s.shape[0], 2, 3
+    x = rng.standard_normal((n, H, D)).astype(np.float32)
+    w = (rng.uniform(0.5, 2.0, (e, H)) * rng.choice([-1, 1], (e, H))).astype(np.float32)
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)[:, :, None]
+    forms = {"u_add_e": x64[s] + w64, "u_sub_e": x64[s] - w64, "u_div_e": x64[s] / w64}
+    nonempty = np.diff(ptr) > 0
+    for op, msg in forms.items():
+        want = np.zeros((n, H, D))
+        np.add.at(want, d, msg)
+        got = oracle.spmm(ptr, nbr, eid, x.reshape(n, H * D), w, op=op, heads=H)
+        np.testing.assert_allclose(got, want.reshape(n, H * D), rtol=1e-5, atol=1e-5, err_msg=op)
+        grouped = msg.reshape(e, H * D)[eid]                 # messages in group order
+        wmax = np.full((n, H * D), -np.inf)
+        wmax[nonempty] = np.maximum.reduceat(grouped, ptr[:-1][nonempty], axis=0)
+        gmax = oracle.spmm(ptr, nbr, eid, x.reshape(n, H * D), w, op=op, reduce="max", heads=H)
+        np.testing.assert_allclose(gmax, wmax.astype(np.float32), rtol=1e-6, err_msg=op)
+    # u_sub_e is not e_sub_u, u_div_e is not e_div_u
+    a = oracle.spmm(ptr, nbr, eid, x.reshape(n, H * D), w, op="u_sub_e", heads=H)
+    b = oracle.spmm(ptr, nbr, eid, x.reshape(n, H * D), w, op="u_add_e", heads=H)
+    deg_w = np.zeros((n, H))
+    np.add.at(deg_w, d, w.astype(np.float64))
+    np.testing.assert_allclose((b - a).reshape(n, H, D), 2 * deg_w[:, :, None] * np.ones(D),
+                               rtol=1e-4, atol=1e-4)
+
+
 def test_sddmm_against_numpy_indexing():
     rng = np.random.default_rng(6)
     n, s, d, *_ = _graph(rng)
