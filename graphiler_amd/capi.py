@@ -26,6 +26,8 @@ SIGNATURES = {
     "ga_version": (_int, []),
     "ga_error_string": (ctypes.c_char_p, [_int]),
     "ga_csr_row_ids": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "ga_group_edges_workspace_bytes": (_sz, [_i64, _i64]),
+    "ga_group_edges": (_int, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "ga_spmm_workspace_bytes": (_sz, [_i64, _i64]),
     "ga_spmm_csr": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                            _i64, _int, _int, _int, _vp, _sz, _vp]),

@@ -206,26 +206,75 @@ class DGLGraph:
         return ws
 
 
+def group_on_device(key: torch.Tensor, other: Optional[torch.Tensor], n_keys: int):
+    """Stable grouping of item ids by ``key`` on the GPU (setup.py:116-146):
+    returns (pointer int32 (n_keys+1), other[order] int32 or None, order int32,
+    status int32 (1,)).  ``status`` is left on the device: 1 means a key outside
+    [0, n_keys); read it when convenient."""
+    from . import capi
+    if key.dtype != torch.int64 or not key.is_cuda or not key.is_contiguous():
+        raise RuntimeError("key must be a contiguous int64 CUDA tensor")
+    if other is not None and (other.dtype != torch.int64 or other.shape != key.shape
+                              or not other.is_cuda or not other.is_contiguous()):
+        raise RuntimeError("other must match key (contiguous int64 CUDA tensor)")
+    n, dev = int(key.numel()), key.device
+    if n >= 2 ** 31 or n_keys >= 2 ** 31 - 1:
+        raise ValueError("graphs are limited to int32 node and edge ids")
+    lib = capi.load()
+    pointer = torch.empty(n_keys + 1, dtype=torch.int32, device=dev)
+    order = torch.empty(n, dtype=torch.int32, device=dev)
+    nbr = torch.empty(n, dtype=torch.int32, device=dev) if other is not None else None
+    status = torch.empty(1, dtype=torch.int32, device=dev)
+    ws = torch.empty(max(int(lib.ga_group_edges_workspace_bytes(n_keys, n)), 256),
+                     dtype=torch.uint8, device=dev)
+    capi.check(lib.ga_group_edges(
+        key.data_ptr(), None if other is None else other.data_ptr(), n_keys, n,
+        pointer.data_ptr(), None if nbr is None else nbr.data_ptr(), order.data_ptr(),
+        status.data_ptr(), ws.data_ptr(), ws.numel(),
+        torch.cuda.current_stream(dev).cuda_stream), "ga_group_edges")
+    return pointer, nbr, order, status
+
+
+def _type_columns(type_of, num_types: int, dev):
+    """Type pointer + type COO column on the device; items must be sorted by
+    type (ids of one type contiguous, include/dglgraph.h:68-69)."""
+    t = torch.as_tensor(np.ascontiguousarray(type_of, dtype=np.int64)).to(dev)
+    pointer, _, _, status = group_on_device(t, None, num_types)
+    unsorted = bool((t[1:] < t[:-1]).any().item()) if t.numel() > 1 else False
+    if unsorted:
+        raise ValueError("items must be sorted by type")
+    if int(status.item()):
+        raise ValueError("type outside [0, num_types)")
+    return pointer, t
+
+
 def prepare_graph(src, dst, num_nodes: int, device="cuda:0",
                   ntype_of=None, num_ntypes: int = 0, etype_of=None,
                   num_etypes: int = 0) -> DGLGraph:
     """Build the device graph from an edge list (setup.py:116-146); when type
     columns are given also install the type pointers and type COO columns the
-    way load_data does for heterogeneous graphs (setup.py:87-100)."""
-    arr = build_graph_arrays(src, dst, num_nodes)
+    way load_data does for heterogeneous graphs (setup.py:87-100).  The edge
+    list is uploaded once and grouped on the GPU (both adjacencies and the type
+    pointers); nothing is sorted on the host."""
     dev = torch.device(device)
-
-    def up(a):
-        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-
-    g = DGLGraph(up(arr.in_pointer), up(arr.in_node_indices),
-                 up(arr.in_edge_indices), up(arr.out_pointer),
-                 up(arr.out_node_indices), up(arr.out_edge_indices),
-                 up(arr.COO_src), up(arr.COO_dst), None, None)
+    src = np.ascontiguousarray(src, dtype=np.int64)
+    dst = np.ascontiguousarray(dst, dtype=np.int64)
+    if src.shape != dst.shape or src.ndim != 1:
+        raise ValueError("src and dst must be 1-D arrays of equal length")
+    if src.shape[0] >= 2 ** 31 or num_nodes >= 2 ** 31 - 1:
+        raise ValueError("graphs are limited to int32 node and edge ids")
+    coo_src, coo_dst = torch.from_numpy(src).to(dev), torch.from_numpy(dst).to(dev)
+    ip, inb, ie, st_in = group_on_device(coo_dst, coo_src, num_nodes)
+    op, onb, oe, st_out = group_on_device(coo_src, coo_dst, num_nodes)
+    if int((st_in | st_out).item()):
+        raise ValueError("edge endpoint outside [0, num_nodes)")
+    g = DGLGraph(ip, inb, ie, op, onb, oe, coo_src, coo_dst, None, None)
     if ntype_of is not None:
-        g.SetNtypePointer(up(type_pointer(ntype_of, num_ntypes)))
-        g.SetNtypeCOO(up(np.asarray(ntype_of, dtype=np.int64)))
+        p, t = _type_columns(ntype_of, num_ntypes, dev)
+        g.SetNtypePointer(p)
+        g.SetNtypeCOO(t)
     if etype_of is not None:
-        g.SetEtypePointer(up(type_pointer(etype_of, num_etypes)))
-        g.SetEtypeCOO(up(np.asarray(etype_of, dtype=np.int64)))
+        p, t = _type_columns(etype_of, num_etypes, dev)
+        g.SetEtypePointer(p)
+        g.SetEtypeCOO(t)
     return g

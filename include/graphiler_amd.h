@@ -63,6 +63,25 @@ const char *ga_error_string(int code);
 int ga_csr_row_ids(const int32_t *pointer, int64_t n_rows, int64_t n_edges,
                    int32_t *row_of_slot, ga_stream_t stream);
 
+/* Stable grouping of items by key on the device: the construction of the
+ * in_* / out_* columns (python/graphiler/utils/setup.py:116-146: key = COO_dst,
+ * other = COO_src for the in-adjacency; key = COO_src, other = COO_dst for the
+ * out-adjacency) and of the type pointers (setup.py:147-161 with
+ * include/dglgraph.h:68-71: key = type of each item, nbr = NULL; eid is then
+ * the stable permutation that makes types contiguous).
+ *   key, other  (n_items) int64      pointer (n_keys+1) int32
+ *   nbr         (n_items) int32 or NULL: other[eid[i]]
+ *   eid         (n_items) int32: item ids, ascending inside one key
+ *   status      one int32 on the device: 0, or 1 when a key lies outside
+ *               [0, n_keys) (the outputs are then meaningless but in bounds)
+ *   workspace   ga_group_edges_workspace_bytes() bytes, 256-byte aligned
+ */
+size_t ga_group_edges_workspace_bytes(int64_t n_keys, int64_t n_items);
+int ga_group_edges(const int64_t *key, const int64_t *other, int64_t n_keys,
+                   int64_t n_items, int32_t *pointer, int32_t *nbr, int32_t *eid,
+                   int32_t *status, void *workspace, size_t workspace_bytes,
+                   ga_stream_t stream);
+
 /* ------------------------------------------------------------------- SpMM --
  * out[v, h, d] = reduce_{i in [pointer[v], pointer[v+1])} msg_i[h, d]
  * Replaces SpMMSrc (spmm.cu:375-389; op GA_COPY_U, gather by nbr),

@@ -33,6 +33,12 @@ def test_config2_gat_full(device):
     g = prepare_graph(wl.src, wl.dst, n, device=device)
     ptr, nbr, eid = _host(g)
     assert g.in_eid_is_identity and np.array_equal(eid, np.arange(e, dtype=np.int32))
+    # the grouping done on the GPU against the oracle's, both directions, bit-exact
+    for want, got in zip(oracle.group_edges(n, wl.dst, wl.src), (ptr, nbr, eid)):
+        assert np.array_equal(want, got)
+    for want, got in zip(oracle.group_edges(n, wl.src, wl.dst),
+                         (g.out_pointer, g.out_node_indices, g.out_edge_indices)):
+        assert np.array_equal(want, got.cpu().numpy())
     rng = np.random.default_rng(1)
     z = rng.standard_normal((n, 64), dtype=np.float32)
     el = rng.standard_normal((n, 1), dtype=np.float32)

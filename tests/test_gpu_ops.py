@@ -53,6 +53,43 @@ def test_row_ids_bit_exact(graph):
     assert np.array_equal(g.out_row_of_slot.cpu().numpy(), want)
 
 
+def test_graph_prep_on_device_bit_exact(graph):
+    """prepare_graph groups the edge list on the GPU; every column must equal the
+    oracle's stable grouping and the host construction, bit for bit."""
+    name, g, arr = graph
+    for side, key, other in (("in", arr.COO_dst, arr.COO_src), ("out", arr.COO_src, arr.COO_dst)):
+        ptr, nbr, eid = oracle.group_edges(arr.num_nodes, key, other)
+        assert np.array_equal(getattr(g, side + "_pointer").cpu().numpy(), ptr), f"{name} {side} pointer"
+        assert np.array_equal(getattr(g, side + "_node_indices").cpu().numpy(), nbr), f"{name} {side} nbr"
+        assert np.array_equal(getattr(g, side + "_edge_indices").cpu().numpy(), eid), f"{name} {side} eid"
+        assert np.array_equal(ptr, getattr(arr, side + "_pointer"))
+        assert np.array_equal(eid, getattr(arr, side + "_edge_indices"))
+    assert g.in_pointer.dtype == torch.int32 and g.COO_src.dtype == torch.int64
+
+
+def test_graph_prep_rejects_bad_endpoints_and_sorts_types(device):
+    from graphiler_amd.graph import group_on_device
+    src = np.array([0, 1, 2, 7], np.int64)
+    dst = np.array([1, 2, 0, 1], np.int64)
+    with pytest.raises(ValueError, match="outside"):
+        prepare_graph(src, dst, 3, device)
+    with pytest.raises(ValueError, match="outside"):
+        prepare_graph(dst, np.array([0, -1, 2, 1], np.int64), 3, device)
+    # grouping by type: pointer = running count, order = stable permutation
+    rng = np.random.default_rng(9)
+    et = rng.integers(0, 7, 5000).astype(np.int64)
+    ptr, _, order, status = group_on_device(torch.from_numpy(et).to(device), None, 9)
+    assert int(status.item()) == 0
+    assert np.array_equal(order.cpu().numpy(), np.argsort(et, kind="stable").astype(np.int32))
+    assert np.array_equal(ptr.cpu().numpy(), oracle.type_pointer(np.sort(et), 9))
+    with pytest.raises(ValueError, match="sorted by type"):
+        prepare_graph(np.array([0, 1], np.int64), np.array([1, 0], np.int64), 2, device,
+                      etype_of=np.array([1, 0]), num_etypes=2)
+    g = prepare_graph(np.array([0, 1], np.int64), np.array([1, 0], np.int64), 2, device,
+                      etype_of=np.array([0, 1]), num_etypes=3)
+    assert g.etype_pointer.cpu().tolist() == [0, 1, 2, 2]
+
+
 @pytest.mark.parametrize("feat", [1, 3, 16, 64, 100, 256, 602])
 @pytest.mark.parametrize("op", ["copy_u", "copy_e"])
 def test_spmm_copy_sum_f32(graph, device, feat, op):
