@@ -6,19 +6,18 @@
 // Order contract (what the operators rely on): slots of one key are contiguous,
 // keys ascend, and inside a key the edge ids ascend, i.e. a STABLE sort of the
 // edge ids by key.  Steps, all on the caller's stream:
-//   1. narrow the int64 keys to int32, check their range, count items per key
-//      (integer atomics: the counts do not depend on the order of arrival),
+//   1. narrow the int64 keys to int32 and check their range,
 //   2. stable LSD radix sort of (key, edge id) pairs over the bits the keys
 //      use (rocPRIM device radix sort: a library sort, like a library GEMM),
-//   3. exclusive scan of the counts -> pointer,
+//   3. pointer[v] = first slot whose key is >= v, by binary search in the sorted
+//      keys (no counting with atomics: a hub node of a power-law graph would
+//      serialise tens of thousands of them on one address),
 //   4. gather the other endpoint through the sorted edge ids.
 #include "common.h"
 
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/device/device_scan.hpp>
-#include <rocprim/functional.hpp>
 
 namespace ga {
 namespace {
@@ -26,7 +25,7 @@ namespace {
 __global__ __launch_bounds__(kBlock) void prep_keys_kernel(
     const int64_t *__restrict__ key, int64_t n_keys, int64_t n_items,
     int32_t *__restrict__ key32, int32_t *__restrict__ ids,
-    int32_t *__restrict__ count, int32_t *__restrict__ status) {
+    int32_t *__restrict__ status) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= n_items) return;
   int64_t k = key[i];
@@ -36,7 +35,20 @@ __global__ __launch_bounds__(kBlock) void prep_keys_kernel(
   }
   key32[i] = (int32_t)k;
   ids[i] = (int32_t)i;
-  atomicAdd(&count[k], 1);
+}
+
+// pointer[v] = number of items with key < v, v in [0, n_keys]
+__global__ __launch_bounds__(kBlock) void pointer_kernel(
+    const int32_t *__restrict__ key_sorted, int64_t n_keys, int64_t n_items,
+    int32_t *__restrict__ pointer) {
+  const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (v > n_keys) return;
+  int64_t lo = 0, hi = n_items;          // first index with key_sorted[index] >= v
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if ((int64_t)key_sorted[mid] < v) lo = mid + 1; else hi = mid;
+  }
+  pointer[v] = (int32_t)lo;
 }
 
 __global__ __launch_bounds__(kBlock) void gather_other_kernel(
@@ -55,7 +67,7 @@ __global__ __launch_bounds__(kBlock) void fill_zero_kernel(int32_t *p, int64_t n
 inline size_t round_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct PrepLayout {
-  size_t key32, key_sorted, ids, count, temp, total;
+  size_t key32, key_sorted, ids, temp, total;
   size_t temp_bytes;
 };
 
@@ -68,22 +80,18 @@ int end_bit_for(int64_t n_keys) {
 // Sizes only; nothing is launched (rocPRIM's calls with a null temporary
 // buffer just report what they need).
 int prep_layout(int64_t n_keys, int64_t n_items, PrepLayout &L) {
-  size_t sort_bytes = 0, scan_bytes = 0;
+  size_t sort_bytes = 0;
   int32_t *k = nullptr;
   if (n_items > 0) {
     hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, k, k, k, k,
                                              (size_t)n_items, 0, end_bit_for(n_keys));
     if (e != hipSuccess) return (int)e;
   }
-  hipError_t e = rocprim::exclusive_scan(nullptr, scan_bytes, k, k, 0,
-                                         (size_t)(n_keys + 1), rocprim::plus<int32_t>());
-  if (e != hipSuccess) return (int)e;
-  L.temp_bytes = sort_bytes > scan_bytes ? sort_bytes : scan_bytes;
+  L.temp_bytes = sort_bytes;
   size_t off = 0;
   L.key32 = off;       off += round_up((size_t)n_items * 4);
   L.key_sorted = off;  off += round_up((size_t)n_items * 4);
   L.ids = off;         off += round_up((size_t)n_items * 4);
-  L.count = off;       off += round_up((size_t)(n_keys + 1) * 4);
   L.temp = off;        off += round_up(L.temp_bytes);
   L.total = off;
   return GA_OK;
@@ -120,28 +128,23 @@ int ga_group_edges(const int64_t *key, const int64_t *other, int64_t n_keys,
   int32_t *key32 = (int32_t *)(ws + L.key32);
   int32_t *key_sorted = (int32_t *)(ws + L.key_sorted);
   int32_t *ids = (int32_t *)(ws + L.ids);
-  int32_t *count = (int32_t *)(ws + L.count);
   void *temp = ws + L.temp;
 
-  // counts (n_keys + 1 entries, the last stays 0) and the status word start at 0;
-  // a fill kernel rather than a memset node keeps the sequence capturable
-  const int64_t cblocks = (n_keys + 1 + kBlock - 1) / kBlock;
-  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)cblocks), dim3(kBlock), 0, s, count,
-                     n_keys + 1);
+  // the status word starts at 0; a fill kernel rather than a memset node keeps
+  // the sequence capturable
   hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(kBlock), 0, s, status, (int64_t)1);
   if (n_items > 0) {
     const int64_t blocks = (n_items + kBlock - 1) / kBlock;
     hipLaunchKernelGGL(prep_keys_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, key,
-                       n_keys, n_items, key32, ids, count, status);
+                       n_keys, n_items, key32, ids, status);
     size_t tb = L.temp_bytes;
     hipError_t e = rocprim::radix_sort_pairs(temp, tb, key32, key_sorted, ids, eid,
                                              (size_t)n_items, 0, end_bit_for(n_keys), s);
     if (e != hipSuccess) return (int)e;
   }
-  size_t tb = L.temp_bytes;
-  hipError_t e = rocprim::exclusive_scan(temp, tb, count, pointer, 0, (size_t)(n_keys + 1),
-                                         rocprim::plus<int32_t>(), s);
-  if (e != hipSuccess) return (int)e;
+  const int64_t pblocks = (n_keys + 1 + kBlock - 1) / kBlock;
+  hipLaunchKernelGGL(pointer_kernel, dim3((unsigned)pblocks), dim3(kBlock), 0, s, key_sorted,
+                     n_keys, n_items, pointer);
   if (n_items > 0 && nbr) {
     const int64_t blocks = (n_items + kBlock - 1) / kBlock;
     hipLaunchKernelGGL(gather_other_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, other,
