@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 # HBM bytes per dominant-kernel launch measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); the summary
 # lives under profiles/.  None until measured for the kernel named below.
-MEASURED_TRAFFIC_BYTES = {"plan": 1_480_080_486, "fused": 1_534_816_358}
+MEASURED_TRAFFIC_BYTES = {"plan": 1_486_204_723, "fused": 1_509_594_829}
 
 
 def main():
