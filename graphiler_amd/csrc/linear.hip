@@ -57,7 +57,11 @@ template <> struct XVec<1> { using type = float; };
 // one, the row's last vector) and zero by select at commit time, where the
 // value is consumed anyway; no lane is ever predicated off in the k loop.
 template <bool HAS_ATTN, int VK>
-__global__ __launch_bounds__(kBlock) void linear_attn_kernel(
+// two waves per SIMD: with that register budget the accumulators stay in place
+// across the loop (left to itself the allocator splits them over both register
+// files and copies 48 of them every trip)
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2, 2))) void
+linear_attn_kernel(
     const float *__restrict__ X, const float *__restrict__ W,
     const float *__restrict__ a_l, const float *__restrict__ a_r,
     float *__restrict__ Z, float *__restrict__ el, float *__restrict__ er,
@@ -125,9 +129,9 @@ __global__ __launch_bounds__(kBlock) void linear_attn_kernel(
 #pragma unroll
     for (int j = 0; j < kWPieces; ++j) {
       const int i = threadIdx.x + j * kBlock;
+      float4 v = st.w[j];
       const int cc = col0 + (i & 15) * 4;
       const bool kin = sl * kSliceK + (i >> 4) < K;
-      float4 v = st.w[j];
       v.x = kin && cc < M ? v.x : 0.0f;
       v.y = kin && cc + 1 < M ? v.y : 0.0f;
       v.z = kin && cc + 2 < M ? v.z : 0.0f;

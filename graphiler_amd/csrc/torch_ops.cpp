@@ -416,6 +416,32 @@ torch::Tensor gat_aggregate(torch::Tensor el, torch::Tensor er, torch::Tensor z,
   return out;
 }
 
+// z = x @ w with the GAT attention terms from the same kernel (GAT.py:25-29)
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> linear_attn(
+    torch::Tensor x, torch::Tensor w, torch::Tensor a_l, torch::Tensor a_r) {
+  check_input(x, "x");
+  check_input(w, "weight");
+  check_input(a_l, "a_l");
+  check_input(a_r, "a_r");
+  TORCH_CHECK(x.scalar_type() == at::kFloat && w.scalar_type() == at::kFloat &&
+                  a_l.scalar_type() == at::kFloat && a_r.scalar_type() == at::kFloat,
+              "linear_attn is float32 only");
+  TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && w.size(0) == x.size(1), "weight must be (K, M)");
+  const int64_t rows = x.size(0), K = x.size(1), M = w.size(1);
+  TORCH_CHECK(a_l.dim() == 2 && a_l.numel() == M && a_r.numel() == M && a_r.dim() == 2 &&
+                  a_r.size(0) == a_l.size(0),
+              "a_l and a_r must be (heads, M / heads)");
+  const int64_t heads = a_l.size(0);
+  torch::Tensor z = torch::empty({rows, M}, x.options());
+  torch::Tensor el = torch::empty({rows, heads}, x.options());
+  torch::Tensor er = torch::empty({rows, heads}, x.options());
+  check_ga(ga_linear_attn(x.data_ptr<float>(), w.data_ptr<float>(), a_l.data_ptr<float>(),
+                          a_r.data_ptr<float>(), z.data_ptr<float>(), el.data_ptr<float>(),
+                          er.data_ptr<float>(), rows, K, M, heads, current_stream(x)),
+           "ga_linear_attn");
+  return std::make_tuple(z, el, er);
+}
+
 }  // namespace
 
 TORCH_LIBRARY(my_classes, m) {
@@ -467,4 +493,7 @@ static auto registry =
             &gspmm)
         .op("my_ops::gat_aggregate(Tensor el, Tensor er, Tensor z, float slope, " GRAPH_T
             " g) -> Tensor y",
-            &gat_aggregate);
+            &gat_aggregate)
+        .op("my_ops::linear_attn(Tensor x, Tensor w, Tensor a_l, Tensor a_r) -> "
+            "(Tensor z, Tensor el, Tensor er)",
+            &linear_attn);

@@ -82,6 +82,23 @@ def test_scripted_gat_plan_runs_unchanged(setup, device):
     assert_close(fused.cpu().numpy(), ref, TOL_F32, "fused GAT op")
 
 
+def test_linear_attn_op(setup, device):
+    """The projection kernel through the TorchScript boundary: z = x @ w in fp32
+    (fp64 numpy product as the reference) and both attention terms."""
+    sg, arr, rng = setup
+    n = arr.num_nodes
+    x = rng.standard_normal((n, 50), dtype=np.float32)
+    w = rng.standard_normal((50, 64), dtype=np.float32) / 7
+    al = rng.standard_normal((2, 32), dtype=np.float32)
+    ar = rng.standard_normal((2, 32), dtype=np.float32)
+    z, el, er = torch.ops.my_ops.linear_attn(_t(x, device), _t(w, device), _t(al, device),
+                                             _t(ar, device))
+    zr = x.astype(np.float64) @ w.astype(np.float64)
+    assert_close(z.cpu().numpy(), zr, TOL_F32, "linear_attn z")
+    assert_close(el.cpu().numpy(), np.einsum("nhd,hd->nh", zr.reshape(n, 2, 32), al), TOL_F32, "el")
+    assert_close(er.cpu().numpy(), np.einsum("nhd,hd->nh", zr.reshape(n, 2, 32), ar), TOL_F32, "er")
+
+
 def test_error_convention(setup, device):
     sg, arr, rng = setup
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
