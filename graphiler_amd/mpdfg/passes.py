@@ -1,0 +1,355 @@
+"""Rewrites of a built plan: split, reorder, fusion (src/optimizer/split.cpp,
+reorder.cpp, fusion.cpp, dedup.cpp), written as direct graph surgery so that a
+rewrite can ask where a value lives (the reference matches on operator names
+only and notes residency as a to-do, reorder.cpp:14-15, split.cpp:8).
+
+* split:   ``mm(cat([a, b], 1), w)`` -> ``mm(a, w[:fa]) + mm(b, w[fa:])`` so each
+  half can move to node data on its own (the GAT attention product).
+* reorder: an operator that acts row by row commutes with a broadcast: ``op(
+  Broadcast(x))`` -> ``Broadcast(op(x))`` does the work once per node instead of
+  once per edge.  Allowed when every other operand is shared (a weight, a
+  constant); two broadcasts of the same kind under one binary operator merge.
+* fusion:  broadcast + compute + reduce chains into the fused graph operators:
+  ``SpMMSrc``, ``gspmm_{src,dst}_mul_e_sum``, ``gsddmm_u_add_v_mul_alpha``,
+  ``SegmentMMNode/Edge`` for per-type ``bmm``, and (not in the reference) the
+  whole attention chain into ``gat_aggregate``.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .builder import EDGE, ETYPE, MPDFG, NODE, NTYPE, SHARED
+
+_BCAST = {"my_ops::BroadcastSrcNode", "my_ops::BroadcastDstNode", "my_ops::BroadcastSrcNodeType",
+          "my_ops::BroadcastDstNodeType", "my_ops::BroadcastEdgeType", "my_ops::BroadcastNodeType"}
+# row-wise operators whose first operand is the data and the rest are shared
+_ROWWISE = {"aten::relu", "aten::sigmoid", "aten::tanh", "aten::exp", "aten::neg",
+            "aten::leaky_relu", "aten::squeeze", "aten::mm", "aten::pow", "aten::unsqueeze"}
+_INPLACE = {"aten::relu_": "aten::relu", "aten::leaky_relu_": "aten::leaky_relu",
+            "aten::sigmoid_": "aten::sigmoid", "aten::tanh_": "aten::tanh"}
+_PAIRWISE = {"aten::mul", "aten::add", "aten::sub", "aten::div"}
+
+
+def dedup(graph: torch._C.Graph) -> None:
+    """Dead code, pooled constants, common subexpressions; the graph operators
+    are pure functions of their inputs too, which TorchScript cannot know."""
+    torch._C._jit_pass_dce(graph)
+    torch._C._jit_pass_constant_pooling(graph)
+    torch._C._jit_pass_cse(graph)
+    # repeated reads of one feature (ndata["h"] for the source and again for the
+    # destination): TorchScript keeps both because dictionaries are mutable; they
+    # are the same tensor as long as no _set_item on that dictionary lies between
+    known = {}
+    for n in list(graph.nodes()):
+        if n.kind() == "aten::_set_item":
+            d = n.inputsAt(0).unique()
+            known = {k: v for k, v in known.items() if k[0] != d}
+        elif n.kind() == "aten::__getitem__" and n.inputsAt(1).node().kind() == "prim::Constant":
+            key = (n.inputsAt(0).unique(), n.inputsAt(1).unique())
+            if key in known:
+                n.output().replaceAllUsesWith(known[key])
+                n.destroy()
+            else:
+                known[key] = n.output()
+    torch._C._jit_pass_cse(graph)
+
+    def mutated(v) -> bool:
+        return any(u.user.kind().endswith("_") or u.user.kind() == "aten::_set_item"
+                   for u in v.uses())
+
+    changed = True
+    while changed:
+        changed = False
+        seen = {}
+        for n in list(graph.nodes()):
+            ours = n.kind().startswith("my_ops::")
+            # TorchScript's own pass will not merge two equal aten nodes once a
+            # custom operator reads their results (it must assume it writes them)
+            pure_aten = (n.kind().startswith("aten::") and not n.kind().endswith("_")
+                         and n.kind() not in ("aten::__getitem__", "aten::_set_item")
+                         and n.outputsSize() == 1 and not n.attributeNames()
+                         and not any(mutated(i) for i in n.inputs())
+                         and not mutated(n.output()))
+            if not ours and not pure_aten:
+                continue
+            if ours and not any(o.uses() for o in n.outputs()):
+                n.destroy()
+                changed = True
+                continue
+            key = (n.kind(), tuple(i.unique() for i in n.inputs()))
+            if key in seen:
+                n.replaceAllUsesWith(seen[key])
+                n.destroy()
+                changed = True
+            else:
+                seen[key] = n
+    torch._C._jit_pass_dce(graph)
+
+
+class _Rewriter:
+    def __init__(self, plan: MPDFG):
+        self.plan = plan
+        self.G = plan.graph
+        self.res = plan.residency
+        self.dglgraph = list(self.G.inputs())[0]
+
+    def where(self, v) -> str:
+        return self.res.get(v.unique(), SHARED)
+
+    def make(self, kind, inputs, before, residency, ty=None, like=None):
+        node = self.G.create(kind, list(inputs), 1)
+        if like is not None:
+            node.copyAttributes(like)
+            node.output().copyMetadata(like.output())
+        node.insertBefore(before)
+        node.output().setType(ty if ty is not None else
+                              (like.output().type() if like is not None
+                               else torch._C.TensorType.get()))
+        self.res[node.output().unique()] = residency
+        return node.output()
+
+    def const(self, value, before):
+        with self.G.insert_point_guard(before):
+            v = self.G.insertConstant(value)
+        self.res[v.unique()] = SHARED
+        return v
+
+    @staticmethod
+    def single_use(v) -> bool:
+        return len(v.uses()) == 1
+
+    @staticmethod
+    def const_of(v):
+        from .builder import _const_of
+        return _const_of(v)
+
+    # ------------------------------------------------------------- split ----
+    def split(self) -> bool:
+        changed = False
+        for n in list(self.G.nodes()):
+            if n.kind() != "aten::mm":
+                continue
+            cat = n.inputsAt(0).node()
+            if cat.kind() != "aten::cat" or self.const_of(cat.inputsAt(1)) != 1:
+                continue
+            lst = cat.inputsAt(0).node()
+            if lst.kind() != "prim::ListConstruct" or lst.inputsSize() != 2:
+                continue
+            a, b = lst.inputsAt(0), lst.inputsAt(1)
+            w = n.inputsAt(1)
+            if self.where(w) != SHARED:
+                continue
+            r = self.where(n.output())
+            int_t = torch._C.IntType.get()
+            fa = self.make("my_ops::get_feat_dim", [a], n, SHARED, ty=int_t)
+            zero, one = self.const(0, n), self.const(1, n)
+            none = self.const(None, n)
+            w_a = self.make("aten::slice", [w, zero, zero, fa, one], n, SHARED)
+            w_b = self.make("aten::slice", [w, zero, fa, none, one], n, SHARED)
+            m_a = self.make("aten::mm", [a, w_a], n, self.where(a))
+            m_b = self.make("aten::mm", [b, w_b], n, self.where(b))
+            out = self.make("aten::add", [m_a, m_b, one], n, r)
+            n.output().replaceAllUsesWith(out)
+            n.destroy()
+            changed = True
+        return changed
+
+    # ----------------------------------------------------------- reorder ----
+    def _target_residency(self, bkind: str, src_res: str) -> str:
+        return NODE if bkind == "my_ops::BroadcastNodeType" else EDGE
+
+    def reorder(self) -> bool:
+        changed = False
+        for n in list(self.G.nodes()):
+            kind = _INPLACE.get(n.kind(), n.kind())
+            if n.inputsSize() == 0:
+                continue
+            first = n.inputsAt(0).node()
+            if kind == "my_ops::get_feat_dim" and first.kind() in _BCAST:
+                n.replaceInput(0, first.inputsAt(0))
+                changed = True
+                continue
+            if kind in _PAIRWISE and n.inputsSize() >= 2:
+                second = n.inputsAt(1).node()
+                if (first.kind() in _BCAST and second.kind() == first.kind()
+                        and first.inputsAt(1).unique() == second.inputsAt(1).unique()
+                        and self.where(first.inputsAt(0)) == self.where(second.inputsAt(0))
+                        and all(self.where(i) == SHARED for i in list(n.inputs())[2:])):
+                    src_res = self.where(first.inputsAt(0))
+                    ins = [first.inputsAt(0), second.inputsAt(0)] + list(n.inputs())[2:]
+                    small = self.make(kind, ins, n, src_res, like=n)
+                    back = self.make(first.kind(), [small, self.dglgraph], n,
+                                     self.where(n.output()))
+                    n.output().replaceAllUsesWith(back)
+                    n.destroy()
+                    changed = True
+                    continue
+            if kind not in _ROWWISE or first.kind() not in _BCAST:
+                continue
+            if any(self.where(i) != SHARED for i in list(n.inputs())[1:]):
+                continue
+            if kind == "aten::unsqueeze" and self.const_of(n.inputsAt(1)) in (0, None):
+                continue                      # a new leading dimension is not row-wise
+            if kind == "aten::squeeze" and n.inputsSize() > 1 and self.const_of(n.inputsAt(1)) in (0, None):
+                continue
+            src = first.inputsAt(0)
+            small = self.make(kind, [src] + list(n.inputs())[1:], n, self.where(src), like=n)
+            back = self.make(first.kind(), [small, self.dglgraph], n, self.where(n.output()))
+            n.output().replaceAllUsesWith(back)
+            n.destroy()
+            changed = True
+        return changed
+
+    # ------------------------------------------------------------ fusion ----
+    def fusion(self) -> bool:
+        changed = False
+        for n in list(self.G.nodes()):
+            kind = n.kind()
+            if kind == "my_ops::SpMMEdge":
+                changed |= self._fuse_spmm(n)
+            elif kind == "aten::add":
+                changed |= self._fuse_u_add_v(n)
+            elif kind == "aten::squeeze" and n.inputsSize() == 1:
+                inner = n.input().node()
+                if inner.kind() == "aten::unsqueeze":
+                    n.output().replaceAllUsesWith(inner.inputsAt(0))
+                    n.destroy()
+                    changed = True
+            elif kind == "aten::bmm":
+                changed |= self._fuse_bmm(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::gspmm_src_mul_e_sum":
+                changed |= self._fuse_gat_chain(n)
+        return changed
+
+    def _fuse_spmm(self, n) -> bool:
+        x = n.inputsAt(0).node()
+        rest = list(n.inputs())[1:]                 # dims, keep, dtype, graph
+        if x.kind() == "my_ops::BroadcastSrcNode":
+            out = self.make("my_ops::SpMMSrc", [x.inputsAt(0)] + rest, n, NODE)
+        elif x.kind() == "aten::mul":
+            a, b = x.inputsAt(0), x.inputsAt(1)
+            for msg, bc in ((a, b), (b, a)):
+                k = bc.node().kind()
+                if k in ("my_ops::BroadcastSrcNode", "my_ops::BroadcastDstNode") \
+                        and self.where(msg) == EDGE:
+                    op = "my_ops::gspmm_src_mul_e_sum" if "Src" in k else "my_ops::gspmm_dst_mul_e_sum"
+                    out = self.make(op, [bc.node().inputsAt(0), msg] + rest, n, NODE)
+                    break
+            else:
+                return False
+        else:
+            return False
+        n.output().replaceAllUsesWith(out)
+        n.destroy()
+        return True
+
+    def _fuse_u_add_v(self, n) -> bool:
+        if n.inputsSize() != 3:
+            return False
+        a, b = n.inputsAt(0).node(), n.inputsAt(1).node()
+        if a.kind() != "my_ops::BroadcastSrcNode" or b.kind() != "my_ops::BroadcastDstNode":
+            return False
+        alpha = self.const_of(n.inputsAt(2))
+        if alpha != 1:                              # the operator ignores alpha (sddmm.cu:116-121)
+            return False
+        out = self.make("my_ops::gsddmm_u_add_v_mul_alpha",
+                        [a.inputsAt(0), b.inputsAt(0), n.inputsAt(2), self.dglgraph], n, EDGE)
+        n.output().replaceAllUsesWith(out)
+        n.destroy()
+        return True
+
+    def _fuse_bmm(self, n) -> bool:
+        x, w = n.inputsAt(0), n.inputsAt(1)
+        wk = w.node().kind()
+        one = None
+        if wk in ("my_ops::BroadcastSrcNodeType", "my_ops::BroadcastDstNodeType"):
+            need = "my_ops::BroadcastSrcNode" if "Src" in wk else "my_ops::BroadcastDstNode"
+            if x.node().kind() != need:
+                return False
+            nd = x.node().inputsAt(0)
+            flat = self.make("aten::squeeze", [nd], n, NODE)
+            mm = self.make("my_ops::SegmentMMNode", [flat, w.node().inputsAt(0), self.dglgraph], n, NODE)
+            wide = self.make(need, [mm, self.dglgraph], n, EDGE)
+            one = self.const(1, n)
+            out = self.make("aten::unsqueeze", [wide, one], n, EDGE)
+        elif wk in ("my_ops::BroadcastEdgeType", "my_ops::BroadcastNodeType"):
+            seg = "my_ops::SegmentMMEdge" if wk.endswith("EdgeType") else "my_ops::SegmentMMNode"
+            r = EDGE if wk.endswith("EdgeType") else NODE
+            if self.where(x) != r:
+                return False
+            flat = self.make("aten::squeeze", [x], n, r)
+            mm = self.make(seg, [flat, w.node().inputsAt(0), self.dglgraph], n, r)
+            one = self.const(1, n)
+            out = self.make("aten::unsqueeze", [mm, one], n, r)
+        else:
+            return False
+        n.output().replaceAllUsesWith(out)
+        n.destroy()
+        return True
+
+    def _fuse_gat_chain(self, n) -> bool:
+        """gspmm_src_mul_e_sum(z, SegmentSoftmax(leaky_relu(u_add_v(el, er)))) with
+        no other reader of the intermediates -> gat_aggregate(el, er, z, slope)."""
+        z, att = n.inputsAt(0), n.inputsAt(1)
+        sm = att.node()
+        if sm.kind() != "my_ops::SegmentSoftmax" or not self.single_use(att):
+            return False
+        act = sm.inputsAt(0).node()
+        if act.kind() not in ("aten::leaky_relu", "aten::leaky_relu_") or \
+                not self.single_use(act.output()):
+            return False
+        add = act.inputsAt(0).node()
+        if add.kind() != "my_ops::gsddmm_u_add_v_mul_alpha" or not self.single_use(add.output()):
+            return False
+        slope = self.const_of(act.inputsAt(1))
+        if slope is None:
+            return False
+        slope_v = self.const(float(slope), n)
+        out = self.make("my_ops::gat_aggregate",
+                        [add.inputsAt(0), add.inputsAt(1), z, slope_v, self.dglgraph], n, NODE)
+        n.output().replaceAllUsesWith(out)
+        for dead in (n, sm, act, add):      # the in-place activation would not be swept
+            dead.destroy()
+        return True
+
+
+def split(plan: MPDFG) -> None:
+    _Rewriter(plan).split()
+    dedup(plan.graph)
+    plan.invalidate()
+
+
+def reorder(plan: MPDFG) -> None:
+    rw = _Rewriter(plan)
+    for _ in range(16):
+        if not rw.reorder():
+            break
+        dedup(plan.graph)
+    dedup(plan.graph)
+    plan.invalidate()
+
+
+def fusion(plan: MPDFG) -> None:
+    rw = _Rewriter(plan)
+    for _ in range(8):
+        if not rw.fusion():
+            break
+        dedup(plan.graph)
+    dedup(plan.graph)
+    plan.invalidate()
+
+
+def optimize(plan: MPDFG, opt_level: int) -> None:
+    """python/graphiler/mpdfg_optimizer.py:4-16: level 1 = split + reorder,
+    level 2 = + alternating reorder / fusion until nothing changes."""
+    if opt_level <= 0:
+        return
+    split(plan)
+    reorder(plan)
+    if opt_level > 1:
+        for _ in range(3):
+            reorder(plan)
+            fusion(plan)

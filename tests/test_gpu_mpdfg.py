@@ -1,0 +1,123 @@
+"""Compiled plans (MP-DFG builder + optimizer) run on the GPU and must give the
+model's result at every optimisation level.  The expected values are computed
+here in numpy / with the oracle from the model's definition, edge by edge."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import udf_models as U
+from graphiler_amd import prepare_graph
+from graphiler_amd.graph import build_graph_arrays
+from graphiler_amd.mpdfg import GraphData, mpdfg_builder, update_all
+from helpers import TOL_F32, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def _homo(rng, n=300, e=2500):
+    src = rng.integers(0, n, e).astype(np.int64)
+    dst = rng.integers(0, n, e).astype(np.int64)
+    dst[: e // 10] = 7                                  # one busy row
+    return n, src, dst
+
+
+@pytest.mark.parametrize("level", [0, 1, 2])
+def test_gcn_plan(device, level):
+    rng = np.random.default_rng(21)
+    n, src, dst = _homo(rng)
+    g = GraphData(prepare_graph(src, dst, n, device))
+    h = rng.standard_normal((n, 16), dtype=np.float32)
+    deg = rng.integers(1, 9, (n, 1)).astype(np.float32)
+    g.ndata['h'], g.ndata['degree'] = _t(h, device), _t(deg, device)
+    update_all(g, mpdfg_builder(U.gcn_message, U.gcn_reduce, opt_level=level))
+    arr = build_graph_arrays(src, dst, n)
+    want = np.maximum(oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                                  (h * deg ** -0.5).astype(np.float32), op="copy_u"), 0)
+    assert_close(g.ndata['h'].cpu().numpy(), want, TOL_F32, f"GCN plan level {level}")
+
+
+@pytest.mark.parametrize("level", [0, 1, 2])
+def test_gat_plan(device, level):
+    rng = np.random.default_rng(22)
+    n, src, dst = _homo(rng)
+    g = GraphData(prepare_graph(src, dst, n, device))
+    h = rng.standard_normal((n, 24), dtype=np.float32)
+    fc = (rng.standard_normal((24, 32)) / 5).astype(np.float32)
+    attn = (rng.standard_normal((64, 1)) / 5).astype(np.float32)
+    g.ndata['h'] = _t(h, device)
+    update_all(g, mpdfg_builder(U.gat_message, U.gat_reduce, opt_level=level),
+               msg_params=(_t(fc, device), _t(attn, device)))
+    z = h.astype(np.float64) @ fc
+    el, er = (z @ attn[:32]).astype(np.float32), (z @ attn[32:]).astype(np.float32)
+    arr = build_graph_arrays(src, dst, n)
+    want = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er,
+                                z.astype(np.float32), heads=1, slope=0.2)
+    assert_close(g.ndata['h'].cpu().numpy(), want, 2e-5, f"GAT plan level {level}")
+
+
+def _hetero(rng, n_per_type=(60, 50, 40), e_per_rel=(400, 300, 500, 200)):
+    n = sum(n_per_type)
+    ntype = np.repeat(np.arange(len(n_per_type)), n_per_type).astype(np.int64)
+    etype = np.repeat(np.arange(len(e_per_rel)), e_per_rel).astype(np.int64)   # sorted by type
+    e = etype.shape[0]
+    src = rng.integers(0, n, e).astype(np.int64)
+    dst = rng.integers(0, n, e).astype(np.int64)
+    return n, src, dst, ntype, etype
+
+
+@pytest.mark.parametrize("level", [0, 1, 2])
+def test_rgcn_plan(device, level):
+    rng = np.random.default_rng(23)
+    n, src, dst, ntype, etype = _hetero(rng)
+    g = GraphData(prepare_graph(src, dst, n, device, etype_of=etype, num_etypes=4))
+    h = rng.standard_normal((n, 16), dtype=np.float32)
+    w = (rng.standard_normal((4, 16, 8)) / 4).astype(np.float32)
+    norm = rng.uniform(0.2, 1.0, (src.shape[0], 1)).astype(np.float32)
+    g.ndata['h'], g.edata['norm'], g.etype_data['weight'] = _t(h, device), _t(norm, device), _t(w, device)
+    update_all(g, mpdfg_builder(U.rgcn_message, U.rgcn_reduce, opt_level=level))
+    msg = np.einsum("ek,ekm->em", h[src].astype(np.float64), w[etype]) * norm
+    want = np.zeros((n, 8))
+    np.add.at(want, dst, msg)
+    assert_close(g.ndata['h'].cpu().numpy(), want, TOL_F32, f"RGCN plan level {level}")
+
+
+@pytest.mark.parametrize("level", [0, 1, 2])
+def test_hgt_plan(device, level):
+    rng = np.random.default_rng(24)
+    n, src, dst, ntype, etype = _hetero(rng)
+    g = GraphData(prepare_graph(src, dst, n, device, ntype_of=ntype, num_ntypes=3,
+                                etype_of=etype, num_etypes=4))
+    d_in, d = 12, 16
+    h = rng.standard_normal((n, d_in), dtype=np.float32)
+    kw, qw, vw = ((rng.standard_normal((3, d_in, d)) / 3).astype(np.float32) for _ in range(3))
+    aw = (rng.standard_normal((3, d, d)) / 4).astype(np.float32)
+    skip = rng.standard_normal(3).astype(np.float32)           # one scalar per node type
+    r_att, r_msg = ((rng.standard_normal((4, d, d)) / 4).astype(np.float32) for _ in range(2))
+    r_pri = rng.uniform(0.5, 1.5, (4, 1)).astype(np.float32)
+    g.ndata['h'] = _t(h, device)
+    for k, v in (("k_weight", kw), ("q_weight", qw), ("v_weight", vw), ("a_weight", aw), ("skip", skip)):
+        g.ntype_data[k] = _t(v, device)
+    for k, v in (("relation_att", r_att), ("relation_msg", r_msg), ("relation_pri", r_pri)):
+        g.etype_data[k] = _t(v, device)
+    sqrt_dk = float(np.sqrt(d))
+    plan = mpdfg_builder(U.hgt_message, U.hgt_reduce, U.hgt_update, opt_level=level)
+    update_all(g, plan, msg_params=(sqrt_dk,))
+
+    h64 = h.astype(np.float64)
+    k = np.einsum("nk,nkm->nm", h64, kw[ntype])[src]
+    v = np.einsum("nk,nkm->nm", h64, vw[ntype])[src]
+    q = np.einsum("nk,nkm->nm", h64, qw[ntype])[dst]
+    k = np.einsum("ek,ekm->em", k, r_att[etype])
+    v = np.einsum("ek,ekm->em", v, r_msg[etype])
+    score = (k * q).sum(1, keepdims=True) * r_pri[etype] / sqrt_dk
+    arr = build_graph_arrays(src, dst, n)
+    att = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, score.astype(np.float32))
+    t = np.zeros((n, d))
+    np.add.at(t, dst, att.astype(np.float64) * v)
+    want = np.einsum("nk,nkm->nm", t, aw[ntype]) / (1 + np.exp(-skip[ntype]))[:, None]
+    assert_close(g.ndata['h'].cpu().numpy(), want, 5e-5, f"HGT plan level {level}")

@@ -1,0 +1,103 @@
+"""Structure of the plans the MP-DFG builder emits (no GPU needed: the plans are
+built and linted, not run)."""
+import pytest
+import torch
+
+import udf_models as U
+from graphiler_amd.mpdfg import BuildError, EdgeBatchDummy, NodeBatchDummy, mpdfg_builder
+
+MODELS = {
+    "gcn": (U.gcn_message, U.gcn_reduce),
+    "gat": (U.gat_message, U.gat_reduce),
+    "rgcn": (U.rgcn_message, U.rgcn_reduce),
+    "hgt": (U.hgt_message, U.hgt_reduce, U.hgt_update),
+}
+
+
+def _kinds(name, level):
+    plan = mpdfg_builder(*MODELS[name], opt_level=level)
+    plan.forward                                    # lints and compiles
+    return plan, [k for k in plan.op_kinds() if k.startswith(("my_ops::", "aten::"))]
+
+
+def test_plan_signature_and_parameters():
+    plan, _ = _kinds("gat", 0)
+    names = [v.debugName() for v in plan.graph.inputs()]
+    assert names[:5] == ["dglgraph", "ndata", "edata", "ntypedata", "etypedata"]
+    assert names[5:] == ["fc_weight_msg", "attn_weight_msg"]
+    plan, _ = _kinds("hgt", 0)
+    assert [v.debugName() for v in plan.graph.inputs()][5:] == ["sqrt_dk_msg"]
+    assert str(list(plan.graph.inputs())[5].type()) == "float"
+
+
+def test_level0_is_broadcast_compute_reduce():
+    """Unoptimised: every batch read is a Broadcast operator, the mailbox
+    reductions are SegmentSoftmax / SpMMEdge (builder.cpp:24-42, 205-238)."""
+    _, k = _kinds("gat", 0)
+    assert k.count("my_ops::BroadcastSrcNode") == 1 and k.count("my_ops::BroadcastDstNode") == 1
+    assert "aten::cat" in k and "my_ops::SegmentSoftmax" in k and "my_ops::SpMMEdge" in k
+    assert k.index("my_ops::SegmentSoftmax") < k.index("my_ops::SpMMEdge")
+    _, k = _kinds("hgt", 0)
+    assert k.count("my_ops::BroadcastSrcNodeType") == 2 and k.count("my_ops::BroadcastDstNodeType") == 1
+    assert k.count("my_ops::BroadcastEdgeType") == 3 and k.count("my_ops::BroadcastNodeType") == 2
+    assert "aten::_set_item" in k               # reduce results stored for the update function
+    _, k = _kinds("rgcn", 0)
+    assert "my_ops::BroadcastEdgeType" in k and "aten::bmm" in k
+
+
+def test_level1_moves_dense_work_to_the_nodes():
+    _, k = _kinds("gat", 1)
+    assert "aten::cat" not in k                                 # split
+    assert k.index("aten::mm") < k.index("my_ops::BroadcastSrcNode")   # reorder
+    assert k.count("aten::mm") == 3             # z once (source and destination share it), el, er
+    _, k = _kinds("gcn", 1)
+    assert k.index("aten::mul") < k.index("my_ops::BroadcastSrcNode")
+    assert k.count("my_ops::BroadcastSrcNode") == 1
+
+
+def test_level2_fuses_into_graph_operators():
+    _, k = _kinds("gcn", 2)
+    assert "my_ops::SpMMSrc" in k and not any(x.startswith("my_ops::Broadcast") for x in k)
+    _, k = _kinds("gat", 2)
+    ours = [x for x in k if x.startswith("my_ops::")]
+    assert ours == ["my_ops::get_feat_dim", "my_ops::gat_aggregate"]
+    _, k = _kinds("rgcn", 2)
+    assert "my_ops::SegmentMMEdge" in k and "aten::bmm" not in k and "my_ops::BroadcastEdgeType" not in k
+    _, k = _kinds("hgt", 2)
+    assert k.count("my_ops::SegmentMMNode") == 4 and k.count("my_ops::SegmentMMEdge") == 2
+    assert "aten::bmm" not in k and "aten::squeeze" not in k
+
+
+def gat_reference_style_message(edges: EdgeBatchDummy, fc_weight, attn_weight):
+    z_s = torch.mm(edges.src['h'], fc_weight)
+    z_d = torch.mm(edges.dst['h'], fc_weight)
+    a = torch.mm(torch.cat([z_s, z_d], dim=1), attn_weight)
+    return {'z': z_s, 'e': torch.nn.functional.leaky_relu_(a)}      # in place, default slope
+
+
+def test_inplace_activation_chain_is_fused_and_removed():
+    plan = mpdfg_builder(gat_reference_style_message, U.gat_reduce, opt_level=2)
+    k = plan.op_kinds()
+    assert "my_ops::gat_aggregate" in k and "aten::leaky_relu_" not in k
+    assert "my_ops::gsddmm_u_add_v_mul_alpha" not in k
+
+
+def bad_reduce(nodes: NodeBatchDummy):
+    return {'h': torch.sum(nodes.mailbox['missing'], dim=1)}
+
+
+def bad_softmax(nodes: NodeBatchDummy):
+    return {'h': torch.sum(torch.softmax(nodes.mailbox['m'], dim=0), dim=1)}
+
+
+def untyped_message(edges, w):
+    return {'m': edges.src['h']}
+
+
+def test_build_errors():
+    with pytest.raises(BuildError, match="mailbox"):
+        mpdfg_builder(U.gcn_message, bad_reduce)
+    with pytest.raises(BuildError, match="dim 1"):
+        mpdfg_builder(U.gcn_message, bad_softmax)
+    with pytest.raises(BuildError, match="annotated"):
+        mpdfg_builder(untyped_message, U.gcn_reduce)
