@@ -442,6 +442,29 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> linear_attn(
   return std::make_tuple(z, el, er);
 }
 
+// The dense head of a GAT layer after the split / reorder passes
+// (GAT.py:25-29): z = h @ fc, el = z @ w_src, er = z @ w_dst with w_src / w_dst
+// the two (M, 1) halves of the attention vector.  One kernel when the shape
+// allows (fp32, a single attention column, M in {16, 32, 64}); otherwise three
+// GPU GEMMs through ATen, still on the device.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> gat_project(
+    torch::Tensor h, torch::Tensor fc, torch::Tensor w_src, torch::Tensor w_dst) {
+  check_input(h, "h");
+  check_input(fc, "fc_weight");
+  TORCH_CHECK(w_src.is_cuda() && w_dst.is_cuda(), "attention weights must be a CUDA tensor");
+  TORCH_CHECK(h.dim() == 2 && fc.dim() == 2 && fc.size(0) == h.size(1), "fc_weight must be (K, M)");
+  const int64_t M = fc.size(1);
+  const bool one_kernel = h.scalar_type() == at::kFloat && fc.scalar_type() == at::kFloat &&
+                          w_src.scalar_type() == at::kFloat && w_dst.scalar_type() == at::kFloat &&
+                          w_src.dim() == 2 && w_dst.dim() == 2 && w_src.size(1) == 1 &&
+                          w_dst.size(1) == 1 && w_src.size(0) == M && w_dst.size(0) == M &&
+                          (M == 16 || M == 32 || M == 64);
+  if (one_kernel)   // an (M, 1) column read as one (1, M) head vector
+    return linear_attn(h, fc, w_src.contiguous().view({1, M}), w_dst.contiguous().view({1, M}));
+  torch::Tensor z = at::mm(h, fc);
+  return std::make_tuple(z, at::mm(z, w_src), at::mm(z, w_dst));
+}
+
 }  // namespace
 
 TORCH_LIBRARY(my_classes, m) {
@@ -496,4 +519,7 @@ static auto registry =
             &gat_aggregate)
         .op("my_ops::linear_attn(Tensor x, Tensor w, Tensor a_l, Tensor a_r) -> "
             "(Tensor z, Tensor el, Tensor er)",
-            &linear_attn);
+            &linear_attn)
+        .op("my_ops::gat_project(Tensor h, Tensor fc, Tensor w_src, Tensor w_dst) -> "
+            "(Tensor z, Tensor el, Tensor er)",
+            &gat_project);

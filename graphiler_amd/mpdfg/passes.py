@@ -171,6 +171,16 @@ class _Rewriter:
                 n.replaceInput(0, first.inputsAt(0))
                 changed = True
                 continue
+            if kind == "my_ops::get_feat_dim" and first.kind() == "aten::mm":
+                # width of a product = columns of its right operand: frees the
+                # consumer (a weight slice) from depending on the product itself
+                one = self.const(1, n)
+                cols = self.make("aten::size", [first.inputsAt(1), one], n, SHARED,
+                                 ty=torch._C.IntType.get())
+                n.output().replaceAllUsesWith(cols)
+                n.destroy()
+                changed = True
+                continue
             if kind in _PAIRWISE and n.inputsSize() >= 2:
                 second = n.inputsAt(1).node()
                 if (first.kind() in _BCAST and second.kind() == first.kind()
@@ -222,6 +232,9 @@ class _Rewriter:
         for n in list(self.G.nodes()):
             if n.kind() == "my_ops::gspmm_src_mul_e_sum":
                 changed |= self._fuse_gat_chain(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::gat_aggregate":
+                changed |= self._fuse_gat_project(n)
         return changed
 
     def _fuse_spmm(self, n) -> bool:
@@ -312,6 +325,54 @@ class _Rewriter:
                         [add.inputsAt(0), add.inputsAt(1), z, slope_v, self.dglgraph], n, NODE)
         n.output().replaceAllUsesWith(out)
         for dead in (n, sm, act, add):      # the in-place activation would not be swept
+            dead.destroy()
+        return True
+
+
+    def _fuse_gat_project(self, n) -> bool:
+        """gat_aggregate(mm(z, w_src), mm(z, w_dst), z = mm(h, fc), ...) with node
+        data h and shared weights -> (z, el, er) = gat_project(h, fc, w_src, w_dst):
+        the projection and both attention products in one operator."""
+        el, er, z = n.inputsAt(0).node(), n.inputsAt(1).node(), n.inputsAt(2).node()
+        if not (el.kind() == er.kind() == z.kind() == "aten::mm"):
+            return False
+        if el.inputsAt(0).unique() != z.output().unique() or \
+                er.inputsAt(0).unique() != z.output().unique():
+            return False
+        h, fc = z.inputsAt(0), z.inputsAt(1)
+        w_s, w_d = el.inputsAt(1), er.inputsAt(1)
+        if self.where(h) != NODE or any(self.where(v) != SHARED for v in (fc, w_s, w_d)):
+            return False
+        # the weights must be defined before the place the product is computed
+        def depends_on(v, target, depth=0) -> bool:
+            node = v.node()
+            if node.kind() == "prim::Param" or depth > 32:
+                return False
+            return node is target or node == target or \
+                any(depends_on(i, target, depth + 1) for i in node.inputs())
+
+        def hoist(v):
+            node = v.node()
+            if node.kind() == "prim::Param" or node.isBefore(z):
+                return
+            for i in node.inputs():
+                hoist(i)
+            node.moveBefore(z)
+
+        if depends_on(w_s, z) or depends_on(w_d, z):
+            return False
+        hoist(w_s)
+        hoist(w_d)
+        node = self.G.create("my_ops::gat_project", [h, fc, w_s, w_d], 3)
+        node.insertBefore(z)
+        for o in node.outputs():
+            o.setType(torch._C.TensorType.get())
+            self.res[o.unique()] = NODE
+        outs = list(node.outputs())
+        z.output().replaceAllUsesWith(outs[0])
+        el.output().replaceAllUsesWith(outs[1])
+        er.output().replaceAllUsesWith(outs[2])
+        for dead in (el, er, z):
             dead.destroy()
         return True
 

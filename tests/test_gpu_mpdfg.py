@@ -41,19 +41,21 @@ def test_gcn_plan(device, level):
     assert_close(g.ndata['h'].cpu().numpy(), want, TOL_F32, f"GCN plan level {level}")
 
 
-@pytest.mark.parametrize("level", [0, 1, 2])
-def test_gat_plan(device, level):
+@pytest.mark.parametrize("level,width", [(0, 32), (1, 32), (2, 32), (2, 64), (2, 24)])
+def test_gat_plan(device, level, width):
+    """width 32 / 64: the projection runs as one kernel at level 2; width 24:
+    the same operator takes its three-GEMM route."""
     rng = np.random.default_rng(22)
     n, src, dst = _homo(rng)
     g = GraphData(prepare_graph(src, dst, n, device))
     h = rng.standard_normal((n, 24), dtype=np.float32)
-    fc = (rng.standard_normal((24, 32)) / 5).astype(np.float32)
-    attn = (rng.standard_normal((64, 1)) / 5).astype(np.float32)
+    fc = (rng.standard_normal((24, width)) / 5).astype(np.float32)
+    attn = (rng.standard_normal((2 * width, 1)) / 5).astype(np.float32)
     g.ndata['h'] = _t(h, device)
     update_all(g, mpdfg_builder(U.gat_message, U.gat_reduce, opt_level=level),
                msg_params=(_t(fc, device), _t(attn, device)))
     z = h.astype(np.float64) @ fc
-    el, er = (z @ attn[:32]).astype(np.float32), (z @ attn[32:]).astype(np.float32)
+    el, er = (z @ attn[:width]).astype(np.float32), (z @ attn[width:]).astype(np.float32)
     arr = build_graph_arrays(src, dst, n)
     want = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er,
                                 z.astype(np.float32), heads=1, slope=0.2)

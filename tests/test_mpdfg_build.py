@@ -50,6 +50,7 @@ def test_level1_moves_dense_work_to_the_nodes():
     assert "aten::cat" not in k                                 # split
     assert k.index("aten::mm") < k.index("my_ops::BroadcastSrcNode")   # reorder
     assert k.count("aten::mm") == 3             # z once (source and destination share it), el, er
+    assert "my_ops::get_feat_dim" not in k and "aten::size" in k   # slice width from the weight
     _, k = _kinds("gcn", 1)
     assert k.index("aten::mul") < k.index("my_ops::BroadcastSrcNode")
     assert k.count("my_ops::BroadcastSrcNode") == 1
@@ -60,7 +61,8 @@ def test_level2_fuses_into_graph_operators():
     assert "my_ops::SpMMSrc" in k and not any(x.startswith("my_ops::Broadcast") for x in k)
     _, k = _kinds("gat", 2)
     ours = [x for x in k if x.startswith("my_ops::")]
-    assert ours == ["my_ops::get_feat_dim", "my_ops::gat_aggregate"]
+    assert ours == ["my_ops::gat_project", "my_ops::gat_aggregate"]    # two kernels end to end
+    assert "aten::mm" not in k
     _, k = _kinds("rgcn", 2)
     assert "my_ops::SegmentMMEdge" in k and "aten::bmm" not in k and "my_ops::BroadcastEdgeType" not in k
     _, k = _kinds("hgt", 2)
