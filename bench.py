@@ -23,7 +23,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 # HBM bytes per dominant-kernel launch measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); the summary
 # lives under profiles/.  None until measured for the kernel named below.
-MEASURED_TRAFFIC_BYTES = {"plan": 1_486_204_723, "fused": 1_509_594_829}
+MEASURED_TRAFFIC_BYTES = {"plan": 1_486_204_723, "fused": 1_509_594_829,
+                          "compiled": 1_509_594_829}
 
 
 def main():
@@ -31,7 +32,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--path", choices=["fused", "plan"], default="fused")
+    ap.add_argument("--path", choices=["fused", "plan", "compiled"], default="fused",
+                    help="fused: projection + one aggregation pass; plan: the reference's "
+                         "four graph operators (GAT.py:25-36 after fusion); compiled: the "
+                         "GAT user-defined functions of bench_udf.py through the MP-DFG "
+                         "builder (opt level 2) and the TorchScript interpreter")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device-to-device elementwise copy "
@@ -65,7 +70,7 @@ def main():
     g.in_row_of_slot                              # per-graph schedule, built once
     assert g.in_eid_is_identity
 
-    fused = args.path == "fused"
+    fused = args.path != "plan"
     if args.calibrate_copy:
         big = torch.zeros(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB
         for _ in range(3):
@@ -73,8 +78,19 @@ def main():
         torch.cuda.synchronize()
         del big, big2
 
-    def step():
-        return layers.gat_layer(g, x, w, a, heads, slope, fused=fused)
+    if args.path == "compiled":
+        import bench_udf
+        from graphiler_amd.mpdfg import GraphData, mpdfg_builder, update_all
+        plan = mpdfg_builder(bench_udf.gat_message, bench_udf.gat_reduce, opt_level=2)
+        gd = GraphData(g)
+        attn_col = torch.cat([a[0].reshape(-1, 1), a[1].reshape(-1, 1)]).contiguous()
+
+        def step():
+            gd.ndata["h"] = x            # update_all stores its result under "h"
+            return update_all(gd, plan, msg_params=(w, attn_col))["h"]
+    else:
+        def step():
+            return layers.gat_layer(g, x, w, a, heads, slope, fused=fused)
 
     for _ in range(args.warmup):
         step()
