@@ -32,6 +32,7 @@ struct GatPolicy {
     int heads;
     int dph;
     float slope;
+    bool ids_vec;   // row_of_slot and nbr are 16-byte aligned
   };
   static __device__ __forceinline__ void init(float (&st)[VEC + 2]) {
 #pragma unroll
@@ -74,23 +75,19 @@ struct GatPolicy {
     typedef Frag<T, VEC> IO;
     const int h = f0 / A.dph;
     for (int64_t j = a; j < b; j += kUnroll) {
-      int r[kUnroll];
-      int64_t g[kUnroll];
+      int r[kUnroll], g[kUnroll];
       float s[kUnroll];
       typename IO::raw_t x[kUnroll];
+      load_ids8(row_of_slot, j, b, A.ids_vec, r);
+      load_ids8(A.nbr, j, b, A.ids_vec, g);
 #pragma unroll
       for (int t = 0; t < kUnroll; ++t) {
-        const int64_t jj = j + t < b ? j + t : b - 1;
-        r[t] = row_of_slot[jj];
-        g[t] = A.nbr[jj];
-      }
-#pragma unroll
-      for (int t = 0; t < kUnroll; ++t) {
-        x[t] = IO::load(A.z + g[t] * feat + f0);
-        s[t] = leaky(A.el[g[t] * A.heads + h] + A.er[(int64_t)r[t] * A.heads + h],
+        x[t] = IO::load(A.z + (int64_t)g[t] * feat + f0);
+        s[t] = leaky(A.el[(int64_t)g[t] * A.heads + h] + A.er[(int64_t)r[t] * A.heads + h],
                      A.slope);
       }
-      if (j + kUnroll <= b && r[0] == cur && r[kUnroll - 1] == cur) {
+      const bool one_row = j + kUnroll <= b && r[0] == cur && r[kUnroll - 1] == cur;
+      if (one_row) {
         // whole batch inside the open row (rows are sorted): one rescale
         float bm = s[0];
 #pragma unroll
@@ -141,7 +138,8 @@ int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const void *z, void *out, int64_t n_rows, int64_t n_edges,
                int heads, int dim, float slope, float *ws, hipStream_t stream) {
   typedef GatPolicy<T, VEC> P;
-  typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope};
+  const bool ids_vec = aligned(row_of_slot, 16) && aligned(nbr, 16);
+  typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges,
                         heads * dim, ws, stream);
 }

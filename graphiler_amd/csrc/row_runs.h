@@ -33,6 +33,25 @@ namespace ga {
 
 constexpr int kUnroll = 8;
 
+static_assert(kUnroll == 8, "load_ids8 reads two int4");
+
+// Eight consecutive int32 of a slot-indexed column starting at slot j (a
+// multiple of 8: runs start at multiples of 32).  Two 16-byte loads when the
+// column is 16-byte aligned and the batch is whole; otherwise element loads
+// clamped to the run's last slot.
+__device__ __forceinline__ void load_ids8(const int32_t *__restrict__ p, int64_t j, int64_t b,
+                                          bool vec, int (&out)[kUnroll]) {
+  if (vec && j + kUnroll <= b) {
+    const int4 lo = *reinterpret_cast<const int4 *>(p + j);
+    const int4 hi = *reinterpret_cast<const int4 *>(p + j + 4);
+    out[0] = lo.x; out[1] = lo.y; out[2] = lo.z; out[3] = lo.w;
+    out[4] = hi.x; out[5] = hi.y; out[6] = hi.z; out[7] = hi.w;
+  } else {
+#pragma unroll
+    for (int t = 0; t < kUnroll; ++t) out[t] = p[j + t < b ? j + t : b - 1];
+  }
+}
+
 struct RunGeom {
   int64_t n_edges;
   int64_t n_runs;

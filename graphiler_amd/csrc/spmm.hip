@@ -56,6 +56,7 @@ struct SpmmPolicy {
     const float *w;
     int heads;
     int dph;
+    bool ids_vec;   // row_of_slot, gidx and eid (where given) are 16-byte aligned
   };
   static __device__ __forceinline__ void init(float (&st)[VEC]) {
 #pragma unroll
@@ -88,22 +89,28 @@ struct SpmmPolicy {
     typedef Frag<T, VEC> IO;
     const int h = HASW ? f0 / A.dph : 0;
     for (int64_t j = a; j < b; j += kUnroll) {
-      int r[kUnroll];
-      int64_t g[kUnroll];
+      int r[kUnroll], g[kUnroll], e[kUnroll];
       float ww[kUnroll];
       typename IO::raw_t x[kUnroll];
+      load_ids8(row_of_slot, j, b, A.ids_vec, r);
+      if (A.gidx) {
+        load_ids8(A.gidx, j, b, A.ids_vec, g);
+      } else {
 #pragma unroll
-      for (int t = 0; t < kUnroll; ++t) {
-        const int64_t jj = j + t < b ? j + t : b - 1;
-        r[t] = row_of_slot[jj];
-        g[t] = A.gidx ? (int64_t)A.gidx[jj] : jj;
-        if (HASW) {
-          const int64_t e = A.eid ? (int64_t)A.eid[jj] : jj;
-          ww[t] = A.w[e * A.heads + h];
+        for (int t = 0; t < kUnroll; ++t) g[t] = (int)(j + t < b ? j + t : b - 1);
+      }
+      if (HASW) {
+        if (A.eid) {
+          load_ids8(A.eid, j, b, A.ids_vec, e);
+        } else {
+#pragma unroll
+          for (int t = 0; t < kUnroll; ++t) e[t] = (int)(j + t < b ? j + t : b - 1);
         }
+#pragma unroll
+        for (int t = 0; t < kUnroll; ++t) ww[t] = A.w[(int64_t)e[t] * A.heads + h];
       }
 #pragma unroll
-      for (int t = 0; t < kUnroll; ++t) x[t] = IO::load(A.u + g[t] * feat + f0);
+      for (int t = 0; t < kUnroll; ++t) x[t] = IO::load(A.u + (int64_t)g[t] * feat + f0);
 #pragma unroll
       for (int t = 0; t < kUnroll; ++t) {
         if (j + t < b) {
@@ -129,7 +136,9 @@ int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
                 const float *w, void *out, int64_t n_rows, int64_t n_edges,
                 int feat, int heads, float *partial, hipStream_t stream) {
   typedef SpmmPolicy<T, VEC, RED, BOP> P;
-  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads};
+  const bool ids_vec = aligned(row_of_slot, 16) && (!gidx || aligned(gidx, 16)) &&
+                       (!eid || aligned(eid, 16));
+  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads, ids_vec};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, feat,
                         partial, stream);
 }
