@@ -60,6 +60,8 @@ struct RunGeom {
   int run_shift;
   int tpr_shift;
   int lanes_total;  // ceil(feat / VEC): state slots per partial row
+  int64_t n_wg;     // workgroups of the main kernel that walk runs; the blocks
+                    // after them write the rows without edges
 };
 
 // Per-run bookkeeping shared through LDS.
@@ -88,11 +90,22 @@ __device__ __forceinline__ void emit_empty_row(typename Policy::out_t *out, int6
 
 template <class Policy>
 __global__ __launch_bounds__(kBlock) void runs_kernel(
-    typename Policy::Args args, const int32_t *__restrict__ row_of_slot,
-    typename Policy::out_t *__restrict__ out, float *__restrict__ partial,
-    RunGeom geo) {
+    typename Policy::Args args, const int32_t *__restrict__ pointer,
+    const int32_t *__restrict__ row_of_slot, typename Policy::out_t *__restrict__ out,
+    float *__restrict__ partial, RunGeom geo) {
   constexpr int VEC = Policy::kVec;
   constexpr int SF = Policy::kState;
+  if ((int64_t)blockIdx.x >= geo.n_wg) {
+    // Trailing blocks: one lane group per row, rows without edges get the empty
+    // value.  They share the launch with the gathers, so this small amount of
+    // streaming work hides behind them instead of costing a pass of its own.
+    const int tpr_ = 1 << geo.tpr_shift;
+    const int f0_ = ((int)blockIdx.y * tpr_ + (threadIdx.x & (tpr_ - 1))) * VEC;
+    const int64_t row = (((int64_t)blockIdx.x - geo.n_wg) * kBlock + threadIdx.x) >> geo.tpr_shift;
+    if (f0_ < geo.feat && row < geo.n_rows && pointer[row] == pointer[row + 1])
+      Policy::emit_empty(args, out, row, geo.feat, f0_);
+    return;
+  }
   // LDS: [run in block][A|B][lane in group][SF]
   extern __shared__ float lds_state[];
   __shared__ RunFlags flags[kBlock];
@@ -214,7 +227,8 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
 // Blocks [0, fix_blocks): one lane group per main-kernel workgroup q; the group
 // whose slot range holds the END of a row that began in an earlier workgroup
 // combines that row's global partial states in workgroup order.  Remaining
-// blocks: one lane group per row, rows without edges get Policy::empty_row.
+// blocks (only for a graph without edges, where the main kernel does not run):
+// one lane group per row, every row gets Policy::empty_row.
 template <class Policy>
 __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
     typename Policy::Args args, const int32_t *__restrict__ pointer,
@@ -284,16 +298,18 @@ int launch_runs(typename Policy::Args args, const int32_t *pointer,
   geo.lanes_total = lanes;
   const int G = kBlock >> geo.tpr_shift;
   const int64_t n_wg = (geo.n_runs + G - 1) / G;
+  const int64_t row_blocks = (n_rows + G - 1) / G;
+  geo.n_wg = n_wg;
   typedef typename Policy::out_t out_t;
-  if (n_wg > 0x7fffffff) return GA_EUNSUPPORTED;
+  if (n_wg + row_blocks > 0x7fffffff) return GA_EUNSUPPORTED;
   if (n_wg > 0) {
     const size_t lds = (size_t)kBlock * 2 * SF * sizeof(float);
-    hipLaunchKernelGGL((runs_kernel<Policy>), dim3((unsigned)n_wg, ftiles),
-                       dim3(kBlock), lds, stream, args, row_of_slot,
+    hipLaunchKernelGGL((runs_kernel<Policy>), dim3((unsigned)(n_wg + row_blocks), ftiles),
+                       dim3(kBlock), lds, stream, args, pointer, row_of_slot,
                        (out_t *)out, partial, geo);
   }
   const int64_t fix_blocks = (n_wg + G - 1) / G;
-  const int64_t fill_blocks = (n_rows + G - 1) / G;
+  const int64_t fill_blocks = n_wg > 0 ? 0 : row_blocks;
   if (fix_blocks + fill_blocks > 0x7fffffff) return GA_EUNSUPPORTED;
   if (fix_blocks + fill_blocks > 0)
     hipLaunchKernelGGL((runs_fixup_kernel<Policy>),
