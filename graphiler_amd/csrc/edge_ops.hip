@@ -16,10 +16,19 @@ __device__ __forceinline__ float load_f32<bf16_t>(const bf16_t *p) {
   return bf16_lo(*p);
 }
 
-// ---- u_add_v ---------------------------------------------------------------
+// ---- u (op) v --------------------------------------------------------------
 // One thread per output element; FEAT1 specialisation handles four consecutive
-// edges per thread so index and output accesses are 16 bytes wide.
-template <typename IdxT, typename T>
+// edges per thread so index and output accesses are 16 bytes wide.  OP is the
+// binary functor (functor.cuh:19-72): one fp32 operation per element.
+template <int OP>
+__device__ __forceinline__ float edge_op(float a, float b) {
+  if (OP == GA_SDDMM_SUB) return a - b;
+  if (OP == GA_SDDMM_MUL) return a * b;
+  if (OP == GA_SDDMM_DIV) return a / b;
+  return a + b;
+}
+
+template <typename IdxT, typename T, int OP>
 __global__ __launch_bounds__(kBlock) void u_add_v_kernel(
     const IdxT *__restrict__ lhs, const IdxT *__restrict__ rhs,
     const T *__restrict__ u, const T *__restrict__ v, float *__restrict__ out,
@@ -28,11 +37,11 @@ __global__ __launch_bounds__(kBlock) void u_add_v_kernel(
   if (t >= n_edges * feat) return;
   const int64_t i = t / feat;
   const int k = (int)(t - i * feat);
-  out[t] = load_f32(u + (int64_t)lhs[i] * feat + k) +
-           load_f32(v + (int64_t)rhs[i] * feat + k);
+  out[t] = edge_op<OP>(load_f32(u + (int64_t)lhs[i] * feat + k),
+                       load_f32(v + (int64_t)rhs[i] * feat + k));
 }
 
-template <typename IdxT, typename T>
+template <typename IdxT, typename T, int OP>
 __global__ __launch_bounds__(kBlock) void u_add_v_feat1_kernel(
     const IdxT *__restrict__ lhs, const IdxT *__restrict__ rhs,
     const T *__restrict__ u, const T *__restrict__ v, float *__restrict__ out,
@@ -45,11 +54,11 @@ __global__ __launch_bounds__(kBlock) void u_add_v_feat1_kernel(
     for (int q = 0; q < 4; ++q) { l[q] = lhs[i0 + q]; r[q] = rhs[i0 + q]; }
     float o[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) o[q] = load_f32(u + l[q]) + load_f32(v + r[q]);
+    for (int q = 0; q < 4; ++q) o[q] = edge_op<OP>(load_f32(u + l[q]), load_f32(v + r[q]));
     *reinterpret_cast<float4 *>(out + i0) = make_float4(o[0], o[1], o[2], o[3]);
   } else {
     for (int64_t i = i0; i < n_edges; ++i)
-      out[i] = load_f32(u + lhs[i]) + load_f32(v + rhs[i]);
+      out[i] = edge_op<OP>(load_f32(u + lhs[i]), load_f32(v + rhs[i]));
   }
 }
 
@@ -140,20 +149,20 @@ int pick_gather_unit(const void *idx, const void *x, void *y, int64_t n_out,
   return launch_gather<IdxT, uint8_t>(idx, x, y, n_out, row_bytes, s);
 }
 
-template <typename IdxT, typename T>
-int launch_u_add_v(const void *lhs, const void *rhs, const void *u,
+template <typename IdxT, typename T, int OP>
+int launch_u_op_v(const void *lhs, const void *rhs, const void *u,
                    const void *v, float *out, int64_t n_edges, int feat,
                    hipStream_t s) {
   if (feat == 1 && aligned(out, 16)) {
     const int64_t threads = (n_edges + 3) / 4;
     const int64_t blocks = (threads + kBlock - 1) / kBlock;
-    hipLaunchKernelGGL((u_add_v_feat1_kernel<IdxT, T>), dim3((unsigned)blocks),
+    hipLaunchKernelGGL((u_add_v_feat1_kernel<IdxT, T, OP>), dim3((unsigned)blocks),
                        dim3(kBlock), 0, s, (const IdxT *)lhs, (const IdxT *)rhs,
                        (const T *)u, (const T *)v, out, n_edges);
   } else {
     const int64_t blocks = (n_edges * feat + kBlock - 1) / kBlock;
     if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-    hipLaunchKernelGGL((u_add_v_kernel<IdxT, T>), dim3((unsigned)blocks),
+    hipLaunchKernelGGL((u_add_v_kernel<IdxT, T, OP>), dim3((unsigned)blocks),
                        dim3(kBlock), 0, s, (const IdxT *)lhs, (const IdxT *)rhs,
                        (const T *)u, (const T *)v, out, n_edges, feat);
   }
@@ -207,24 +216,39 @@ int check_edge_args(const void *lhs, const void *rhs, int idx_bits,
 
 extern "C" {
 
-int ga_sddmm_u_add_v(const void *lhs, const void *rhs, int idx_bits,
-                     const void *u, const void *v, float *out, int64_t n_edges,
-                     int64_t feat, int dtype, ga_stream_t stream) {
+int ga_sddmm_u_op_v(const void *lhs, const void *rhs, int idx_bits,
+                    const void *u, const void *v, float *out, int64_t n_edges,
+                    int64_t feat, int op, int dtype, ga_stream_t stream) {
   if (feat <= 0 || feat > 0x7fffffff) return GA_EINVAL;
+  if (op < GA_SDDMM_ADD || op > GA_SDDMM_DIV) return GA_EINVAL;
   int rc = ga::check_edge_args(lhs, rhs, idx_bits, u, v, out, n_edges, dtype);
   if (rc != GA_OK || n_edges == 0) return rc;
   hipStream_t s = (hipStream_t)stream;
-  if (idx_bits == 64)
-    return dtype == GA_F32
-               ? ga::launch_u_add_v<int64_t, float>(lhs, rhs, u, v, out, n_edges,
-                                                    (int)feat, s)
-               : ga::launch_u_add_v<int64_t, ga::bf16_t>(lhs, rhs, u, v, out,
-                                                         n_edges, (int)feat, s);
-  return dtype == GA_F32
-             ? ga::launch_u_add_v<int32_t, float>(lhs, rhs, u, v, out, n_edges,
-                                                  (int)feat, s)
-             : ga::launch_u_add_v<int32_t, ga::bf16_t>(lhs, rhs, u, v, out,
-                                                       n_edges, (int)feat, s);
+#define GA_U_OP_V(IDX, T)                                                             \
+  switch (op) {                                                                       \
+    case GA_SDDMM_SUB:                                                                \
+      return ga::launch_u_op_v<IDX, T, GA_SDDMM_SUB>(lhs, rhs, u, v, out, n_edges, (int)feat, s); \
+    case GA_SDDMM_MUL:                                                                \
+      return ga::launch_u_op_v<IDX, T, GA_SDDMM_MUL>(lhs, rhs, u, v, out, n_edges, (int)feat, s); \
+    case GA_SDDMM_DIV:                                                                \
+      return ga::launch_u_op_v<IDX, T, GA_SDDMM_DIV>(lhs, rhs, u, v, out, n_edges, (int)feat, s); \
+    default:                                                                          \
+      return ga::launch_u_op_v<IDX, T, GA_SDDMM_ADD>(lhs, rhs, u, v, out, n_edges, (int)feat, s); \
+  }
+  if (idx_bits == 64) {
+    if (dtype == GA_F32) GA_U_OP_V(int64_t, float)
+    GA_U_OP_V(int64_t, ga::bf16_t)
+  }
+  if (dtype == GA_F32) GA_U_OP_V(int32_t, float)
+  GA_U_OP_V(int32_t, ga::bf16_t)
+#undef GA_U_OP_V
+}
+
+int ga_sddmm_u_add_v(const void *lhs, const void *rhs, int idx_bits,
+                     const void *u, const void *v, float *out, int64_t n_edges,
+                     int64_t feat, int dtype, ga_stream_t stream) {
+  return ga_sddmm_u_op_v(lhs, rhs, idx_bits, u, v, out, n_edges, feat, GA_SDDMM_ADD, dtype,
+                         stream);
 }
 
 int ga_sddmm_u_dot_v(const void *lhs, const void *rhs, int idx_bits,

@@ -194,6 +194,30 @@ def gsddmm_u_add_v_mul_alpha(src_feature, dst_feature, alpha: int,
     return out
 
 
+def gsddmm_u_op_v(op: str, src_feature, dst_feature, graph: DGLGraph) -> torch.Tensor:
+    """Generic SDDMM of the reference (sddmm.cuh:34-71 with the add / sub / mul /
+    div functors, functor.cuh:19-72): out[e] = src_feature[src[e]] (op)
+    dst_feature[dst[e]] in edge-id order, fp32 (E, feat)."""
+    code = {"add": capi.GA_SDDMM_ADD, "sub": capi.GA_SDDMM_SUB, "mul": capi.GA_SDDMM_MUL,
+            "div": capi.GA_SDDMM_DIV}[op]
+    _check_input(src_feature, "src_feature")
+    _check_input(dst_feature, "dst_feature")
+    dt = _feat_dtype(src_feature, "src_feature")
+    if dst_feature.dtype != src_feature.dtype:
+        raise RuntimeError("src_feature and dst_feature must share a dtype")
+    feat = get_feat_dim(src_feature)
+    if get_feat_dim(dst_feature) != feat:
+        raise RuntimeError("src_feature and dst_feature must share a width")
+    out = torch.empty(_out_shape(graph.num_edges, src_feature),
+                      dtype=torch.float32, device=src_feature.device)
+    lhs, rhs, bits = _edge_columns(graph)
+    capi.check(capi.load().ga_sddmm_u_op_v(
+        lhs.data_ptr(), rhs.data_ptr(), bits, src_feature.data_ptr(),
+        dst_feature.data_ptr(), out.data_ptr(), graph.num_edges, feat, code, dt,
+        _stream(out)), "ga_sddmm_u_op_v")
+    return out
+
+
 def gsddmm_u_dot_v(src_feature, dst_feature, graph: DGLGraph) -> torch.Tensor:
     """u_dot_v over the last dimension (functor.cuh:103-116, sddmm.cuh:80-120):
     (N, H, D) x (N, H, D) -> (E, H) fp32; 2-D inputs are one head."""

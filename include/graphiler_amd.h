@@ -41,6 +41,7 @@ typedef void *ga_stream_t;
 
 enum ga_dtype { GA_F32 = 0, GA_BF16 = 1 };
 /* message = u[nbr] | e[eid] | u[nbr] * w[eid]   (functor.cuh:18-121)         */
+enum ga_sddmm_op { GA_SDDMM_ADD = 0, GA_SDDMM_SUB = 1, GA_SDDMM_MUL = 2, GA_SDDMM_DIV = 3 };
 enum ga_spmm_op {
   GA_COPY_U = 0, GA_COPY_E = 1,
   GA_U_MUL_E = 2, GA_U_ADD_E = 3, GA_U_SUB_E = 4, GA_U_DIV_E = 5 /* u[src] (op) w[edge] */
@@ -138,6 +139,14 @@ int ga_spmm_csr_arg(const int32_t *pointer, const int32_t *row_of_slot,
 int ga_sddmm_u_add_v(const void *lhs, const void *rhs, int idx_bits,
                      const void *u, const void *v, float *out, int64_t n_edges,
                      int64_t feat, int dtype, ga_stream_t stream);
+
+/* The same kernel with the other binary functors of the reference's generic
+ * SDDMM (SDDMMCooKernel<..., BinaryOp, ...>, sddmm.cuh:34-71 with
+ * functor.cuh:19-72): out[i, k] = u[lhs[i], k] (op) v[rhs[i], k], one fp32
+ * operation per element.  op: GA_SDDMM_ADD / SUB / MUL / DIV. */
+int ga_sddmm_u_op_v(const void *lhs, const void *rhs, int idx_bits,
+                    const void *u, const void *v, float *out, int64_t n_edges,
+                    int64_t feat, int op, int dtype, ga_stream_t stream);
 
 /* out[i, h] = sum_d u[lhs[i], h, d] * v[rhs[i], h, d], fp32 output (E, heads).
  * The Dot functor (functor.cuh:103-116) with the reduction over the last

@@ -147,6 +147,20 @@ def sddmm_u_add_v(src, dst, u, v):
     return out
 
 
+def sddmm_u_op_v(op, src, dst, u, v):
+    """Generic SDDMM: out[e] = u[src[e]] (op) v[dst[e]], op in add/sub/mul/div."""
+    src = _c(src, np.int64)
+    dst = _c(dst, np.int64)
+    u = _c(u, np.float32)
+    v = _c(v, np.float32)
+    feat = int(np.prod(u.shape[1:])) if u.ndim > 1 else 1
+    out = np.empty((src.shape[0], feat), np.float32)
+    code = {"add": 0, "sub": 1, "mul": 2, "div": 3}[op]
+    _check(lib().orc_sddmm_u_op_v(_i64(src.shape[0]), _p(src), _p(dst), _p(u), _p(v),
+                                  _p(out), _i64(feat), ctypes.c_int(code)), "u_op_v")
+    return out
+
+
 def sddmm_u_dot_v(src, dst, u, v):
     """u_dot_v over the last dimension: u, v are (N, H, D) -> (E, H)."""
     src = _c(src, np.int64)

@@ -229,6 +229,24 @@ int orc_sddmm_u_add_v(int64_t n_edges, const int64_t *src, const int64_t *dst,
 }
 
 /*
+ * The same with the other binary functors (functor.cuh:19-72): op 0 add, 1 sub,
+ * 2 mul, 3 div; one fp32 operation per element, as SDDMMCooKernel computes it
+ * (sddmm.cuh:34-71).
+ */
+int orc_sddmm_u_op_v(int64_t n_edges, const int64_t *src, const int64_t *dst,
+                     const float *u, const float *v, float *out, int64_t feat,
+                     int op) {
+  if (feat <= 0 || op < 0 || op > 3) return ORC_EINVAL;
+#pragma omp parallel for schedule(static)
+  for (int64_t e = 0; e < n_edges; ++e)
+    for (int64_t k = 0; k < feat; ++k) {
+      const float a = u[src[e] * feat + k], b = v[dst[e] * feat + k];
+      out[e * feat + k] = op == 0 ? a + b : op == 1 ? a - b : op == 2 ? a * b : a / b;
+    }
+  return ORC_OK;
+}
+
+/*
  * SDDMM u_dot_v: out[e, h] = sum_k u[src[e], h, k] * v[dst[e], h, k].
  * Follows the Dot functor (functor.cuh:103-116) with the reduction over the
  * last feature dimension (bcast.cc:37-39, 57-60).

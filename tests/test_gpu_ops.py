@@ -260,6 +260,21 @@ def test_sddmm_u_add_v_bit_exact(graph, device, feat, bf16):
     assert np.array_equal(got.cpu().numpy(), ref), f"u_add_v {name} F={feat}"
 
 
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+@pytest.mark.parametrize("feat", [1, 4, 5])
+def test_sddmm_u_op_v_bit_exact(graph, device, op, feat):
+    """One fp32 operation per element: the result must equal the oracle's bit
+    for bit (division included: it is correctly rounded on both sides)."""
+    name, g, arr = graph
+    rng = np.random.default_rng(feat)
+    u = rng.standard_normal((arr.num_nodes, feat), dtype=np.float32)
+    v = rng.standard_normal((arr.num_nodes, feat), dtype=np.float32)
+    v = np.where(np.abs(v) < 0.1, 1.0, v).astype(np.float32)
+    got = ops.gsddmm_u_op_v(op, _dev(u, device), _dev(v, device), g).cpu().numpy()
+    ref = oracle.sddmm_u_op_v(op, arr.COO_src, arr.COO_dst, u, v)
+    assert np.array_equal(got, ref), f"{op} {name}"
+
+
 @pytest.mark.parametrize("heads,dim", [(1, 64), (8, 16), (4, 64), (3, 5),
                                        (1, 1), (2, 256)])
 @pytest.mark.parametrize("bf16", [False, True])

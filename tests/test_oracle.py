@@ -238,6 +238,12 @@ def test_sddmm_against_numpy_indexing():
     assert np.array_equal(oracle.sddmm_u_add_v(s, d, u, v), u[s] + v[d])
     # a swapped (src, dst) pair must not pass
     assert not np.array_equal(oracle.sddmm_u_add_v(s, d, u, v), u[d] + v[s])
+    # the other functors: numpy's own fp32 arithmetic on the indexed rows, bit for bit
+    v_nz = np.where(np.abs(v) < 0.1, 1.0, v).astype(np.float32)
+    for op, fn in (("add", np.add), ("sub", np.subtract), ("mul", np.multiply),
+                   ("div", np.divide)):
+        assert np.array_equal(oracle.sddmm_u_op_v(op, s, d, u, v_nz), fn(u[s], v_nz[d])), op
+    assert not np.array_equal(oracle.sddmm_u_op_v("sub", s, d, u, v_nz), v_nz[d] - u[s])
     a = rng.standard_normal((n, 4, 7)).astype(np.float32)
     b = rng.standard_normal((n, 4, 7)).astype(np.float32)
     want = np.einsum("ehk,ehk->eh", a[s].astype(np.float64), b[d].astype(np.float64))
