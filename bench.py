@@ -23,8 +23,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 # HBM bytes per dominant-kernel launch measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); the summary
 # lives under profiles/.  None until measured for the kernel named below.
-MEASURED_TRAFFIC_BYTES = {"plan": 1_486_204_723, "fused": 1_509_594_829,
-                          "compiled": 1_509_594_829}
+MEASURED_TRAFFIC_BYTES = {"plan": 1_517_519_171, "fused": 1_513_213_043,
+                          "compiled": 1_513_213_043}
 
 
 def main():
@@ -147,6 +147,7 @@ def main():
         "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES[args.path],
+        "traffic_GBps": round(MEASURED_TRAFFIC_BYTES[args.path] / (ops_ms[dom] * 1e-3) / 1e9, 1),
         "algorithmic_bytes": alg[dom], "launch_ms": round(ops_ms[dom], 4),
         "note": ("algorithmic bytes credit no cache reuse (one gathered row per "
                  "edge); a fraction above 1 means the gathers are cache-served: "
@@ -193,7 +194,7 @@ def main():
     roofline_dense = {
         "kernel": "linear_attn", "bound": "mfma", "achieved": round(dense_tflops, 2),
         "peak": 157.3, "unit": "TFLOP/s", "frac": round(dense_tflops / 157.3, 4),
-        "traffic": 663_342_080, "algorithmic_bytes": 4 * (N * in_dim + in_dim * out_dim
+        "traffic": 662_814_541, "algorithmic_bytes": 4 * (N * in_dim + in_dim * out_dim
                                                          + N * out_dim + 2 * N * heads),
         "launch_ms": round(ops_ms["dense_project"], 4),
     }
