@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import oracle
-import udf_models as U
+from graphiler_amd.examples import udf as U
 from graphiler_amd import prepare_graph
 from graphiler_amd.graph import build_graph_arrays
 from graphiler_amd.mpdfg import GraphData, mpdfg_builder, update_all

@@ -3,7 +3,7 @@ built and linted, not run)."""
 import pytest
 import torch
 
-import udf_models as U
+from graphiler_amd.examples import udf as U
 from graphiler_amd.mpdfg import BuildError, EdgeBatchDummy, NodeBatchDummy, mpdfg_builder
 
 MODELS = {
