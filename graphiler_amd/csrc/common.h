@@ -31,6 +31,21 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
 }
 
+// Sums over lane groups with DPP moves (all VALU, no LDS), result in every lane
+// of the group: swaps inside quads, then the half-row mirror (8 lanes:
+// 8j..8j+7) and the row mirror (16 lanes: 16j..16j+15).
+__device__ __forceinline__ float row8_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v = row8_sum(v);
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));  // row_mirror
+  return v;
+}
+
 // Row fragment I/O: VEC consecutive features of element type T, widened to
 // fp32 registers.  VEC > 1 uses one 16-byte access.
 template <typename T, int VEC>

@@ -34,16 +34,6 @@ constexpr int kSliceK = 32;                              // k per LDS slice
 constexpr int kXs = kSliceK + 4;                         // LDS row stride of the X tile
 constexpr int kWs = kPassCols + 4;                       // LDS row stride of the W tile
 
-// Sum over the 16 lanes of a DPP row (lanes 16j..16j+15), result in every lane:
-// swaps inside quads, then the half-row and row mirrors; all VALU, no LDS.
-__device__ __forceinline__ float row16_sum(float v) {
-  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));  // row_mirror
-  return v;
-}
-
 template <int VK> struct XVec;
 template <> struct XVec<4> { using type = float4; };
 template <> struct XVec<2> { using type = float2; };

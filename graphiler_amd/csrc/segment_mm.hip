@@ -22,6 +22,14 @@
 // two neighbouring outputs into one 4-byte store.  The type of a chunk is found
 // on the device from type_pointer (block-wide prefix sum of chunks per type):
 // no host copy, no synchronisation.
+//
+// Two fused forms of the exact-shape kernel serve per-edge products whose
+// operand lives on the nodes (Y[e] = X[endpoint(e)] @ W[type(e)], the
+// Broadcast -> bmm pairs of examples/RGCN/RGCN.py:26-28 and
+// examples/HGT/HGT.py:35-44): rows of X are read through an index instead of
+// being materialised per edge first, and the product can be reduced on the spot
+// against a second gathered row, out[e, h] = <Y[e, h, :], Q[q_index[e], h, :]>
+// (HGT's sum(k * q)), in which case Y never reaches memory.
 #include "common.h"
 
 namespace ga {
@@ -56,6 +64,17 @@ struct MmGeom {
   int KB, MB;          // k blocks / 16-column blocks of the tile
   int64_t ldx, ldy;    // row strides of X and Y (elements)
   int64_t w_type_stride;  // elements between W[t] and W[t+1]
+};
+
+// Optional gather / dot-product operands of the exact-shape kernel.
+struct MmExt {
+  const int64_t *x_index;   // row r reads X[x_index[r]]; null: X[r]
+  const void *Q;            // dot operand rows (ldq elements apart); null: store Y
+  const int64_t *q_index;   // row r is reduced against Q[q_index[r]]; null: Q[r]
+  float *dot;               // (rows, ldd) fp32, column = head
+  int64_t ldq, ldd;
+  unsigned head_end;        // bit cb: a head's columns end with column block cb
+  int half_heads;           // bf16, M == 16: a block pair holds two heads
 };
 
 // Column of the tile held by lane column j of column block cb.
@@ -340,6 +359,16 @@ __global__ __launch_bounds__(kBlock) void segment_mm_kernel(
   }
 }
 
+// element loads / stores widened to fp32
+template <typename T>
+__device__ __forceinline__ float ldf(const T *p);
+template <>
+__device__ __forceinline__ float ldf<float>(const float *p) { return *p; }
+template <>
+__device__ __forceinline__ float ldf<bf16_t>(const bf16_t *p) { return bf16_lo(*p); }
+__device__ __forceinline__ void stf(float *p, float v) { *p = v; }
+__device__ __forceinline__ void stf(bf16_t *p, float v) { *p = (bf16_t)f32_to_bf16_bits(v); }
+
 // ---- exact-shape kernel ------------------------------------------------------
 // NF = k blocks and CG = 16-column blocks of the tile, both compile-time (the
 // tile is zero padded up to them), so the LDS layout, every LDS / global offset
@@ -382,10 +411,10 @@ struct Tight<bf16_t, 32, NF, CG> {
   }
 };
 
-template <typename T, int KBLK, int NF, int CG>
+template <typename T, int KBLK, int NF, int CG, bool DOT>
 __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
     const int32_t *__restrict__ tp, const T *__restrict__ X,
-    const T *__restrict__ W, T *__restrict__ Y, MmGeom g) {
+    const T *__restrict__ W, T *__restrict__ Y, MmGeom g, MmExt e) {
   typedef Mma<T, KBLK> MM;
   typedef Tight<T, KBLK, NF, CG> TT;
   typedef typename MM::frag_t frag_t;
@@ -411,21 +440,30 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
   const bool full_cols = g.Mt == CG * 16;
   const bool pack_ok = (g.Mt & 1) == 0 && (g.ldy & 1) == 0;
 
-  const T *xp = X + (int64_t)(row0 + wave * kTileRows + lr) * g.ldx + klane;
+  // source row of X for tile row `row` (rows at or beyond row1 are never read)
+  const int64_t *__restrict__ xi = e.x_index;
+  auto src_row = [&](int row) -> int64_t {
+    if (row >= row1) return 0;
+    return xi ? xi[row] : (int64_t)row;
+  };
+  const int first = row0 + wave * kTileRows + lr;
   T *yp = Y + (int64_t)(row0 + wave * kTileRows + lk * 4) * g.ldy +
           (MM::kPaired ? 2 * lr : lr);
-  const int64_t xstep = (int64_t)kTileBlock * g.ldx, ystep = (int64_t)kTileBlock * g.ldy;
+  const int64_t ystep = (int64_t)kTileBlock * g.ldy;
 
-  // fragments of the next tile are requested before the current tile's MFMAs
+  // fragments of the next tile are requested before the current tile's MFMAs,
+  // and the source row of the tile after that before those loads are needed
   frag_t xn[NF];
   {
-    const bool xlive = row0 + wave * kTileRows + lr < row1;
+    const T *xp = X + src_row(first) * g.ldx + klane;
+    const bool xlive = first < row1;
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
       xn[f] = MM::zero();
       if (xlive && (kmask >> f & 1)) xn[f] = MM::load(xp + f * KBLK);
     }
   }
+  int64_t inext = src_row(first + kTileBlock);
   for (int tile0 = row0 + wave * kTileRows; tile0 < row1;
        tile0 += kTileBlock, yp += ystep) {
     // With many weight fragments the compiler would otherwise keep them all in
@@ -435,13 +473,16 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
     frag_t xa[NF];
 #pragma unroll
     for (int f = 0; f < NF; ++f) xa[f] = xn[f];
-    xp += xstep;
-    const bool xlive = tile0 + kTileBlock + lr < row1;
+    {
+      const T *xp = X + inext * g.ldx + klane;
+      const bool xlive = tile0 + kTileBlock + lr < row1;
 #pragma unroll
-    for (int f = 0; f < NF; ++f) {
-      xn[f] = MM::zero();
-      if (xlive && (kmask >> f & 1)) xn[f] = MM::load(xp + f * KBLK);
+      for (int f = 0; f < NF; ++f) {
+        xn[f] = MM::zero();
+        if (xlive && (kmask >> f & 1)) xn[f] = MM::load(xp + f * KBLK);
+      }
     }
+    inext = src_row(tile0 + 2 * kTileBlock + lr);
     floatx4 acc[CG];
 #pragma unroll
     for (int cb = 0; cb < CG; ++cb) acc[cb] = floatx4{0, 0, 0, 0};
@@ -452,6 +493,56 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
         acc[cb] = TT::mma(acc[cb], wl, f, cb, xa[f]);
     }
     // lane holds rows tile0 + 4*lk + r, lane column lr of every column block
+    if (DOT) {
+      const T *__restrict__ Q = static_cast<const T *>(e.Q);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = tile0 + lk * 4 + r;
+        const bool live = row < row1;          // uniform over the 16 lanes of a row
+        const int64_t qr = live ? (e.q_index ? e.q_index[row] : (int64_t)row) : 0;
+        const T *qrow = Q + qr * e.ldq;
+        float *drow = e.dot + (int64_t)row * e.ldd;
+        float s = 0.0f;
+        int head = 0;
+        if constexpr (MM::kPaired) {
+#pragma unroll
+          for (int cb = 0; cb < CG; cb += 2) {
+            const int m = (cb >> 1) * 32 + 2 * lr;          // even column of the pair
+            uint32_t qv = 0;
+            if (live && (full_cols || m + 1 < g.Mt))
+              qv = *reinterpret_cast<const uint32_t *>(qrow + m);
+            s = fmaf(acc[cb][r], bf16_lo(qv), s);
+            s = fmaf(acc[cb + 1 < CG ? cb + 1 : cb][r], bf16_hi(qv), s);
+            if (e.half_heads) {                  // lanes 0-7: one head, 8-15: the next
+              const float t = row8_sum(s);
+              const int h = (cb >> 1) * 2 + (lr >> 3);
+              if (live && (lr & 7) == 0 && h < g.hb) drow[h] = t;
+              s = 0.0f;
+            } else if (e.head_end >> (cb + 1) & 1) {
+              const float t = row16_sum(s);
+              if (live && lr == 0) drow[head] = t;
+              ++head;
+              s = 0.0f;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int cb = 0; cb < CG; ++cb) {
+            const int m = cb * 16 + lr;
+            float qv = 0.0f;
+            if (live && (full_cols || m < g.Mt)) qv = ldf(qrow + m);
+            s = fmaf(acc[cb][r], qv, s);
+            if (e.head_end >> cb & 1) {
+              const float t = row16_sum(s);
+              if (live && lr == 0) drow[head] = t;
+              ++head;
+              s = 0.0f;
+            }
+          }
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       if (tile0 + lk * 4 + r < row1) {
@@ -479,15 +570,6 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
 }
 
 // ---- any shape: one thread per output element ------------------------------
-template <typename T>
-__device__ __forceinline__ float ldf(const T *p);
-template <>
-__device__ __forceinline__ float ldf<float>(const float *p) { return *p; }
-template <>
-__device__ __forceinline__ float ldf<bf16_t>(const bf16_t *p) { return bf16_lo(*p); }
-__device__ __forceinline__ void stf(float *p, float v) { *p = v; }
-__device__ __forceinline__ void stf(bf16_t *p, float v) { *p = (bf16_t)f32_to_bf16_bits(v); }
-
 template <typename T>
 __global__ __launch_bounds__(kBlock) void segment_mm_scalar_kernel(
     const int32_t *__restrict__ tp, int n_types, const T *__restrict__ X,
@@ -518,39 +600,46 @@ void launch_cg(const int32_t *tp, const T *X, const T *W, T *Y, const MmGeom &g,
                      dim3(kBlock), lds, s, tp, X, W, Y, g);
 }
 
-template <typename T, int KBLK, int NF, int CG>
-int launch_tight(const int32_t *tp, const T *X, const T *W, T *Y, MmGeom g,
-                 int64_t grid, hipStream_t s) {
+template <typename T, int KBLK, int NF, int CG, bool DOT>
+int launch_tight_as(const int32_t *tp, const T *X, const T *W, T *Y, MmGeom g,
+                    const MmExt &e, int64_t grid, hipStream_t s) {
   typedef Tight<T, KBLK, NF, CG> TT;
   const size_t lds = (size_t)TT::kTileElems * sizeof(T);
-  if (!allow_lds((const void *)segment_mm_tight_kernel<T, KBLK, NF, CG>, lds))
+  if (!allow_lds((const void *)segment_mm_tight_kernel<T, KBLK, NF, CG, DOT>, lds))
     return GA_EUNSUPPORTED;
   g.KB = NF;   // the tile is padded to the compile-time shape
   g.MB = CG;
-  hipLaunchKernelGGL((segment_mm_tight_kernel<T, KBLK, NF, CG>),
-                     dim3((unsigned)grid), dim3(kBlock), lds, s, tp, X, W, Y, g);
+  hipLaunchKernelGGL((segment_mm_tight_kernel<T, KBLK, NF, CG, DOT>),
+                     dim3((unsigned)grid), dim3(kBlock), lds, s, tp, X, W, Y, g, e);
   return launch_status();
+}
+
+template <typename T, int KBLK, int NF, int CG>
+int launch_tight(const int32_t *tp, const T *X, const T *W, T *Y, const MmGeom &g,
+                 const MmExt &e, int64_t grid, hipStream_t s) {
+  if (e.Q) return launch_tight_as<T, KBLK, NF, CG, true>(tp, X, W, Y, g, e, grid, s);
+  return launch_tight_as<T, KBLK, NF, CG, false>(tp, X, W, Y, g, e, grid, s);
 }
 
 template <typename T, int KBLK, int NF>
 int pick_tight_cg(int cg, const int32_t *tp, const T *X, const T *W, T *Y,
-                  const MmGeom &g, int64_t grid, hipStream_t s) {
+                  const MmGeom &g, const MmExt &e, int64_t grid, hipStream_t s) {
   switch (cg) {
-    case 1: return launch_tight<T, KBLK, NF, Mma<T, KBLK>::kPaired ? 2 : 1>(tp, X, W, Y, g, grid, s);
-    case 2: return launch_tight<T, KBLK, NF, 2>(tp, X, W, Y, g, grid, s);
-    case 4: return launch_tight<T, KBLK, NF, 4>(tp, X, W, Y, g, grid, s);
-    default: return launch_tight<T, KBLK, NF, 8>(tp, X, W, Y, g, grid, s);
+    case 1: return launch_tight<T, KBLK, NF, Mma<T, KBLK>::kPaired ? 2 : 1>(tp, X, W, Y, g, e, grid, s);
+    case 2: return launch_tight<T, KBLK, NF, 2>(tp, X, W, Y, g, e, grid, s);
+    case 4: return launch_tight<T, KBLK, NF, 4>(tp, X, W, Y, g, e, grid, s);
+    default: return launch_tight<T, KBLK, NF, 8>(tp, X, W, Y, g, e, grid, s);
   }
 }
 
 template <typename T, int KBLK>
 int pick_tight(int nf, int cg, const int32_t *tp, const T *X, const T *W, T *Y,
-               const MmGeom &g, int64_t grid, hipStream_t s) {
+               const MmGeom &g, const MmExt &e, int64_t grid, hipStream_t s) {
   switch (nf) {
-    case 1: return pick_tight_cg<T, KBLK, 1>(cg, tp, X, W, Y, g, grid, s);
-    case 2: return pick_tight_cg<T, KBLK, 2>(cg, tp, X, W, Y, g, grid, s);
-    case 4: return pick_tight_cg<T, KBLK, 4>(cg, tp, X, W, Y, g, grid, s);
-    default: return pick_tight_cg<T, KBLK, 8>(cg, tp, X, W, Y, g, grid, s);
+    case 1: return pick_tight_cg<T, KBLK, 1>(cg, tp, X, W, Y, g, e, grid, s);
+    case 2: return pick_tight_cg<T, KBLK, 2>(cg, tp, X, W, Y, g, e, grid, s);
+    case 4: return pick_tight_cg<T, KBLK, 4>(cg, tp, X, W, Y, g, e, grid, s);
+    default: return pick_tight_cg<T, KBLK, 8>(cg, tp, X, W, Y, g, e, grid, s);
   }
 }
 
@@ -564,7 +653,7 @@ inline int pow2_ceil_int(int v) {
 template <typename T, int KBLK>
 int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
                 int64_t rows, int heads, int K, int M, int h0, int hb,
-                hipStream_t s) {
+                const MmExt &ext, hipStream_t s) {
   typedef Mma<T, KBLK> MM;
   MmGeom g;
   g.n_types = n_types;
@@ -585,14 +674,31 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
   if (grid > 0x7fffffff) return GA_EUNSUPPORTED;
   const T *Xh = X + (int64_t)h0 * K;
   const T *Wh = W + (int64_t)h0 * K * M;
-  T *Yh = Y + (int64_t)h0 * M;
+  T *Yh = Y ? Y + (int64_t)h0 * M : nullptr;
+  const bool fused = ext.x_index || ext.Q;
   if (KBLK != 16 || sizeof(T) == 4) {   // exact-shape kernels: fp32 and bf16 x32
     if (g.KB <= 8 && g.MB <= 8) {
+      MmExt e = ext;
+      if (e.Q) {
+        // heads must end on column-block (fp32) / block-pair (bf16) boundaries,
+        // or be exactly half a pair
+        constexpr bool paired = Mma<T, KBLK>::kPaired;
+        e.half_heads = paired && M == 16;
+        if (!e.half_heads && M % (paired ? 32 : 16) != 0) return GA_EUNSUPPORTED;
+        e.Q = static_cast<const T *>(ext.Q) + (int64_t)h0 * M;
+        e.dot = ext.dot + h0;
+        e.head_end = 0;
+        for (int b = 0; b < 32; ++b) {
+          const int end_col = paired ? ((b >> 1) + 1) * 32 : (b + 1) * 16;
+          if ((!paired || (b & 1)) && end_col % M == 0) e.head_end |= 1u << b;
+        }
+      }
       const int rc = pick_tight<T, (sizeof(T) == 4 ? 16 : 32)>(
-          pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), tp, Xh, Wh, Yh, g, grid, s);
-      if (rc != GA_EUNSUPPORTED) return rc;
+          pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), tp, Xh, Wh, Yh, g, e, grid, s);
+      if (rc != GA_EUNSUPPORTED || fused) return rc;
     }
   }
+  if (fused) return GA_EUNSUPPORTED;   // only the exact-shape kernel gathers
   const size_t lds = (size_t)MM::tile_elems(g.KB, g.MB) * sizeof(T);
   if (lds > (size_t)kMaxLds) return GA_EUNSUPPORTED;
   const int mbp = MM::mb_pad(g.MB);
@@ -610,19 +716,22 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
 
 template <typename T, int KBLK>
 int launch_mfma(const int32_t *tp, int n_types, const void *X, const void *W,
-                void *Y, int64_t rows, int heads, int K, int M, hipStream_t s) {
+                void *Y, int64_t rows, int heads, int K, int M, const MmExt &ext,
+                hipStream_t s) {
   // all heads folded into one block-diagonal tile when that fits the LDS and
   // the fragment budget; otherwise one launch per head
   if (heads > 1) {
     int rc = GA_EUNSUPPORTED;
     if ((int64_t)heads * K <= kMaxFrags * KBLK)
       rc = launch_fold<T, KBLK>(tp, n_types, (const T *)X, (const T *)W, (T *)Y,
-                                rows, heads, K, M, 0, heads, s);
+                                rows, heads, K, M, 0, heads, ext, s);
     if (rc != GA_EUNSUPPORTED) return rc;
   }
   for (int h = 0; h < heads; ++h) {
     const int rc = launch_fold<T, KBLK>(tp, n_types, (const T *)X, (const T *)W,
-                                        (T *)Y, rows, heads, K, M, h, 1, s);
+                                        (T *)Y, rows, heads, K, M, h, 1, ext, s);
+    // a fused form that does not fit fails on its first launch, before
+    // anything was written
     if (rc != GA_OK) return rc;
   }
   return GA_OK;
@@ -631,35 +740,26 @@ int launch_mfma(const int32_t *tp, int n_types, const void *X, const void *W,
 }  // namespace
 }  // namespace ga
 
-extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
-                             const void *X, const void *W, void *Y, int64_t rows,
-                             int64_t heads, int64_t K, int64_t M, int dtype,
-                             ga_stream_t stream) {
-  using namespace ga;
-  if (n_types < 0 || rows < 0 || heads <= 0 || K <= 0 || M <= 0) return GA_EINVAL;
-  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
-  if (rows > 0x7fffffff || n_types > 0x7fffffff || heads * K > 0x7fffffff ||
-      heads * M > 0x7fffffff)
-    return GA_EINVAL;
-  if (rows == 0 || n_types == 0) return GA_OK;
-  if (!type_pointer || !X || !W || !Y) return GA_EINVAL;
-  const size_t esz = dtype == GA_F32 ? 4 : 2;
-  if (!aligned(X, esz) || !aligned(W, esz) || !aligned(Y, esz)) return GA_EALIGN;
-  hipStream_t s = (hipStream_t)stream;
+namespace ga {
+namespace {
 
+int segment_mm_any(const int32_t *type_pointer, int64_t n_types, const void *X,
+                   const void *W, void *Y, int64_t rows, int64_t heads, int64_t K,
+                   int64_t M, int dtype, const MmExt &ext, hipStream_t s) {
+  const bool fused = ext.x_index || ext.Q;
   int rc = GA_EUNSUPPORTED;
-  if (aligned(X, 16) && aligned(Y, 16)) {
+  if (aligned(X, 16) && (!Y || aligned(Y, 16)) && (!ext.Q || aligned(ext.Q, 16))) {
     if (dtype == GA_F32 && K % 4 == 0)
       rc = launch_mfma<float, 16>(type_pointer, (int)n_types, X, W, Y, rows,
-                                  (int)heads, (int)K, (int)M, s);
+                                  (int)heads, (int)K, (int)M, ext, s);
     else if (dtype == GA_BF16 && K % 8 == 0)
       rc = launch_mfma<bf16_t, 32>(type_pointer, (int)n_types, X, W, Y, rows,
-                                   (int)heads, (int)K, (int)M, s);
-    else if (dtype == GA_BF16 && K % 4 == 0)
+                                   (int)heads, (int)K, (int)M, ext, s);
+    else if (dtype == GA_BF16 && K % 4 == 0 && !fused)
       rc = launch_mfma<bf16_t, 16>(type_pointer, (int)n_types, X, W, Y, rows,
-                                   (int)heads, (int)K, (int)M, s);
+                                   (int)heads, (int)K, (int)M, ext, s);
   }
-  if (rc != GA_EUNSUPPORTED) return rc;
+  if (rc != GA_EUNSUPPORTED || fused) return rc;
 
   // shapes the MFMA path does not take (odd K, weights beyond the LDS budget)
   const int64_t total = rows * heads * M;
@@ -676,4 +776,63 @@ extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
                        (const bf16_t *)X, (const bf16_t *)W, (bf16_t *)Y, rows,
                        (int)heads, (int)K, (int)M);
   return launch_status();
+}
+
+int check_mm_args(int64_t n_types, int64_t rows, int64_t heads, int64_t K, int64_t M,
+                  int dtype) {
+  if (n_types < 0 || rows < 0 || heads <= 0 || K <= 0 || M <= 0) return GA_EINVAL;
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  if (rows > 0x7fffffff || n_types > 0x7fffffff || heads * K > 0x7fffffff ||
+      heads * M > 0x7fffffff)
+    return GA_EINVAL;
+  return GA_OK;
+}
+
+}  // namespace
+}  // namespace ga
+
+extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
+                             const void *X, const void *W, void *Y, int64_t rows,
+                             int64_t heads, int64_t K, int64_t M, int dtype,
+                             ga_stream_t stream) {
+  using namespace ga;
+  const int bad = check_mm_args(n_types, rows, heads, K, M, dtype);
+  if (bad != GA_OK) return bad;
+  if (rows == 0 || n_types == 0) return GA_OK;
+  if (!type_pointer || !X || !W || !Y) return GA_EINVAL;
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!aligned(X, esz) || !aligned(W, esz) || !aligned(Y, esz)) return GA_EALIGN;
+  MmExt ext = {};
+  return segment_mm_any(type_pointer, n_types, X, W, Y, rows, heads, K, M, dtype, ext,
+                        (hipStream_t)stream);
+}
+
+extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types,
+                                    const void *X, const int64_t *x_index,
+                                    const void *W, void *Y, const void *Q,
+                                    const int64_t *q_index, float *dot, int64_t rows,
+                                    int64_t heads, int64_t K, int64_t M, int dtype,
+                                    ga_stream_t stream) {
+  using namespace ga;
+  const int bad = check_mm_args(n_types, rows, heads, K, M, dtype);
+  if (bad != GA_OK) return bad;
+  if ((Y != nullptr) == (dot != nullptr)) return GA_EINVAL;   // exactly one result
+  if ((Q != nullptr) != (dot != nullptr)) return GA_EINVAL;
+  if (q_index && !Q) return GA_EINVAL;
+  if (rows == 0 || n_types == 0) return GA_OK;
+  if (!type_pointer || !X || !W) return GA_EINVAL;
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!aligned(X, esz) || !aligned(W, esz) || (Y && !aligned(Y, esz)) ||
+      (Q && !aligned(Q, esz)) || (dot && !aligned(dot, 4)) ||
+      (x_index && !aligned(x_index, 8)) || (q_index && !aligned(q_index, 8)))
+    return GA_EALIGN;
+  MmExt ext = {};
+  ext.x_index = x_index;
+  ext.Q = Q;
+  ext.q_index = q_index;
+  ext.dot = dot;
+  ext.ldq = heads * M;
+  ext.ldd = heads;
+  return segment_mm_any(type_pointer, n_types, X, W, Y, rows, heads, K, M, dtype, ext,
+                        (hipStream_t)stream);
 }

@@ -163,14 +163,18 @@ using GraphPtr = c10::intrusive_ptr<DGLGraph>;
 
 namespace {
 
+// edge_rows: u is per-edge in edge-id order and is read through the edge-id
+// column in place of the neighbour column (u[e] op w[e])
 torch::Tensor spmm(const GraphPtr &g, int op, int reduce, const torch::Tensor &u,
-                   const at::optional<torch::Tensor> &w, bool reverse) {
+                   const at::optional<torch::Tensor> &w, bool reverse,
+                   bool edge_rows = false) {
   check_input(u, "features");
   const int dt = feat_dtype(u, "features");
   const auto &side = g->side(reverse);
   const torch::Tensor &ptr = reverse ? g->out_pointer : g->in_pointer;
-  const torch::Tensor &nbr = reverse ? g->out_node_indices : g->in_node_indices;
   const torch::Tensor &eid = reverse ? g->out_edge_indices : g->in_edge_indices;
+  const torch::Tensor &nbr =
+      edge_rows ? eid : reverse ? g->out_node_indices : g->in_node_indices;
   const int64_t feat = feat_dim(u);
   int64_t heads = 1;
   if (op >= GA_U_MUL_E) {
@@ -182,7 +186,7 @@ torch::Tensor spmm(const GraphPtr &g, int op, int reduce, const torch::Tensor &u
     TORCH_CHECK(heads > 0 && feat % heads == 0,
                 "feature width is not a multiple of the heads");
   }
-  TORCH_CHECK(u.size(0) == (op == GA_COPY_E ? g->num_edges : g->num_nodes),
+  TORCH_CHECK(u.size(0) == (op == GA_COPY_E || edge_rows ? g->num_edges : g->num_nodes),
               "features have the wrong number of rows");
   torch::Tensor out = torch::empty(out_shape(g->num_nodes, u), u.options());
   const size_t ws_bytes = ga_spmm_workspace_bytes(g->num_edges, feat);
@@ -235,6 +239,20 @@ torch::Tensor gspmm(torch::Tensor ufeature, at::optional<torch::Tensor> efeature
   TORCH_CHECK(o >= 0, "Unsupported SpMM binary operator: ", op);
   TORCH_CHECK(r >= 0, "Unsupported SpMM reducer: ", reduce);
   return spmm(graph, o, r, ufeature, efeature, false);
+}
+
+// SpMMEdge(x * y) for two per-edge operands without the product tensor: one of
+// them must be a per-edge / per-head fp32 weight; otherwise multiply, then copy_e
+torch::Tensor e_mul_e_sum(torch::Tensor x, torch::Tensor y, const GraphPtr &graph) {
+  for (int pass = 0; pass < 2; ++pass) {
+    const torch::Tensor &a = pass ? y : x, &b = pass ? x : y;
+    if (b.scalar_type() != at::kFloat || a.dim() < 2 || a.size(0) != b.size(0)) continue;
+    const bool scalar = b.dim() <= 2 && feat_dim(b) == 1;
+    bool per_head = b.dim() == a.dim() && a.dim() >= 3 && b.size(b.dim() - 1) == 1;
+    for (int64_t d = 0; per_head && d + 1 < a.dim(); ++d) per_head = a.size(d) == b.size(d);
+    if (scalar || per_head) return spmm(graph, GA_U_MUL_E, GA_SUM, a, b, false, true);
+  }
+  return spmm(graph, GA_COPY_E, GA_SUM, (x * y).contiguous(), at::nullopt, false);
 }
 
 struct EdgeColumns {
@@ -351,6 +369,82 @@ torch::Tensor SegmentMMEdge(torch::Tensor features, torch::Tensor weights,
                             const GraphPtr &graph) {
   return segment_mm(features, weights, graph->etype_pointer, graph->num_etypes,
                     graph->num_edges);
+}
+
+torch::Tensor gather(const torch::Tensor &features, const torch::Tensor &index);
+
+struct MmShape { int64_t heads, K, M; int dt; };
+MmShape edge_mm_shape(const torch::Tensor &features, const torch::Tensor &weights,
+                      const GraphPtr &graph) {
+  check_input(features, "features");
+  check_input(weights, "weights");
+  MmShape s;
+  s.dt = feat_dtype(features, "features");
+  TORCH_CHECK(weights.scalar_type() == features.scalar_type(),
+              "features and weights must share a dtype");
+  TORCH_CHECK(graph->etype_pointer.has_value(),
+              "the graph has no type pointer for this operator");
+  TORCH_CHECK(weights.dim() == 3 || weights.dim() == 4,
+              "weights must be (T, K, M) or (T, H, K, M)");
+  s.heads = weights.dim() == 4 ? weights.size(1) : 1;
+  s.K = weights.size(weights.dim() - 2);
+  s.M = weights.size(weights.dim() - 1);
+  TORCH_CHECK(weights.size(0) == graph->num_etypes, "weights must have one matrix per type");
+  TORCH_CHECK(features.size(0) == graph->num_nodes && feat_dim(features) == s.heads * s.K,
+              "features must be (nodes, heads*K)");
+  return s;
+}
+const torch::Tensor &endpoint_column(const GraphPtr &graph, int64_t which) {
+  TORCH_CHECK(which == 0 || which == 1, "endpoint must be 0 (source) or 1 (destination)");
+  return which == 0 ? graph->COO_src : graph->COO_dst;
+}
+
+// broadcast.cu:58-69 + segment_mm.cu:29-33 as one pass:
+// out[e] = features[endpoint(e)] @ weights[type(e)]
+torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
+                                  int64_t endpoint, const GraphPtr &graph) {
+  const MmShape s = edge_mm_shape(features, weights, graph);
+  const torch::Tensor &index = endpoint_column(graph, endpoint);
+  torch::Tensor out = torch::empty({graph->num_edges, s.heads * s.M}, features.options());
+  const int rc = ga_segment_mm_gather(
+      graph->etype_pointer.value().data_ptr<int>(), graph->num_etypes, features.data_ptr(),
+      index.data_ptr<int64_t>(), weights.data_ptr(), out.data_ptr(), nullptr, nullptr,
+      nullptr, graph->num_edges, s.heads, s.K, s.M, s.dt, current_stream(out));
+  if (rc == GA_EUNSUPPORTED)       // shape outside the matrix-core tile
+    return segment_mm(gather(features, index), weights, graph->etype_pointer,
+                      graph->num_etypes, graph->num_edges);
+  check_ga(rc, "ga_segment_mm_gather");
+  return out;
+}
+
+// out[e, h] = <features[endpoint(e)] @ weights[type(e)], other[other_endpoint(e)]>
+// (examples/HGT/HGT.py:42-45), fp32 (E, heads)
+torch::Tensor SegmentMMEdgeDot(torch::Tensor features, torch::Tensor weights,
+                               int64_t endpoint, torch::Tensor other,
+                               int64_t other_endpoint, const GraphPtr &graph) {
+  const MmShape s = edge_mm_shape(features, weights, graph);
+  check_input(other, "other");
+  TORCH_CHECK(other.scalar_type() == features.scalar_type() &&
+                  other.size(0) == graph->num_nodes && feat_dim(other) == s.heads * s.M,
+              "other must be (nodes, heads*M) of the features' dtype");
+  const torch::Tensor &xi = endpoint_column(graph, endpoint);
+  const torch::Tensor &qi = endpoint_column(graph, other_endpoint);
+  torch::Tensor out =
+      torch::empty({graph->num_edges, s.heads}, features.options().dtype(at::kFloat));
+  const int rc = ga_segment_mm_gather(
+      graph->etype_pointer.value().data_ptr<int>(), graph->num_etypes, features.data_ptr(),
+      xi.data_ptr<int64_t>(), weights.data_ptr(), nullptr, other.data_ptr(),
+      qi.data_ptr<int64_t>(), out.data_ptr<float>(), graph->num_edges, s.heads, s.K, s.M,
+      s.dt, current_stream(out));
+  if (rc == GA_EUNSUPPORTED) {
+    torch::Tensor y = SegmentMMEdgeGather(features, weights, endpoint, graph);
+    torch::Tensor q = gather(other, qi).reshape(y.sizes());
+    return (y.to(at::kFloat) * q.to(at::kFloat))
+        .reshape({graph->num_edges, s.heads, s.M})
+        .sum(-1);
+  }
+  check_ga(rc, "ga_segment_mm_gather");
+  return out;
 }
 
 torch::Tensor gather(const torch::Tensor &features, const torch::Tensor &index) {
@@ -514,6 +608,14 @@ static auto registry =
         .op("my_ops::gsddmm_u_dot_v(Tensor x, Tensor y, " GRAPH_T " g) -> Tensor z", &u_dot_v)
         .op("my_ops::gspmm(Tensor x, Tensor? y, str op, str reduce, " GRAPH_T " g) -> Tensor z",
             &gspmm)
+        .op("my_ops::gspmm_e_mul_e_sum(Tensor x, Tensor y, " GRAPH_T " g) -> Tensor z",
+            &e_mul_e_sum)
+        .op("my_ops::SegmentMMEdgeGather(Tensor x, Tensor w, int endpoint, " GRAPH_T
+            " g) -> Tensor z",
+            &SegmentMMEdgeGather)
+        .op("my_ops::SegmentMMEdgeDot(Tensor x, Tensor w, int endpoint, Tensor q, "
+            "int q_endpoint, " GRAPH_T " g) -> Tensor z",
+            &SegmentMMEdgeDot)
         .op("my_ops::gat_aggregate(Tensor el, Tensor er, Tensor z, float slope, " GRAPH_T
             " g) -> Tensor y",
             &gat_aggregate)

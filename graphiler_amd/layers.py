@@ -71,9 +71,15 @@ def gat_layer(g: DGLGraph, h, fc_weight, attn_weight, heads: int = 1,
     return gat_aggregate_plan(g, z, el, er, negative_slope)
 
 
-def rgcn_layer(g: DGLGraph, h, weight, norm):
-    """examples/RGCN/RGCN.py:25-33: BroadcastSrcNode -> SegmentMMEdge ->
-    mul(norm) -> SpMMEdge.  weight (R, K, M); norm (E, 1); edges sorted by type."""
+def rgcn_layer(g: DGLGraph, h, weight, norm, fused: bool = True):
+    """examples/RGCN/RGCN.py:25-33.  weight (R, K, M); norm (E, 1) fp32; edges
+    sorted by type.  ``fused``: the typed product reads the source rows through
+    the COO column and the norm multiplies inside the reduction (two passes);
+    otherwise the reference's plan BroadcastSrcNode -> SegmentMMEdge ->
+    mul(norm) -> SpMMEdge."""
+    if fused:
+        msg = ops.SegmentMMEdgeGather(h, weight, 0, g)
+        return ops.gspmm_e_mul_e_sum(msg, norm.float(), g)
     hs = ops.BroadcastSrcNode(h, g)
     msg = ops.SegmentMMEdge(hs, weight, g)
     msg = msg * norm.to(msg.dtype)
@@ -81,7 +87,8 @@ def rgcn_layer(g: DGLGraph, h, weight, norm):
 
 
 def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
-              relation_att, relation_msg, relation_pri, skip, heads: int = 1):
+              relation_att, relation_msg, relation_pri, skip, heads: int = 1,
+              fused: bool = True):
     """examples/HGT/HGT.py:28-60 as the operator sequence of its optimised plan,
     generalised from one head to ``heads`` heads of width D = hidden / heads:
 
@@ -95,6 +102,11 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
 
     k/q/v/a_weight: (T_n, hidden, hidden); relation_att / relation_msg:
     (T_e, heads, D, D); relation_pri: (T_e, heads); skip: (T_n,).
+
+    ``fused`` replaces the per-edge copies and products by
+      attn = SegmentMMEdgeDot(K, relation_att, src, Q, dst) * pri / sqrt(D)
+      t    = gspmm_e_mul_e_sum(SegmentMMEdgeGather(V, relation_msg, src), softmax(attn))
+    so the only per-edge tensors are the scores and the transformed values.
     """
     n, hidden = h.shape
     d = hidden // heads
@@ -102,14 +114,20 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
     k = ops.SegmentMMNode(h, k_weight, g)
     v = ops.SegmentMMNode(h, v_weight, g)
     q = ops.SegmentMMNode(h, q_weight, g)
-    k_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(k, g), relation_att, g)
-    v_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(v, g), relation_msg, g)
-    q_e = ops.BroadcastDstNode(q, g)
-    attn = (k_e.view(e, heads, d).float() * q_e.view(e, heads, d).float()).sum(-1)
-    attn = attn * ops.BroadcastEdgeType(relation_pri.float(), g) / (d ** 0.5)
-    a = ops.SegmentSoftmax(attn.contiguous(), 1, None, g)          # (E, heads) fp32
-    m = (v_e.view(e, heads, d).float() * a.unsqueeze(-1)).to(h.dtype).view(e, hidden)
-    t = ops.SpMMEdge(m, [1], False, None, g)
+    pri = ops.BroadcastEdgeType(relation_pri.float(), g) / (d ** 0.5)
+    if fused:
+        attn = ops.SegmentMMEdgeDot(k, relation_att, 0, q, 1, g) * pri
+        a = ops.SegmentSoftmax(attn.contiguous(), 1, None, g)      # (E, heads) fp32
+        v_e = ops.SegmentMMEdgeGather(v, relation_msg, 0, g)
+        t = ops.spmm(g, "e_mul_e", "sum", v_e, a)
+    else:
+        k_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(k, g), relation_att, g)
+        v_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(v, g), relation_msg, g)
+        q_e = ops.BroadcastDstNode(q, g)
+        attn = (k_e.view(e, heads, d).float() * q_e.view(e, heads, d).float()).sum(-1) * pri
+        a = ops.SegmentSoftmax(attn.contiguous(), 1, None, g)      # (E, heads) fp32
+        m = (v_e.view(e, heads, d).float() * a.unsqueeze(-1)).to(h.dtype).view(e, hidden)
+        t = ops.SpMMEdge(m, [1], False, None, g)
     alpha = torch.sigmoid(ops.BroadcastNodeType(skip.float().unsqueeze(1), g))
     out = ops.SegmentMMNode(t, a_weight, g)
     return (out.float() * alpha).to(h.dtype)

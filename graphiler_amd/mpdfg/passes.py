@@ -377,6 +377,81 @@ class _Rewriter:
         return True
 
 
+    # ------------------------------------------------- late fusion ----
+    def late_fusion(self) -> bool:
+        """Rewrites that remove per-edge copies of node rows and per-edge product
+        tensors; run once the other passes have settled, because they consume the
+        Broadcast nodes those passes match on."""
+        changed = False
+        for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::SegmentMMEdge":
+                changed |= self._fuse_gather_mm(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "aten::sum":
+                changed |= self._fuse_mm_dot(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::SpMMEdge":
+                changed |= self._fuse_e_mul_e(n)
+        return changed
+
+    def _fuse_gather_mm(self, n) -> bool:
+        """SegmentMMEdge(BroadcastSrcNode | BroadcastDstNode (x), w) ->
+        SegmentMMEdgeGather(x, w, endpoint): the product reads the node rows
+        through the COO column."""
+        bc = n.inputsAt(0).node()
+        if bc.kind() not in ("my_ops::BroadcastSrcNode", "my_ops::BroadcastDstNode"):
+            return False
+        which = self.const(0 if bc.kind().endswith("SrcNode") else 1, n)
+        out = self.make("my_ops::SegmentMMEdgeGather",
+                        [bc.inputsAt(0), n.inputsAt(1), which, self.dglgraph], n, EDGE)
+        n.output().replaceAllUsesWith(out)
+        n.destroy()
+        return True
+
+    def _fuse_mm_dot(self, n) -> bool:
+        """sum(SegmentMMEdgeGather(x, w, i) * Broadcast{Src,Dst}Node(q), [1], keepdim=True)
+        -> SegmentMMEdgeDot(x, w, i, q, j).  The typed products in a plan come
+        from bmm (_fuse_bmm), so w is (T, K, M), one head, and the (E, 1) result
+        of the sum is the operator's (E, heads) result."""
+        if n.inputsSize() != 4 or self.const_of(n.inputsAt(1)) != [1] \
+                or self.const_of(n.inputsAt(2)) is not True \
+                or n.inputsAt(3).node().kind() != "prim::Constant" \
+                or n.inputsAt(3).toIValue() is not None:
+            return False
+        mul = n.inputsAt(0).node()
+        if mul.kind() != "aten::mul" or not self.single_use(mul.output()):
+            return False
+        for a, b in ((mul.inputsAt(0), mul.inputsAt(1)), (mul.inputsAt(1), mul.inputsAt(0))):
+            mm, bc = a.node(), b.node()
+            if mm.kind() == "my_ops::SegmentMMEdgeGather" and self.single_use(a) and \
+                    bc.kind() in ("my_ops::BroadcastSrcNode", "my_ops::BroadcastDstNode"):
+                which = self.const(0 if bc.kind().endswith("SrcNode") else 1, n)
+                out = self.make("my_ops::SegmentMMEdgeDot",
+                                [mm.inputsAt(0), mm.inputsAt(1), mm.inputsAt(2),
+                                 bc.inputsAt(0), which, self.dglgraph], n, EDGE)
+                n.output().replaceAllUsesWith(out)
+                n.destroy()
+                return True
+        return False
+
+    def _fuse_e_mul_e(self, n) -> bool:
+        """SpMMEdge(a * b) with both operands per-edge -> gspmm_e_mul_e_sum(a, b):
+        the product tensor is not formed (the operator multiplies first itself
+        when neither operand is a per-edge weight)."""
+        mul = n.inputsAt(0).node()
+        if mul.kind() != "aten::mul" or not self.single_use(mul.output()):
+            return False
+        a, b = mul.inputsAt(0), mul.inputsAt(1)
+        if self.where(a) != EDGE or self.where(b) != EDGE:
+            return False
+        if not (isinstance(a.type(), torch._C.TensorType) and isinstance(b.type(), torch._C.TensorType)):
+            return False
+        out = self.make("my_ops::gspmm_e_mul_e_sum", [a, b, self.dglgraph], n, NODE)
+        n.output().replaceAllUsesWith(out)
+        n.destroy()
+        return True
+
+
 def split(plan: MPDFG) -> None:
     _Rewriter(plan).split()
     dedup(plan.graph)
@@ -414,3 +489,9 @@ def optimize(plan: MPDFG, opt_level: int) -> None:
         for _ in range(3):
             reorder(plan)
             fusion(plan)
+        rw = _Rewriter(plan)
+        for _ in range(4):
+            if not rw.late_fusion():
+                break
+            dedup(plan.graph)
+        plan.invalidate()

@@ -69,7 +69,9 @@ def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
 
     op: "copy_u" (u is (N, ...)), "copy_e" (u is (E, ...)), "u_mul_e" /
     "u_add_e" / "u_sub_e" / "u_div_e" (functor.cuh:19-72; w is (E,), (E, 1) or
-    (E, H) fp32).  reduce: "sum" | "max" | "min".
+    (E, H) fp32), "e_mul_e" (u is (E, ...) in edge-id order, times w: the rows
+    are read through the edge-id column in place of the neighbour column).
+    reduce: "sum" | "max" | "min".
     ``return_arg`` (max / min only): also return ``(arg_u, arg_e)``, the int32
     neighbour id and edge id that supplied each output element (spmm.cuh:30-71);
     the one the operator has no use for is None.
@@ -84,7 +86,11 @@ def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
         rows, ident = g.in_row_of_slot, g.in_eid_is_identity
     feat = get_feat_dim(u)
     heads = 1
+    edge_rows = op in ("copy_e", "e_mul_e")
+    if op == "e_mul_e":
+        nbr = eid            # "neighbour" row of a slot = its edge id
     code = {"copy_u": capi.GA_COPY_U, "copy_e": capi.GA_COPY_E,
+            "e_mul_e": capi.GA_U_MUL_E,
             "u_mul_e": capi.GA_U_MUL_E, "u_add_e": capi.GA_U_ADD_E,
             "u_sub_e": capi.GA_U_SUB_E, "u_div_e": capi.GA_U_DIV_E}[op]
     if code >= capi.GA_U_MUL_E:
@@ -105,7 +111,7 @@ def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
                     or not np.array_equal(b.rhs_offset, per_head):
                 raise RuntimeError("unsupported broadcast between features "
                                    f"{tuple(u.shape)} and edge weights {tuple(w.shape)}")
-    n_src = g.num_edges if op == "copy_e" else g.num_nodes
+    n_src = g.num_edges if edge_rows else g.num_nodes
     if u.shape[0] != n_src:
         raise RuntimeError("features have the wrong number of rows")
     out = torch.empty(_out_shape(g.num_nodes, u), dtype=u.dtype, device=u.device)
@@ -160,6 +166,23 @@ def gspmm_dst_mul_e_sum(ufeature, efeature, dims: Sequence[int], keep_dim: bool,
     """spmm.cu:322-356: the same contraction over the out-adjacency:
     out[v] = sum over out-edges of ufeature[dst] * efeature[e]."""
     return spmm(graph, "u_mul_e", "sum", ufeature, efeature, reverse=True)
+
+
+def gspmm_e_mul_e_sum(x, y, graph: DGLGraph) -> torch.Tensor:
+    """out[v] = sum over in-edges e of x[e] * y[e] for two per-edge operands,
+    the ``SpMMEdge(x * y)`` of the reference's plans (reduce of
+    examples/HGT/HGT.py:50-53, message of examples/RGCN/RGCN.py:29) without the
+    product tensor.  One operand must be a per-edge (or per-head) fp32 weight;
+    two full-width operands are multiplied first and summed with copy_e."""
+    for a, b in ((x, y), (y, x)):
+        if b.dtype != torch.float32 or a.dim() < 2 or a.shape[0] != b.shape[0]:
+            continue
+        scalar = b.dim() <= 2 and get_feat_dim(b) == 1                  # (E,) / (E, 1)
+        per_head = (b.dim() == a.dim() >= 3 and b.shape[-1] == 1
+                    and b.shape[:-1] == a.shape[:-1])                   # (E, H, 1)
+        if scalar or per_head:
+            return spmm(graph, "e_mul_e", "sum", a, b)
+    return spmm(graph, "copy_e", "sum", (x * y).contiguous())
 
 
 # ---------------------------------------------------------------- SDDMM ----
@@ -308,6 +331,74 @@ def SegmentMMEdge(features, weights, graph: DGLGraph) -> torch.Tensor:
     """segment_mm.cu:29-33: per-edge-type linear, edges sorted by type."""
     return _segment_mm(features, weights, graph.etype_pointer,
                        graph.num_etypes, graph.num_edges)
+
+
+def _endpoint(graph: DGLGraph, which: int) -> torch.Tensor:
+    if which not in (0, 1):
+        raise RuntimeError("endpoint must be 0 (source) or 1 (destination)")
+    return graph.COO_src if which == 0 else graph.COO_dst
+
+
+def _mm_shapes(features, weights, graph: DGLGraph):
+    _check_input(features, "features")
+    _check_input(weights, "weights")
+    if weights.dtype != features.dtype:
+        raise RuntimeError("features and weights must share a dtype")
+    if graph.etype_pointer is None:
+        raise RuntimeError("the graph has no type pointer for this operator")
+    if weights.dim() not in (3, 4):
+        raise RuntimeError("weights must be (T, K, M) or (T, H, K, M)")
+    heads = 1 if weights.dim() == 3 else int(weights.shape[1])
+    K, M = int(weights.shape[-2]), int(weights.shape[-1])
+    if int(weights.shape[0]) != graph.num_etypes:
+        raise RuntimeError("weights must have one matrix per type")
+    if int(features.shape[0]) != graph.num_nodes or get_feat_dim(features) != heads * K:
+        raise RuntimeError("features must be (nodes, heads*K)")
+    return heads, K, M
+
+
+def SegmentMMEdgeGather(features, weights, endpoint: int, graph: DGLGraph) -> torch.Tensor:
+    """``SegmentMMEdge(BroadcastSrcNode(features), weights)`` (endpoint 0) or
+    the same with ``BroadcastDstNode`` (endpoint 1) as one pass: row e of the
+    result is features[endpoint(e)] @ weights[type(e)] (broadcast.cu:58-69 +
+    segment_mm.cu:29-33); the (E, heads*K) copy of the node rows is never made."""
+    heads, K, M = _mm_shapes(features, weights, graph)
+    index = _endpoint(graph, endpoint)
+    out = torch.empty((graph.num_edges, heads * M), dtype=features.dtype,
+                      device=features.device)
+    rc = capi.load().ga_segment_mm_gather(
+        graph.etype_pointer.data_ptr(), graph.num_etypes, features.data_ptr(),
+        index.data_ptr(), weights.data_ptr(), out.data_ptr(), None, None, None,
+        graph.num_edges, heads, K, M, _feat_dtype(features, "features"), _stream(out))
+    if rc == capi.GA_EUNSUPPORTED:      # shape outside the matrix-core tile
+        return SegmentMMEdge(_gather(features, index), weights, graph)
+    capi.check(rc, "ga_segment_mm_gather")
+    return out
+
+
+def SegmentMMEdgeDot(features, weights, endpoint: int, other, other_endpoint: int,
+                     graph: DGLGraph) -> torch.Tensor:
+    """out[e, h] = <features[endpoint(e)] @ weights[type(e)], other[other_endpoint(e)]>
+    per head, fp32 (E, heads): the ``sum(bmm(k, W) * q, dim=1, keepdim=True)`` of
+    examples/HGT/HGT.py:42-45 with neither per-edge operand materialised."""
+    heads, K, M = _mm_shapes(features, weights, graph)
+    _check_input(other, "other")
+    if other.dtype != features.dtype or int(other.shape[0]) != graph.num_nodes \
+            or get_feat_dim(other) != heads * M:
+        raise RuntimeError("other must be (nodes, heads*M) of the features' dtype")
+    xi, qi = _endpoint(graph, endpoint), _endpoint(graph, other_endpoint)
+    out = torch.empty((graph.num_edges, heads), dtype=torch.float32, device=features.device)
+    rc = capi.load().ga_segment_mm_gather(
+        graph.etype_pointer.data_ptr(), graph.num_etypes, features.data_ptr(),
+        xi.data_ptr(), weights.data_ptr(), None, other.data_ptr(), qi.data_ptr(),
+        out.data_ptr(), graph.num_edges, heads, K, M,
+        _feat_dtype(features, "features"), _stream(out))
+    if rc == capi.GA_EUNSUPPORTED:
+        y = SegmentMMEdgeGather(features, weights, endpoint, graph)
+        prod = y.float() * _gather(other, qi).float().reshape(y.shape)
+        return prod.reshape(graph.num_edges, heads, M).sum(-1)
+    capi.check(rc, "ga_segment_mm_gather")
+    return out
 
 
 # ------------------------------------------------------------ broadcast ----

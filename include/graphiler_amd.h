@@ -188,6 +188,28 @@ int ga_segment_mm(const int32_t *type_pointer, int64_t n_types, const void *X,
                   const void *W, void *Y, int64_t rows, int64_t heads,
                   int64_t K, int64_t M, int dtype, ga_stream_t stream);
 
+/* Per-edge typed linear whose operand lives on the nodes, without the per-edge
+ * copy: Y[r] = X[x_index[r]] @ W[type(r)] (x_index NULL: X[r]).  Replaces the
+ * pair BroadcastSrcNode / BroadcastDstNode (broadcast.cu:58-66) -> SegmentMMEdge
+ * (segment_mm.cu:29-33) that the reference's plans execute for
+ * examples/RGCN/RGCN.py:26-28 and examples/HGT/HGT.py:35-44.  Exactly one of
+ * two results:
+ *   Y   (rows, heads*M) `dtype`, with Q / q_index / dot NULL;
+ *   dot (rows, heads) fp32 with Y NULL: dot[r, h] = <Y[r, h, :], Q[q_index[r], h, :]>
+ *       (q_index NULL: Q[r]); Q (*, heads*M) `dtype`.  The product rows stay in
+ *       registers (HGT's sum(k * q, dim=1), HGT.py:44-45).
+ * x_index / q_index are int64 (the COO columns of the graph); entries are not
+ * checked on the device.  Returns GA_EUNSUPPORTED, having launched nothing, for
+ * shapes outside the matrix-core tile (heads*K > 128 fp32 / 256 bf16,
+ * heads*M > 128, K % 4 (fp32) or K % 8 (bf16) != 0; for dot also M % 16 (fp32),
+ * M % 32 and M != 16 (bf16)); the caller then gathers with ga_gather_rows.
+ */
+int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types, const void *X,
+                         const int64_t *x_index, const void *W, void *Y,
+                         const void *Q, const int64_t *q_index, float *dot,
+                         int64_t rows, int64_t heads, int64_t K, int64_t M,
+                         int dtype, ga_stream_t stream);
+
 /* ---------------------------------------------------------------- gather --
  * y[i, :] = x[idx[i], :], a bit-exact row copy of row_bytes bytes.
  * Replaces BroadcastSrcNode / DstNode / NodeType / EdgeType

@@ -67,8 +67,9 @@ def test_gat_layer(device, heads, bf16):
     assert_close(plan.float().cpu().numpy(), ref, tol, "GAT plan")
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("bf16", [False, True])
-def test_rgcn_two_layers(device, bf16):
+def test_rgcn_two_layers(device, bf16, fused):
     wl = datasets.rgcn_zipf(num_nodes=10_000, n_edges=100_000)
     n = wl.num_nodes
     g = prepare_graph(wl.src, wl.dst, n, device=device, etype_of=wl.etype,
@@ -89,16 +90,18 @@ def test_rgcn_two_layers(device, bf16):
                            msg.astype(np.float32), op="copy_e")
 
     dn = _t(norm, device)
-    h1 = torch.relu(layers.rgcn_layer(g, _t(x, device, bf16), _t(w1, device, bf16), dn))
-    h2 = layers.rgcn_layer(g, h1, _t(w2, device, bf16), dn)
+    h1 = torch.relu(layers.rgcn_layer(g, _t(x, device, bf16), _t(w1, device, bf16), dn,
+                                      fused=fused))
+    h2 = layers.rgcn_layer(g, h1, _t(w2, device, bf16), dn, fused=fused)
     r1 = np.maximum(ref_layer(x, w1), 0).astype(np.float32)
     tol = TOL_BF16 if bf16 else 2 * TOL_F32
     assert_close(h1.float().cpu().numpy(), r1, tol, "RGCN layer 1")
     assert_close(h2.float().cpu().numpy(), ref_layer(r1, w2), 2 * tol, "RGCN layer 2")
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("bf16", [False, True])
-def test_hgt_layer(device, bf16):
+def test_hgt_layer(device, bf16, fused):
     wl = datasets.hgt_hetero(counts=(800, 600, 400, 200), edges_per_type=4000)
     n, e = wl.num_nodes, wl.num_edges
     heads, d = 8, 16
@@ -117,7 +120,7 @@ def test_hgt_layer(device, bf16):
                            _t(wq, device, bf16), _t(wv, device, bf16),
                            _t(wa, device, bf16), _t(ratt, device, bf16),
                            _t(rmsg, device, bf16), _t(rpri, device, bf16),
-                           _t(skip, device), heads)
+                           _t(skip, device), heads, fused=fused)
     # the same plan on the oracle (fp64 accumulation; bf16 rounding applied where
     # the device stores bf16 tensors)
     ntp, etp = oracle.type_pointer(wl.ntype, 4), oracle.type_pointer(wl.etype, 10)

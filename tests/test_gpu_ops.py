@@ -443,6 +443,117 @@ def test_segment_mm_ops_and_rgcn_layer(device):
         ops.SegmentMMEdge(_dev(h[:1], device), _dev(W, device), g2)
 
 
+@pytest.mark.parametrize("K,M,heads,bf16", [
+    (16, 64, 1, False), (64, 64, 1, False), (16, 16, 8, False), (64, 8, 1, False),
+    (12, 48, 2, False), (128, 128, 1, False), (200, 16, 1, False),
+    (16, 16, 8, True), (64, 64, 1, True), (32, 32, 4, True), (16, 64, 1, True),
+    (64, 48, 1, True)])
+def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
+    """Y[e] = X[endpoint(e)] @ W[type(e)] read through the COO columns, and its
+    reduction against a second gathered row; expected values: the oracle's
+    segment_mm on numpy-gathered rows and a float64 einsum.  (64, 8), (200, 16)
+    and bf16 (64, 48) fall outside the fused kernel's shapes: the entry point
+    must say so and the operator wrapper must still give the result."""
+    rng = np.random.default_rng(K * 131 + M * 7 + heads + 1000 * bf16)
+    counts = [70, 0, 1, 333, 0, 64, 15, 129, 2001, 0]
+    n_nodes, n_rel = 500, len(counts)
+    etype = np.repeat(np.arange(n_rel), counts).astype(np.int64)
+    e = etype.shape[0]
+    src = rng.integers(0, n_nodes, e, dtype=np.int64)
+    dst = rng.integers(0, n_nodes, e, dtype=np.int64)
+    g = prepare_graph(src, dst, n_nodes, device=device, etype_of=etype, num_etypes=n_rel)
+    X = rng.standard_normal((n_nodes, heads * K), dtype=np.float32)
+    Q = rng.standard_normal((n_nodes, heads * M), dtype=np.float32)
+    W = (rng.standard_normal((n_rel, heads, K, M)) / np.sqrt(K)).astype(np.float32)
+    if bf16:
+        X, Q, W = to_bf16_f32(X), to_bf16_f32(Q), to_bf16_f32(W)
+    dX, dQ, dW = _dev(X, device, bf16), _dev(Q, device, bf16), _dev(W, device, bf16)
+    tol = TOL_BF16 if bf16 else TOL_F32
+    tp = oracle.type_pointer(etype, n_rel)
+    lib = capi.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    dt = capi.GA_BF16 if bf16 else capi.GA_F32
+    kb = 32 if bf16 else 16
+    fits = heads * K <= 8 * kb and heads * M <= 128 and K % (8 if bf16 else 4) == 0
+    dot_fits = fits and (M % 16 == 0 if not bf16 else (M % 32 == 0 or M == 16))
+    for which, col in ((0, src), (1, dst)):
+        ref = oracle.segment_mm(tp, X[col], W, heads=heads)
+        Y = torch.full((e, heads * M), float("nan"), dtype=dX.dtype, device=device)
+        rc = lib.ga_segment_mm_gather(
+            g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(),
+            (g.COO_src if which == 0 else g.COO_dst).data_ptr(), dW.data_ptr(), Y.data_ptr(),
+            None, None, None, e, heads, K, M, dt, stream)
+        assert rc == (0 if fits else capi.GA_EUNSUPPORTED)
+        if fits:
+            assert_close(Y.float().cpu().numpy(), ref, tol, f"segment_mm_gather {which}")
+        got = ops.SegmentMMEdgeGather(dX, dW, which, g)
+        assert_close(got.float().cpu().numpy(), ref, tol, f"SegmentMMEdgeGather {which}")
+        # dot against the other endpoint's row of Q
+        other = dst if which == 0 else src
+        y64 = np.einsum("ehk,ehkm->ehm", X[col].reshape(e, heads, K).astype(np.float64),
+                        W[etype].astype(np.float64))
+        want = np.einsum("ehm,ehm->eh", y64, Q[other].reshape(e, heads, M).astype(np.float64))
+        D = torch.full((e, heads), float("nan"), dtype=torch.float32, device=device)
+        rc = lib.ga_segment_mm_gather(
+            g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(),
+            (g.COO_src if which == 0 else g.COO_dst).data_ptr(), dW.data_ptr(), None,
+            dQ.data_ptr(), (g.COO_dst if which == 0 else g.COO_src).data_ptr(), D.data_ptr(),
+            e, heads, K, M, dt, stream)
+        assert rc == (0 if dot_fits else capi.GA_EUNSUPPORTED)
+        if dot_fits:
+            assert_close(D.cpu().numpy(), want, tol, f"segment_mm dot {which}")
+        got = ops.SegmentMMEdgeDot(dX, dW, which, dQ, 1 - which, g)
+        assert got.shape == (e, heads) and got.dtype == torch.float32
+        assert_close(got.cpu().numpy(), want, tol, f"SegmentMMEdgeDot {which}")
+    # identity index (NULL) = plain segment_mm on per-edge rows
+    Xe = rng.standard_normal((e, heads * K), dtype=np.float32)
+    if bf16:
+        Xe = to_bf16_f32(Xe)
+    dXe = _dev(Xe, device, bf16)
+    if fits:
+        Y = torch.full((e, heads * M), float("nan"), dtype=dX.dtype, device=device)
+        assert lib.ga_segment_mm_gather(g.etype_pointer.data_ptr(), n_rel, dXe.data_ptr(), None,
+                                        dW.data_ptr(), Y.data_ptr(), None, None, None, e,
+                                        heads, K, M, dt, stream) == 0
+        assert_close(Y.float().cpu().numpy(), oracle.segment_mm(tp, Xe, W, heads=heads), tol,
+                     "segment_mm_gather identity")
+    # argument errors: both or neither result, dot without Q
+    assert lib.ga_segment_mm_gather(g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(), None,
+                                    dW.data_ptr(), None, None, None, None, e, heads, K, M, dt,
+                                    stream) == capi.GA_EINVAL
+
+
+def test_e_mul_e_sum(device):
+    """out[v] = sum over in-edges of m[e] * a[e]: SpMMEdge of the product without
+    forming it; edge ids shuffled against the adjacency order."""
+    rng = np.random.default_rng(77)
+    src, dst = skewed_graph(rng, 400, 6000, 1500)
+    n, e = 400, src.shape[0]
+    g = prepare_graph(src, dst, n, device=device)
+    arr = build_graph_arrays(src, dst, n)
+    m = rng.standard_normal((e, 64), dtype=np.float32)
+    a = rng.uniform(0.1, 1.0, (e, 1)).astype(np.float32)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      (m * a).astype(np.float32), op="copy_e")
+    for x, y in ((m, a), (a, m)):
+        got = ops.gspmm_e_mul_e_sum(_dev(x, device), _dev(y, device), g)
+        assert_close(got.cpu().numpy(), ref, TOL_F32, "e_mul_e")
+    # per-head weights on shaped operands, bf16 messages
+    mh = to_bf16_f32(rng.standard_normal((e, 4, 16), dtype=np.float32))
+    ah = rng.uniform(0.1, 1.0, (e, 4, 1)).astype(np.float32)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      (mh * ah).reshape(e, 64).astype(np.float32), op="copy_e")
+    got = ops.gspmm_e_mul_e_sum(_dev(mh, device, True), _dev(ah, device), g)
+    assert got.shape == (n, 4, 16)
+    assert_close(got.float().cpu().numpy().reshape(n, 64), ref, TOL_BF16, "e_mul_e heads bf16")
+    # two full-width operands: product first
+    m2 = rng.standard_normal((e, 64), dtype=np.float32)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      (m * m2).astype(np.float32), op="copy_e")
+    got = ops.gspmm_e_mul_e_sum(_dev(m, device), _dev(m2, device), g)
+    assert_close(got.cpu().numpy(), ref, TOL_F32, "e_mul_e full width")
+
+
 @pytest.mark.parametrize("rows,K,M,heads", [(1000, 602, 64, 1), (333, 77, 64, 2),
                                             (777, 64, 64, 4),
                                             (300, 100, 256, 4), (5000, 16, 32, 2),
