@@ -6,10 +6,12 @@ achieved algorithmic GB/s and, for the matrix products, TFLOP/s.
     python bench_kernels.py [c1] [c3] [c4] [c5]        # default: c1 c3 c4
 
   c1  GCN, 19,717 nodes / 108,368 edges: SpMM copy_u at F = 16 and 3
-  c3  RGCN, 100 k nodes / 1 M edges / 60 relations: segment_mm 16->64 and 64->8,
-      SpMM copy_e, source gather (fp32 and bf16)
+  c3  RGCN, 100 k nodes / 1 M edges / 60 relations: segment_mm 16->64 and 64->8
+      (on per-edge rows and reading the source rows through the COO column),
+      SpMM copy_e and e_mul_e, source gather, the whole layer (fp32 and bf16)
   c4  HGT, 100 k nodes / 2 M edges / 4 node types / 10 relations, 8 heads x 16:
-      segment_mm on nodes and on edges, SDDMM u_dot_v, 8-head softmax, SpMM u_mul_e
+      segment_mm on nodes and on edges (plain, gathered, with the dot-product
+      epilogue), SDDMM u_dot_v, 8-head softmax, SpMM u_mul_e / e_mul_e, the layer
   c5  GAT, 2.45 M nodes / 64.3 M edges, 4 heads x 64 bf16: fused aggregation,
       SpMM u_mul_e, SDDMM u_add_v, 4-head softmax
 
@@ -37,7 +39,7 @@ def main():
     import numpy as np
     import torch
 
-    from graphiler_amd import datasets, ops, prepare_graph
+    from graphiler_amd import datasets, layers, ops, prepare_graph
 
     if not torch.cuda.is_available():
         sys.exit("bench_kernels.py: no GPU visible")
@@ -88,10 +90,24 @@ def main():
                 X, W = rnd(E, K, dtype=dt), rnd(R, K, M, dtype=dt)
                 report("c3", f"segment_mm edge {K}->{M} {tag}", lambda: ops.SegmentMMEdge(X, W, g),
                        E * (K + M) * b + R * K * M * b, 2 * E * K * M)
+                Xn = rnd(N, K, dtype=dt)
+                report("c3", f"segment_mm gather src {K}->{M} {tag}",
+                       lambda: ops.SegmentMMEdgeGather(Xn, W, 0, g),
+                       E * (8 + (K + M) * b) + R * K * M * b, 2 * E * K * M)
+            norm = torch.rand(E, 1, device=dev)
             for F in (64, 8):
                 m = rnd(E, F, dtype=dt)
                 report("c3", f"spmm copy_e F={F} {tag}", lambda: ops.SpMMEdge(m, [1], False, None, g),
                        4 * (N + 1) + E * (4 + 4 + F * b) + N * F * b)
+                report("c3", f"spmm e_mul_e F={F} {tag}", lambda: ops.gspmm_e_mul_e_sum(m, norm, g),
+                       4 * (N + 1) + E * (4 + 4 + 4 + F * b) + N * F * b)
+            for K, M in ((16, 64), (64, 8)):
+                Xn, W = rnd(N, K, dtype=dt), rnd(R, K, M, dtype=dt)
+                for fused in (False, True):
+                    report("c3", f"rgcn layer {K}->{M} {tag} {'fused' if fused else 'plan'}",
+                           lambda: layers.rgcn_layer(g, Xn, W, norm, fused=fused),
+                           4 * (N + 1) + E * (8 + 4 + 4 + K * b) + R * K * M * b + N * M * b,
+                           2 * E * K * M)
         h = rnd(N, 16)
         report("c3", "gather src (N,16)->(E,16) f32", lambda: ops.BroadcastSrcNode(h, g),
                E * (8 + 64 + 64))
@@ -109,6 +125,12 @@ def main():
         Xe, Wr = rnd(E, 128, dtype=dt), rnd(wl.num_etypes, H, D, D, dtype=dt)
         report("c4", "segment_mm edge 8 x (16->16) bf16", lambda: ops.SegmentMMEdge(Xe, Wr, g),
                E * 256 * b + wl.num_etypes * H * D * D * b, 2 * E * H * D * D)
+        report("c4", "segment_mm gather src 8 x (16->16) bf16",
+               lambda: ops.SegmentMMEdgeGather(X, Wr, 0, g),
+               E * (8 + 512) + wl.num_etypes * H * D * D * b, 2 * E * H * D * D)
+        report("c4", "segment_mm dot (src rows, dst rows) 8 x (16->16) bf16",
+               lambda: ops.SegmentMMEdgeDot(X, Wr, 0, X, 1, g),
+               E * (16 + 512 + 4 * H) + wl.num_etypes * H * D * D * b, 2 * E * H * D * D)
         q, k = rnd(N, H, D, dtype=dt), rnd(N, H, D, dtype=dt)
         report("c4", "sddmm u_dot_v 8x16 bf16", lambda: ops.gsddmm_u_dot_v(k, q, g),
                4 * (N + 1) + E * (4 + 2 * H * D * b + 4 * H))
@@ -119,8 +141,21 @@ def main():
         report("c4", "spmm u_mul_e H=8 F=128 bf16",
                lambda: ops.gspmm_src_mul_e_sum(v, a, [1], False, None, g),
                4 * (N + 1) + E * (4 + 4 * H + H * D * b) + N * H * D * b)
+        report("c4", "spmm e_mul_e H=8 F=128 bf16", lambda: ops.spmm(g, "e_mul_e", "sum", Xe, a),
+               4 * (N + 1) + E * (4 + 4 + 4 * H + H * D * b) + N * H * D * b)
         report("c4", "gather src (N,128)->(E,128) bf16", lambda: ops.BroadcastSrcNode(X, g),
                E * (8 + 256 + 256))
+        wk, wq, wv, wa = (rnd(wl.num_ntypes, 128, 128, dtype=dt) / 11 for _ in range(4))
+        ra, rm = (rnd(wl.num_etypes, H, D, D, dtype=dt) / 4 for _ in range(2))
+        rp = torch.rand(wl.num_etypes, H, device=dev).to(dt)
+        skip = torch.ones(wl.num_ntypes, device=dev)
+        # bytes of the fused layer: h in, K/V/Q/t/out node rows, three gathered
+        # rows per edge, the transformed values written and read once, scores
+        layer_bytes = N * 128 * b * 9 + E * (3 * 128 * b + 2 * 128 * b + 24 + 6 * 4 * H)
+        for fused in (False, True):
+            report("c4", f"hgt layer bf16 {'fused' if fused else 'plan'}",
+                   lambda: layers.hgt_layer(g, X, wk, wq, wv, wa, ra, rm, rp, skip, H, fused=fused),
+                   layer_bytes, 2 * N * 128 * 128 * 4 + 4 * E * H * D * D)
 
     if "c5" in args.configs:
         wl = datasets.gat_rmat_large()

@@ -32,6 +32,8 @@
 // (HGT's sum(k * q)), in which case Y never reaches memory.
 #include "common.h"
 
+#include <type_traits>
+
 namespace ga {
 namespace {
 
@@ -72,6 +74,7 @@ struct MmExt {
   const void *Q;            // dot operand rows (ldq elements apart); null: store Y
   const int64_t *q_index;   // row r is reduced against Q[q_index[r]]; null: Q[r]
   float *dot;               // (rows, ldd) fp32, column = head
+  const float *scale;       // (n_types, ldd) factor per type and head; null: 1
   int64_t ldq, ldd;
   unsigned head_end;        // bit cb: a head's columns end with column block cb
   int half_heads;           // bf16, M == 16: a block pair holds two heads
@@ -464,6 +467,54 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
     }
   }
   int64_t inext = src_row(first + kTileBlock);
+
+  // dot operand: the values this lane needs from Q (4 rows x its column of every
+  // block; a packed bf16 pair per block pair) are requested one tile ahead as
+  // well, their row indices two tiles ahead
+  constexpr int NQ = DOT ? (MM::kPaired ? CG / 2 : CG) : 1;
+  typedef typename std::conditional<MM::kPaired, uint32_t, float>::type qv_t;
+  const T *__restrict__ Qb = static_cast<const T *>(e.Q);
+  const int64_t *__restrict__ qix = e.q_index;
+  auto q_row = [&](int row) -> int64_t {
+    if (row >= row1) return 0;
+    return qix ? qix[row] : (int64_t)row;
+  };
+  auto load_q = [&](int64_t qr, bool live, qv_t (&dst)[NQ]) {
+    const T *qrow = Qb + qr * e.ldq;
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      dst[i] = 0;
+      if constexpr (MM::kPaired) {
+        const int m = i * 32 + 2 * lr;                      // even column of the pair
+        if (live && (full_cols || m + 1 < g.Mt))
+          dst[i] = *reinterpret_cast<const uint32_t *>(qrow + m);
+      } else {
+        const int m = i * 16 + lr;
+        if (live && (full_cols || m < g.Mt)) dst[i] = ldf(qrow + m);
+      }
+    }
+  };
+  // per-head factors of this chunk's type, read once: a load inside the tile
+  // loop would make every tile wait for the prefetches issued before it
+  float scv[CG];
+#pragma unroll
+  for (int i = 0; i < CG; ++i) {
+    scv[i] = 1.0f;
+    if (DOT && e.scale) {
+      const int h = e.half_heads ? i * 2 + (lr >> 3) : i;
+      if (h < g.hb) scv[i] = e.scale[(int64_t)type * e.ldd + h];
+    }
+  }
+  qv_t qn[4][NQ];
+  int64_t qinext[4];
+  if (DOT) {
+    const int t0 = row0 + wave * kTileRows + lk * 4;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      load_q(q_row(t0 + r), t0 + r < row1, qn[r]);
+      qinext[r] = q_row(t0 + kTileBlock + r);
+    }
+  }
   for (int tile0 = row0 + wave * kTileRows; tile0 < row1;
        tile0 += kTileBlock, yp += ystep) {
     // With many weight fragments the compiler would otherwise keep them all in
@@ -483,6 +534,17 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
       }
     }
     inext = src_row(tile0 + 2 * kTileBlock + lr);
+    qv_t qa[4][NQ];
+    if (DOT) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) qa[r][i] = qn[r][i];
+        const int nrow = tile0 + kTileBlock + lk * 4 + r;
+        load_q(qinext[r], nrow < row1, qn[r]);
+        qinext[r] = q_row(nrow + kTileBlock);
+      }
+    }
     floatx4 acc[CG];
 #pragma unroll
     for (int cb = 0; cb < CG; ++cb) acc[cb] = floatx4{0, 0, 0, 0};
@@ -494,33 +556,27 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
     }
     // lane holds rows tile0 + 4*lk + r, lane column lr of every column block
     if (DOT) {
-      const T *__restrict__ Q = static_cast<const T *>(e.Q);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int row = tile0 + lk * 4 + r;
         const bool live = row < row1;          // uniform over the 16 lanes of a row
-        const int64_t qr = live ? (e.q_index ? e.q_index[row] : (int64_t)row) : 0;
-        const T *qrow = Q + qr * e.ldq;
         float *drow = e.dot + (int64_t)row * e.ldd;
         float s = 0.0f;
         int head = 0;
         if constexpr (MM::kPaired) {
 #pragma unroll
           for (int cb = 0; cb < CG; cb += 2) {
-            const int m = (cb >> 1) * 32 + 2 * lr;          // even column of the pair
-            uint32_t qv = 0;
-            if (live && (full_cols || m + 1 < g.Mt))
-              qv = *reinterpret_cast<const uint32_t *>(qrow + m);
+            const uint32_t qv = qa[r][cb >> 1];
             s = fmaf(acc[cb][r], bf16_lo(qv), s);
             s = fmaf(acc[cb + 1 < CG ? cb + 1 : cb][r], bf16_hi(qv), s);
             if (e.half_heads) {                  // lanes 0-7: one head, 8-15: the next
               const float t = row8_sum(s);
               const int h = (cb >> 1) * 2 + (lr >> 3);
-              if (live && (lr & 7) == 0 && h < g.hb) drow[h] = t;
+              if (live && (lr & 7) == 0 && h < g.hb) drow[h] = t * scv[cb >> 1];
               s = 0.0f;
             } else if (e.head_end >> (cb + 1) & 1) {
               const float t = row16_sum(s);
-              if (live && lr == 0) drow[head] = t;
+              if (live && lr == 0) drow[head] = t * scv[head < CG ? head : 0];
               ++head;
               s = 0.0f;
             }
@@ -528,13 +584,10 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
         } else {
 #pragma unroll
           for (int cb = 0; cb < CG; ++cb) {
-            const int m = cb * 16 + lr;
-            float qv = 0.0f;
-            if (live && (full_cols || m < g.Mt)) qv = ldf(qrow + m);
-            s = fmaf(acc[cb][r], qv, s);
+            s = fmaf(acc[cb][r], qa[r][cb], s);
             if (e.head_end >> cb & 1) {
               const float t = row16_sum(s);
-              if (live && lr == 0) drow[head] = t;
+              if (live && lr == 0) drow[head] = t * scv[head < CG ? head : 0];
               ++head;
               s = 0.0f;
             }
@@ -687,6 +740,7 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
         if (!e.half_heads && M % (paired ? 32 : 16) != 0) return GA_EUNSUPPORTED;
         e.Q = static_cast<const T *>(ext.Q) + (int64_t)h0 * M;
         e.dot = ext.dot + h0;
+        if (e.scale) e.scale = ext.scale + h0;
         e.head_end = 0;
         for (int b = 0; b < 32; ++b) {
           const int end_col = paired ? ((b >> 1) + 1) * 32 : (b + 1) * 16;
@@ -810,20 +864,22 @@ extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
 extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types,
                                     const void *X, const int64_t *x_index,
                                     const void *W, void *Y, const void *Q,
-                                    const int64_t *q_index, float *dot, int64_t rows,
-                                    int64_t heads, int64_t K, int64_t M, int dtype,
+                                    const int64_t *q_index, const float *scale,
+                                    float *dot, int64_t rows, int64_t heads,
+                                    int64_t K, int64_t M, int dtype,
                                     ga_stream_t stream) {
   using namespace ga;
   const int bad = check_mm_args(n_types, rows, heads, K, M, dtype);
   if (bad != GA_OK) return bad;
   if ((Y != nullptr) == (dot != nullptr)) return GA_EINVAL;   // exactly one result
   if ((Q != nullptr) != (dot != nullptr)) return GA_EINVAL;
-  if (q_index && !Q) return GA_EINVAL;
+  if ((q_index || scale) && !Q) return GA_EINVAL;
   if (rows == 0 || n_types == 0) return GA_OK;
   if (!type_pointer || !X || !W) return GA_EINVAL;
   const size_t esz = dtype == GA_F32 ? 4 : 2;
   if (!aligned(X, esz) || !aligned(W, esz) || (Y && !aligned(Y, esz)) ||
       (Q && !aligned(Q, esz)) || (dot && !aligned(dot, 4)) ||
+      (scale && !aligned(scale, 4)) ||
       (x_index && !aligned(x_index, 8)) || (q_index && !aligned(q_index, 8)))
     return GA_EALIGN;
   MmExt ext = {};
@@ -831,6 +887,7 @@ extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types
   ext.Q = Q;
   ext.q_index = q_index;
   ext.dot = dot;
+  ext.scale = scale;
   ext.ldq = heads * M;
   ext.ldd = heads;
   return segment_mm_any(type_pointer, n_types, X, W, Y, rows, heads, K, M, dtype, ext,

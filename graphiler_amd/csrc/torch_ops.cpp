@@ -409,7 +409,7 @@ torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
   const int rc = ga_segment_mm_gather(
       graph->etype_pointer.value().data_ptr<int>(), graph->num_etypes, features.data_ptr(),
       index.data_ptr<int64_t>(), weights.data_ptr(), out.data_ptr(), nullptr, nullptr,
-      nullptr, graph->num_edges, s.heads, s.K, s.M, s.dt, current_stream(out));
+      nullptr, nullptr, graph->num_edges, s.heads, s.K, s.M, s.dt, current_stream(out));
   if (rc == GA_EUNSUPPORTED)       // shape outside the matrix-core tile
     return segment_mm(gather(features, index), weights, graph->etype_pointer,
                       graph->num_etypes, graph->num_edges);
@@ -421,8 +421,16 @@ torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
 // (examples/HGT/HGT.py:42-45), fp32 (E, heads)
 torch::Tensor SegmentMMEdgeDot(torch::Tensor features, torch::Tensor weights,
                                int64_t endpoint, torch::Tensor other,
-                               int64_t other_endpoint, const GraphPtr &graph) {
+                               int64_t other_endpoint, at::optional<torch::Tensor> scale,
+                               const GraphPtr &graph) {
   const MmShape s = edge_mm_shape(features, weights, graph);
+  torch::Tensor sc;      // (T, heads) fp32: out[e, h] *= scale[type(e), h]
+  if (scale.has_value()) {
+    check_input(scale.value(), "scale");
+    TORCH_CHECK(scale.value().numel() == graph->num_etypes * s.heads,
+                "scale must have one value per type and head");
+    sc = scale.value().to(at::kFloat).contiguous();
+  }
   check_input(other, "other");
   TORCH_CHECK(other.scalar_type() == features.scalar_type() &&
                   other.size(0) == graph->num_nodes && feat_dim(other) == s.heads * s.M,
@@ -434,14 +442,19 @@ torch::Tensor SegmentMMEdgeDot(torch::Tensor features, torch::Tensor weights,
   const int rc = ga_segment_mm_gather(
       graph->etype_pointer.value().data_ptr<int>(), graph->num_etypes, features.data_ptr(),
       xi.data_ptr<int64_t>(), weights.data_ptr(), nullptr, other.data_ptr(),
-      qi.data_ptr<int64_t>(), out.data_ptr<float>(), graph->num_edges, s.heads, s.K, s.M,
-      s.dt, current_stream(out));
+      qi.data_ptr<int64_t>(), sc.defined() ? sc.data_ptr<float>() : nullptr,
+      out.data_ptr<float>(), graph->num_edges, s.heads, s.K, s.M, s.dt, current_stream(out));
   if (rc == GA_EUNSUPPORTED) {
     torch::Tensor y = SegmentMMEdgeGather(features, weights, endpoint, graph);
     torch::Tensor q = gather(other, qi).reshape(y.sizes());
-    return (y.to(at::kFloat) * q.to(at::kFloat))
-        .reshape({graph->num_edges, s.heads, s.M})
-        .sum(-1);
+    torch::Tensor d = (y.to(at::kFloat) * q.to(at::kFloat))
+                          .reshape({graph->num_edges, s.heads, s.M})
+                          .sum(-1);
+    TORCH_CHECK(!sc.defined() || graph->etype_COO.has_value(),
+                "the graph has no edge-type column");
+    if (sc.defined())
+      d = d * gather(sc.reshape({graph->num_etypes, s.heads}), graph->etype_COO.value());
+    return d;
   }
   check_ga(rc, "ga_segment_mm_gather");
   return out;
@@ -614,7 +627,7 @@ static auto registry =
             " g) -> Tensor z",
             &SegmentMMEdgeGather)
         .op("my_ops::SegmentMMEdgeDot(Tensor x, Tensor w, int endpoint, Tensor q, "
-            "int q_endpoint, " GRAPH_T " g) -> Tensor z",
+            "int q_endpoint, Tensor? scale, " GRAPH_T " g) -> Tensor z",
             &SegmentMMEdgeDot)
         .op("my_ops::gat_aggregate(Tensor el, Tensor er, Tensor z, float slope, " GRAPH_T
             " g) -> Tensor y",

@@ -114,13 +114,14 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
     k = ops.SegmentMMNode(h, k_weight, g)
     v = ops.SegmentMMNode(h, v_weight, g)
     q = ops.SegmentMMNode(h, q_weight, g)
-    pri = ops.BroadcastEdgeType(relation_pri.float(), g) / (d ** 0.5)
     if fused:
-        attn = ops.SegmentMMEdgeDot(k, relation_att, 0, q, 1, g) * pri
-        a = ops.SegmentSoftmax(attn.contiguous(), 1, None, g)      # (E, heads) fp32
+        attn = ops.SegmentMMEdgeDot(k, relation_att, 0, q, 1, g,
+                                    scale=relation_pri.float() / (d ** 0.5))
+        a = ops.SegmentSoftmax(attn, 1, None, g)                   # (E, heads) fp32
         v_e = ops.SegmentMMEdgeGather(v, relation_msg, 0, g)
         t = ops.spmm(g, "e_mul_e", "sum", v_e, a)
     else:
+        pri = ops.BroadcastEdgeType(relation_pri.float(), g) / (d ** 0.5)
         k_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(k, g), relation_att, g)
         v_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(v, g), relation_msg, g)
         q_e = ops.BroadcastDstNode(q, g)

@@ -390,6 +390,9 @@ class _Rewriter:
             if n.kind() == "aten::sum":
                 changed |= self._fuse_mm_dot(n)
         for n in list(self.G.nodes()):
+            if n.kind() == "aten::mul":
+                changed |= self._fuse_dot_scale(n)
+        for n in list(self.G.nodes()):
             if n.kind() == "my_ops::SpMMEdge":
                 changed |= self._fuse_e_mul_e(n)
         return changed
@@ -428,7 +431,27 @@ class _Rewriter:
                 which = self.const(0 if bc.kind().endswith("SrcNode") else 1, n)
                 out = self.make("my_ops::SegmentMMEdgeDot",
                                 [mm.inputsAt(0), mm.inputsAt(1), mm.inputsAt(2),
-                                 bc.inputsAt(0), which, self.dglgraph], n, EDGE)
+                                 bc.inputsAt(0), which, self.const(None, n), self.dglgraph],
+                                n, EDGE)
+                n.output().replaceAllUsesWith(out)
+                n.destroy()
+                return True
+        return False
+
+    def _fuse_dot_scale(self, n) -> bool:
+        """SegmentMMEdgeDot(..., scale=None) * BroadcastEdgeType(p) with p one value
+        per type (the dot has one head, see _fuse_mm_dot) -> the factor goes into
+        the operator's per-type scale table."""
+        for a, b in ((n.inputsAt(0), n.inputsAt(1)), (n.inputsAt(1), n.inputsAt(0))):
+            dot, bc = a.node(), b.node()
+            if dot.kind() == "my_ops::SegmentMMEdgeDot" and self.single_use(a) and \
+                    dot.inputsAt(5).node().kind() == "prim::Constant" and \
+                    dot.inputsAt(5).toIValue() is None and \
+                    isinstance(dot.inputsAt(5).type(), torch._C.NoneType) and \
+                    bc.kind() == "my_ops::BroadcastEdgeType":
+                ins = list(dot.inputs())
+                ins[5] = bc.inputsAt(0)
+                out = self.make("my_ops::SegmentMMEdgeDot", ins, n, EDGE)
                 n.output().replaceAllUsesWith(out)
                 n.destroy()
                 return True

@@ -368,7 +368,7 @@ def SegmentMMEdgeGather(features, weights, endpoint: int, graph: DGLGraph) -> to
                       device=features.device)
     rc = capi.load().ga_segment_mm_gather(
         graph.etype_pointer.data_ptr(), graph.num_etypes, features.data_ptr(),
-        index.data_ptr(), weights.data_ptr(), out.data_ptr(), None, None, None,
+        index.data_ptr(), weights.data_ptr(), out.data_ptr(), None, None, None, None,
         graph.num_edges, heads, K, M, _feat_dtype(features, "features"), _stream(out))
     if rc == capi.GA_EUNSUPPORTED:      # shape outside the matrix-core tile
         return SegmentMMEdge(_gather(features, index), weights, graph)
@@ -377,11 +377,18 @@ def SegmentMMEdgeGather(features, weights, endpoint: int, graph: DGLGraph) -> to
 
 
 def SegmentMMEdgeDot(features, weights, endpoint: int, other, other_endpoint: int,
-                     graph: DGLGraph) -> torch.Tensor:
+                     graph: DGLGraph, scale=None) -> torch.Tensor:
     """out[e, h] = <features[endpoint(e)] @ weights[type(e)], other[other_endpoint(e)]>
     per head, fp32 (E, heads): the ``sum(bmm(k, W) * q, dim=1, keepdim=True)`` of
-    examples/HGT/HGT.py:42-45 with neither per-edge operand materialised."""
+    examples/HGT/HGT.py:42-45 with neither per-edge operand materialised.
+    ``scale`` (T, heads) or (T,) multiplies row e by scale[type(e)] (the
+    ``* relation_pri`` of HGT.py:45)."""
     heads, K, M = _mm_shapes(features, weights, graph)
+    if scale is not None:
+        _check_input(scale, "scale")
+        if scale.numel() != graph.num_etypes * heads:
+            raise RuntimeError("scale must have one value per type and head")
+        scale = scale.float().contiguous()
     _check_input(other, "other")
     if other.dtype != features.dtype or int(other.shape[0]) != graph.num_nodes \
             or get_feat_dim(other) != heads * M:
@@ -391,12 +398,15 @@ def SegmentMMEdgeDot(features, weights, endpoint: int, other, other_endpoint: in
     rc = capi.load().ga_segment_mm_gather(
         graph.etype_pointer.data_ptr(), graph.num_etypes, features.data_ptr(),
         xi.data_ptr(), weights.data_ptr(), None, other.data_ptr(), qi.data_ptr(),
-        out.data_ptr(), graph.num_edges, heads, K, M,
+        _ptr(scale), out.data_ptr(), graph.num_edges, heads, K, M,
         _feat_dtype(features, "features"), _stream(out))
     if rc == capi.GA_EUNSUPPORTED:
         y = SegmentMMEdgeGather(features, weights, endpoint, graph)
         prod = y.float() * _gather(other, qi).float().reshape(y.shape)
-        return prod.reshape(graph.num_edges, heads, M).sum(-1)
+        out = prod.reshape(graph.num_edges, heads, M).sum(-1)
+        if scale is not None:
+            out = out * BroadcastEdgeType(scale.reshape(graph.num_etypes, heads), graph)
+        return out
     capi.check(rc, "ga_segment_mm_gather")
     return out
 

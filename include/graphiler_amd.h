@@ -197,7 +197,9 @@ int ga_segment_mm(const int32_t *type_pointer, int64_t n_types, const void *X,
  *   Y   (rows, heads*M) `dtype`, with Q / q_index / dot NULL;
  *   dot (rows, heads) fp32 with Y NULL: dot[r, h] = <Y[r, h, :], Q[q_index[r], h, :]>
  *       (q_index NULL: Q[r]); Q (*, heads*M) `dtype`.  The product rows stay in
- *       registers (HGT's sum(k * q, dim=1), HGT.py:44-45).
+ *       registers (HGT's sum(k * q, dim=1), HGT.py:44-45).  scale, when not
+ *       NULL, is (n_types, heads) fp32 and multiplies dot[r, h] by
+ *       scale[type(r), h] (the relation_pri factor of HGT.py:45).
  * x_index / q_index are int64 (the COO columns of the graph); entries are not
  * checked on the device.  Returns GA_EUNSUPPORTED, having launched nothing, for
  * shapes outside the matrix-core tile (heads*K > 128 fp32 / 256 bf16,
@@ -206,9 +208,9 @@ int ga_segment_mm(const int32_t *type_pointer, int64_t n_types, const void *X,
  */
 int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types, const void *X,
                          const int64_t *x_index, const void *W, void *Y,
-                         const void *Q, const int64_t *q_index, float *dot,
-                         int64_t rows, int64_t heads, int64_t K, int64_t M,
-                         int dtype, ga_stream_t stream);
+                         const void *Q, const int64_t *q_index, const float *scale,
+                         float *dot, int64_t rows, int64_t heads, int64_t K,
+                         int64_t M, int dtype, ga_stream_t stream);
 
 /* ---------------------------------------------------------------- gather --
  * y[i, :] = x[idx[i], :], a bit-exact row copy of row_bytes bytes.

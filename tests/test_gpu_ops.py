@@ -482,7 +482,7 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
         rc = lib.ga_segment_mm_gather(
             g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(),
             (g.COO_src if which == 0 else g.COO_dst).data_ptr(), dW.data_ptr(), Y.data_ptr(),
-            None, None, None, e, heads, K, M, dt, stream)
+            None, None, None, None, e, heads, K, M, dt, stream)
         assert rc == (0 if fits else capi.GA_EUNSUPPORTED)
         if fits:
             assert_close(Y.float().cpu().numpy(), ref, tol, f"segment_mm_gather {which}")
@@ -497,14 +497,17 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
         rc = lib.ga_segment_mm_gather(
             g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(),
             (g.COO_src if which == 0 else g.COO_dst).data_ptr(), dW.data_ptr(), None,
-            dQ.data_ptr(), (g.COO_dst if which == 0 else g.COO_src).data_ptr(), D.data_ptr(),
-            e, heads, K, M, dt, stream)
+            dQ.data_ptr(), (g.COO_dst if which == 0 else g.COO_src).data_ptr(), None,
+            D.data_ptr(), e, heads, K, M, dt, stream)
         assert rc == (0 if dot_fits else capi.GA_EUNSUPPORTED)
         if dot_fits:
             assert_close(D.cpu().numpy(), want, tol, f"segment_mm dot {which}")
         got = ops.SegmentMMEdgeDot(dX, dW, which, dQ, 1 - which, g)
         assert got.shape == (e, heads) and got.dtype == torch.float32
         assert_close(got.cpu().numpy(), want, tol, f"SegmentMMEdgeDot {which}")
+        scale = rng.uniform(0.5, 2.0, (n_rel, heads)).astype(np.float32)
+        got = ops.SegmentMMEdgeDot(dX, dW, which, dQ, 1 - which, g, scale=_dev(scale, device))
+        assert_close(got.cpu().numpy(), want * scale[etype], tol, f"SegmentMMEdgeDot scaled {which}")
     # identity index (NULL) = plain segment_mm on per-edge rows
     Xe = rng.standard_normal((e, heads * K), dtype=np.float32)
     if bf16:
@@ -513,14 +516,14 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
     if fits:
         Y = torch.full((e, heads * M), float("nan"), dtype=dX.dtype, device=device)
         assert lib.ga_segment_mm_gather(g.etype_pointer.data_ptr(), n_rel, dXe.data_ptr(), None,
-                                        dW.data_ptr(), Y.data_ptr(), None, None, None, e,
+                                        dW.data_ptr(), Y.data_ptr(), None, None, None, None, e,
                                         heads, K, M, dt, stream) == 0
         assert_close(Y.float().cpu().numpy(), oracle.segment_mm(tp, Xe, W, heads=heads), tol,
                      "segment_mm_gather identity")
     # argument errors: both or neither result, dot without Q
     assert lib.ga_segment_mm_gather(g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(), None,
-                                    dW.data_ptr(), None, None, None, None, e, heads, K, M, dt,
-                                    stream) == capi.GA_EINVAL
+                                    dW.data_ptr(), None, None, None, None, None, e, heads, K, M,
+                                    dt, stream) == capi.GA_EINVAL
 
 
 def test_e_mul_e_sum(device):
