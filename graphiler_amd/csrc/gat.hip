@@ -8,6 +8,11 @@
 // acc.  Two states merge as
 //   M = max(m1, m2); l = l1 e^(m1-M) + l2 e^(m2-M); acc likewise,
 // so partial rows combine exactly like partial sums, in run order.
+//
+// The same pass with per-edge operands (EDGE): the logits are given per edge
+// and the weighted rows are per-edge rows, both read through the edge-id
+// column: out[v] = sum_e softmax_v(logit)[e] * m[e], the SegmentSoftmax ->
+// mul -> SpMMEdge tail of examples/HGT/HGT.py:50-53 with no attention tensor.
 #include "row_runs.h"
 
 namespace ga {
@@ -19,16 +24,16 @@ __device__ __forceinline__ float leaky(float t, float slope) {
 
 // State per lane: VEC un-normalised weighted sums, then the running maximum m
 // and the running denominator l of the lane's head.
-template <typename T, int VEC>
+template <typename T, int VEC, bool EDGE = false>
 struct GatPolicy {
   typedef T out_t;
   static constexpr int kVec = VEC;
   static constexpr int kState = VEC + 2;
   struct Args {
-    const int32_t *nbr;
-    const float *el;
-    const float *er;
-    const T *z;
+    const int32_t *nbr;   // EDGE: the edge-id column, or null when slot = edge id
+    const float *el;      // EDGE: per-edge logits (E, heads)
+    const float *er;      // EDGE: unused
+    const T *z;           // EDGE: per-edge rows (E, heads*dph)
     int heads;
     int dph;
     float slope;
@@ -79,12 +84,20 @@ struct GatPolicy {
       float s[kUnroll];
       typename IO::raw_t x[kUnroll];
       load_ids8(row_of_slot, j, b, A.ids_vec, r);
-      load_ids8(A.nbr, j, b, A.ids_vec, g);
+      if (EDGE && !A.nbr) {
+#pragma unroll
+        for (int t = 0; t < kUnroll; ++t) g[t] = (int)(j + t < b ? j + t : b - 1);
+      } else {
+        load_ids8(A.nbr, j, b, A.ids_vec, g);
+      }
 #pragma unroll
       for (int t = 0; t < kUnroll; ++t) {
         x[t] = IO::load(A.z + (int64_t)g[t] * feat + f0);
-        s[t] = leaky(A.el[(int64_t)g[t] * A.heads + h] + A.er[(int64_t)r[t] * A.heads + h],
-                     A.slope);
+        if constexpr (EDGE)
+          s[t] = A.el[(int64_t)g[t] * A.heads + h];
+        else
+          s[t] = leaky(A.el[(int64_t)g[t] * A.heads + h] + A.er[(int64_t)r[t] * A.heads + h],
+                       A.slope);
       }
       const bool one_row = j + kUnroll <= b && r[0] == cur && r[kUnroll - 1] == cur;
       if (one_row) {
@@ -132,13 +145,13 @@ struct GatPolicy {
   }
 };
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool EDGE = false>
 int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const int32_t *nbr, const float *el, const float *er,
                const void *z, void *out, int64_t n_rows, int64_t n_edges,
                int heads, int dim, float slope, float *ws, hipStream_t stream) {
-  typedef GatPolicy<T, VEC> P;
-  const bool ids_vec = aligned(row_of_slot, 16) && aligned(nbr, 16);
+  typedef GatPolicy<T, VEC, EDGE> P;
+  const bool ids_vec = aligned(row_of_slot, 16) && (!nbr || aligned(nbr, 16));
   typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges,
                         heads * dim, ws, stream);
@@ -198,6 +211,46 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
   return ga::launch_gat<ga::bf16_t, 1>(pointer, row_of_slot, nbr, el, er, z, out,
                                        n_rows, n_edges, (int)heads, (int)dim,
                                        slope, ws, s);
+}
+
+int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,
+                        const int32_t *eid, const float *logit, const void *m,
+                        void *out, int64_t n_rows, int64_t n_edges, int64_t heads,
+                        int64_t dim, int dtype, void *workspace,
+                        size_t workspace_bytes, ga_stream_t stream) {
+  if (n_rows < 0 || n_edges < 0 || heads <= 0 || dim <= 0) return GA_EINVAL;
+  if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || heads * dim > 0x7fffffff)
+    return GA_EINVAL;
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  if (n_rows == 0) return GA_OK;
+  if (!pointer || !out) return GA_EINVAL;
+  const int64_t feat = heads * dim;
+  if (n_edges > 0) {
+    if (!row_of_slot || !logit || !m) return GA_EINVAL;
+    if (!workspace || !ga::aligned(workspace, 16) ||
+        ga_gat_workspace_bytes(n_edges, feat, heads) > workspace_bytes)
+      return GA_EWORKSPACE;
+  }
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!ga::aligned(out, esz) || (m && !ga::aligned(m, esz)) ||
+      (logit && !ga::aligned(logit, 4)))
+    return GA_EALIGN;
+  const bool vec_ok = ga::aligned(out, 16) && (!m || ga::aligned(m, 16));
+  hipStream_t s = (hipStream_t)stream;
+  float *ws = (float *)workspace;
+  const int h = (int)heads, d = (int)dim;
+  if (dtype == GA_F32) {
+    if (vec_ok && dim % 4 == 0)
+      return ga::launch_gat<float, 4, true>(pointer, row_of_slot, eid, logit, nullptr, m,
+                                            out, n_rows, n_edges, h, d, 0.0f, ws, s);
+    return ga::launch_gat<float, 1, true>(pointer, row_of_slot, eid, logit, nullptr, m, out,
+                                          n_rows, n_edges, h, d, 0.0f, ws, s);
+  }
+  if (vec_ok && dim % 8 == 0)
+    return ga::launch_gat<ga::bf16_t, 8, true>(pointer, row_of_slot, eid, logit, nullptr, m,
+                                               out, n_rows, n_edges, h, d, 0.0f, ws, s);
+  return ga::launch_gat<ga::bf16_t, 1, true>(pointer, row_of_slot, eid, logit, nullptr, m,
+                                             out, n_rows, n_edges, h, d, 0.0f, ws, s);
 }
 
 }  // extern "C"

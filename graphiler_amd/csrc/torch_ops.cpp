@@ -523,6 +523,35 @@ torch::Tensor gat_aggregate(torch::Tensor el, torch::Tensor er, torch::Tensor z,
   return out;
 }
 
+// SegmentSoftmax -> mul -> SpMMEdge (examples/HGT/HGT.py:50-53) in one pass:
+// out[v] = sum over in-edges e of softmax_v(logits)[e] * messages[e]
+torch::Tensor edge_softmax_sum(torch::Tensor logits, torch::Tensor messages,
+                               const GraphPtr &graph) {
+  check_input(logits, "logits");
+  check_input(messages, "messages");
+  const int64_t heads = feat_dim(logits), feat = feat_dim(messages);
+  const bool fits = logits.scalar_type() == at::kFloat && messages.dim() >= 2 &&
+                    heads > 0 && feat % heads == 0 &&
+                    (messages.scalar_type() == at::kFloat ||
+                     messages.scalar_type() == at::kBFloat16);
+  if (!fits)      // the two operators it stands for
+    return e_mul_e_sum(SegmentSoftmaxForward(logits, 1, at::nullopt, graph), messages, graph);
+  const int dt = feat_dtype(messages, "messages");
+  TORCH_CHECK(logits.size(0) == graph->num_edges && messages.size(0) == graph->num_edges,
+              "logits and messages must have one row per edge");
+  const auto &side = graph->side(false);
+  torch::Tensor out = torch::empty(out_shape(graph->num_nodes, messages), messages.options());
+  torch::Tensor ws = graph->workspace(ga_gat_workspace_bytes(graph->num_edges, feat, heads));
+  check_ga(ga_edge_softmax_sum(graph->in_pointer.data_ptr<int>(), side.rows.data_ptr<int>(),
+                               side.identity ? nullptr
+                                             : graph->in_edge_indices.data_ptr<int>(),
+                               logits.data_ptr<float>(), messages.data_ptr(), out.data_ptr(),
+                               graph->num_nodes, graph->num_edges, heads, feat / heads, dt,
+                               ws.data_ptr(), (size_t)ws.numel(), current_stream(out)),
+           "ga_edge_softmax_sum");
+  return out;
+}
+
 // z = x @ w with the GAT attention terms from the same kernel (GAT.py:25-29)
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> linear_attn(
     torch::Tensor x, torch::Tensor w, torch::Tensor a_l, torch::Tensor a_r) {
@@ -623,6 +652,8 @@ static auto registry =
             &gspmm)
         .op("my_ops::gspmm_e_mul_e_sum(Tensor x, Tensor y, " GRAPH_T " g) -> Tensor z",
             &e_mul_e_sum)
+        .op("my_ops::edge_softmax_sum(Tensor x, Tensor m, " GRAPH_T " g) -> Tensor z",
+            &edge_softmax_sum)
         .op("my_ops::SegmentMMEdgeGather(Tensor x, Tensor w, int endpoint, " GRAPH_T
             " g) -> Tensor z",
             &SegmentMMEdgeGather)

@@ -105,7 +105,7 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
 
     ``fused`` replaces the per-edge copies and products by
       attn = SegmentMMEdgeDot(K, relation_att, src, Q, dst) * pri / sqrt(D)
-      t    = gspmm_e_mul_e_sum(SegmentMMEdgeGather(V, relation_msg, src), softmax(attn))
+      t    = edge_softmax_sum(attn, SegmentMMEdgeGather(V, relation_msg, src))
     so the only per-edge tensors are the scores and the transformed values.
     """
     n, hidden = h.shape
@@ -117,9 +117,8 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
     if fused:
         attn = ops.SegmentMMEdgeDot(k, relation_att, 0, q, 1, g,
                                     scale=relation_pri.float() / (d ** 0.5))
-        a = ops.SegmentSoftmax(attn, 1, None, g)                   # (E, heads) fp32
         v_e = ops.SegmentMMEdgeGather(v, relation_msg, 0, g)
-        t = ops.spmm(g, "e_mul_e", "sum", v_e, a)
+        t = ops.edge_softmax_sum(attn, v_e, g)
     else:
         pri = ops.BroadcastEdgeType(relation_pri.float(), g) / (d ** 0.5)
         k_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(k, g), relation_att, g)

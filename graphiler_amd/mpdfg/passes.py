@@ -395,6 +395,9 @@ class _Rewriter:
         for n in list(self.G.nodes()):
             if n.kind() == "my_ops::SpMMEdge":
                 changed |= self._fuse_e_mul_e(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::gspmm_e_mul_e_sum":
+                changed |= self._fuse_softmax_sum(n)
         return changed
 
     def _fuse_gather_mm(self, n) -> bool:
@@ -454,6 +457,20 @@ class _Rewriter:
                 out = self.make("my_ops::SegmentMMEdgeDot", ins, n, EDGE)
                 n.output().replaceAllUsesWith(out)
                 n.destroy()
+                return True
+        return False
+
+    def _fuse_softmax_sum(self, n) -> bool:
+        """gspmm_e_mul_e_sum(SegmentSoftmax(x), m) with no other reader of the
+        attention -> edge_softmax_sum(x, m): softmax and weighted sum in one pass."""
+        for a, b in ((n.inputsAt(0), n.inputsAt(1)), (n.inputsAt(1), n.inputsAt(0))):
+            sm = a.node()
+            if sm.kind() == "my_ops::SegmentSoftmax" and self.single_use(a):
+                out = self.make("my_ops::edge_softmax_sum",
+                                [sm.inputsAt(0), b, self.dglgraph], n, NODE)
+                n.output().replaceAllUsesWith(out)
+                n.destroy()
+                sm.destroy()
                 return True
         return False
 

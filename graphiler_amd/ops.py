@@ -487,6 +487,34 @@ def gat_aggregate(el, er, z, graph: DGLGraph, negative_slope: float = 0.01):
     return out
 
 
+def edge_softmax_sum(logits, messages, graph: DGLGraph) -> torch.Tensor:
+    """out[v] = sum over in-edges e of softmax_v(logits)[e] * messages[e]: the
+    SegmentSoftmax -> mul -> SpMMEdge tail of the reference's HGT plan
+    (examples/HGT/HGT.py:50-53) in one pass.  logits (E,), (E, 1) or (E, H) fp32;
+    messages (E, H*D) or (E, H, D), both in edge-id order."""
+    _check_input(logits, "logits")
+    _check_input(messages, "messages")
+    dt = _feat_dtype(messages, "messages")
+    if logits.dtype != torch.float32:
+        raise RuntimeError("logits must be float32")
+    heads, feat = get_feat_dim(logits), get_feat_dim(messages)
+    if logits.shape[0] != graph.num_edges or messages.shape[0] != graph.num_edges:
+        raise RuntimeError("logits and messages must have one row per edge")
+    if feat % heads:
+        raise RuntimeError("message width is not a multiple of the heads")
+    out = torch.empty(_out_shape(graph.num_nodes, messages), dtype=messages.dtype,
+                      device=messages.device)
+    lib = capi.load()
+    ws = graph.workspace(lib.ga_gat_workspace_bytes(graph.num_edges, feat, heads))
+    capi.check(lib.ga_edge_softmax_sum(
+        graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
+        None if graph.in_eid_is_identity else graph.in_edge_indices.data_ptr(),
+        logits.data_ptr(), messages.data_ptr(), out.data_ptr(), graph.num_nodes,
+        graph.num_edges, heads, feat // heads, dt, ws.data_ptr(), ws.numel(),
+        _stream(out)), "ga_edge_softmax_sum")
+    return out
+
+
 # ------------------------------------------------------ dense projection ----
 def linear_attn(x, weight, a_l=None, a_r=None):
     """z = x @ weight and, when a_l / a_r (heads, D) are given, the GAT attention

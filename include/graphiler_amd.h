@@ -240,6 +240,22 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
                      void *workspace, size_t workspace_bytes,
                      ga_stream_t stream);
 
+/* The softmax-weighted reduction with per-edge operands:
+ *   a = softmax_v(logit[e, h] over the in-edges e of v),
+ *   out[v, h, :] = sum_e a_e * m[e, h, :]
+ * replacing the tail SegmentSoftmax -> mul -> SpMMEdge (segment_softmax.cu:3-24,
+ * spmm.cu:359-373) of the reference's HGT plan (examples/HGT/HGT.py:50-53) in
+ * one pass, with no (E, heads) attention tensor.  logit (E, heads) fp32 and
+ * m (E, heads*dim) `dtype` are in edge-id order and are read through `eid`
+ * (NULL when slot i holds edge i).  Rows without edges get 0.  workspace:
+ * ga_gat_workspace_bytes(n_edges, heads*dim, heads) bytes, 16-byte aligned.
+ */
+int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,
+                        const int32_t *eid, const float *logit, const void *m,
+                        void *out, int64_t n_rows, int64_t n_edges, int64_t heads,
+                        int64_t dim, int dtype, void *workspace,
+                        size_t workspace_bytes, ga_stream_t stream);
+
 /* ------------------------------------------- dense projection (fp32) ------
  * Z = X @ W and, optionally, the per-head attention terms of a GAT layer
  * el[n, h] = <Z[n, h, :], a_l[h, :]>, er likewise, in the same kernel.

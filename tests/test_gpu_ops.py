@@ -526,6 +526,41 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
                                     dt, stream) == capi.GA_EINVAL
 
 
+@pytest.mark.parametrize("heads,dim,bf16", [(1, 64, False), (8, 16, True), (4, 5, False),
+                                            (2, 24, True), (1, 1, False)])
+def test_edge_softmax_sum(device, heads, dim, bf16):
+    """softmax over the in-edges of per-edge logits times per-edge rows, summed:
+    expected = the oracle's segment softmax, a numpy product and the oracle's
+    copy_e sum.  Edge ids are shuffled against the adjacency order, one node
+    owns a third of the edges and half the nodes have none."""
+    rng = np.random.default_rng(heads * 100 + dim)
+    src, dst = skewed_graph(rng, 600, 9000, 4000)
+    n, e = 600, src.shape[0]
+    g = prepare_graph(src, dst, n, device=device)
+    arr = build_graph_arrays(src, dst, n)
+    logit = (rng.standard_normal((e, heads)) * 3).astype(np.float32)
+    m = rng.standard_normal((e, heads * dim), dtype=np.float32)
+    if bf16:
+        m = to_bf16_f32(m)
+    att = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, logit)
+    prod = (m.reshape(e, heads, dim).astype(np.float64) * att[:, :, None]).reshape(e, -1)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      prod.astype(np.float32), op="copy_e")
+    got = ops.edge_softmax_sum(_dev(logit, device), _dev(m, device, bf16), g)
+    assert got.shape == (n, heads * dim)
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else 2 * TOL_F32,
+                 f"edge_softmax_sum H={heads} D={dim}")
+    assert not got[n // 2:].float().abs().sum().item()         # rows without edges: 0
+    # edge ids already in adjacency order (no edge-id column passed)
+    s2, d2 = datasets.sort_by_dst(src, dst)
+    g2 = prepare_graph(s2, d2, n, device=device)
+    assert g2.in_eid_is_identity
+    order = np.argsort(dst, kind="stable")
+    got2 = ops.edge_softmax_sum(_dev(logit[order], device), _dev(m[order], device, bf16), g2)
+    assert_close(got2.float().cpu().numpy(), ref, TOL_BF16 if bf16 else 2 * TOL_F32,
+                 "edge_softmax_sum identity order")
+
+
 def test_e_mul_e_sum(device):
     """out[v] = sum over in-edges of m[e] * a[e]: SpMMEdge of the product without
     forming it; edge ids shuffled against the adjacency order."""

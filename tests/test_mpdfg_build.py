@@ -73,7 +73,8 @@ def test_level2_fuses_into_graph_operators():
     ours = [x for x in k if x.startswith("my_ops::")]
     assert ours.count("my_ops::SegmentMMNode") == 4
     assert "my_ops::SegmentMMEdgeDot" in ours            # sum(bmm(k, W_att) * q) in one pass
-    assert "my_ops::SegmentMMEdgeGather" in ours and "my_ops::gspmm_e_mul_e_sum" in ours
+    assert "my_ops::SegmentMMEdgeGather" in ours and "my_ops::edge_softmax_sum" in ours
+    assert "my_ops::SegmentSoftmax" not in ours and "my_ops::gspmm_e_mul_e_sum" not in ours
     assert not any(x in ("my_ops::BroadcastSrcNode", "my_ops::BroadcastDstNode",
                          "my_ops::SegmentMMEdge", "my_ops::SpMMEdge") for x in ours)
     assert "aten::bmm" not in k and "aten::squeeze" not in k and "aten::sum" not in k
