@@ -13,7 +13,8 @@ achieved algorithmic GB/s and, for the matrix products, TFLOP/s.
       segment_mm on nodes and on edges (plain, gathered, with the dot-product
       epilogue), SDDMM u_dot_v, 8-head softmax, SpMM u_mul_e / e_mul_e, the layer
   c5  GAT, 2.45 M nodes / 64.3 M edges, 4 heads x 64 bf16: fused aggregation,
-      SpMM u_mul_e, SDDMM u_add_v, 4-head softmax
+      SpMM u_mul_e, SDDMM u_add_v, 4-head softmax, the dense projection with its
+      attention terms (100 -> 256 and 256 -> 256) beside the three ATen GEMMs it replaces
 
 Inputs are resident on the device; each operator is timed with HIP events over
 `--reps` calls after `--warmup` calls.  Byte counts credit one gathered row
@@ -175,6 +176,16 @@ def main():
         lg = rnd(E, H)
         report("c5", "segment_softmax H=4 f32", lambda: ops.SegmentSoftmax(lg, 1, None, g),
                4 * (N + 1) + 8 * E * H)
+        al, ar = rnd(H, F // H), rnd(H, F // H)
+        bl, br = rnd(F, H, dtype=dt), rnd(F, H, dtype=dt)     # block-diagonal (F, H) forms
+        for K in (100, 256):          # first and hidden layers
+            x, w = rnd(N, K, dtype=dt), rnd(K, F, dtype=dt) / 16
+            report("c5", f"projection + attention terms {K}->256 bf16",
+                   lambda: ops.linear_attn(x, w, al, ar),
+                   N * (K + F) * b + K * F * b + 2 * N * H * 4, 2 * N * K * F + 4 * N * F)
+            report("c5", f"three ATen GEMMs {K}->256 bf16 (z, el, er)",
+                   lambda: (lambda z: (z, z @ bl, z @ br))(x @ w),
+                   N * (K + F) * b + K * F * b + 2 * N * H * 4, 2 * N * K * F + 4 * N * F)
 
 
 if __name__ == "__main__":

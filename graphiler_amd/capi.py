@@ -51,6 +51,8 @@ SIGNATURES = {
     "ga_gather_rows": (_int, [_vp, _int, _vp, _vp, _i64, _i64, _vp]),
     "ga_linear_attn": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                               _i64, _vp]),
+    "ga_project_attn": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+                               _i64, _int, _vp]),
     "ga_gat_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "ga_edge_softmax_sum": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                    _int, _vp, _sz, _vp]),

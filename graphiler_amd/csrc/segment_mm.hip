@@ -66,6 +66,8 @@ struct MmGeom {
   int KB, MB;          // k blocks / 16-column blocks of the tile
   int64_t ldx, ldy;    // row strides of X and Y (elements)
   int64_t w_type_stride;  // elements between W[t] and W[t+1]
+  int64_t ldw;            // elements between rows k and k+1 of one (K x M) block
+  int64_t rows;           // used when there is no type pointer: one type, rows [0, rows)
 };
 
 // Optional gather / dot-product operands of the exact-shape kernel.
@@ -76,6 +78,9 @@ struct MmExt {
   float *dot;               // (rows, ldd) fp32, column = head
   const float *scale;       // (n_types, ldd) factor per type and head; null: 1
   int64_t ldq, ldd;
+  const float *a_l, *a_r;   // attention vectors over the tile's columns (kEpiAttn)
+  float *el, *er;           // (rows, ldd) fp32
+  int n_heads;              // heads inside the tile (kEpiAttn)
   unsigned head_end;        // bit cb: a head's columns end with column block cb
   int half_heads;           // bf16, M == 16: a block pair holds two heads
 };
@@ -121,21 +126,22 @@ struct Mma<float, 16> {          // LDS: [k][col], row stride ws floats
       reinterpret_cast<float4 *>(tile)[i] = make_float4(0, 0, 0, 0);
     __syncthreads();
     const int tx = threadIdx.x & (kWave - 1), ty = threadIdx.x / kWave;
-    const bool vec = (g.M & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
+    const bool vec = (g.M & 3) == 0 && (g.ldw & 3) == 0 &&
+                     (reinterpret_cast<uintptr_t>(w) & 15) == 0;
     for (int h = 0; h < g.hb; ++h) {
-      const float *wh = w + (int64_t)h * g.K * g.M;
+      const float *wh = w + (int64_t)h * g.K * g.ldw;
       float *th = tile + (h * g.K) * wsv + h * g.M;
       if (vec) {
         for (int k = ty; k < g.K; k += kBlock / kWave)
           for (int m = tx * 4; m < g.M; m += kWave * 4) {
-            const float4 v = *reinterpret_cast<const float4 *>(wh + (int64_t)k * g.M + m);
+            const float4 v = *reinterpret_cast<const float4 *>(wh + (int64_t)k * g.ldw + m);
             float *d = th + k * wsv + m;       // 16-byte aligned only when h*M is
             d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
           }
       } else {
         for (int k = ty; k < g.K; k += kBlock / kWave)
           for (int m = tx; m < g.M; m += kWave)
-            th[k * wsv + m] = wh[(int64_t)k * g.M + m];
+            th[k * wsv + m] = wh[(int64_t)k * g.ldw + m];
       }
     }
   }
@@ -164,13 +170,13 @@ struct MmaBf16Base {
     __syncthreads();
     const int tx = threadIdx.x & (kWave - 1), ty = threadIdx.x / kWave;
     for (int h = 0; h < g.hb; ++h) {
-      const bf16_t *wh = w + (int64_t)h * g.K * g.M;
+      const bf16_t *wh = w + (int64_t)h * g.K * g.ldw;
       for (int kc = ty * 8; kc < g.K; kc += (kBlock / kWave) * 8)
         for (int m = tx; m < g.M; m += kWave) {
           uint32_t v[8];
 #pragma unroll
           for (int q = 0; q < 8; ++q)
-            v[q] = kc + q < g.K ? (uint32_t)wh[(int64_t)(kc + q) * g.M + m] : 0u;
+            v[q] = kc + q < g.K ? (uint32_t)wh[(int64_t)(kc + q) * g.ldw + m] : 0u;
           const int c = h * g.M + m;                       // tile column
           const int lrow = ((c >> 5) * 2 + (c & 1)) * 16 + ((c & 31) >> 1);
           bf16_t *d = tile + lrow * wsv + h * g.K + kc;
@@ -236,6 +242,12 @@ __device__ __forceinline__ bool locate_chunk(const int32_t *__restrict__ tp,
                                              int &type, int &row0, int &row1) {
   __shared__ int scan[kBlock];
   __shared__ int found[3];
+  if (!tp) {               // one type; the caller passes the row count as n_types
+    type = 0;
+    row0 = blockIdx.x * chunk_rows;
+    row1 = min(n_types, row0 + chunk_rows);
+    return row0 < n_types;
+  }
   if (threadIdx.x == 0) found[0] = -1;
   const int target = blockIdx.x;
   int base = 0;
@@ -414,7 +426,28 @@ struct Tight<bf16_t, 32, NF, CG> {
   }
 };
 
-template <typename T, int KBLK, int NF, int CG, bool DOT>
+template <int NF, int CG>
+struct Tight<bf16_t, 16, NF, CG> {
+  static constexpr int kWs = NF * 16 + 8;
+  static constexpr int kTileElems = CG * 16 * kWs;
+  static __device__ __forceinline__ floatx4 mma(floatx4 acc, const bf16_t *wl, int f,
+                                                int cb, const uint2 &x) {
+    const uint2 w = *reinterpret_cast<const uint2 *>(wl + cb * 16 * kWs + f * 16);
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(shortx4, x),
+                                                     __builtin_bit_cast(shortx4, w),
+                                                     acc, 0, 0, 0);
+  }
+  static __device__ __forceinline__ const bf16_t *lane_base(const bf16_t *tile, int lr, int lk) {
+    return tile + lr * kWs + lk * 4;
+  }
+};
+
+// What happens to a finished tile.
+constexpr int kEpiStore = 0;   // Y
+constexpr int kEpiDot = 1;     // dot[r, h] = <Y[r, h, :], Q[q_index[r], h, :]> only
+constexpr int kEpiAttn = 2;    // Y and el / er[r, h] = <Y[r, h, :], a_l / a_r[h, :]>
+
+template <typename T, int KBLK, int NF, int CG, int EPI>
 __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
     const int32_t *__restrict__ tp, const T *__restrict__ X,
     const T *__restrict__ W, T *__restrict__ Y, MmGeom g, MmExt e) {
@@ -424,7 +457,7 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   T *tile = reinterpret_cast<T *>(lds_raw);
   int type, row0, row1;
-  if (!locate_chunk(tp, g.n_types, g.chunk_rows, type, row0, row1)) return;
+  if (!locate_chunk(tp, tp ? g.n_types : (int)g.rows, g.chunk_rows, type, row0, row1)) return;
   MM::stage(W + (int64_t)type * g.w_type_stride, tile, g);   // g.KB == NF, g.MB == CG
   __syncthreads();
 
@@ -471,6 +504,7 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
   // dot operand: the values this lane needs from Q (4 rows x its column of every
   // block; a packed bf16 pair per block pair) are requested one tile ahead as
   // well, their row indices two tiles ahead
+  constexpr bool DOT = EPI == kEpiDot;
   constexpr int NQ = DOT ? (MM::kPaired ? CG / 2 : CG) : 1;
   typedef typename std::conditional<MM::kPaired, uint32_t, float>::type qv_t;
   const T *__restrict__ Qb = static_cast<const T *>(e.Q);
@@ -503,6 +537,19 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
     if (DOT && e.scale) {
       const int h = e.half_heads ? i * 2 + (lr >> 3) : i;
       if (h < g.hb) scv[i] = e.scale[(int64_t)type * e.ldd + h];
+    }
+  }
+  // attention vectors at this lane's column of every block (0 beyond the tile)
+  float alv[CG], arv[CG];
+#pragma unroll
+  for (int cb = 0; cb < CG; ++cb) {
+    alv[cb] = arv[cb] = 0.0f;
+    if (EPI == kEpiAttn) {
+      const int m = tile_col<MM::kPaired>(cb, lr);
+      if (m < g.Mt) {
+        alv[cb] = e.a_l[m];
+        arv[cb] = e.a_r[m];
+      }
     }
   }
   qv_t qn[4][NQ];
@@ -576,7 +623,7 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
               s = 0.0f;
             } else if (e.head_end >> (cb + 1) & 1) {
               const float t = row16_sum(s);
-              if (live && lr == 0) drow[head] = t * scv[head < CG ? head : 0];
+              if (live && lr == 0 && head < g.hb) drow[head] = t * scv[head < CG ? head : 0];
               ++head;
               s = 0.0f;
             }
@@ -587,7 +634,7 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
             s = fmaf(acc[cb][r], qa[r][cb], s);
             if (e.head_end >> cb & 1) {
               const float t = row16_sum(s);
-              if (live && lr == 0) drow[head] = t * scv[head < CG ? head : 0];
+              if (live && lr == 0 && head < g.hb) drow[head] = t * scv[head < CG ? head : 0];
               ++head;
               s = 0.0f;
             }
@@ -595,6 +642,41 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
         }
       }
       continue;
+    }
+    if (EPI == kEpiAttn) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = tile0 + lk * 4 + r;
+        const bool live = row < row1;
+        float sl = 0.0f, sr = 0.0f;
+        int head = 0;
+        constexpr int step = MM::kPaired ? 2 : 1;
+#pragma unroll
+        for (int cb = 0; cb < CG; cb += step) {
+#pragma unroll
+          for (int i = 0; i < step; ++i) {
+            sl = fmaf(acc[cb + i < CG ? cb + i : cb][r], alv[cb + i < CG ? cb + i : cb], sl);
+            sr = fmaf(acc[cb + i < CG ? cb + i : cb][r], arv[cb + i < CG ? cb + i : cb], sr);
+          }
+          if (MM::kPaired && e.half_heads) {     // lanes 0-7: one head, 8-15: the next
+            const float tl = row8_sum(sl), tr = row8_sum(sr);
+            const int h = (cb >> 1) * 2 + (lr >> 3);
+            if (live && (lr & 7) == 0 && h < (int)e.n_heads) {
+              e.el[(int64_t)row * e.ldd + h] = tl;
+              e.er[(int64_t)row * e.ldd + h] = tr;
+            }
+            sl = sr = 0.0f;
+          } else if (e.head_end >> (cb + step - 1) & 1) {
+            const float tl = row16_sum(sl), tr = row16_sum(sr);
+            if (live && lr == 0 && head < e.n_heads) {   // blocks past the tile are padding
+              e.el[(int64_t)row * e.ldd + head] = tl;
+              e.er[(int64_t)row * e.ldd + head] = tr;
+            }
+            ++head;
+            sl = sr = 0.0f;
+          }
+        }
+      }
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -653,16 +735,16 @@ void launch_cg(const int32_t *tp, const T *X, const T *W, T *Y, const MmGeom &g,
                      dim3(kBlock), lds, s, tp, X, W, Y, g);
 }
 
-template <typename T, int KBLK, int NF, int CG, bool DOT>
+template <typename T, int KBLK, int NF, int CG, int EPI>
 int launch_tight_as(const int32_t *tp, const T *X, const T *W, T *Y, MmGeom g,
                     const MmExt &e, int64_t grid, hipStream_t s) {
   typedef Tight<T, KBLK, NF, CG> TT;
   const size_t lds = (size_t)TT::kTileElems * sizeof(T);
-  if (!allow_lds((const void *)segment_mm_tight_kernel<T, KBLK, NF, CG, DOT>, lds))
+  if (!allow_lds((const void *)segment_mm_tight_kernel<T, KBLK, NF, CG, EPI>, lds))
     return GA_EUNSUPPORTED;
   g.KB = NF;   // the tile is padded to the compile-time shape
   g.MB = CG;
-  hipLaunchKernelGGL((segment_mm_tight_kernel<T, KBLK, NF, CG, DOT>),
+  hipLaunchKernelGGL((segment_mm_tight_kernel<T, KBLK, NF, CG, EPI>),
                      dim3((unsigned)grid), dim3(kBlock), lds, s, tp, X, W, Y, g, e);
   return launch_status();
 }
@@ -670,8 +752,9 @@ int launch_tight_as(const int32_t *tp, const T *X, const T *W, T *Y, MmGeom g,
 template <typename T, int KBLK, int NF, int CG>
 int launch_tight(const int32_t *tp, const T *X, const T *W, T *Y, const MmGeom &g,
                  const MmExt &e, int64_t grid, hipStream_t s) {
-  if (e.Q) return launch_tight_as<T, KBLK, NF, CG, true>(tp, X, W, Y, g, e, grid, s);
-  return launch_tight_as<T, KBLK, NF, CG, false>(tp, X, W, Y, g, e, grid, s);
+  if (e.Q) return launch_tight_as<T, KBLK, NF, CG, kEpiDot>(tp, X, W, Y, g, e, grid, s);
+  if (e.a_l) return launch_tight_as<T, KBLK, NF, CG, kEpiAttn>(tp, X, W, Y, g, e, grid, s);
+  return launch_tight_as<T, KBLK, NF, CG, kEpiStore>(tp, X, W, Y, g, e, grid, s);
 }
 
 template <typename T, int KBLK, int NF>
@@ -717,6 +800,8 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
   g.ldx = (int64_t)heads * K;
   g.ldy = (int64_t)heads * M;
   g.w_type_stride = (int64_t)heads * K * M;
+  g.ldw = M;
+  g.rows = rows;
   // rows per workgroup: a multiple of the 64-row step, large enough to
   // amortise the weight staging, small enough to keep every CU busy
   int64_t steps = rows / (kTileBlock * 2048);
@@ -729,7 +814,7 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
   const T *Wh = W + (int64_t)h0 * K * M;
   T *Yh = Y ? Y + (int64_t)h0 * M : nullptr;
   const bool fused = ext.x_index || ext.Q;
-  if (KBLK != 16 || sizeof(T) == 4) {   // exact-shape kernels: fp32 and bf16 x32
+  {
     if (g.KB <= 8 && g.MB <= 8) {
       MmExt e = ext;
       if (e.Q) {
@@ -747,8 +832,8 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
           if ((!paired || (b & 1)) && end_col % M == 0) e.head_end |= 1u << b;
         }
       }
-      const int rc = pick_tight<T, (sizeof(T) == 4 ? 16 : 32)>(
-          pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), tp, Xh, Wh, Yh, g, e, grid, s);
+      const int rc = pick_tight<T, KBLK>(pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), tp, Xh,
+                                         Wh, Yh, g, e, grid, s);
       if (rc != GA_EUNSUPPORTED || fused) return rc;
     }
   }
@@ -844,6 +929,99 @@ int check_mm_args(int64_t n_types, int64_t rows, int64_t heads, int64_t K, int64
 
 }  // namespace
 }  // namespace ga
+
+namespace ga {
+namespace {
+
+// Z = X @ W for one weight matrix plus el / er = <Z_h, a_l[h]>, <Z_h, a_r[h]>:
+// the exact-shape kernel with a single type, one launch per pass of up to 128
+// output columns (whole heads); X is re-read per pass (from cache for all but
+// the first).
+template <typename T, int KBLK>
+int launch_dense_attn(const T *X, const T *W, T *Z, const float *a_l, const float *a_r,
+                      float *el, float *er, int64_t rows, int K, int M, int heads,
+                      hipStream_t s) {
+  typedef Mma<T, KBLK> MM;
+  constexpr bool paired = MM::kPaired;
+  const int dph = M / heads;
+  if (dph > 128 || (K + KBLK - 1) / KBLK > 8) return GA_EUNSUPPORTED;
+  const bool half = paired && dph == 16;
+  if (!half && dph % (paired ? 32 : 16) != 0) return GA_EUNSUPPORTED;
+  const int pass = (128 / dph) * dph;              // columns per launch: whole heads
+  for (int col0 = 0; col0 < M; col0 += pass) {
+    const int pw = M - col0 < pass ? M - col0 : pass;
+    MmGeom g;
+    g.n_types = 1;
+    g.K = K; g.M = pw; g.hb = 1;
+    g.Kt = K; g.Mt = pw;
+    g.KB = (K + KBLK - 1) / KBLK;
+    g.MB = (pw + 15) / 16;
+    g.ldx = K;
+    g.ldy = M;
+    g.w_type_stride = 0;
+    g.ldw = M;
+    g.rows = rows;
+    int64_t steps = rows / (kTileBlock * 2048);
+    if (steps < 1) steps = 1;
+    if (steps > 16) steps = 16;
+    g.chunk_rows = (int)steps * kTileBlock;
+    const int64_t grid = (rows + g.chunk_rows - 1) / g.chunk_rows;
+    if (grid > 0x7fffffff) return GA_EUNSUPPORTED;
+    MmExt e = {};
+    e.a_l = a_l + col0;
+    e.a_r = a_r + col0;
+    e.el = el + col0 / dph;
+    e.er = er + col0 / dph;
+    e.ldd = heads;
+    e.n_heads = pw / dph;
+    e.half_heads = half;
+    for (int b = 0; b < 32; ++b) {
+      const int end_col = paired ? ((b >> 1) + 1) * 32 : (b + 1) * 16;
+      if ((!paired || (b & 1)) && end_col % dph == 0) e.head_end |= 1u << b;
+    }
+    const int rc = pick_tight<T, KBLK>(pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), nullptr, X,
+                                       W + col0, Z + col0, g, e, grid, s);
+    if (rc != GA_OK) return rc;     // an unsupported shape fails on the first pass
+  }
+  return GA_OK;
+}
+
+}  // namespace
+}  // namespace ga
+
+extern "C" int ga_project_attn(const void *X, const void *W, const float *a_l,
+                               const float *a_r, void *Z, float *el, float *er,
+                               int64_t rows, int64_t K, int64_t M, int64_t heads,
+                               int dtype, ga_stream_t stream) {
+  using namespace ga;
+  if (rows < 0 || K <= 0 || M <= 0 || heads <= 0 || M % heads) return GA_EINVAL;
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  if (rows > 0x7fffffff || K > 0x7fffffff || M > 0x7fffffff) return GA_EINVAL;
+  if (rows == 0) return GA_OK;
+  if (!X || !W || !a_l || !a_r || !Z || !el || !er) return GA_EINVAL;
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!aligned(X, esz) || !aligned(W, esz) || !aligned(Z, esz) || !aligned(a_l, 4) ||
+      !aligned(a_r, 4) || !aligned(el, 4) || !aligned(er, 4))
+    return GA_EALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == GA_F32) {
+    const int rc = ga_linear_attn((const float *)X, (const float *)W, a_l, a_r, (float *)Z,
+                                  el, er, rows, K, M, heads, stream);
+    if (rc != GA_EUNSUPPORTED) return rc;
+    if (aligned(X, 16) && aligned(Z, 16) && K % 4 == 0)
+      return launch_dense_attn<float, 16>((const float *)X, (const float *)W, (float *)Z, a_l,
+                                          a_r, el, er, rows, (int)K, (int)M, (int)heads, s);
+    return GA_EUNSUPPORTED;
+  }
+  if ((M & 1) || !aligned(Z, 4)) return GA_EUNSUPPORTED;      // packed bf16 pair stores
+  if (aligned(X, 16) && K % 8 == 0)
+    return launch_dense_attn<bf16_t, 32>((const bf16_t *)X, (const bf16_t *)W, (bf16_t *)Z,
+                                         a_l, a_r, el, er, rows, (int)K, (int)M, (int)heads, s);
+  if (aligned(X, 8) && K % 4 == 0)
+    return launch_dense_attn<bf16_t, 16>((const bf16_t *)X, (const bf16_t *)W, (bf16_t *)Z,
+                                         a_l, a_r, el, er, rows, (int)K, (int)M, (int)heads, s);
+  return GA_EUNSUPPORTED;
+}
 
 extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
                              const void *X, const void *W, void *Y, int64_t rows,

@@ -552,37 +552,48 @@ torch::Tensor edge_softmax_sum(torch::Tensor logits, torch::Tensor messages,
   return out;
 }
 
-// z = x @ w with the GAT attention terms from the same kernel (GAT.py:25-29)
+// z = x @ w with the GAT attention terms from the same kernel (GAT.py:25-29);
+// fp32 or bf16 storage, el / er always fp32.  Returns the C-ABI code so that a
+// caller can fall back on GA_EUNSUPPORTED.
+int project_attn(const torch::Tensor &x, const torch::Tensor &w, const torch::Tensor &a_l,
+                 const torch::Tensor &a_r, int64_t heads, torch::Tensor &z, torch::Tensor &el,
+                 torch::Tensor &er) {
+  const int64_t rows = x.size(0), K = x.size(1), M = w.size(1);
+  z = torch::empty({rows, M}, x.options());
+  el = torch::empty({rows, heads}, x.options().dtype(at::kFloat));
+  er = torch::empty({rows, heads}, x.options().dtype(at::kFloat));
+  return ga_project_attn(x.data_ptr(), w.data_ptr(), a_l.data_ptr<float>(),
+                         a_r.data_ptr<float>(), z.data_ptr(), el.data_ptr<float>(),
+                         er.data_ptr<float>(), rows, K, M, heads,
+                         x.scalar_type() == at::kFloat ? GA_F32 : GA_BF16, current_stream(x));
+}
+
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> linear_attn(
     torch::Tensor x, torch::Tensor w, torch::Tensor a_l, torch::Tensor a_r) {
   check_input(x, "x");
   check_input(w, "weight");
   check_input(a_l, "a_l");
   check_input(a_r, "a_r");
-  TORCH_CHECK(x.scalar_type() == at::kFloat && w.scalar_type() == at::kFloat &&
-                  a_l.scalar_type() == at::kFloat && a_r.scalar_type() == at::kFloat,
-              "linear_attn is float32 only");
+  feat_dtype(x, "x");
+  TORCH_CHECK(w.scalar_type() == x.scalar_type(), "x and weight must share a dtype");
+  TORCH_CHECK(a_l.scalar_type() == at::kFloat && a_r.scalar_type() == at::kFloat,
+              "a_l and a_r must be float32");
   TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && w.size(0) == x.size(1), "weight must be (K, M)");
-  const int64_t rows = x.size(0), K = x.size(1), M = w.size(1);
+  const int64_t M = w.size(1);
   TORCH_CHECK(a_l.dim() == 2 && a_l.numel() == M && a_r.numel() == M && a_r.dim() == 2 &&
                   a_r.size(0) == a_l.size(0),
               "a_l and a_r must be (heads, M / heads)");
-  const int64_t heads = a_l.size(0);
-  torch::Tensor z = torch::empty({rows, M}, x.options());
-  torch::Tensor el = torch::empty({rows, heads}, x.options());
-  torch::Tensor er = torch::empty({rows, heads}, x.options());
-  check_ga(ga_linear_attn(x.data_ptr<float>(), w.data_ptr<float>(), a_l.data_ptr<float>(),
-                          a_r.data_ptr<float>(), z.data_ptr<float>(), el.data_ptr<float>(),
-                          er.data_ptr<float>(), rows, K, M, heads, current_stream(x)),
-           "ga_linear_attn");
+  torch::Tensor z, el, er;
+  check_ga(project_attn(x, w, a_l, a_r, a_l.size(0), z, el, er), "ga_project_attn");
   return std::make_tuple(z, el, er);
 }
 
 // The dense head of a GAT layer after the split / reorder passes
 // (GAT.py:25-29): z = h @ fc, el = z @ w_src, er = z @ w_dst with w_src / w_dst
 // the two (M, 1) halves of the attention vector.  One kernel when the shape
-// allows (fp32, a single attention column, M in {16, 32, 64}); otherwise three
-// GPU GEMMs through ATen, still on the device.
+// allows (fp32 or bf16, a single attention column, a width the kernels take);
+// otherwise three GPU GEMMs through ATen, still on the device.  el / er are fp32
+// either way (the aggregation that follows reads them as fp32).
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> gat_project(
     torch::Tensor h, torch::Tensor fc, torch::Tensor w_src, torch::Tensor w_dst) {
   check_input(h, "h");
@@ -590,15 +601,21 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> gat_project(
   TORCH_CHECK(w_src.is_cuda() && w_dst.is_cuda(), "attention weights must be a CUDA tensor");
   TORCH_CHECK(h.dim() == 2 && fc.dim() == 2 && fc.size(0) == h.size(1), "fc_weight must be (K, M)");
   const int64_t M = fc.size(1);
-  const bool one_kernel = h.scalar_type() == at::kFloat && fc.scalar_type() == at::kFloat &&
-                          w_src.scalar_type() == at::kFloat && w_dst.scalar_type() == at::kFloat &&
-                          w_src.dim() == 2 && w_dst.dim() == 2 && w_src.size(1) == 1 &&
-                          w_dst.size(1) == 1 && w_src.size(0) == M && w_dst.size(0) == M &&
-                          (M == 16 || M == 32 || M == 64);
-  if (one_kernel)   // an (M, 1) column read as one (1, M) head vector
-    return linear_attn(h, fc, w_src.contiguous().view({1, M}), w_dst.contiguous().view({1, M}));
+  const bool candidate =
+      (h.scalar_type() == at::kFloat || h.scalar_type() == at::kBFloat16) &&
+      fc.scalar_type() == h.scalar_type() && w_src.dim() == 2 && w_dst.dim() == 2 &&
+      w_src.size(1) == 1 && w_dst.size(1) == 1 && w_src.size(0) == M && w_dst.size(0) == M;
+  if (candidate) {   // an (M, 1) column read as one (1, M) head vector
+    torch::Tensor z, el, er;
+    const int rc = project_attn(h, fc, w_src.to(at::kFloat).contiguous().view({1, M}),
+                                w_dst.to(at::kFloat).contiguous().view({1, M}), 1, z, el, er);
+    if (rc != GA_EUNSUPPORTED) {
+      check_ga(rc, "ga_project_attn");
+      return std::make_tuple(z, el, er);
+    }
+  }
   torch::Tensor z = at::mm(h, fc);
-  return std::make_tuple(z, at::mm(z, w_src), at::mm(z, w_dst));
+  return std::make_tuple(z, at::mm(z, w_src).to(at::kFloat), at::mm(z, w_dst).to(at::kFloat));
 }
 
 }  // namespace

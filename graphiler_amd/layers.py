@@ -32,11 +32,13 @@ def gcn_layer(g: DGLGraph, h: torch.Tensor, weight: torch.Tensor,
 def gat_project(h, fc_weight, attn_weight, heads: int = 1):
     """Dense part of the GAT plan (GAT.py:25-29 after the split and reorder
     passes): z = h @ W, el = <z, a_l>, er = <z, a_r> per head."""
-    d = fc_weight.shape[1] // heads
-    if h.dtype == torch.float32 and d in (16, 32, 64):
-        # one kernel: the GEMM with the attention terms in its epilogue
-        return ops.linear_attn(h, fc_weight, attn_weight[0].contiguous(),
-                               attn_weight[1].contiguous())
+    from . import capi
+    try:        # one kernel: the GEMM with the attention terms in its epilogue
+        return ops.linear_attn(h, fc_weight, attn_weight[0].float().contiguous(),
+                               attn_weight[1].float().contiguous())
+    except capi.GraphilerError as err:
+        if err.code != capi.GA_EUNSUPPORTED:
+            raise
     z = torch.mm(h, fc_weight)                               # (N, H*D)
     # per-head dot products as two skinny GEMMs with block-diagonal (H*D, H)
     # matrices: the reference's mm(z2, attn_weight) after its split pass

@@ -517,29 +517,40 @@ def edge_softmax_sum(logits, messages, graph: DGLGraph) -> torch.Tensor:
 
 # ------------------------------------------------------ dense projection ----
 def linear_attn(x, weight, a_l=None, a_r=None):
-    """z = x @ weight and, when a_l / a_r (heads, D) are given, the GAT attention
-    terms el = <z_h, a_l[h]>, er = <z_h, a_r[h]> from the same kernel (fp32).
-    Returns z or (z, el, er).  A head width other than 16/32/64 raises
+    """z = x @ weight and, when a_l / a_r (heads, D) fp32 are given, the GAT
+    attention terms el = <z_h, a_l[h]>, er = <z_h, a_r[h]> (fp32) from the same
+    kernel.  Returns z or (z, el, er).  fp32 or bf16 storage with the attention
+    terms; fp32 only without them.  A shape the kernels do not take raises
     GraphilerError with GA_EUNSUPPORTED."""
     _check_input(x, "x")
     _check_input(weight, "weight")
-    if x.dtype != torch.float32 or weight.dtype != torch.float32:
-        raise RuntimeError("linear_attn is float32 only")
+    dt = _feat_dtype(x, "x")
+    if weight.dtype != x.dtype:
+        raise RuntimeError("x and weight must share a dtype")
+    if x.dim() != 2 or weight.dim() != 2:
+        raise RuntimeError("x must be (rows, K) and weight (K, M)")
     rows, K = int(x.shape[0]), int(x.shape[1])
     if int(weight.shape[0]) != K:
         raise RuntimeError("weight must be (K, M)")
     M = int(weight.shape[1])
     z = torch.empty((rows, M), dtype=x.dtype, device=x.device)
-    heads, el, er = 1, None, None
-    if a_l is not None:
-        _check_input(a_l, "a_l")
-        _check_input(a_r, "a_r")
-        heads = int(a_l.shape[0])
-        if a_l.numel() != M or a_r.numel() != M:
-            raise RuntimeError("a_l and a_r must be (heads, M / heads)")
-        el = torch.empty((rows, heads), dtype=x.dtype, device=x.device)
-        er = torch.empty((rows, heads), dtype=x.dtype, device=x.device)
-    capi.check(capi.load().ga_linear_attn(
-        x.data_ptr(), weight.data_ptr(), _ptr(a_l), _ptr(a_r), z.data_ptr(),
-        _ptr(el), _ptr(er), rows, K, M, heads, _stream(x)), "ga_linear_attn")
-    return z if a_l is None else (z, el, er)
+    if a_l is None:
+        if x.dtype != torch.float32:
+            raise RuntimeError("the plain projection is float32 only")
+        capi.check(capi.load().ga_linear_attn(
+            x.data_ptr(), weight.data_ptr(), None, None, z.data_ptr(), None, None,
+            rows, K, M, 1, _stream(x)), "ga_linear_attn")
+        return z
+    _check_input(a_l, "a_l")
+    _check_input(a_r, "a_r")
+    if a_l.dtype != torch.float32 or a_r.dtype != torch.float32:
+        raise RuntimeError("a_l and a_r must be float32")
+    heads = int(a_l.shape[0])
+    if a_l.numel() != M or a_r.numel() != M or M % heads:
+        raise RuntimeError("a_l and a_r must be (heads, M / heads)")
+    el = torch.empty((rows, heads), dtype=torch.float32, device=x.device)
+    er = torch.empty((rows, heads), dtype=torch.float32, device=x.device)
+    capi.check(capi.load().ga_project_attn(
+        x.data_ptr(), weight.data_ptr(), a_l.data_ptr(), a_r.data_ptr(), z.data_ptr(),
+        el.data_ptr(), er.data_ptr(), rows, K, M, heads, dt, _stream(x)), "ga_project_attn")
+    return z, el, er

@@ -273,6 +273,22 @@ int ga_linear_attn(const float *X, const float *W, const float *a_l,
                    int64_t rows, int64_t K, int64_t M, int64_t heads,
                    ga_stream_t stream);
 
+/* The same projection with the attention terms for fp32 or bf16 storage (fp32
+ * accumulation; el / er are fp32 and are taken from the accumulators, before Z
+ * is rounded): the 100 -> 256 (4 heads x 64, bf16) layer of the larger GAT
+ * configuration as one operator instead of three GEMMs.  fp32 with M/heads in
+ * {16, 32, 64} runs ga_linear_attn; other cases run the typed-linear tile
+ * kernel with a single type, one launch per 128 output columns.  X (rows, K),
+ * W (K, M), Z (rows, M) `dtype`; a_l / a_r (heads, M/heads), el / er
+ * (rows, heads) fp32, all required.  GA_EUNSUPPORTED (nothing launched) when
+ * K > 128 (fp32) / 256 (bf16, K % 8 == 0) / 128 (bf16, K % 4 == 0), K % 4 != 0,
+ * M/heads > 128, or M/heads not a multiple of 16 (fp32) / of 32 and not 16 (bf16).
+ */
+int ga_project_attn(const void *X, const void *W, const float *a_l,
+                    const float *a_r, void *Z, float *el, float *er,
+                    int64_t rows, int64_t K, int64_t M, int64_t heads, int dtype,
+                    ga_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

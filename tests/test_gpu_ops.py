@@ -447,7 +447,7 @@ def test_segment_mm_ops_and_rgcn_layer(device):
     (16, 64, 1, False), (64, 64, 1, False), (16, 16, 8, False), (64, 8, 1, False),
     (12, 48, 2, False), (128, 128, 1, False), (200, 16, 1, False),
     (16, 16, 8, True), (64, 64, 1, True), (32, 32, 4, True), (16, 64, 1, True),
-    (64, 48, 1, True)])
+    (64, 48, 1, True), (32, 32, 3, True), (8, 16, 5, True), (8, 16, 3, False)])
 def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
     """Y[e] = X[endpoint(e)] @ W[type(e)] read through the COO columns, and its
     reduction against a second gathered row; expected values: the oracle's
@@ -610,6 +610,33 @@ def test_linear_attn(device, rows, K, M, heads):
     assert_close(er.cpu().numpy(), (zh * a[1]).sum(-1), 2 * TOL_F32, "linear er")
     z2 = ops.linear_attn(_dev(x, device), _dev(w, device))
     assert np.array_equal(z2.cpu().numpy(), z.cpu().numpy())
+
+
+@pytest.mark.parametrize("rows,K,M,heads,bf16", [
+    (3000, 100, 256, 4, True),      # the larger GAT configuration's first layer (K % 8 != 0)
+    (1500, 256, 256, 4, True),      # ... and its hidden layers
+    (777, 64, 128, 8, True),        # heads of width 16: two per column-block pair
+    (500, 32, 96, 3, True), (129, 8, 32, 1, True), (1, 16, 64, 2, True),
+    (1000, 100, 128, 1, False),     # fp32 head of width 128: tile kernel, not linear.hip
+    (640, 128, 256, 2, False)])
+def test_project_attn_tile_kernel(device, rows, K, M, heads, bf16):
+    """Projection + attention terms through the typed-linear tile kernel (bf16
+    storage, and the fp32 head widths the dedicated fp32 kernel does not take)."""
+    rng = np.random.default_rng(K * 3 + M + heads)
+    x = rng.standard_normal((rows, K), dtype=np.float32)
+    w = datasets.glorot(rng, (K, M))
+    a = rng.standard_normal((2, heads, M // heads), dtype=np.float32)
+    if bf16:
+        x, w = to_bf16_f32(x), to_bf16_f32(w)
+    z, el, er = ops.linear_attn(_dev(x, device, bf16), _dev(w, device, bf16),
+                                _dev(a[0], device), _dev(a[1], device))
+    assert el.dtype == torch.float32 and z.dtype == (torch.bfloat16 if bf16 else torch.float32)
+    zr = x.astype(np.float64) @ w.astype(np.float64)
+    assert_close(z.float().cpu().numpy(), zr, TOL_BF16 if bf16 else TOL_F32, "project z")
+    zh = zr.reshape(rows, heads, -1)
+    # el / er come from the fp32 accumulators, not from the rounded z
+    assert_close(el.cpu().numpy(), (zh * a[0]).sum(-1), 2 * TOL_F32, "project el")
+    assert_close(er.cpu().numpy(), (zh * a[1]).sum(-1), 2 * TOL_F32, "project er")
 
 
 def test_linear_attn_unsupported_shapes(device):
