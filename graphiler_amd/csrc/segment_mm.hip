@@ -68,6 +68,9 @@ struct MmGeom {
   int64_t w_type_stride;  // elements between W[t] and W[t+1]
   int64_t ldw;            // elements between rows k and k+1 of one (K x M) block
   int64_t rows;           // used when there is no type pointer: one type, rows [0, rows)
+  // dense projection wider than one tile: column passes of pass_cols columns
+  // (whole heads of dph columns) inside one launch; n_pass <= 1: a single tile
+  int n_pass, pass_cols, m_total, dph;
 };
 
 // Optional gather / dot-product operands of the exact-shape kernel.
@@ -238,18 +241,18 @@ struct Mma<bf16_t, 16> : MmaBf16Base<16> {
 // Which chunk of which type does this workgroup own?  chunks(t) =
 // ceil(rows_t / chunk_rows); workgroup id -> (t, first row, end row).
 __device__ __forceinline__ bool locate_chunk(const int32_t *__restrict__ tp,
-                                             int n_types, int chunk_rows,
+                                             int n_types, int chunk_rows, int target,
                                              int &type, int &row0, int &row1) {
   __shared__ int scan[kBlock];
   __shared__ int found[3];
   if (!tp) {               // one type; the caller passes the row count as n_types
     type = 0;
-    row0 = blockIdx.x * chunk_rows;
+    if ((int64_t)target * chunk_rows >= n_types) return false;
+    row0 = target * chunk_rows;
     row1 = min(n_types, row0 + chunk_rows);
-    return row0 < n_types;
+    return true;
   }
   if (threadIdx.x == 0) found[0] = -1;
-  const int target = blockIdx.x;
   int base = 0;
   for (int t0 = 0; t0 < n_types; t0 += kBlock) {
     const int t = t0 + threadIdx.x;
@@ -297,7 +300,7 @@ __global__ __launch_bounds__(kBlock) void segment_mm_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   T *tile = reinterpret_cast<T *>(lds_raw);
   int type, row0, row1;
-  if (!locate_chunk(tp, g.n_types, g.chunk_rows, type, row0, row1)) return;
+  if (!locate_chunk(tp, g.n_types, g.chunk_rows, blockIdx.x, type, row0, row1)) return;
   MM::stage(W + (int64_t)type * g.w_type_stride, tile, g);
   __syncthreads();
 
@@ -457,7 +460,26 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   T *tile = reinterpret_cast<T *>(lds_raw);
   int type, row0, row1;
-  if (!locate_chunk(tp, tp ? g.n_types : (int)g.rows, g.chunk_rows, type, row0, row1)) return;
+  int chunk = blockIdx.x;
+  if (g.n_pass > 1) {
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2:
+    // the passes of one row chunk get ids 8 apart, so they run on the same XCD
+    // at about the same time and the later ones find the chunk's rows in its L2.
+    const int group = blockIdx.x / (8 * g.n_pass), within = blockIdx.x % (8 * g.n_pass);
+    const int pass = within >> 3;
+    chunk = group * 8 + (within & 7);
+    const int col0 = pass * g.pass_cols;
+    W += col0;
+    Y += col0;
+    e.a_l += col0;
+    e.a_r += col0;
+    e.el += col0 / g.dph;
+    e.er += col0 / g.dph;
+    g.M = g.Mt = min(g.pass_cols, g.m_total - col0);
+    e.n_heads = g.Mt / g.dph;
+  }
+  if (!locate_chunk(tp, tp ? g.n_types : (int)g.rows, g.chunk_rows, chunk, type, row0, row1))
+    return;
   MM::stage(W + (int64_t)type * g.w_type_stride, tile, g);   // g.KB == NF, g.MB == CG
   __syncthreads();
 
@@ -791,7 +813,7 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
                 int64_t rows, int heads, int K, int M, int h0, int hb,
                 const MmExt &ext, hipStream_t s) {
   typedef Mma<T, KBLK> MM;
-  MmGeom g;
+  MmGeom g = {};
   g.n_types = n_types;
   g.K = K; g.M = M; g.hb = hb;
   g.Kt = hb * K; g.Mt = hb * M;
@@ -934,9 +956,8 @@ namespace ga {
 namespace {
 
 // Z = X @ W for one weight matrix plus el / er = <Z_h, a_l[h]>, <Z_h, a_r[h]>:
-// the exact-shape kernel with a single type, one launch per pass of up to 128
-// output columns (whole heads); X is re-read per pass (from cache for all but
-// the first).
+// the exact-shape kernel with a single type; output columns beyond 128 are
+// covered by further column passes of the same launch (whole heads each).
 template <typename T, int KBLK>
 int launch_dense_attn(const T *X, const T *W, T *Z, const float *a_l, const float *a_r,
                       float *el, float *er, int64_t rows, int K, int M, int heads,
@@ -947,43 +968,46 @@ int launch_dense_attn(const T *X, const T *W, T *Z, const float *a_l, const floa
   if (dph > 128 || (K + KBLK - 1) / KBLK > 8) return GA_EUNSUPPORTED;
   const bool half = paired && dph == 16;
   if (!half && dph % (paired ? 32 : 16) != 0) return GA_EUNSUPPORTED;
-  const int pass = (128 / dph) * dph;              // columns per launch: whole heads
-  for (int col0 = 0; col0 < M; col0 += pass) {
-    const int pw = M - col0 < pass ? M - col0 : pass;
-    MmGeom g;
-    g.n_types = 1;
-    g.K = K; g.M = pw; g.hb = 1;
-    g.Kt = K; g.Mt = pw;
-    g.KB = (K + KBLK - 1) / KBLK;
-    g.MB = (pw + 15) / 16;
-    g.ldx = K;
-    g.ldy = M;
-    g.w_type_stride = 0;
-    g.ldw = M;
-    g.rows = rows;
-    int64_t steps = rows / (kTileBlock * 2048);
-    if (steps < 1) steps = 1;
-    if (steps > 16) steps = 16;
-    g.chunk_rows = (int)steps * kTileBlock;
-    const int64_t grid = (rows + g.chunk_rows - 1) / g.chunk_rows;
-    if (grid > 0x7fffffff) return GA_EUNSUPPORTED;
-    MmExt e = {};
-    e.a_l = a_l + col0;
-    e.a_r = a_r + col0;
-    e.el = el + col0 / dph;
-    e.er = er + col0 / dph;
-    e.ldd = heads;
-    e.n_heads = pw / dph;
-    e.half_heads = half;
-    for (int b = 0; b < 32; ++b) {
-      const int end_col = paired ? ((b >> 1) + 1) * 32 : (b + 1) * 16;
-      if ((!paired || (b & 1)) && end_col % dph == 0) e.head_end |= 1u << b;
-    }
-    const int rc = pick_tight<T, KBLK>(pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), nullptr, X,
-                                       W + col0, Z + col0, g, e, grid, s);
-    if (rc != GA_OK) return rc;     // an unsupported shape fails on the first pass
+  const int pass = (128 / dph) * dph;              // columns per pass: whole heads
+  const int pw = M < pass ? M : pass;              // widest pass fixes the tile shape
+  MmGeom g = {};
+  g.n_types = 1;
+  g.K = K; g.M = pw; g.hb = 1;
+  g.Kt = K; g.Mt = pw;
+  g.KB = (K + KBLK - 1) / KBLK;
+  g.MB = (pw + 15) / 16;
+  g.ldx = K;
+  g.ldy = M;
+  g.w_type_stride = 0;
+  g.ldw = M;
+  g.rows = rows;
+  g.n_pass = (M + pass - 1) / pass;
+  g.pass_cols = pass;
+  g.m_total = M;
+  g.dph = dph;
+  int64_t steps = rows / (kTileBlock * 2048);
+  if (steps < 1) steps = 1;
+  if (steps > 16) steps = 16;
+  g.chunk_rows = (int)steps * kTileBlock;
+  const int64_t chunks = (rows + g.chunk_rows - 1) / g.chunk_rows;
+  // with several passes the chunk count is padded to a multiple of 8 (surplus
+  // workgroups return at once)
+  const int64_t grid = g.n_pass > 1 ? (chunks + 7) / 8 * 8 * g.n_pass : chunks;
+  if (grid > 0x7fffffff) return GA_EUNSUPPORTED;
+  MmExt e = {};
+  e.a_l = a_l;
+  e.a_r = a_r;
+  e.el = el;
+  e.er = er;
+  e.ldd = heads;
+  e.n_heads = pw / dph;
+  e.half_heads = half;
+  for (int b = 0; b < 32; ++b) {
+    const int end_col = paired ? ((b >> 1) + 1) * 32 : (b + 1) * 16;
+    if ((!paired || (b & 1)) && end_col % dph == 0) e.head_end |= 1u << b;
   }
-  return GA_OK;
+  return pick_tight<T, KBLK>(pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), nullptr, X, W, Z, g, e,
+                             grid, s);
 }
 
 }  // namespace

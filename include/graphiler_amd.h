@@ -278,7 +278,7 @@ int ga_linear_attn(const float *X, const float *W, const float *a_l,
  * is rounded): the 100 -> 256 (4 heads x 64, bf16) layer of the larger GAT
  * configuration as one operator instead of three GEMMs.  fp32 with M/heads in
  * {16, 32, 64} runs ga_linear_attn; other cases run the typed-linear tile
- * kernel with a single type, one launch per 128 output columns.  X (rows, K),
+ * kernel with a single type, column passes of 128 inside one launch.  X (rows, K),
  * W (K, M), Z (rows, M) `dtype`; a_l / a_r (heads, M/heads), el / er
  * (rows, heads) fp32, all required.  GA_EUNSUPPORTED (nothing launched) when
  * K > 128 (fp32) / 256 (bf16, K % 8 == 0) / 128 (bf16, K % 4 == 0), K % 4 != 0,
