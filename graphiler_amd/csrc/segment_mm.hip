@@ -1073,10 +1073,10 @@ extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types
   using namespace ga;
   const int bad = check_mm_args(n_types, rows, heads, K, M, dtype);
   if (bad != GA_OK) return bad;
+  if (rows == 0 || n_types == 0) return GA_OK;   // empty results may have no address
   if ((Y != nullptr) == (dot != nullptr)) return GA_EINVAL;   // exactly one result
   if ((Q != nullptr) != (dot != nullptr)) return GA_EINVAL;
   if ((q_index || scale) && !Q) return GA_EINVAL;
-  if (rows == 0 || n_types == 0) return GA_OK;
   if (!type_pointer || !X || !W) return GA_EINVAL;
   const size_t esz = dtype == GA_F32 ? 4 : 2;
   if (!aligned(X, esz) || !aligned(W, esz) || (Y && !aligned(Y, esz)) ||

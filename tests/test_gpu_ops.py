@@ -520,10 +520,16 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
                                         heads, K, M, dt, stream) == 0
         assert_close(Y.float().cpu().numpy(), oracle.segment_mm(tp, Xe, W, heads=heads), tol,
                      "segment_mm_gather identity")
-    # argument errors: both or neither result, dot without Q
-    assert lib.ga_segment_mm_gather(g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(), None,
-                                    dW.data_ptr(), None, None, None, None, None, e, heads, K, M,
-                                    dt, stream) == capi.GA_EINVAL
+    # argument errors: neither result; both results; scale without a dot operand
+    args = (g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(), None, dW.data_ptr())
+    tail = (e, heads, K, M, dt, stream)
+    Y = torch.empty((e, heads * M), dtype=dX.dtype, device=device)
+    D = torch.empty((e, heads), dtype=torch.float32, device=device)
+    assert lib.ga_segment_mm_gather(*args, None, None, None, None, None, *tail) == capi.GA_EINVAL
+    assert lib.ga_segment_mm_gather(*args, Y.data_ptr(), dQ.data_ptr(), None, None,
+                                    D.data_ptr(), *tail) == capi.GA_EINVAL
+    assert lib.ga_segment_mm_gather(*args, Y.data_ptr(), None, None, D.data_ptr(), None,
+                                    *tail) == capi.GA_EINVAL
 
 
 @pytest.mark.parametrize("heads,dim,bf16", [(1, 64, False), (8, 16, True), (4, 5, False),
@@ -559,6 +565,43 @@ def test_edge_softmax_sum(device, heads, dim, bf16):
     got2 = ops.edge_softmax_sum(_dev(logit[order], device), _dev(m[order], device, bf16), g2)
     assert_close(got2.float().cpu().numpy(), ref, TOL_BF16 if bf16 else 2 * TOL_F32,
                  "edge_softmax_sum identity order")
+
+
+@pytest.mark.parametrize("heads,dim", [(1, 64), (4, 8)])
+def test_edge_reductions_on_every_graph(graph, device, heads, dim):
+    """edge_softmax_sum and e_mul_e on the debug graph, the graph without edges,
+    the single busy row, the skewed and the R-MAT graphs."""
+    name, g, arr = graph
+    e, n = int(arr.in_node_indices.shape[0]), arr.num_nodes
+    rng = np.random.default_rng(5)
+    logit = (rng.standard_normal((e, heads)) * 2).astype(np.float32)
+    m = rng.standard_normal((e, heads * dim), dtype=np.float32)
+    got = ops.edge_softmax_sum(_dev(logit, device), _dev(m, device), g)
+    att = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, logit)
+    prod = (m.reshape(e, heads, dim).astype(np.float64) * att[:, :, None]).reshape(e, heads * dim)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      prod.astype(np.float32), op="copy_e")
+    assert got.shape == (n, heads * dim)
+    assert_close(got.cpu().numpy(), ref, 2 * TOL_F32, f"edge_softmax_sum on {name}")
+    w = rng.uniform(0.1, 1.0, (e, 1)).astype(np.float32)
+    got = ops.gspmm_e_mul_e_sum(_dev(m, device), _dev(w, device), g)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      (m * w).astype(np.float32), op="copy_e")
+    assert_close(got.cpu().numpy(), ref, TOL_F32, f"e_mul_e on {name}")
+
+
+def test_fused_typed_products_without_rows(device):
+    """Zero edges / zero rows: the entry points return GA_OK and touch nothing."""
+    g = prepare_graph(np.zeros(0, np.int64), np.zeros(0, np.int64), 9, device=device,
+                      etype_of=np.zeros(0, np.int64), num_etypes=3)
+    x = torch.randn(9, 16, device=device)
+    w = torch.randn(3, 16, 32, device=device)
+    assert ops.SegmentMMEdgeGather(x, w, 0, g).shape == (0, 32)
+    assert ops.SegmentMMEdgeDot(x, w, 0, torch.randn(9, 32, device=device), 1, g).shape == (0, 1)
+    z, el, er = ops.linear_attn(torch.zeros(0, 16, device=device, dtype=torch.bfloat16),
+                                torch.zeros(16, 32, device=device, dtype=torch.bfloat16),
+                                torch.zeros(1, 32, device=device), torch.zeros(1, 32, device=device))
+    assert z.shape == (0, 32) and el.shape == (0, 1) and er.shape == (0, 1)
 
 
 def test_e_mul_e_sum(device):
