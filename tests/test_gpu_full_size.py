@@ -110,6 +110,40 @@ def test_config4_hgt_operators_full(device):
     assert_close(out.float().cpu().numpy(), ref, TOL_BF16, "config 4 u_mul_e")
 
 
+def test_config4_hgt_fused_operators_full(device):
+    """The fused forms at config 4's size (2 M edges, 8 heads x 16, bf16): typed
+    product through the COO column, its dot epilogue with the relation prior,
+    and the softmax-weighted sum of per-edge rows; expected values from the
+    oracle's segment_mm / softmax / copy_e sum on numpy-gathered rows."""
+    wl = datasets.hgt_hetero()
+    n, e, heads, d = wl.num_nodes, wl.num_edges, 8, 16
+    g = prepare_graph(wl.src, wl.dst, n, device=device, ntype_of=wl.ntype,
+                      num_ntypes=4, etype_of=wl.etype, num_etypes=10)
+    ptr, nbr, eid = _host(g)
+    rng = np.random.default_rng(33)
+    k = to_bf16_f32(rng.standard_normal((n, 128), dtype=np.float32))
+    q = to_bf16_f32(rng.standard_normal((n, 128), dtype=np.float32))
+    ratt = to_bf16_f32(datasets.glorot(rng, (10, heads, d, d)))
+    pri = rng.uniform(0.5, 1.5, (10, heads)).astype(np.float32)
+    etp = oracle.type_pointer(wl.etype, 10)
+    ke = oracle.segment_mm(etp, oracle.gather_rows(wl.src, k), ratt, heads=heads)   # fp32, unrounded
+    got = ops.SegmentMMEdgeGather(_t(k, device, True), _t(ratt, device, True), 0, g)
+    assert_close(got.float().cpu().numpy(), ke, TOL_BF16, "config 4 gathered relation transform")
+    want = (ke.reshape(e, heads, d).astype(np.float64) *
+            oracle.gather_rows(wl.dst, q).reshape(e, heads, d)).sum(-1) * pri[wl.etype]
+    score = ops.SegmentMMEdgeDot(_t(k, device, True), _t(ratt, device, True), 0,
+                                 _t(q, device, True), 1, g, scale=_t(pri, device))
+    assert_close(score.cpu().numpy(), want, 2 * TOL_F32, "config 4 attention scores")
+    # reduce tail on the device's own scores (scaled down to softmax range)
+    logits = (want / 8).astype(np.float32)
+    ve = to_bf16_f32(rng.standard_normal((e, 128), dtype=np.float32))
+    att = oracle.segment_softmax(ptr, eid, logits)
+    msg = (ve.reshape(e, heads, d).astype(np.float64) * att[:, :, None]).reshape(e, 128)
+    ref = oracle.spmm(ptr, nbr, eid, msg.astype(np.float32), op="copy_e")
+    out = ops.edge_softmax_sum(_t(logits, device), _t(ve, device, True), g)
+    assert_close(out.float().cpu().numpy(), ref, TOL_BF16, "config 4 softmax-weighted sum")
+
+
 @pytest.mark.timeout(400)
 def test_config5_large_gat_sampled_and_properties(device):
     wl = datasets.gat_rmat_large()               # N=2,449,029  E=64,308,169
