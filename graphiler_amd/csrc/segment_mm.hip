@@ -71,6 +71,9 @@ struct MmGeom {
   // dense projection wider than one tile: column passes of pass_cols columns
   // (whole heads of dph columns) inside one launch; n_pass <= 1: a single tile
   int n_pass, pass_cols, m_total, dph;
+  // dot form: tile column c sits in column block c % 2^perm_shift at lane column
+  // c >> perm_shift, so a lane's columns are adjacent in memory; -1: natural order
+  int perm_shift;
 };
 
 // Optional gather / dot-product operands of the exact-shape kernel.
@@ -84,8 +87,8 @@ struct MmExt {
   const float *a_l, *a_r;   // attention vectors over the tile's columns (kEpiAttn)
   float *el, *er;           // (rows, ldd) fp32
   int n_heads;              // heads inside the tile (kEpiAttn)
-  unsigned head_end;        // bit cb: a head's columns end with column block cb
-  int half_heads;           // bf16, M == 16: a block pair holds two heads
+  unsigned head_end;        // kEpiAttn: bit cb: a head's columns end with column block cb
+  int half_heads;           // kEpiAttn, bf16, head width 16: a block pair holds two heads
 };
 
 // Column of the tile held by lane column j of column block cb.
@@ -129,7 +132,7 @@ struct Mma<float, 16> {          // LDS: [k][col], row stride ws floats
       reinterpret_cast<float4 *>(tile)[i] = make_float4(0, 0, 0, 0);
     __syncthreads();
     const int tx = threadIdx.x & (kWave - 1), ty = threadIdx.x / kWave;
-    const bool vec = (g.M & 3) == 0 && (g.ldw & 3) == 0 &&
+    const bool vec = (g.M & 3) == 0 && (g.ldw & 3) == 0 && g.perm_shift < 0 &&
                      (reinterpret_cast<uintptr_t>(w) & 15) == 0;
     for (int h = 0; h < g.hb; ++h) {
       const float *wh = w + (int64_t)h * g.K * g.ldw;
@@ -143,8 +146,12 @@ struct Mma<float, 16> {          // LDS: [k][col], row stride ws floats
           }
       } else {
         for (int k = ty; k < g.K; k += kBlock / kWave)
-          for (int m = tx; m < g.M; m += kWave)
-            th[k * wsv + m] = wh[(int64_t)k * g.ldw + m];
+          for (int m = tx; m < g.M; m += kWave) {
+            int c = h * g.M + m;                           // tile column
+            if (g.perm_shift >= 0)
+              c = (c & ((1 << g.perm_shift) - 1)) * 16 + (c >> g.perm_shift);
+            tile[(h * g.K + k) * wsv + c] = wh[(int64_t)k * g.ldw + m];
+          }
       }
     }
   }
@@ -181,7 +188,9 @@ struct MmaBf16Base {
           for (int q = 0; q < 8; ++q)
             v[q] = kc + q < g.K ? (uint32_t)wh[(int64_t)(kc + q) * g.ldw + m] : 0u;
           const int c = h * g.M + m;                       // tile column
-          const int lrow = ((c >> 5) * 2 + (c & 1)) * 16 + ((c & 31) >> 1);
+          const int lrow = g.perm_shift >= 0
+                               ? (c & ((1 << g.perm_shift) - 1)) * 16 + (c >> g.perm_shift)
+                               : ((c >> 5) * 2 + (c & 1)) * 16 + ((c & 31) >> 1);
           bf16_t *d = tile + lrow * wsv + h * g.K + kc;
           if (((h * g.K + kc) & 7) == 0) {
             uint4 o;
@@ -535,32 +544,47 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
     if (row >= row1) return 0;
     return qix ? qix[row] : (int64_t)row;
   };
+  // The dot form stages W with its columns permuted (MmGeom::perm_shift): lane
+  // column lr of block cb is tile column lr * CG + cb, so the CG values of Q that
+  // meet this lane's accumulators are adjacent: one or two wide loads per row.
   auto load_q = [&](int64_t qr, bool live, qv_t (&dst)[NQ]) {
-    const T *qrow = Qb + qr * e.ldq;
+    const T *p = Qb + qr * e.ldq + lr * CG;
+    const bool on = live && lr * CG < g.Mt;      // Mt is a multiple of CG
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) {
-      dst[i] = 0;
-      if constexpr (MM::kPaired) {
-        const int m = i * 32 + 2 * lr;                      // even column of the pair
-        if (live && (full_cols || m + 1 < g.Mt))
-          dst[i] = *reinterpret_cast<const uint32_t *>(qrow + m);
+    for (int i = 0; i < NQ; ++i) dst[i] = 0;
+    if (!on) return;
+    if constexpr (MM::kPaired) {
+      if constexpr (CG == 8) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+      } else if constexpr (CG == 4) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(p);
+        dst[0] = v.x; dst[1] = v.y;
       } else {
-        const int m = i * 16 + lr;
-        if (live && (full_cols || m < g.Mt)) dst[i] = ldf(qrow + m);
+        dst[0] = *reinterpret_cast<const uint32_t *>(p);
+      }
+    } else {
+      if constexpr (CG >= 4) {
+#pragma unroll
+        for (int i = 0; i < CG; i += 4) {
+          const float4 v = *reinterpret_cast<const float4 *>(p + i);
+          dst[i] = v.x; dst[i + 1] = v.y; dst[i + 2] = v.z; dst[i + 3] = v.w;
+        }
+      } else if constexpr (CG == 2) {
+        const float2 v = *reinterpret_cast<const float2 *>(p);
+        dst[0] = v.x; dst[1] = v.y;
+      } else {
+        dst[0] = *p;
       }
     }
   };
-  // per-head factors of this chunk's type, read once: a load inside the tile
-  // loop would make every tile wait for the prefetches issued before it
-  float scv[CG];
-#pragma unroll
-  for (int i = 0; i < CG; ++i) {
-    scv[i] = 1.0f;
-    if (DOT && e.scale) {
-      const int h = e.half_heads ? i * 2 + (lr >> 3) : i;
-      if (h < g.hb) scv[i] = e.scale[(int64_t)type * e.ldd + h];
-    }
-  }
+  // lanes per head, the head of this lane and its factor for this chunk's type
+  // (read once: a load inside the tile loop would make every tile wait for the
+  // prefetches issued before it)
+  const int lph = DOT ? g.M / CG : 1;
+  const int my_head = lr / lph;
+  float my_scale = 1.0f;
+  if (DOT && e.scale && my_head < g.hb) my_scale = e.scale[(int64_t)type * e.ldd + my_head];
   // attention vectors at this lane's column of every block (0 beyond the tile)
   float alv[CG], arv[CG];
 #pragma unroll
@@ -628,40 +652,23 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int row = tile0 + lk * 4 + r;
-        const bool live = row < row1;          // uniform over the 16 lanes of a row
-        float *drow = e.dot + (int64_t)row * e.ldd;
-        float s = 0.0f;
-        int head = 0;
-        if constexpr (MM::kPaired) {
+        float v = 0.0f;
 #pragma unroll
-          for (int cb = 0; cb < CG; cb += 2) {
-            const uint32_t qv = qa[r][cb >> 1];
-            s = fmaf(acc[cb][r], bf16_lo(qv), s);
-            s = fmaf(acc[cb + 1 < CG ? cb + 1 : cb][r], bf16_hi(qv), s);
-            if (e.half_heads) {                  // lanes 0-7: one head, 8-15: the next
-              const float t = row8_sum(s);
-              const int h = (cb >> 1) * 2 + (lr >> 3);
-              if (live && (lr & 7) == 0 && h < g.hb) drow[h] = t * scv[cb >> 1];
-              s = 0.0f;
-            } else if (e.head_end >> (cb + 1) & 1) {
-              const float t = row16_sum(s);
-              if (live && lr == 0 && head < g.hb) drow[head] = t * scv[head < CG ? head : 0];
-              ++head;
-              s = 0.0f;
-            }
-          }
-        } else {
-#pragma unroll
-          for (int cb = 0; cb < CG; ++cb) {
-            s = fmaf(acc[cb][r], qa[r][cb], s);
-            if (e.head_end >> cb & 1) {
-              const float t = row16_sum(s);
-              if (live && lr == 0 && head < g.hb) drow[head] = t * scv[head < CG ? head : 0];
-              ++head;
-              s = 0.0f;
-            }
-          }
+        for (int cb = 0; cb < CG; ++cb) {
+          float qf;
+          if constexpr (MM::kPaired)
+            qf = (cb & 1) ? bf16_hi(qa[r][cb >> 1]) : bf16_lo(qa[r][cb >> 1]);
+          else
+            qf = qa[r][cb];
+          v = fmaf(acc[cb][r], qf, v);
         }
+        // sum over the lanes of the head (a power of two, at most the 16 of a row)
+        if (lph >= 2) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
+        if (lph >= 4) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));
+        if (lph >= 8) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));
+        if (lph >= 16) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));
+        if (row < row1 && (lr & (lph - 1)) == 0 && my_head < g.hb)
+          e.dot[(int64_t)row * e.ldd + my_head] = v * my_scale;
       }
       continue;
     }
@@ -824,6 +831,7 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
   g.w_type_stride = (int64_t)heads * K * M;
   g.ldw = M;
   g.rows = rows;
+  g.perm_shift = -1;
   // rows per workgroup: a multiple of the 64-row step, large enough to
   // amortise the weight staging, small enough to keep every CU busy
   int64_t steps = rows / (kTileBlock * 2048);
@@ -840,19 +848,16 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
     if (g.KB <= 8 && g.MB <= 8) {
       MmExt e = ext;
       if (e.Q) {
-        // heads must end on column-block (fp32) / block-pair (bf16) boundaries,
-        // or be exactly half a pair
-        constexpr bool paired = Mma<T, KBLK>::kPaired;
-        e.half_heads = paired && M == 16;
-        if (!e.half_heads && M % (paired ? 32 : 16) != 0) return GA_EUNSUPPORTED;
+        // a head must cover a power-of-two number of lane columns: with the
+        // permuted tile lane column j holds columns [j * CG, (j + 1) * CG)
+        int cg = pow2_ceil_int(g.MB);
+        if (Mma<T, KBLK>::kPaired && cg < 2) cg = 2;
+        const int lph = M / cg;
+        if (M % cg != 0 || lph > 16 || (lph & (lph - 1)) != 0) return GA_EUNSUPPORTED;
+        g.perm_shift = ilog2_floor((uint64_t)cg);
         e.Q = static_cast<const T *>(ext.Q) + (int64_t)h0 * M;
         e.dot = ext.dot + h0;
         if (e.scale) e.scale = ext.scale + h0;
-        e.head_end = 0;
-        for (int b = 0; b < 32; ++b) {
-          const int end_col = paired ? ((b >> 1) + 1) * 32 : (b + 1) * 16;
-          if ((!paired || (b & 1)) && end_col % M == 0) e.head_end |= 1u << b;
-        }
       }
       const int rc = pick_tight<T, KBLK>(pow2_ceil_int(g.KB), pow2_ceil_int(g.MB), tp, Xh,
                                          Wh, Yh, g, e, grid, s);
@@ -985,6 +990,7 @@ int launch_dense_attn(const T *X, const T *W, T *Z, const float *a_l, const floa
   g.pass_cols = pass;
   g.m_total = M;
   g.dph = dph;
+  g.perm_shift = -1;
   int64_t steps = rows / (kTileBlock * 2048);
   if (steps < 1) steps = 1;
   if (steps > 16) steps = 16;

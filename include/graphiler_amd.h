@@ -203,8 +203,10 @@ int ga_segment_mm(const int32_t *type_pointer, int64_t n_types, const void *X,
  * x_index / q_index are int64 (the COO columns of the graph); entries are not
  * checked on the device.  Returns GA_EUNSUPPORTED, having launched nothing, for
  * shapes outside the matrix-core tile (heads*K > 128 fp32 / 256 bf16,
- * heads*M > 128, K % 4 (fp32) or K % 8 (bf16) != 0; for dot also M % 16 (fp32),
- * M % 32 and M != 16 (bf16)); the caller then gathers with ga_gather_rows.
+ * heads*M > 128, K % 4 (fp32) or K % 8 (bf16) != 0; for dot also a head width M
+ * that is not c, 2c, 4c, 8c or 16c with c = ceil(heads*M / 16) rounded up to a
+ * power of two (at least 2 for bf16)); the caller then gathers with
+ * ga_gather_rows.
  */
 int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types, const void *X,
                          const int64_t *x_index, const void *W, void *Y,

@@ -451,9 +451,10 @@ def test_segment_mm_ops_and_rgcn_layer(device):
 def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
     """Y[e] = X[endpoint(e)] @ W[type(e)] read through the COO columns, and its
     reduction against a second gathered row; expected values: the oracle's
-    segment_mm on numpy-gathered rows and a float64 einsum.  (64, 8), (200, 16)
-    and bf16 (64, 48) fall outside the fused kernel's shapes: the entry point
-    must say so and the operator wrapper must still give the result."""
+    segment_mm on numpy-gathered rows and a float64 einsum.  (200, 16) falls outside
+    the fused kernel's shapes and (12, 48, 2 heads) / bf16 (64, 48) outside the dot
+    form's: the entry point must say so and the operator wrapper must still give the
+    result."""
     rng = np.random.default_rng(K * 131 + M * 7 + heads + 1000 * bf16)
     counts = [70, 0, 1, 333, 0, 64, 15, 129, 2001, 0]
     n_nodes, n_rel = 500, len(counts)
@@ -475,7 +476,9 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
     dt = capi.GA_BF16 if bf16 else capi.GA_F32
     kb = 32 if bf16 else 16
     fits = heads * K <= 8 * kb and heads * M <= 128 and K % (8 if bf16 else 4) == 0
-    dot_fits = fits and (M % 16 == 0 if not bf16 else (M % 32 == 0 or M == 16))
+    blocks = -(-heads * M // 16)
+    cg = max(1 << (blocks - 1).bit_length(), 2 if bf16 else 1)     # column blocks, power of two
+    dot_fits = fits and M % cg == 0 and M // cg in (1, 2, 4, 8, 16)
     for which, col in ((0, src), (1, dst)):
         ref = oracle.segment_mm(tp, X[col], W, heads=heads)
         Y = torch.full((e, heads * M), float("nan"), dtype=dX.dtype, device=device)
