@@ -553,28 +553,30 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
 #pragma unroll
     for (int i = 0; i < NQ; ++i) dst[i] = 0;
     if (!on) return;
-    if constexpr (MM::kPaired) {
-      if constexpr (CG == 8) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(p);
-        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
-      } else if constexpr (CG == 4) {
-        const uint2 v = *reinterpret_cast<const uint2 *>(p);
-        dst[0] = v.x; dst[1] = v.y;
-      } else {
-        dst[0] = *reinterpret_cast<const uint32_t *>(p);
-      }
-    } else {
-      if constexpr (CG >= 4) {
-#pragma unroll
-        for (int i = 0; i < CG; i += 4) {
-          const float4 v = *reinterpret_cast<const float4 *>(p + i);
-          dst[i] = v.x; dst[i + 1] = v.y; dst[i + 2] = v.z; dst[i + 3] = v.w;
+    if constexpr (DOT) {
+      if constexpr (MM::kPaired) {
+        if constexpr (CG == 8) {
+          const uint4 v = *reinterpret_cast<const uint4 *>(p);
+          dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+        } else if constexpr (CG == 4) {
+          const uint2 v = *reinterpret_cast<const uint2 *>(p);
+          dst[0] = v.x; dst[1] = v.y;
+        } else {
+          dst[0] = *reinterpret_cast<const uint32_t *>(p);
         }
-      } else if constexpr (CG == 2) {
-        const float2 v = *reinterpret_cast<const float2 *>(p);
-        dst[0] = v.x; dst[1] = v.y;
       } else {
-        dst[0] = *p;
+        if constexpr (CG >= 4) {
+#pragma unroll
+          for (int i = 0; i < CG; i += 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(p + i);
+            dst[i] = v.x; dst[i + 1] = v.y; dst[i + 2] = v.z; dst[i + 3] = v.w;
+          }
+        } else if constexpr (CG == 2) {
+          const float2 v = *reinterpret_cast<const float2 *>(p);
+          dst[0] = v.x; dst[1] = v.y;
+        } else {
+          dst[0] = *p;
+        }
       }
     }
   };
