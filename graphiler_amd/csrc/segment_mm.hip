@@ -709,6 +709,41 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
         }
       }
     }
+    if (EPI == kEpiStore && g.perm_shift >= 0) {
+      // permuted tile: this lane holds columns [lr * CG, (lr + 1) * CG) of its four
+      // rows, so a row leaves as one vector store per lane (a whole 256-byte row
+      // per 16 lanes at CG = 8 bf16 / CG = 4 fp32)
+      if (lr * CG < g.Mt) {                        // Mt is a multiple of CG
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (tile0 + lk * 4 + r >= row1) continue;
+          T *yw = yp + (int64_t)r * g.ldy - (MM::kPaired ? 2 * lr : lr) + lr * CG;
+          if constexpr (MM::kPaired) {
+            uint32_t pk[CG / 2];
+#pragma unroll
+            for (int i = 0; i < CG / 2; ++i) pk[i] = pack_bf16(acc[2 * i][r], acc[2 * i + 1][r]);
+            if constexpr (CG == 8)
+              *reinterpret_cast<uint4 *>(yw) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            else if constexpr (CG == 4)
+              *reinterpret_cast<uint2 *>(yw) = make_uint2(pk[0], pk[1]);
+            else
+              *reinterpret_cast<uint32_t *>(yw) = pk[0];
+          } else {
+            if constexpr (CG >= 4) {
+#pragma unroll
+              for (int i = 0; i < CG; i += 4)
+                *reinterpret_cast<float4 *>(yw + i) =
+                    make_float4(acc[i][r], acc[i + 1][r], acc[i + 2][r], acc[i + 3][r]);
+            } else if constexpr (CG == 2) {
+              *reinterpret_cast<float2 *>(yw) = make_float2(acc[0][r], acc[1][r]);
+            } else {
+              *yw = acc[0][r];
+            }
+          }
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       if (tile0 + lk * 4 + r < row1) {
@@ -849,11 +884,15 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
   {
     if (g.KB <= 8 && g.MB <= 8) {
       MmExt e = ext;
+      int cg = pow2_ceil_int(g.MB);        // column blocks of the tile as compiled
+      if (Mma<T, KBLK>::kPaired && cg < 2) cg = 2;
+      // stores: with the permuted tile (lane column j holds columns
+      // [j * cg, (j + 1) * cg)) a lane writes its part of a row as one vector
+      if (!e.Q && !e.a_l && g.Mt % cg == 0 && (g.ldy % cg) == 0 &&
+          aligned(Yh, (size_t)cg * sizeof(T)))
+        g.perm_shift = ilog2_floor((uint64_t)cg);
       if (e.Q) {
-        // a head must cover a power-of-two number of lane columns: with the
-        // permuted tile lane column j holds columns [j * CG, (j + 1) * CG)
-        int cg = pow2_ceil_int(g.MB);
-        if (Mma<T, KBLK>::kPaired && cg < 2) cg = 2;
+        // a head must cover a power-of-two number of lane columns
         const int lph = M / cg;
         if (M % cg != 0 || lph > 16 || (lph & (lph - 1)) != 0) return GA_EUNSUPPORTED;
         g.perm_shift = ilog2_floor((uint64_t)cg);
