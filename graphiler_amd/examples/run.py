@@ -24,6 +24,7 @@ import numpy as np
 import torch
 
 from .. import datasets, prepare_graph
+from ..hipgraph import Graphed
 from ..mpdfg import GraphData
 from ..report import (bench, check_equal, empty_cache, init_log, mark_unavailable,
                       save_logs)
@@ -133,9 +134,11 @@ def profile(model: str, dataset: str, feat_dim: int, repeat: int = 1000, device=
 
 def breakdown(model: str, dataset: str, feat_dim: int, repeat: int = 1000, device="cuda:0"):
     """examples/GAT/GAT.py:140-163: the eager baseline, then the plan at
-    optimisation levels 0, 1 and 2; every level is checked against the eager
-    network evaluated with float64 sums."""
-    log = init_log(["0-" + EAGER_TAG, "1+compile", "2+reorder", "3+fusion"], ["time", "mem"])
+    optimisation levels 0, 1 and 2 and the level-2 network replayed as a HIP
+    graph; every result is checked against the eager network evaluated with
+    float64 sums."""
+    log = init_log(["0-" + EAGER_TAG, "1+compile", "2+reorder", "3+fusion", "4+hipgraph"],
+                   ["time", "mem"])
     print("benchmarking on: " + dataset)
     torch.cuda.empty_cache()
     g, feats = load_data(dataset, feat_dim, device)
@@ -148,6 +151,11 @@ def breakdown(model: str, dataset: str, feat_dim: int, repeat: int = 1000, devic
             res = bench(net, (g, feats) + extra + (level,), tag=tag, repeat=repeat,
                         memory=True, log=log)
             check_equal(res, base)
+        # the level-2 network recorded once and replayed as a single HIP graph
+        # (memory of a replay is the graph's own pool, held since the recording)
+        graphed = Graphed(net, (g, feats) + extra + (2,))
+        res = bench(graphed, (), tag="4+hipgraph", repeat=repeat, memory=False, log=log)
+        check_equal(res, base)
     return log
 
 
