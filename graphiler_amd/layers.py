@@ -5,15 +5,16 @@ TorchScript graph of ``my_ops::*`` nodes (python/graphiler/mpdfg_builder.py:35-7
 src/optimizer/fusion.cpp:15-145) and executes it in ``update_all``
 (python/graphiler/update_all.py:1-5).  The functions below are those
 opt-level-2 operator sequences written out by hand for the four example models,
-calling :mod:`graphiler_amd.ops`; dense per-node linears stay on ``torch.mm``
-exactly as in the reference plans.
+calling :mod:`graphiler_amd.ops`; the GAT projection uses the kernel that also
+produces the attention terms, other dense per-node linears stay on ``torch.mm``
+as in the reference plans.
 """
 from __future__ import annotations
 
 import torch
 import torch.nn.functional as F
 
-from . import ops
+from . import capi, ops
 from .graph import DGLGraph
 
 
@@ -32,7 +33,6 @@ def gcn_layer(g: DGLGraph, h: torch.Tensor, weight: torch.Tensor,
 def gat_project(h, fc_weight, attn_weight, heads: int = 1):
     """Dense part of the GAT plan (GAT.py:25-29 after the split and reorder
     passes): z = h @ W, el = <z, a_l>, er = <z, a_r> per head."""
-    from . import capi
     try:        # one kernel: the GEMM with the attention terms in its epilogue
         return ops.linear_attn(h, fc_weight, attn_weight[0].float().contiguous(),
                                attn_weight[1].float().contiguous())
