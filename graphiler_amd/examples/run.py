@@ -26,7 +26,7 @@ import torch
 from .. import datasets, prepare_graph
 from ..hipgraph import Graphed
 from ..mpdfg import GraphData
-from ..report import (bench, check_equal, empty_cache, init_log, mark_unavailable,
+from ..report import (is_out_of_memory, bench, check_equal, empty_cache, init_log, mark_unavailable,
                       save_logs)
 from . import models
 
@@ -101,7 +101,7 @@ def _expected(net, params):
     try:
         return net(*params, "eager64")
     except RuntimeError as err:
-        if "out of memory" not in str(err).lower():
+        if not is_out_of_memory(err):
             raise
         torch.cuda.empty_cache()
         return None

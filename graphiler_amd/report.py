@@ -35,48 +35,63 @@ def check_equal(first, second, rtol: float = 1e-3) -> bool:
     return True
 
 
+WARM_UP_CALLS = 5
+
+
+def is_out_of_memory(err: RuntimeError) -> bool:
+    # torch.cuda.OutOfMemoryError is a RuntimeError; raised inside a TorchScript
+    # plan it arrives as a plain RuntimeError with the same text
+    return "out of memory" in str(err).lower()
+
+
+def _timed_calls(net: Callable, params: tuple, repeat: int, mark_range: bool):
+    """``repeat`` back-to-back calls between two device synchronisations;
+    returns (last result, wall-clock milliseconds per call)."""
+    result = None
+    if mark_range:
+        torch.cuda.profiler.start()
+    t0 = time.perf_counter()
+    for _ in range(repeat):
+        result = net(*params)
+    torch.cuda.synchronize()
+    per_call_ms = (time.perf_counter() - t0) * 1e3 / max(repeat, 1)
+    if mark_range:
+        torch.cuda.profiler.stop()
+    return result, per_call_ms
+
+
 def bench(net: Callable, net_params: Iterable, tag: str = "", nvprof: bool = False,
           memory: bool = False, repeat: int = 1000, log: Optional[pd.Series] = None):
-    """bench.py:19-49: five warm-up calls, ``repeat`` timed calls between two
-    device synchronisations, wall clock per call in ms into ``log[tag, "time"]``;
-    with ``memory`` the peak of newly allocated device memory in MiB into
-    ``log[tag, "mem"]``.  ``nvprof`` brackets the timed loop with the profiler's
-    start / stop marks (a range for rocprofv3's marker trace).  Out of memory
-    prints "<tag> OOM", leaves the log entries at 0 and returns None."""
-    net_params = tuple(net_params)
+    """Same contract as bench.py:19-49: five warm-up calls, ``repeat`` timed calls
+    between two device synchronisations, wall clock per call in ms into
+    ``log[tag, "time"]``; with ``memory`` the peak of newly allocated device
+    memory in MiB into ``log[tag, "mem"]``.  ``nvprof`` brackets the timed loop
+    with the profiler's start / stop marks (a range for rocprofv3's marker trace).
+    Out of memory prints "<tag> OOM", leaves the log entries at 0 and returns
+    None; any other error propagates."""
+    params = tuple(net_params)
     try:
-        for _ in range(5):
-            net(*net_params)
+        for _ in range(WARM_UP_CALLS):
+            net(*params)
         torch.cuda.synchronize()
-        offset = torch.cuda.memory_allocated()
+        baseline_bytes = torch.cuda.memory_allocated()
         torch.cuda.reset_peak_memory_stats()
-        if nvprof:
-            torch.cuda.profiler.start()
-        start = time.time()
-        logits = None
-        for _ in range(repeat):
-            logits = net(*net_params)
-        torch.cuda.synchronize()
-        if nvprof:
-            torch.cuda.profiler.stop()
-        elapsed = (time.time() - start) / repeat * 1000
-        print("{} elapsed time: {} ms/infer".format(tag, elapsed))
-        if log is not None:
-            log.at[(tag, "time")] = elapsed
-        if memory:
-            used = (torch.cuda.max_memory_allocated() - offset) / 1048576
-            print("intermediate data memory usage: {} MB".format(used))
-            if log is not None:
-                log.at[(tag, "mem")] = used
+        result, per_call_ms = _timed_calls(net, params, repeat, nvprof)
     except RuntimeError as err:
-        # torch.cuda.OutOfMemoryError is a RuntimeError; raised inside a
-        # TorchScript plan it arrives as a plain RuntimeError with the same text
-        if "out of memory" not in str(err).lower():
+        if not is_out_of_memory(err):
             raise
         print("{} OOM".format(tag))
         torch.cuda.empty_cache()
         return None
-    return logits
+    print("{} elapsed time: {} ms/infer".format(tag, per_call_ms))
+    if log is not None:
+        log.at[(tag, "time")] = per_call_ms
+    if memory:
+        peak_mib = (torch.cuda.max_memory_allocated() - baseline_bytes) / 2 ** 20
+        print("intermediate data memory usage: {} MB".format(peak_mib))
+        if log is not None:
+            log.at[(tag, "mem")] = peak_mib
+    return result
 
 
 def init_log(tags, metrics) -> pd.Series:
