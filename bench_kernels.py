@@ -167,6 +167,10 @@ def main():
         z, el, er = rnd(N, F, dtype=dt), rnd(N, H), rnd(N, H)
         report("c5", "gat_aggregate H=4 F=256 bf16", lambda: ops.gat_aggregate(el, er, z, g, 0.2),
                4 * (N + 1) + E * (4 + H * 4 + F * b) + N * (H * 4 + F * b))
+        a_l = rnd(H, F // H) / 8
+        report("c5", "gat_aggregate, source term from z, H=4 F=256 bf16",
+               lambda: ops.gat_aggregate_from_z(a_l, er, z, g, 0.2),
+               4 * (N + 1) + E * (4 + F * b) + N * (H * 4 + F * b))
         a = torch.rand(E, H, device=dev)
         report("c5", "spmm u_mul_e H=4 F=256 bf16",
                lambda: ops.gspmm_src_mul_e_sum(z, a, [1], False, None, g),

@@ -54,6 +54,8 @@ SIGNATURES = {
     "ga_project_attn": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                                _i64, _int, _vp]),
     "ga_gat_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "ga_gat_aggregate_from_z": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+                                       _i64, _i64, ctypes.c_float, _int, _vp, _sz, _vp]),
     "ga_edge_softmax_sum": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                    _int, _vp, _sz, _vp]),
     "ga_gat_aggregate": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,

@@ -24,20 +24,40 @@ __device__ __forceinline__ float leaky(float t, float slope) {
 
 // State per lane: VEC un-normalised weighted sums, then the running maximum m
 // and the running denominator l of the lane's head.
-template <typename T, int VEC, bool EDGE = false>
+// MODE selects where the logits come from:
+//   kGatNode  el[src] + er[dst] through leaky_relu (the GAT chain),
+//   kGatEdge  given per edge (EDGE operands, see the header comment),
+//   kGatFromZ <z[src, h, :], a_l[h, :]> + er[dst] through leaky_relu: the source
+//             term is recomputed from the row that is gathered anyway instead of
+//             being gathered itself -- a separate (N, heads) table costs one more
+//             memory sector per edge once it no longer fits the caches.
+constexpr int kGatNode = 0, kGatEdge = 1, kGatFromZ = 2;
+
+// Sum over `lanes` adjacent lanes (a power of two <= 16, aligned), in every lane.
+__device__ __forceinline__ float lanes_sum(float v, int lanes) {
+  if (lanes >= 2) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
+  if (lanes >= 4) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));
+  if (lanes >= 8) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));
+  if (lanes >= 16) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));
+  return v;
+}
+
+template <typename T, int VEC, int MODE = kGatNode>
 struct GatPolicy {
+  static constexpr bool EDGE = MODE == kGatEdge;
   typedef T out_t;
   static constexpr int kVec = VEC;
   static constexpr int kState = VEC + 2;
   struct Args {
-    const int32_t *nbr;   // EDGE: the edge-id column, or null when slot = edge id
-    const float *el;      // EDGE: per-edge logits (E, heads)
-    const float *er;      // EDGE: unused
-    const T *z;           // EDGE: per-edge rows (E, heads*dph)
+    const int32_t *nbr;   // kGatEdge: the edge-id column, or null when slot = edge id
+    const float *el;      // kGatEdge: per-edge logits (E, heads); kGatFromZ: a_l (heads*dph)
+    const float *er;      // kGatEdge: unused
+    const T *z;           // kGatEdge: per-edge rows (E, heads*dph)
     int heads;
     int dph;
     float slope;
     bool ids_vec;   // row_of_slot and nbr are 16-byte aligned
+    int head_lanes; // kGatFromZ: lanes that share a head (dph / VEC)
   };
   static __device__ __forceinline__ void init(float (&st)[VEC + 2]) {
 #pragma unroll
@@ -79,6 +99,9 @@ struct GatPolicy {
                                               Close &&close_segment) {
     typedef Frag<T, VEC> IO;
     const int h = f0 / A.dph;
+    float al[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) al[v] = MODE == kGatFromZ ? A.el[f0 + v] : 0.0f;
     for (int64_t j = a; j < b; j += kUnroll) {
       int r[kUnroll], g[kUnroll];
       float s[kUnroll];
@@ -93,11 +116,25 @@ struct GatPolicy {
 #pragma unroll
       for (int t = 0; t < kUnroll; ++t) {
         x[t] = IO::load(A.z + (int64_t)g[t] * feat + f0);
-        if constexpr (EDGE)
+        if constexpr (MODE == kGatEdge)
           s[t] = A.el[(int64_t)g[t] * A.heads + h];
-        else
+        else if constexpr (MODE == kGatNode)
           s[t] = leaky(A.el[(int64_t)g[t] * A.heads + h] + A.er[(int64_t)r[t] * A.heads + h],
                        A.slope);
+        else
+          s[t] = A.er[(int64_t)r[t] * A.heads + h];
+      }
+      if constexpr (MODE == kGatFromZ) {
+        // every live lane of a head runs this together (heads tile the row)
+#pragma unroll
+        for (int t = 0; t < kUnroll; ++t) {
+          float xf[VEC];
+          IO::widen(x[t], xf);
+          float d = 0.0f;
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) d = fmaf(xf[v], al[v], d);
+          s[t] = leaky(lanes_sum(d, A.head_lanes) + s[t], A.slope);
+        }
       }
       const bool one_row = j + kUnroll <= b && r[0] == cur && r[kUnroll - 1] == cur;
       if (one_row) {
@@ -145,14 +182,18 @@ struct GatPolicy {
   }
 };
 
-template <typename T, int VEC, bool EDGE = false>
+template <typename T, int VEC, int MODE = kGatNode>
 int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const int32_t *nbr, const float *el, const float *er,
                const void *z, void *out, int64_t n_rows, int64_t n_edges,
                int heads, int dim, float slope, float *ws, hipStream_t stream) {
-  typedef GatPolicy<T, VEC, EDGE> P;
+  typedef GatPolicy<T, VEC, MODE> P;
   const bool ids_vec = aligned(row_of_slot, 16) && (!nbr || aligned(nbr, 16));
-  typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec};
+  const int head_lanes = dim / VEC;
+  if (MODE == kGatFromZ &&
+      (dim % VEC != 0 || head_lanes > 16 || (head_lanes & (head_lanes - 1)) != 0))
+    return GA_EUNSUPPORTED;
+  typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec, head_lanes};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges,
                         heads * dim, ws, stream);
 }
@@ -241,16 +282,56 @@ int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,
   const int h = (int)heads, d = (int)dim;
   if (dtype == GA_F32) {
     if (vec_ok && dim % 4 == 0)
-      return ga::launch_gat<float, 4, true>(pointer, row_of_slot, eid, logit, nullptr, m,
+      return ga::launch_gat<float, 4, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m,
                                             out, n_rows, n_edges, h, d, 0.0f, ws, s);
-    return ga::launch_gat<float, 1, true>(pointer, row_of_slot, eid, logit, nullptr, m, out,
+    return ga::launch_gat<float, 1, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m, out,
                                           n_rows, n_edges, h, d, 0.0f, ws, s);
   }
   if (vec_ok && dim % 8 == 0)
-    return ga::launch_gat<ga::bf16_t, 8, true>(pointer, row_of_slot, eid, logit, nullptr, m,
+    return ga::launch_gat<ga::bf16_t, 8, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m,
                                                out, n_rows, n_edges, h, d, 0.0f, ws, s);
-  return ga::launch_gat<ga::bf16_t, 1, true>(pointer, row_of_slot, eid, logit, nullptr, m,
+  return ga::launch_gat<ga::bf16_t, 1, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m,
                                              out, n_rows, n_edges, h, d, 0.0f, ws, s);
+}
+
+int ga_gat_aggregate_from_z(const int32_t *pointer, const int32_t *row_of_slot,
+                            const int32_t *nbr, const float *a_l, const float *er,
+                            const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                            int64_t heads, int64_t dim, float slope, int dtype,
+                            void *workspace, size_t workspace_bytes, ga_stream_t stream) {
+  if (n_rows < 0 || n_edges < 0 || heads <= 0 || dim <= 0) return GA_EINVAL;
+  if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || heads * dim > 0x7fffffff)
+    return GA_EINVAL;
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  if (n_rows == 0) return GA_OK;
+  if (!pointer || !out) return GA_EINVAL;
+  const int64_t feat = heads * dim;
+  if (n_edges > 0) {
+    if (!row_of_slot || !nbr || !a_l || !er || !z) return GA_EINVAL;
+    if (!workspace || !ga::aligned(workspace, 16) ||
+        ga_gat_workspace_bytes(n_edges, feat, heads) > workspace_bytes)
+      return GA_EWORKSPACE;
+  }
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!ga::aligned(out, esz) || (z && !ga::aligned(z, esz)) ||
+      (a_l && !ga::aligned(a_l, 4)) || (er && !ga::aligned(er, 4)))
+    return GA_EALIGN;
+  const bool vec_ok = ga::aligned(out, 16) && (!z || ga::aligned(z, 16));
+  hipStream_t s = (hipStream_t)stream;
+  float *ws = (float *)workspace;
+  const int h = (int)heads, d = (int)dim;
+  if (dtype == GA_F32) {
+    if (vec_ok && dim % 4 == 0)
+      return ga::launch_gat<float, 4, ga::kGatFromZ>(pointer, row_of_slot, nbr, a_l, er, z, out,
+                                                     n_rows, n_edges, h, d, slope, ws, s);
+    return ga::launch_gat<float, 1, ga::kGatFromZ>(pointer, row_of_slot, nbr, a_l, er, z, out,
+                                                   n_rows, n_edges, h, d, slope, ws, s);
+  }
+  if (vec_ok && dim % 8 == 0)
+    return ga::launch_gat<ga::bf16_t, 8, ga::kGatFromZ>(pointer, row_of_slot, nbr, a_l, er, z,
+                                                        out, n_rows, n_edges, h, d, slope, ws, s);
+  return ga::launch_gat<ga::bf16_t, 1, ga::kGatFromZ>(pointer, row_of_slot, nbr, a_l, er, z, out,
+                                                      n_rows, n_edges, h, d, slope, ws, s);
 }
 
 }  // extern "C"

@@ -56,6 +56,12 @@ def _head_blocks(a: torch.Tensor) -> torch.Tensor:
     return m
 
 
+# An (N, heads) fp32 table above this size (about what the 8 x 4 MB L2s hold
+# besides the feature rows) makes the separate gather of the source term cost a
+# memory sector per edge; measured: no difference at 0.9 MB, 17 % at 39 MB.
+SOURCE_TERM_TABLE_LIMIT = 16 << 20
+
+
 def gat_aggregate_plan(g: DGLGraph, z, el, er, negative_slope: float = 0.01):
     """The four graph operators of the reference's GAT plan, one after another."""
     e = ops.gsddmm_u_add_v_mul_alpha(el, er, 1, g)
@@ -66,10 +72,20 @@ def gat_aggregate_plan(g: DGLGraph, z, el, er, negative_slope: float = 0.01):
 
 def gat_layer(g: DGLGraph, h, fc_weight, attn_weight, heads: int = 1,
               negative_slope: float = 0.01, fused: bool = True):
-    """One GAT layer forward; ``fused`` runs the chain as a single pass."""
+    """One GAT layer forward; ``fused`` runs the chain as a single pass.  When
+    the (N, heads) table of source terms is too large to stay cached
+    (``SOURCE_TERM_TABLE_LIMIT`` bytes), the pass recomputes them from the
+    gathered rows instead of gathering them as well."""
     z, el, er = gat_project(h, fc_weight, attn_weight, heads)
     if fused:
-        return ops.gat_aggregate(el, er, z, g, negative_slope)
+        if el.numel() * el.element_size() >= SOURCE_TERM_TABLE_LIMIT:
+            try:
+                return ops.gat_aggregate_from_z(attn_weight[0].float().contiguous(), er.float(),
+                                                z, g, negative_slope)
+            except capi.GraphilerError as err:      # head width the variant does not take
+                if err.code != capi.GA_EUNSUPPORTED:
+                    raise
+        return ops.gat_aggregate(el.float(), er.float(), z, g, negative_slope)
     return gat_aggregate_plan(g, z, el, er, negative_slope)
 
 

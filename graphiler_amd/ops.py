@@ -487,6 +487,33 @@ def gat_aggregate(el, er, z, graph: DGLGraph, negative_slope: float = 0.01):
     return out
 
 
+def gat_aggregate_from_z(a_l, er, z, graph: DGLGraph, negative_slope: float = 0.01):
+    """``gat_aggregate`` with the source term recomputed from the gathered row:
+    logits leaky_relu(<z[src, h], a_l[h]> + er[dst, h]).  a_l: (H, D) fp32;
+    er: (N, H) fp32; z: (N, H*D).  For node counts whose (N, H) table of source
+    terms no longer fits the caches this saves one memory sector per edge."""
+    _check_input(a_l, "a_l")
+    _check_input(er, "er")
+    _check_input(z, "z")
+    dt = _feat_dtype(z, "z")
+    if a_l.dtype != torch.float32 or er.dtype != torch.float32:
+        raise RuntimeError("a_l and er must be float32")
+    heads = get_feat_dim(er)
+    feat = get_feat_dim(z)
+    if feat % heads or a_l.numel() != feat:
+        raise RuntimeError("inconsistent head count")
+    out = torch.empty(_out_shape(graph.num_nodes, z), dtype=z.dtype, device=z.device)
+    lib = capi.load()
+    ws = graph.workspace(lib.ga_gat_workspace_bytes(graph.num_edges, feat, heads))
+    capi.check(lib.ga_gat_aggregate_from_z(
+        graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
+        graph.in_node_indices.data_ptr(), a_l.data_ptr(), er.data_ptr(), z.data_ptr(),
+        out.data_ptr(), graph.num_nodes, graph.num_edges, heads, feat // heads,
+        float(negative_slope), dt, ws.data_ptr(), ws.numel(), _stream(out)),
+        "ga_gat_aggregate_from_z")
+    return out
+
+
 def edge_softmax_sum(logits, messages, graph: DGLGraph) -> torch.Tensor:
     """out[v] = sum over in-edges e of softmax_v(logits)[e] * messages[e]: the
     SegmentSoftmax -> mul -> SpMMEdge tail of the reference's HGT plan

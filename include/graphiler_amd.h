@@ -242,6 +242,25 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
                      void *workspace, size_t workspace_bytes,
                      ga_stream_t stream);
 
+/* The same chain with the source term recomputed from the gathered row:
+ *   s_i = leaky_relu(<z[nbr[i], h, :], a_l[h, :]> + er[v, h], slope)
+ * instead of reading el[nbr[i], h].  Same result as ga_gat_aggregate with
+ * el = z . a_l (up to fp32 summation order; for bf16 z the products use the
+ * stored, rounded rows, as the reference's plan does when it evaluates
+ * mm(z, attn_weight) on the stored z, examples/GAT/GAT.py:27-29).  It saves the
+ * separate (n, heads) gather, one more memory sector per edge once that table
+ * outgrows the caches (2.4 M nodes x 4 heads: 15 % of the traffic).  a_l is
+ * (heads, dim) fp32.  GA_EUNSUPPORTED when the lanes that share a head
+ * (dim / 8 for bf16, dim / 4 for fp32 with 16-byte aligned rows, else dim) are
+ * not a power of two <= 16.
+ */
+int ga_gat_aggregate_from_z(const int32_t *pointer, const int32_t *row_of_slot,
+                            const int32_t *nbr, const float *a_l, const float *er,
+                            const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                            int64_t heads, int64_t dim, float slope, int dtype,
+                            void *workspace, size_t workspace_bytes,
+                            ga_stream_t stream);
+
 /* The softmax-weighted reduction with per-edge operands:
  *   a = softmax_v(logit[e, h] over the in-edges e of v),
  *   out[v, h, :] = sum_e a_e * m[e, h, :]

@@ -172,6 +172,13 @@ def test_config5_large_gat_sampled_and_properties(device):
     ref = oracle.gat_aggregate(sub_ptr, sub_nbr, el, er[sample], z, heads=heads, slope=0.2)
     assert_close(out[sample], ref, TOL_BF16, "config 5 fused GAT (sampled rows)")
     assert not out[deg == 0].any()
+    # the variant that recomputes the source term from the gathered rows
+    a_l = (rng.standard_normal((heads, d)) / 8).astype(np.float32)
+    el2 = np.einsum("nhd,hd->nh", z.reshape(n, heads, d).astype(np.float64), a_l).astype(np.float32)
+    out2 = ops.gat_aggregate_from_z(_t(a_l, device), dr, dz, g, 0.2).float().cpu().numpy()
+    ref2 = oracle.gat_aggregate(sub_ptr, sub_nbr, el2, er[sample], z, heads=heads, slope=0.2)
+    assert_close(out2[sample], ref2, TOL_BF16, "config 5 fused GAT, source term from z")
+    assert not out2[deg == 0].any()
     # properties over ALL rows: softmax segments sum to one; SpMM column sums
     logits = ops.gsddmm_u_add_v_mul_alpha(dl, dr, 1, g)
     att = ops.SegmentSoftmax(logits, 1, None, g)

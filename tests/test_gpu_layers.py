@@ -43,6 +43,28 @@ def test_gcn_two_layers(device):
                  1e-4, "GCN layer 2")   # two chained fp32 layers
 
 
+@pytest.mark.parametrize("heads", [1, 4])
+def test_gat_layer_switches_to_source_term_from_rows(device, heads, monkeypatch):
+    """gat_layer takes the variant that recomputes the source term once the
+    (N, heads) table passes a size limit; both routes give the layer's result."""
+    wl = datasets.gat_rmat(num_nodes=3000, n_edges=60_000, scale=12, seed=3)
+    n = wl.num_nodes
+    g = prepare_graph(wl.src, wl.dst, n, device=device)
+    rng = np.random.default_rng(3)
+    h = torch.from_numpy(rng.standard_normal((n, 40), dtype=np.float32)).to(device)
+    w = torch.from_numpy(datasets.glorot(rng, (40, heads * 32))).to(device)
+    a = torch.from_numpy(rng.standard_normal((2, heads, 32), dtype=np.float32) / 6).to(device)
+    base = layers.gat_layer(g, h, w, a, heads, 0.2)
+    calls = []
+    real = layers.ops.gat_aggregate_from_z
+    monkeypatch.setattr(layers.ops, "gat_aggregate_from_z",
+                        lambda *args: calls.append(1) or real(*args))
+    monkeypatch.setattr(layers, "SOURCE_TERM_TABLE_LIMIT", 0)
+    alt = layers.gat_layer(g, h, w, a, heads, 0.2)
+    assert calls, "the size limit did not select the variant"
+    assert_close(alt.cpu().numpy(), base.cpu().numpy(), 4 * TOL_F32, "gat_layer, both routes")
+
+
 @pytest.mark.parametrize("heads,bf16", [(1, False), (4, False), (4, True)])
 def test_gat_layer(device, heads, bf16):
     wl = datasets.gat_rmat(num_nodes=20_000, n_edges=600_000, scale=15, seed=1,

@@ -369,6 +369,35 @@ def test_gat_aggregate_fused(graph, device, heads, dim, bf16):
     assert not got.float().cpu().numpy()[np.diff(arr.in_pointer) == 0].any()
 
 
+@pytest.mark.parametrize("heads,dim,bf16", [(1, 64, False), (4, 64, True), (8, 16, True),
+                                            (2, 8, False), (3, 32, False), (1, 16, True)])
+def test_gat_aggregate_from_z(graph, device, heads, dim, bf16):
+    """Source term recomputed from the gathered row: equals the fused chain fed
+    with el = z . a_l (oracle, float64 dot of the stored rows)."""
+    name, g, arr = graph
+    n = arr.num_nodes
+    rng = np.random.default_rng(heads * 31 + dim)
+    z = rng.standard_normal((n, heads * dim), dtype=np.float32)
+    if bf16:
+        z = to_bf16_f32(z)
+    a_l = (rng.standard_normal((heads, dim)) / np.sqrt(dim)).astype(np.float32)
+    er = rng.standard_normal((n, heads), dtype=np.float32)
+    el = np.einsum("nhd,hd->nh", z.reshape(n, heads, dim).astype(np.float64), a_l).astype(np.float32)
+    ref = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er, z, heads=heads,
+                               slope=0.2)
+    got = ops.gat_aggregate_from_z(_dev(a_l, device), _dev(er, device), _dev(z, device, bf16),
+                                   g, 0.2)
+    assert_close(got.float().cpu().numpy().reshape(ref.shape), ref,
+                 TOL_BF16 if bf16 else 4 * TOL_F32, f"gat from z on {name}")
+
+
+def test_gat_aggregate_from_z_unsupported_head_width(device):
+    g = prepare_graph(np.array([0, 1]), np.array([1, 0]), 2, device=device)
+    with pytest.raises(capi.GraphilerError):          # 24 / 4 = 6 lanes per head
+        ops.gat_aggregate_from_z(torch.ones(1, 24, device=device), torch.ones(2, 1, device=device),
+                                 torch.ones(2, 24, device=device), g, 0.2)
+
+
 def test_gat_layer_plan_equals_fused(graph, device):
     from graphiler_amd import layers
     name, g, arr = graph
