@@ -83,6 +83,7 @@ struct MmExt {
   const int64_t *q_index;   // row r is reduced against Q[q_index[r]]; null: Q[r]
   float *dot;               // (rows, ldd) fp32, column = head
   const float *scale;       // (n_types, ldd) factor per type and head; null: 1
+  const float *row_scale;   // kEpiStore: Y[r, :] *= row_scale[r]; null: 1
   int64_t ldq, ldd;
   const float *a_l, *a_r;   // attention vectors over the tile's columns (kEpiAttn)
   float *el, *er;           // (rows, ldd) fp32
@@ -531,6 +532,17 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
     }
   }
   int64_t inext = src_row(first + kTileBlock);
+  // per-row factors of the stored rows (one per edge, in row order), also
+  // requested one tile ahead
+  const float *__restrict__ rsp = EPI == kEpiStore ? e.row_scale : nullptr;
+  float rsn[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+  if (rsp) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = row0 + wave * kTileRows + lk * 4 + r;
+      if (row < row1) rsn[r] = rsp[row];
+    }
+  }
 
   // dot operand: the values this lane needs from Q (4 rows x its column of every
   // block; a packed bf16 pair per block pair) are requested one tile ahead as
@@ -629,6 +641,16 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
       }
     }
     inext = src_row(tile0 + 2 * kTileBlock + lr);
+    float rsa[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) rsa[r] = rsn[r];
+    if (rsp) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = tile0 + kTileBlock + lk * 4 + r;
+        if (row < row1) rsn[r] = rsp[row];
+      }
+    }
     qv_t qa[4][NQ];
     if (DOT) {
 #pragma unroll
@@ -708,6 +730,12 @@ __global__ __launch_bounds__(kBlock) void segment_mm_tight_kernel(
           }
         }
       }
+    }
+    if (EPI == kEpiStore && rsp) {
+#pragma unroll
+      for (int cb = 0; cb < CG; ++cb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[cb][r] *= rsa[r];
     }
     if (EPI == kEpiStore && g.perm_shift >= 0) {
       // permuted tile: this lane holds columns [lr * CG, (lr + 1) * CG) of its four
@@ -1114,8 +1142,8 @@ extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types
                                     const void *X, const int64_t *x_index,
                                     const void *W, void *Y, const void *Q,
                                     const int64_t *q_index, const float *scale,
-                                    float *dot, int64_t rows, int64_t heads,
-                                    int64_t K, int64_t M, int dtype,
+                                    float *dot, const float *row_scale, int64_t rows,
+                                    int64_t heads, int64_t K, int64_t M, int dtype,
                                     ga_stream_t stream) {
   using namespace ga;
   const int bad = check_mm_args(n_types, rows, heads, K, M, dtype);
@@ -1124,11 +1152,12 @@ extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types
   if ((Y != nullptr) == (dot != nullptr)) return GA_EINVAL;   // exactly one result
   if ((Q != nullptr) != (dot != nullptr)) return GA_EINVAL;
   if ((q_index || scale) && !Q) return GA_EINVAL;
+  if (row_scale && !Y) return GA_EINVAL;
   if (!type_pointer || !X || !W) return GA_EINVAL;
   const size_t esz = dtype == GA_F32 ? 4 : 2;
   if (!aligned(X, esz) || !aligned(W, esz) || (Y && !aligned(Y, esz)) ||
       (Q && !aligned(Q, esz)) || (dot && !aligned(dot, 4)) ||
-      (scale && !aligned(scale, 4)) ||
+      (scale && !aligned(scale, 4)) || (row_scale && !aligned(row_scale, 4)) ||
       (x_index && !aligned(x_index, 8)) || (q_index && !aligned(q_index, 8)))
     return GA_EALIGN;
   MmExt ext = {};
@@ -1137,6 +1166,7 @@ extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types
   ext.q_index = q_index;
   ext.dot = dot;
   ext.scale = scale;
+  ext.row_scale = row_scale;
   ext.ldq = heads * M;
   ext.ldd = heads;
   return segment_mm_any(type_pointer, n_types, X, W, Y, rows, heads, K, M, dtype, ext,

@@ -401,20 +401,37 @@ const torch::Tensor &endpoint_column(const GraphPtr &graph, int64_t which) {
 
 // broadcast.cu:58-69 + segment_mm.cu:29-33 as one pass:
 // out[e] = features[endpoint(e)] @ weights[type(e)]
+// row_scale: an (E,) / (E, 1) fp32 tensor multiplies row e of the result (the
+// per-edge norm of examples/RGCN/RGCN.py:29); any other shape multiplies the
+// result afterwards with ATen's broadcasting
 torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
-                                  int64_t endpoint, const GraphPtr &graph) {
+                                  int64_t endpoint, at::optional<torch::Tensor> row_scale,
+                                  const GraphPtr &graph) {
   const MmShape s = edge_mm_shape(features, weights, graph);
   const torch::Tensor &index = endpoint_column(graph, endpoint);
   torch::Tensor out = torch::empty({graph->num_edges, s.heads * s.M}, features.options());
+  const float *rs = nullptr;
+  torch::Tensor late;            // a factor the kernel does not take
+  if (row_scale.has_value()) {
+    const torch::Tensor &r = row_scale.value();
+    if (r.is_cuda() && r.is_contiguous() && r.scalar_type() == at::kFloat &&
+        r.numel() == graph->num_edges && r.dim() <= 2 && r.size(0) == graph->num_edges)
+      rs = r.data_ptr<float>();
+    else
+      late = r;
+  }
   const int rc = ga_segment_mm_gather(
       graph->etype_pointer.value().data_ptr<int>(), graph->num_etypes, features.data_ptr(),
       index.data_ptr<int64_t>(), weights.data_ptr(), out.data_ptr(), nullptr, nullptr,
-      nullptr, nullptr, graph->num_edges, s.heads, s.K, s.M, s.dt, current_stream(out));
-  if (rc == GA_EUNSUPPORTED)       // shape outside the matrix-core tile
-    return segment_mm(gather(features, index), weights, graph->etype_pointer,
-                      graph->num_etypes, graph->num_edges);
-  check_ga(rc, "ga_segment_mm_gather");
-  return out;
+      nullptr, nullptr, rs, graph->num_edges, s.heads, s.K, s.M, s.dt, current_stream(out));
+  if (rc == GA_EUNSUPPORTED) {     // shape outside the matrix-core tile
+    out = segment_mm(gather(features, index), weights, graph->etype_pointer,
+                     graph->num_etypes, graph->num_edges);
+    if (rs) late = row_scale.value();
+  } else {
+    check_ga(rc, "ga_segment_mm_gather");
+  }
+  return late.defined() ? out * late : out;
 }
 
 // out[e, h] = <features[endpoint(e)] @ weights[type(e)], other[other_endpoint(e)]>
@@ -443,9 +460,10 @@ torch::Tensor SegmentMMEdgeDot(torch::Tensor features, torch::Tensor weights,
       graph->etype_pointer.value().data_ptr<int>(), graph->num_etypes, features.data_ptr(),
       xi.data_ptr<int64_t>(), weights.data_ptr(), nullptr, other.data_ptr(),
       qi.data_ptr<int64_t>(), sc.defined() ? sc.data_ptr<float>() : nullptr,
-      out.data_ptr<float>(), graph->num_edges, s.heads, s.K, s.M, s.dt, current_stream(out));
+      out.data_ptr<float>(), nullptr, graph->num_edges, s.heads, s.K, s.M, s.dt,
+      current_stream(out));
   if (rc == GA_EUNSUPPORTED) {
-    torch::Tensor y = SegmentMMEdgeGather(features, weights, endpoint, graph);
+    torch::Tensor y = SegmentMMEdgeGather(features, weights, endpoint, at::nullopt, graph);
     torch::Tensor q = gather(other, qi).reshape(y.sizes());
     torch::Tensor d = (y.to(at::kFloat) * q.to(at::kFloat))
                           .reshape({graph->num_edges, s.heads, s.M})
@@ -671,8 +689,8 @@ static auto registry =
             &e_mul_e_sum)
         .op("my_ops::edge_softmax_sum(Tensor x, Tensor m, " GRAPH_T " g) -> Tensor z",
             &edge_softmax_sum)
-        .op("my_ops::SegmentMMEdgeGather(Tensor x, Tensor w, int endpoint, " GRAPH_T
-            " g) -> Tensor z",
+        .op("my_ops::SegmentMMEdgeGather(Tensor x, Tensor w, int endpoint, Tensor? row_scale, "
+            GRAPH_T " g) -> Tensor z",
             &SegmentMMEdgeGather)
         .op("my_ops::SegmentMMEdgeDot(Tensor x, Tensor w, int endpoint, Tensor q, "
             "int q_endpoint, Tensor? scale, " GRAPH_T " g) -> Tensor z",

@@ -92,12 +92,12 @@ def gat_layer(g: DGLGraph, h, fc_weight, attn_weight, heads: int = 1,
 def rgcn_layer(g: DGLGraph, h, weight, norm, fused: bool = True):
     """examples/RGCN/RGCN.py:25-33.  weight (R, K, M); norm (E, 1) fp32; edges
     sorted by type.  ``fused``: the typed product reads the source rows through
-    the COO column and the norm multiplies inside the reduction (two passes);
+    the COO column and applies the norm to the rows it produces (two passes);
     otherwise the reference's plan BroadcastSrcNode -> SegmentMMEdge ->
     mul(norm) -> SpMMEdge."""
     if fused:
-        msg = ops.SegmentMMEdgeGather(h, weight, 0, g)
-        return ops.gspmm_e_mul_e_sum(msg, norm.float(), g)
+        msg = ops.SegmentMMEdgeGather(h, weight, 0, g, row_scale=norm.float().contiguous())
+        return ops.SpMMEdge(msg, [1], False, None, g)
     hs = ops.BroadcastSrcNode(h, g)
     msg = ops.SegmentMMEdge(hs, weight, g)
     msg = msg * norm.to(msg.dtype)

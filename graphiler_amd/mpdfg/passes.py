@@ -398,6 +398,9 @@ class _Rewriter:
         for n in list(self.G.nodes()):
             if n.kind() == "my_ops::gspmm_e_mul_e_sum":
                 changed |= self._fuse_softmax_sum(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::gspmm_e_mul_e_sum":
+                changed |= self._fuse_row_scale(n)
         return changed
 
     def _fuse_gather_mm(self, n) -> bool:
@@ -409,7 +412,8 @@ class _Rewriter:
             return False
         which = self.const(0 if bc.kind().endswith("SrcNode") else 1, n)
         out = self.make("my_ops::SegmentMMEdgeGather",
-                        [bc.inputsAt(0), n.inputsAt(1), which, self.dglgraph], n, EDGE)
+                        [bc.inputsAt(0), n.inputsAt(1), which, self.const(None, n), self.dglgraph],
+                        n, EDGE)
         n.output().replaceAllUsesWith(out)
         n.destroy()
         return True
@@ -435,7 +439,7 @@ class _Rewriter:
                 out = self.make("my_ops::SegmentMMEdgeDot",
                                 [mm.inputsAt(0), mm.inputsAt(1), mm.inputsAt(2),
                                  bc.inputsAt(0), which, self.const(None, n), self.dglgraph],
-                                n, EDGE)
+                                n, EDGE)                 # (the product's row factor is None here)
                 n.output().replaceAllUsesWith(out)
                 n.destroy()
                 return True
@@ -455,6 +459,32 @@ class _Rewriter:
                 ins = list(dot.inputs())
                 ins[5] = bc.inputsAt(0)
                 out = self.make("my_ops::SegmentMMEdgeDot", ins, n, EDGE)
+                n.output().replaceAllUsesWith(out)
+                n.destroy()
+                return True
+        return False
+
+    def _fuse_row_scale(self, n) -> bool:
+        """gspmm_e_mul_e_sum(SegmentMMEdgeGather(x, w, i, None), s) with s read from
+        the edge data (a stored per-edge tensor such as RGCN's norm, not something
+        computed in the plan) -> SpMMEdge(SegmentMMEdgeGather(x, w, i, s)): the
+        factor is applied where the rows are produced, in edge order, instead of
+        being gathered through the edge ids by the reduction.  The operator
+        multiplies afterwards when s is not one float per edge."""
+        for a, b in ((n.inputsAt(0), n.inputsAt(1)), (n.inputsAt(1), n.inputsAt(0))):
+            mm, sc = a.node(), b.node()
+            if mm.kind() == "my_ops::SegmentMMEdgeGather" and self.single_use(a) and \
+                    mm.inputsAt(3).node().kind() == "prim::Constant" and \
+                    isinstance(mm.inputsAt(3).type(), torch._C.NoneType) and \
+                    sc.kind() == "aten::__getitem__" and self.where(b) == EDGE:
+                ins = list(mm.inputs())
+                ins[3] = b
+                prod = self.make("my_ops::SegmentMMEdgeGather", ins, n, EDGE)
+                with self.G.insert_point_guard(n):
+                    dims = self.G.insertConstant([1])
+                    keep = self.G.insertConstant(False)
+                    none = self.G.insertConstant(None)
+                out = self.make("my_ops::SpMMEdge", [prod, dims, keep, none, self.dglgraph], n, NODE)
                 n.output().replaceAllUsesWith(out)
                 n.destroy()
                 return True

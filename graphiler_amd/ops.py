@@ -357,21 +357,31 @@ def _mm_shapes(features, weights, graph: DGLGraph):
     return heads, K, M
 
 
-def SegmentMMEdgeGather(features, weights, endpoint: int, graph: DGLGraph) -> torch.Tensor:
+def SegmentMMEdgeGather(features, weights, endpoint: int, graph: DGLGraph,
+                        row_scale=None) -> torch.Tensor:
     """``SegmentMMEdge(BroadcastSrcNode(features), weights)`` (endpoint 0) or
     the same with ``BroadcastDstNode`` (endpoint 1) as one pass: row e of the
     result is features[endpoint(e)] @ weights[type(e)] (broadcast.cu:58-69 +
-    segment_mm.cu:29-33); the (E, heads*K) copy of the node rows is never made."""
+    segment_mm.cu:29-33); the (E, heads*K) copy of the node rows is never made.
+    ``row_scale`` (E,) or (E, 1) fp32 multiplies row e (RGCN's per-edge norm)."""
     heads, K, M = _mm_shapes(features, weights, graph)
     index = _endpoint(graph, endpoint)
+    if row_scale is not None:
+        _check_input(row_scale, "row_scale")
+        if row_scale.dtype != torch.float32 or row_scale.numel() != graph.num_edges:
+            raise RuntimeError("row_scale must be one float32 per edge")
     out = torch.empty((graph.num_edges, heads * M), dtype=features.dtype,
                       device=features.device)
     rc = capi.load().ga_segment_mm_gather(
         graph.etype_pointer.data_ptr(), graph.num_etypes, features.data_ptr(),
         index.data_ptr(), weights.data_ptr(), out.data_ptr(), None, None, None, None,
-        graph.num_edges, heads, K, M, _feat_dtype(features, "features"), _stream(out))
+        _ptr(row_scale), graph.num_edges, heads, K, M, _feat_dtype(features, "features"),
+        _stream(out))
     if rc == capi.GA_EUNSUPPORTED:      # shape outside the matrix-core tile
-        return SegmentMMEdge(_gather(features, index), weights, graph)
+        out = SegmentMMEdge(_gather(features, index), weights, graph)
+        if row_scale is not None:
+            out = (out * row_scale.reshape(-1, 1)).to(out.dtype)
+        return out
     capi.check(rc, "ga_segment_mm_gather")
     return out
 
@@ -398,7 +408,7 @@ def SegmentMMEdgeDot(features, weights, endpoint: int, other, other_endpoint: in
     rc = capi.load().ga_segment_mm_gather(
         graph.etype_pointer.data_ptr(), graph.num_etypes, features.data_ptr(),
         xi.data_ptr(), weights.data_ptr(), None, other.data_ptr(), qi.data_ptr(),
-        _ptr(scale), out.data_ptr(), graph.num_edges, heads, K, M,
+        _ptr(scale), out.data_ptr(), None, graph.num_edges, heads, K, M,
         _feat_dtype(features, "features"), _stream(out))
     if rc == capi.GA_EUNSUPPORTED:
         y = SegmentMMEdgeGather(features, weights, endpoint, graph)

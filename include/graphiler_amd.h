@@ -194,7 +194,9 @@ int ga_segment_mm(const int32_t *type_pointer, int64_t n_types, const void *X,
  * (segment_mm.cu:29-33) that the reference's plans execute for
  * examples/RGCN/RGCN.py:26-28 and examples/HGT/HGT.py:35-44.  Exactly one of
  * two results:
- *   Y   (rows, heads*M) `dtype`, with Q / q_index / dot NULL;
+ *   Y   (rows, heads*M) `dtype`, with Q / q_index / dot NULL; row_scale, when
+ *       not NULL, is (rows,) fp32 and multiplies row r of Y (the per-edge norm
+ *       of examples/RGCN/RGCN.py:29, read in edge order with the rows);
  *   dot (rows, heads) fp32 with Y NULL: dot[r, h] = <Y[r, h, :], Q[q_index[r], h, :]>
  *       (q_index NULL: Q[r]); Q (*, heads*M) `dtype`.  The product rows stay in
  *       registers (HGT's sum(k * q, dim=1), HGT.py:44-45).  scale, when not
@@ -211,8 +213,9 @@ int ga_segment_mm(const int32_t *type_pointer, int64_t n_types, const void *X,
 int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types, const void *X,
                          const int64_t *x_index, const void *W, void *Y,
                          const void *Q, const int64_t *q_index, const float *scale,
-                         float *dot, int64_t rows, int64_t heads, int64_t K,
-                         int64_t M, int dtype, ga_stream_t stream);
+                         float *dot, const float *row_scale, int64_t rows,
+                         int64_t heads, int64_t K, int64_t M, int dtype,
+                         ga_stream_t stream);
 
 /* ---------------------------------------------------------------- gather --
  * y[i, :] = x[idx[i], :], a bit-exact row copy of row_bytes bytes.

@@ -514,12 +514,15 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
         rc = lib.ga_segment_mm_gather(
             g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(),
             (g.COO_src if which == 0 else g.COO_dst).data_ptr(), dW.data_ptr(), Y.data_ptr(),
-            None, None, None, None, e, heads, K, M, dt, stream)
+            None, None, None, None, None, e, heads, K, M, dt, stream)
         assert rc == (0 if fits else capi.GA_EUNSUPPORTED)
         if fits:
             assert_close(Y.float().cpu().numpy(), ref, tol, f"segment_mm_gather {which}")
         got = ops.SegmentMMEdgeGather(dX, dW, which, g)
         assert_close(got.float().cpu().numpy(), ref, tol, f"SegmentMMEdgeGather {which}")
+        norm = rng.uniform(0.25, 2.0, (e, 1)).astype(np.float32)        # per-row factor
+        got = ops.SegmentMMEdgeGather(dX, dW, which, g, row_scale=_dev(norm, device))
+        assert_close(got.float().cpu().numpy(), ref * norm, tol, f"SegmentMMEdgeGather scaled {which}")
         # dot against the other endpoint's row of Q
         other = dst if which == 0 else src
         y64 = np.einsum("ehk,ehkm->ehm", X[col].reshape(e, heads, K).astype(np.float64),
@@ -530,7 +533,7 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
             g.etype_pointer.data_ptr(), n_rel, dX.data_ptr(),
             (g.COO_src if which == 0 else g.COO_dst).data_ptr(), dW.data_ptr(), None,
             dQ.data_ptr(), (g.COO_dst if which == 0 else g.COO_src).data_ptr(), None,
-            D.data_ptr(), e, heads, K, M, dt, stream)
+            D.data_ptr(), None, e, heads, K, M, dt, stream)
         assert rc == (0 if dot_fits else capi.GA_EUNSUPPORTED)
         if dot_fits:
             assert_close(D.cpu().numpy(), want, tol, f"segment_mm dot {which}")
@@ -548,8 +551,8 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
     if fits:
         Y = torch.full((e, heads * M), float("nan"), dtype=dX.dtype, device=device)
         assert lib.ga_segment_mm_gather(g.etype_pointer.data_ptr(), n_rel, dXe.data_ptr(), None,
-                                        dW.data_ptr(), Y.data_ptr(), None, None, None, None, e,
-                                        heads, K, M, dt, stream) == 0
+                                        dW.data_ptr(), Y.data_ptr(), None, None, None, None, None,
+                                        e, heads, K, M, dt, stream) == 0
         assert_close(Y.float().cpu().numpy(), oracle.segment_mm(tp, Xe, W, heads=heads), tol,
                      "segment_mm_gather identity")
     # argument errors: neither result; both results; scale without a dot operand
@@ -557,11 +560,14 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
     tail = (e, heads, K, M, dt, stream)
     Y = torch.empty((e, heads * M), dtype=dX.dtype, device=device)
     D = torch.empty((e, heads), dtype=torch.float32, device=device)
-    assert lib.ga_segment_mm_gather(*args, None, None, None, None, None, *tail) == capi.GA_EINVAL
+    none = (None,) * 6
+    assert lib.ga_segment_mm_gather(*args, *none, *tail) == capi.GA_EINVAL
     assert lib.ga_segment_mm_gather(*args, Y.data_ptr(), dQ.data_ptr(), None, None,
-                                    D.data_ptr(), *tail) == capi.GA_EINVAL
-    assert lib.ga_segment_mm_gather(*args, Y.data_ptr(), None, None, D.data_ptr(), None,
+                                    D.data_ptr(), None, *tail) == capi.GA_EINVAL
+    assert lib.ga_segment_mm_gather(*args, Y.data_ptr(), None, None, D.data_ptr(), None, None,
                                     *tail) == capi.GA_EINVAL
+    assert lib.ga_segment_mm_gather(*args, None, dQ.data_ptr(), None, None, D.data_ptr(),
+                                    D.data_ptr(), *tail) == capi.GA_EINVAL      # row factor without Y
 
 
 @pytest.mark.parametrize("heads,dim,bf16", [(1, 64, False), (8, 16, True), (4, 5, False),

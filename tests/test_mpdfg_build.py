@@ -65,9 +65,9 @@ def test_level2_fuses_into_graph_operators():
     assert "aten::mm" not in k
     _, k = _kinds("rgcn", 2)
     ours = [x for x in k if x.startswith("my_ops::")]
-    # the source rows are read through the COO column by the typed product and the
-    # norm multiplies inside the reduction: no per-edge copy, no product tensor
-    assert ours == ["my_ops::SegmentMMEdgeGather", "my_ops::gspmm_e_mul_e_sum"]
+    # the source rows are read through the COO column by the typed product, which
+    # also applies the norm to the rows it writes: no per-edge copy, no product tensor
+    assert ours == ["my_ops::SegmentMMEdgeGather", "my_ops::SpMMEdge"]
     assert "aten::bmm" not in k and "aten::mul" not in k
     _, k = _kinds("hgt", 2)
     ours = [x for x in k if x.startswith("my_ops::")]
