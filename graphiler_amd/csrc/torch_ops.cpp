@@ -442,11 +442,15 @@ torch::Tensor SegmentMMEdgeDot(torch::Tensor features, torch::Tensor weights,
                                const GraphPtr &graph) {
   const MmShape s = edge_mm_shape(features, weights, graph);
   torch::Tensor sc;      // (T, heads) fp32: out[e, h] *= scale[type(e), h]
+  torch::Tensor late;    // a per-type factor of another shape: broadcast afterwards
   if (scale.has_value()) {
     check_input(scale.value(), "scale");
-    TORCH_CHECK(scale.value().numel() == graph->num_etypes * s.heads,
-                "scale must have one value per type and head");
-    sc = scale.value().to(at::kFloat).contiguous();
+    if (scale.value().numel() == graph->num_etypes * s.heads) {
+      sc = scale.value().to(at::kFloat).contiguous();
+    } else {
+      TORCH_CHECK(graph->etype_COO.has_value(), "the graph has no edge-type column");
+      late = gather(scale.value(), graph->etype_COO.value());
+    }
   }
   check_input(other, "other");
   TORCH_CHECK(other.scalar_type() == features.scalar_type() &&
@@ -472,10 +476,10 @@ torch::Tensor SegmentMMEdgeDot(torch::Tensor features, torch::Tensor weights,
                 "the graph has no edge-type column");
     if (sc.defined())
       d = d * gather(sc.reshape({graph->num_etypes, s.heads}), graph->etype_COO.value());
-    return d;
+    return late.defined() ? d * late : d;
   }
   check_ga(rc, "ga_segment_mm_gather");
-  return out;
+  return late.defined() ? out * late : out;
 }
 
 torch::Tensor gather(const torch::Tensor &features, const torch::Tensor &index) {

@@ -394,11 +394,13 @@ def SegmentMMEdgeDot(features, weights, endpoint: int, other, other_endpoint: in
     ``scale`` (T, heads) or (T,) multiplies row e by scale[type(e)] (the
     ``* relation_pri`` of HGT.py:45)."""
     heads, K, M = _mm_shapes(features, weights, graph)
+    late = None            # a per-type factor of another shape: broadcast afterwards
     if scale is not None:
         _check_input(scale, "scale")
-        if scale.numel() != graph.num_etypes * heads:
-            raise RuntimeError("scale must have one value per type and head")
-        scale = scale.float().contiguous()
+        if scale.numel() == graph.num_etypes * heads:
+            scale = scale.float().contiguous()
+        else:
+            late, scale = BroadcastEdgeType(scale, graph), None
     _check_input(other, "other")
     if other.dtype != features.dtype or int(other.shape[0]) != graph.num_nodes \
             or get_feat_dim(other) != heads * M:
@@ -416,9 +418,9 @@ def SegmentMMEdgeDot(features, weights, endpoint: int, other, other_endpoint: in
         out = prod.reshape(graph.num_edges, heads, M).sum(-1)
         if scale is not None:
             out = out * BroadcastEdgeType(scale.reshape(graph.num_etypes, heads), graph)
-        return out
+        return out if late is None else out * late
     capi.check(rc, "ga_segment_mm_gather")
-    return out
+    return out if late is None else out * late
 
 
 # ------------------------------------------------------------ broadcast ----

@@ -570,6 +570,27 @@ def test_segment_mm_gather_and_dot(device, K, M, heads, bf16):
                                     D.data_ptr(), *tail) == capi.GA_EINVAL      # row factor without Y
 
 
+def test_segment_mm_dot_factor_of_another_shape(device):
+    """A per-type factor that is not one value per head (here (T, 3) against a
+    one-head dot) multiplies the result the way the unfused plan's
+    ``* BroadcastEdgeType(p)`` would: by broadcasting, after the kernel."""
+    rng = np.random.default_rng(9)
+    etype = np.repeat(np.arange(4), [30, 0, 50, 21]).astype(np.int64)
+    e, n = etype.shape[0], 40
+    src, dst = rng.integers(0, n, e, dtype=np.int64), rng.integers(0, n, e, dtype=np.int64)
+    g = prepare_graph(src, dst, n, device=device, etype_of=etype, num_etypes=4)
+    X = rng.standard_normal((n, 16), dtype=np.float32)
+    Q = rng.standard_normal((n, 32), dtype=np.float32)
+    W = rng.standard_normal((4, 16, 32)).astype(np.float32) / 4
+    p = rng.uniform(0.5, 2.0, (4, 3)).astype(np.float32)
+    want = np.einsum("em,em->e", np.einsum("ek,ekm->em", X[src].astype(np.float64), W[etype]),
+                     Q[dst].astype(np.float64))[:, None] * p[etype]
+    got = ops.SegmentMMEdgeDot(_dev(X, device), _dev(W, device), 0, _dev(Q, device), 1, g,
+                               scale=_dev(p, device))
+    assert got.shape == (e, 3)
+    assert_close(got.cpu().numpy(), want, 2 * TOL_F32, "dot with a (T, 3) factor")
+
+
 @pytest.mark.parametrize("heads,dim,bf16", [(1, 64, False), (8, 16, True), (4, 5, False),
                                             (2, 24, True), (1, 1, False)])
 def test_edge_softmax_sum(device, heads, dim, bf16):
