@@ -35,7 +35,7 @@ def main():
     ap.add_argument("--path", choices=["fused", "plan", "compiled"], default="fused",
                     help="fused: projection + one aggregation pass; plan: the reference's "
                          "four graph operators (GAT.py:25-36 after fusion); compiled: the "
-                         "GAT user-defined functions of bench_udf.py through the MP-DFG "
+                         "GAT user-defined functions of graphiler_amd/examples/udf.py through the MP-DFG "
                          "builder (opt level 2) and the TorchScript interpreter")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -79,9 +79,9 @@ def main():
         del big, big2
 
     if args.path == "compiled":
-        import bench_udf
+        from graphiler_amd.examples import udf
         from graphiler_amd.mpdfg import GraphData, mpdfg_builder, update_all
-        plan = mpdfg_builder(bench_udf.gat_message, bench_udf.gat_reduce, opt_level=2)
+        plan = mpdfg_builder(udf.gat_message, udf.gat_reduce, opt_level=2)
         gd = GraphData(g)
         attn_col = torch.cat([a[0].reshape(-1, 1), a[1].reshape(-1, 1)]).contiguous()
 
