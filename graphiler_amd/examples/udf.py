@@ -32,6 +32,22 @@ def gat_reduce(nodes: NodeBatchDummy):
     return {'h': torch.sum(alpha * nodes.mailbox['z'], dim=1)}
 
 
+# ---- GAT, four heads of width 16 (the shape literals must be constants for the
+# compiler to see that the view keeps one row per edge) -----------------------------
+def gat4_message(edges: EdgeBatchDummy, fc_weight, attn_l, attn_r):
+    # fc_weight (K, 64); attn_l / attn_r (1, 4, 16)
+    z_src = torch.mm(edges.src['h'], fc_weight).view(-1, 4, 16)
+    z_dst = torch.mm(edges.dst['h'], fc_weight).view(-1, 4, 16)
+    el = torch.sum(z_src * attn_l, dim=2, keepdim=True)          # (E, 4, 1)
+    er = torch.sum(z_dst * attn_r, dim=2, keepdim=True)
+    return {'z': z_src, 'e': F.leaky_relu(el + er, 0.2)}
+
+
+def gat4_reduce(nodes: NodeBatchDummy):
+    alpha = torch.softmax(nodes.mailbox['e'], dim=1)             # over the in-edges, per head
+    return {'h': torch.sum(alpha * nodes.mailbox['z'], dim=1)}
+
+
 # ---- RGCN: per-relation weight, per-edge norm --------------------------------------
 def rgcn_message(edges: EdgeBatchDummy):
     w = edges.type['weight']

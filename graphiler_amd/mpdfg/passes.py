@@ -26,7 +26,8 @@ _BCAST = {"my_ops::BroadcastSrcNode", "my_ops::BroadcastDstNode", "my_ops::Broad
           "my_ops::BroadcastDstNodeType", "my_ops::BroadcastEdgeType", "my_ops::BroadcastNodeType"}
 # row-wise operators whose first operand is the data and the rest are shared
 _ROWWISE = {"aten::relu", "aten::sigmoid", "aten::tanh", "aten::exp", "aten::neg",
-            "aten::leaky_relu", "aten::squeeze", "aten::mm", "aten::pow", "aten::unsqueeze"}
+            "aten::leaky_relu", "aten::squeeze", "aten::mm", "aten::pow", "aten::unsqueeze",
+            "aten::view", "aten::reshape", "aten::sum", "aten::elu"}
 _INPLACE = {"aten::relu_": "aten::relu", "aten::leaky_relu_": "aten::leaky_relu",
             "aten::sigmoid_": "aten::sigmoid", "aten::tanh_": "aten::tanh"}
 _PAIRWISE = {"aten::mul", "aten::add", "aten::sub", "aten::div"}
@@ -196,10 +197,27 @@ class _Rewriter:
                     n.destroy()
                     changed = True
                     continue
+            if kind in _PAIRWISE and n.inputsSize() >= 2 and self._hop_pairwise(n, kind):
+                changed = True
+                continue
             if kind not in _ROWWISE or first.kind() not in _BCAST:
                 continue
             if any(self.where(i) != SHARED for i in list(n.inputs())[1:]):
                 continue
+            if kind in ("aten::view", "aten::reshape"):
+                # row-wise when the rows stay the leading dimension: a leading -1
+                # (a view of per-edge data that regroups rows has no meaning as
+                # per-edge data, so the others are taken to describe one row)
+                shape = self.const_of(n.inputsAt(1))
+                if not isinstance(shape, list) or len(shape) < 2 or shape[0] != -1 \
+                        or any(not isinstance(d, int) or d <= 0 for d in shape[1:]):
+                    continue
+            if kind == "aten::sum":
+                # only reductions inside a row: every listed dimension >= 1
+                dims = self.const_of(n.inputsAt(1)) if n.inputsSize() == 4 else None
+                if not isinstance(dims, list) or not dims or \
+                        any(not isinstance(d, int) or d < 1 for d in dims):
+                    continue
             if kind == "aten::unsqueeze" and self.const_of(n.inputsAt(1)) in (0, None):
                 continue                      # a new leading dimension is not row-wise
             if kind == "aten::squeeze" and n.inputsSize() > 1 and self.const_of(n.inputsAt(1)) in (0, None):
@@ -211,6 +229,27 @@ class _Rewriter:
             n.destroy()
             changed = True
         return changed
+
+    def _hop_pairwise(self, n, kind) -> bool:
+        """``op(Broadcast(x), w)`` / ``op(w, Broadcast(x))`` with a shared tensor or
+        constant ``w`` (a weight that broadcasts against every row alike) ->
+        ``Broadcast(op(x, w))``."""
+        ins = list(n.inputs())
+        for pos in (0, 1):
+            bc, other = ins[pos].node(), ins[1 - pos]
+            if bc.kind() not in _BCAST or self.where(other) != SHARED:
+                continue
+            if any(self.where(i) != SHARED for i in ins[2:]):
+                continue
+            src = bc.inputsAt(0)
+            new_ins = list(ins)
+            new_ins[pos] = src
+            small = self.make(kind, new_ins, n, self.where(src), like=n)
+            back = self.make(bc.kind(), [small, self.dglgraph], n, self.where(n.output()))
+            n.output().replaceAllUsesWith(back)
+            n.destroy()
+            return True
+        return False
 
     # ------------------------------------------------------------ fusion ----
     def fusion(self) -> bool:

@@ -62,6 +62,29 @@ def test_gat_plan(device, level, width):
     assert_close(g.ndata['h'].cpu().numpy(), want, 2e-5, f"GAT plan level {level}")
 
 
+@pytest.mark.parametrize("level", [0, 1, 2])
+def test_multi_head_gat_plan(device, level):
+    rng = np.random.default_rng(25)
+    n, src, dst = _homo(rng)
+    g = GraphData(prepare_graph(src, dst, n, device))
+    heads, d = 4, 16
+    h = rng.standard_normal((n, 24), dtype=np.float32)
+    fc = (rng.standard_normal((24, heads * d)) / 5).astype(np.float32)
+    a_l, a_r = ((rng.standard_normal((1, heads, d)) / 4).astype(np.float32) for _ in range(2))
+    g.ndata['h'] = _t(h, device)
+    update_all(g, mpdfg_builder(U.gat4_message, U.gat4_reduce, opt_level=level),
+               msg_params=(_t(fc, device), _t(a_l, device), _t(a_r, device)))
+    z = (h.astype(np.float64) @ fc).reshape(n, heads, d)
+    el = (z * a_l).sum(-1).astype(np.float32)
+    er = (z * a_r).sum(-1).astype(np.float32)
+    arr = build_graph_arrays(src, dst, n)
+    want = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er,
+                                z.reshape(n, heads * d).astype(np.float32), heads=heads, slope=0.2)
+    got = g.ndata['h'].cpu().numpy()
+    assert got.shape == (n, heads, d)
+    assert_close(got.reshape(n, heads * d), want, 2e-5, f"multi-head GAT plan level {level}")
+
+
 def _hetero(rng, n_per_type=(60, 50, 40), e_per_rel=(400, 300, 500, 200)):
     n = sum(n_per_type)
     ntype = np.repeat(np.arange(len(n_per_type)), n_per_type).astype(np.int64)

@@ -80,6 +80,20 @@ def test_level2_fuses_into_graph_operators():
     assert "aten::bmm" not in k and "aten::squeeze" not in k and "aten::sum" not in k
 
 
+def test_multi_head_attention_reaches_the_fused_kernel():
+    """Four-head GAT written with view / per-head sums: the view, the products
+    with the attention vectors and the in-row sums hop over the broadcasts to
+    node data, and the chain fuses into gat_aggregate."""
+    plan = mpdfg_builder(U.gat4_message, U.gat4_reduce, opt_level=2)
+    k = plan.op_kinds()
+    ours = [x for x in k if x.startswith("my_ops::")]
+    assert ours == ["my_ops::gat_aggregate"]
+    assert k.count("aten::mm") == 1 and k.count("aten::view") == 1
+    plan1 = mpdfg_builder(U.gat4_message, U.gat4_reduce, opt_level=1).op_kinds()
+    # at level 1 the per-head terms are already computed on node data
+    assert plan1.index("aten::sum") < plan1.index("my_ops::BroadcastDstNode")
+
+
 def gat_reference_style_message(edges: EdgeBatchDummy, fc_weight, attn_weight):
     z_s = torch.mm(edges.src['h'], fc_weight)
     z_d = torch.mm(edges.dst['h'], fc_weight)
