@@ -640,6 +640,40 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> gat_project(
   return std::make_tuple(z, at::mm(z, w_src).to(at::kFloat), at::mm(z, w_dst).to(at::kFloat));
 }
 
+// Multi-head form of the same head: zv = (h @ fc).view(-1, heads, dim),
+// el = sum(zv * a_l, 2, keepdim), er likewise, with a_l / a_r of heads * dim
+// elements (any leading unit dimensions).  Returns zv (N, heads, dim) and
+// el / er (N, heads, 1) fp32.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> gat_project_heads(
+    torch::Tensor h, torch::Tensor fc, torch::Tensor a_l, torch::Tensor a_r, int64_t heads,
+    int64_t dim) {
+  check_input(h, "h");
+  check_input(fc, "fc_weight");
+  TORCH_CHECK(a_l.is_cuda() && a_r.is_cuda(), "attention vectors must be a CUDA tensor");
+  TORCH_CHECK(h.dim() == 2 && fc.dim() == 2 && fc.size(0) == h.size(1), "fc_weight must be (K, M)");
+  TORCH_CHECK(heads > 0 && dim > 0 && fc.size(1) == heads * dim,
+              "fc_weight must have heads * dim columns");
+  TORCH_CHECK(a_l.numel() == heads * dim && a_r.numel() == heads * dim,
+              "attention vectors must have heads * dim elements");
+  const int64_t rows = h.size(0);
+  const bool candidate = (h.scalar_type() == at::kFloat || h.scalar_type() == at::kBFloat16) &&
+                         fc.scalar_type() == h.scalar_type();
+  if (candidate) {
+    torch::Tensor z, el, er;
+    const int rc = project_attn(h, fc, a_l.to(at::kFloat).contiguous().view({heads, dim}),
+                                a_r.to(at::kFloat).contiguous().view({heads, dim}), heads, z, el, er);
+    if (rc != GA_EUNSUPPORTED) {
+      check_ga(rc, "ga_project_attn");
+      return std::make_tuple(z.view({rows, heads, dim}), el.view({rows, heads, 1}),
+                             er.view({rows, heads, 1}));
+    }
+  }
+  torch::Tensor zv = at::mm(h, fc).view({rows, heads, dim});
+  torch::Tensor l = (zv * a_l.view({1, heads, dim})).sum(2, true).to(at::kFloat);
+  torch::Tensor r = (zv * a_r.view({1, heads, dim})).sum(2, true).to(at::kFloat);
+  return std::make_tuple(zv, l, r);
+}
+
 }  // namespace
 
 TORCH_LIBRARY(my_classes, m) {
@@ -707,4 +741,7 @@ static auto registry =
             &linear_attn)
         .op("my_ops::gat_project(Tensor h, Tensor fc, Tensor w_src, Tensor w_dst) -> "
             "(Tensor z, Tensor el, Tensor er)",
-            &gat_project);
+            &gat_project)
+        .op("my_ops::gat_project_heads(Tensor h, Tensor fc, Tensor a_l, Tensor a_r, int heads, "
+            "int dim) -> (Tensor z, Tensor el, Tensor er)",
+            &gat_project_heads);

@@ -373,6 +373,8 @@ class _Rewriter:
         data h and shared weights -> (z, el, er) = gat_project(h, fc, w_src, w_dst):
         the projection and both attention products in one operator."""
         el, er, z = n.inputsAt(0).node(), n.inputsAt(1).node(), n.inputsAt(2).node()
+        if z.kind() in ("aten::view", "aten::reshape"):
+            return self._fuse_gat_project_heads(n)
         if not (el.kind() == er.kind() == z.kind() == "aten::mm"):
             return False
         if el.inputsAt(0).unique() != z.output().unique() or \
@@ -415,6 +417,55 @@ class _Rewriter:
             dead.destroy()
         return True
 
+
+    def _fuse_gat_project_heads(self, n) -> bool:
+        """Multi-head form: gat_aggregate(sum(zv * a_l, [2], True), sum(zv * a_r, [2],
+        True), zv = view(mm(h, fc), [-1, H, D]), ...) with shared (.., H, D) attention
+        vectors -> (zv, el, er) = gat_project_heads(h, fc, a_l, a_r): one operator for
+        the projection and the per-head attention terms."""
+        el, er, zv = n.inputsAt(0).node(), n.inputsAt(1).node(), n.inputsAt(2).node()
+        shape = self.const_of(zv.inputsAt(1))
+        mm = zv.inputsAt(0).node()
+        if mm.kind() != "aten::mm" or not isinstance(shape, list) or len(shape) != 3 \
+                or shape[0] != -1 or not self.single_use(mm.output()):
+            return False
+        h, fc = mm.inputsAt(0), mm.inputsAt(1)
+        if self.where(h) != NODE or self.where(fc) != SHARED:
+            return False
+        vecs = []
+        for t in (el, er):
+            if t.kind() != "aten::sum" or t.inputsSize() != 4 or \
+                    self.const_of(t.inputsAt(1)) != [2] or self.const_of(t.inputsAt(2)) is not True \
+                    or not self.single_use(t.output()):
+                return False
+            mul = t.inputsAt(0).node()
+            if mul.kind() != "aten::mul" or not self.single_use(mul.output()):
+                return False
+            a, b = mul.inputsAt(0), mul.inputsAt(1)
+            if a.unique() == zv.output().unique() and self.where(b) == SHARED:
+                vecs.append((b, mul))
+            elif b.unique() == zv.output().unique() and self.where(a) == SHARED:
+                vecs.append((a, mul))
+            else:
+                return False
+        # the attention vectors must already exist where the product is computed
+        for v, _ in vecs:
+            if v.node().kind() != "prim::Param" and not v.node().isBefore(mm):
+                return False
+        heads, dim = self.const(int(shape[1]), mm), self.const(int(shape[2]), mm)
+        node = self.G.create("my_ops::gat_project_heads",
+                             [h, fc, vecs[0][0], vecs[1][0], heads, dim], 3)
+        node.insertBefore(mm)
+        for o in node.outputs():
+            o.setType(torch._C.TensorType.get())
+            self.res[o.unique()] = NODE
+        outs = list(node.outputs())
+        zv.output().replaceAllUsesWith(outs[0])
+        el.output().replaceAllUsesWith(outs[1])
+        er.output().replaceAllUsesWith(outs[2])
+        for dead in (el, er, vecs[0][1], vecs[1][1], zv, mm):
+            dead.destroy()
+        return True
 
     # ------------------------------------------------- late fusion ----
     def late_fusion(self) -> bool:

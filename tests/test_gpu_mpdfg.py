@@ -62,14 +62,16 @@ def test_gat_plan(device, level, width):
     assert_close(g.ndata['h'].cpu().numpy(), want, 2e-5, f"GAT plan level {level}")
 
 
-@pytest.mark.parametrize("level", [0, 1, 2])
-def test_multi_head_gat_plan(device, level):
+@pytest.mark.parametrize("level,k_in", [(0, 24), (1, 24), (2, 24), (2, 200)])
+def test_multi_head_gat_plan(device, level, k_in):
+    """Four heads of width 16 at every level; at level 2 the plan is
+    gat_project_heads + gat_aggregate (two input widths)."""
     rng = np.random.default_rng(25)
     n, src, dst = _homo(rng)
     g = GraphData(prepare_graph(src, dst, n, device))
     heads, d = 4, 16
-    h = rng.standard_normal((n, 24), dtype=np.float32)
-    fc = (rng.standard_normal((24, heads * d)) / 5).astype(np.float32)
+    h = rng.standard_normal((n, k_in), dtype=np.float32)
+    fc = (rng.standard_normal((k_in, heads * d)) / 5).astype(np.float32)
     a_l, a_r = ((rng.standard_normal((1, heads, d)) / 4).astype(np.float32) for _ in range(2))
     g.ndata['h'] = _t(h, device)
     update_all(g, mpdfg_builder(U.gat4_message, U.gat4_reduce, opt_level=level),
