@@ -545,6 +545,37 @@ torch::Tensor gat_aggregate(torch::Tensor el, torch::Tensor er, torch::Tensor z,
   return out;
 }
 
+// gat_aggregate that may recompute the source term from the gathered rows: with
+// a_l (heads * dim elements) at hand, a table of source terms of 16 MB or more
+// (it no longer stays cached, and gathering it costs a memory sector per edge)
+// is not read at all; smaller tables take the ordinary pass.
+torch::Tensor gat_aggregate_al(torch::Tensor a_l, torch::Tensor el, torch::Tensor er,
+                               torch::Tensor z, double negative_slope, const GraphPtr &graph) {
+  constexpr int64_t kTableLimit = 16 << 20;
+  if (el.numel() * 4 < kTableLimit) return gat_aggregate(el, er, z, negative_slope, graph);
+  check_input(er, "er");
+  check_input(z, "z");
+  TORCH_CHECK(a_l.is_cuda(), "a_l must be a CUDA tensor");
+  const int dt = feat_dtype(z, "z");
+  TORCH_CHECK(er.scalar_type() == at::kFloat, "er must be float32");
+  const int64_t heads = feat_dim(er), feat = feat_dim(z);
+  TORCH_CHECK(heads > 0 && feat % heads == 0 && a_l.numel() == feat, "inconsistent head count");
+  TORCH_CHECK(er.size(0) == graph->num_nodes && z.size(0) == graph->num_nodes,
+              "inputs must have one row per node");
+  torch::Tensor al = a_l.to(at::kFloat).contiguous();
+  const auto &side = graph->side(false);
+  torch::Tensor out = torch::empty(out_shape(graph->num_nodes, z), z.options());
+  torch::Tensor ws = graph->workspace(ga_gat_workspace_bytes(graph->num_edges, feat, heads));
+  const int rc = ga_gat_aggregate_from_z(
+      graph->in_pointer.data_ptr<int>(), side.rows.data_ptr<int>(),
+      graph->in_node_indices.data_ptr<int>(), al.data_ptr<float>(), er.data_ptr<float>(),
+      z.data_ptr(), out.data_ptr(), graph->num_nodes, graph->num_edges, heads, feat / heads,
+      (float)negative_slope, dt, ws.data_ptr(), (size_t)ws.numel(), current_stream(out));
+  if (rc == GA_EUNSUPPORTED) return gat_aggregate(el, er, z, negative_slope, graph);
+  check_ga(rc, "ga_gat_aggregate_from_z");
+  return out;
+}
+
 // SegmentSoftmax -> mul -> SpMMEdge (examples/HGT/HGT.py:50-53) in one pass:
 // out[v] = sum over in-edges e of softmax_v(logits)[e] * messages[e]
 torch::Tensor edge_softmax_sum(torch::Tensor logits, torch::Tensor messages,
@@ -736,6 +767,9 @@ static auto registry =
         .op("my_ops::gat_aggregate(Tensor el, Tensor er, Tensor z, float slope, " GRAPH_T
             " g) -> Tensor y",
             &gat_aggregate)
+        .op("my_ops::gat_aggregate_al(Tensor a_l, Tensor el, Tensor er, Tensor z, float slope, "
+            GRAPH_T " g) -> Tensor y",
+            &gat_aggregate_al)
         .op("my_ops::linear_attn(Tensor x, Tensor w, Tensor a_l, Tensor a_r) -> "
             "(Tensor z, Tensor el, Tensor er)",
             &linear_attn)

@@ -465,6 +465,12 @@ class _Rewriter:
         er.output().replaceAllUsesWith(outs[2])
         for dead in (el, er, vecs[0][1], vecs[1][1], zv, mm):
             dead.destroy()
+        # with a_l at hand the aggregation can skip a large table of source terms
+        agg = self.make("my_ops::gat_aggregate_al",
+                        [vecs[0][0], outs[1], outs[2], outs[0], n.inputsAt(3), self.dglgraph],
+                        n, NODE)
+        n.output().replaceAllUsesWith(agg)
+        n.destroy()
         return True
 
     # ------------------------------------------------- late fusion ----

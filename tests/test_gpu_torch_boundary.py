@@ -99,6 +99,28 @@ def test_linear_attn_op(setup, device):
     assert_close(er.cpu().numpy(), np.einsum("nhd,hd->nh", zr.reshape(n, 2, 32), ar), TOL_F32, "er")
 
 
+def test_gat_aggregate_al_small_and_large_tables(setup, device):
+    """gat_aggregate_al = gat_aggregate for a small table of source terms; with
+    1.1 M nodes x 4 heads (17.6 MB) it takes the pass that recomputes the term from
+    the gathered rows, and must still equal gat_aggregate fed with el = z . a_l."""
+    sg, arr, rng = setup
+    heads, d = 4, 16
+    for n_nodes, n_edges, graph in ((arr.num_nodes, None, sg), (1_100_000, 3_000_000, None)):
+        if graph is None:
+            src = rng.integers(0, n_nodes, n_edges, dtype=np.int64)
+            dst = rng.integers(0, n_nodes // 2, n_edges, dtype=np.int64)     # upper half: no in-edges
+            graph = torch_boundary.script_graph(prepare_graph(src, dst, n_nodes, device=device))
+        z = torch.randn(n_nodes, heads, d, device=device)
+        a_l = torch.randn(1, heads, d, device=device) / 4
+        er = torch.randn(n_nodes, heads, 1, device=device)
+        el = (z * a_l).sum(2, keepdim=True)
+        want = torch.ops.my_ops.gat_aggregate(el, er, z, 0.2, graph)
+        got = torch.ops.my_ops.gat_aggregate_al(a_l, el, er, z, 0.2, graph)
+        assert got.shape == want.shape == (n_nodes, heads, d)
+        err = float((got - want).abs().max() / want.abs().max())
+        assert err <= 4 * TOL_F32, f"gat_aggregate_al differs by {err:.2e} at {n_nodes} nodes"
+
+
 def test_error_convention(setup, device):
     sg, arr, rng = setup
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):

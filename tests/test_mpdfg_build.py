@@ -87,7 +87,7 @@ def test_multi_head_attention_reaches_the_fused_kernel():
     plan = mpdfg_builder(U.gat4_message, U.gat4_reduce, opt_level=2)
     k = plan.op_kinds()
     ours = [x for x in k if x.startswith("my_ops::")]
-    assert ours == ["my_ops::gat_project_heads", "my_ops::gat_aggregate"]   # two kernels
+    assert ours == ["my_ops::gat_project_heads", "my_ops::gat_aggregate_al"]   # two kernels
     assert "aten::mm" not in k and "aten::view" not in k and "aten::sum" not in k
     plan1 = mpdfg_builder(U.gat4_message, U.gat4_reduce, opt_level=1).op_kinds()
     # at level 1 the per-head terms are already computed on node data
