@@ -180,6 +180,29 @@ def main():
         lg = rnd(E, H)
         report("c5", "segment_softmax H=4 f32", lambda: ops.SegmentSoftmax(lg, 1, None, g),
                4 * (N + 1) + 8 * E * H)
+        # the whole three-layer network (100 -> 256 -> 256 -> 256, 4 heads x 64, elu
+        # between layers) compiled from its user-defined functions
+        from graphiler_amd.examples import udf
+        from graphiler_amd.mpdfg import GraphData, mpdfg_builder, update_all
+        plan = mpdfg_builder(udf.gat4x64_message, udf.gat4_reduce, opt_level=2)
+        gd = GraphData(g)
+        x0 = rnd(N, 100, dtype=dt)
+        params = [(rnd(k, F, dtype=dt) / 16, rnd(1, H, F // H) / 8, rnd(1, H, F // H) / 8)
+                  for k in (100, F, F)]
+
+        def network():
+            x = x0
+            for fc, a_l, a_r in params:
+                gd.ndata["h"] = x
+                out = update_all(gd, plan, msg_params=(fc, a_l, a_r))["h"]
+                x = torch.nn.functional.elu(out).view(N, F)
+            return x
+
+        layer_bytes = lambda k: (N * (k + F) * b + k * F * b +
+                                 4 * (N + 1) + E * (4 + F * b) + N * (H * 4 + F * b))
+        report("c5", "3-layer GAT compiled from UDFs (gat_project_heads + gat_aggregate_al per layer)",
+               network, sum(layer_bytes(k) for k in (100, F, F)),
+               sum(2 * N * k * F for k in (100, F, F)))
         al, ar = rnd(H, F // H), rnd(H, F // H)
         bl, br = rnd(F, H, dtype=dt), rnd(F, H, dtype=dt)     # block-diagonal (F, H) forms
         for K in (100, 256):          # first and hidden layers

@@ -43,6 +43,16 @@ def gat4_message(edges: EdgeBatchDummy, fc_weight, attn_l, attn_r):
     return {'z': z_src, 'e': F.leaky_relu(el + er, 0.2)}
 
 
+def gat4x64_message(edges: EdgeBatchDummy, fc_weight, attn_l, attn_r):
+    """The same layer with four heads of width 64 (the 256-wide layers of the
+    products-sized GAT configuration); attn_l / attn_r (1, 4, 64)."""
+    z_src = torch.mm(edges.src['h'], fc_weight).view(-1, 4, 64)
+    z_dst = torch.mm(edges.dst['h'], fc_weight).view(-1, 4, 64)
+    el = torch.sum(z_src * attn_l, dim=2, keepdim=True)
+    er = torch.sum(z_dst * attn_r, dim=2, keepdim=True)
+    return {'z': z_src, 'e': F.leaky_relu(el + er, 0.2)}
+
+
 def gat4_reduce(nodes: NodeBatchDummy):
     alpha = torch.softmax(nodes.mailbox['e'], dim=1)             # over the in-edges, per head
     return {'h': torch.sum(alpha * nodes.mailbox['z'], dim=1)}
