@@ -4,14 +4,15 @@ rows, both fused GAT passes and the projection with attention terms, each on a
 random typed graph with random head counts and widths (including shapes the
 kernels refuse, where the wrappers must fall back or say GA_EUNSUPPORTED),
 against numpy float64 and the oracle.  Seeds are fixed; a sweep of 2,300 further
-seeds of the same generator passed when this file was written."""
+seeds of the same generator passed when this file was written.  A second test
+does the same for the reference's own operators on random graphs."""
 import numpy as np
 import pytest
 import torch
 import oracle
 from graphiler_amd import capi, ops, prepare_graph
 from graphiler_amd.graph import build_graph_arrays
-from helpers import to_bf16_f32
+from helpers import rel_err, to_bf16_f32
 pytestmark = pytest.mark.gpu
 
 def rel(got, ref):
@@ -130,3 +131,70 @@ def test_random_shapes(device, seed):
             assert r9 <= 0.0001, ('proj er', r9)
         except capi.GraphilerError as err:
             assert err.code == capi.GA_EUNSUPPORTED
+
+@pytest.mark.parametrize('seed', range(1, 65))
+def test_random_graphs_core_operators(device, seed):
+    """The reference's operators on random graphs (uniform, Zipf-skewed or
+    pre-sorted destinations; 0 to 20,000 edges), random head counts and widths,
+    fp32 or bf16: every SpMM operator x reducer, the out-adjacency form, SDDMM
+    add / sub / mul / div (bit-exact) and dot, multi-head softmax, the gather and
+    the device-side graph preparation (bit-exact)."""
+    dev = device
+
+    def D(a, bf16=False):
+        t = torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+        return t.bfloat16() if bf16 else t
+    rng = np.random.default_rng(seed)
+    bf16 = bool(rng.integers(0, 2))
+    tol = 0.02 if bf16 else 2e-05
+    n = int(rng.integers(1, 600))
+    e = int(rng.choice([0, 1, 5, 60, 700, 5000, 20000]))
+    src = rng.integers(0, n, e, dtype=np.int64)
+    kind = rng.integers(0, 3)
+    if kind == 0:
+        dst = rng.integers(0, n, e, dtype=np.int64)
+    elif kind == 1:
+        dst = (rng.zipf(1.6, e) % n).astype(np.int64)
+    else:
+        dst = np.sort(rng.integers(0, max(1, n // 3), e, dtype=np.int64))
+    g = prepare_graph(src, dst, n, device=dev)
+    arr = build_graph_arrays(src, dst, n)
+    heads = int(rng.choice([1, 1, 2, 4, 8]))
+    dim = int(rng.choice([1, 2, 3, 4, 8, 16, 17, 32, 64, 128]))
+    feat = heads * dim
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    m = rng.standard_normal((e, feat), dtype=np.float32)
+    w = rng.uniform(0.2, 2.0, (e, heads)).astype(np.float32)
+    if bf16:
+        (x, m) = (to_bf16_f32(x), to_bf16_f32(m))
+    op = str(rng.choice(['copy_u', 'copy_e', 'u_mul_e', 'u_add_e', 'u_sub_e', 'u_div_e']))
+    red = str(rng.choice(['sum', 'max', 'min']))
+    u = m if op == 'copy_e' else x
+    ww = None if op in ('copy_u', 'copy_e') else w
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices, u, ww, op=op, reduce=red, heads=heads)
+    got = ops.spmm(g, op, red, D(u, bf16), None if ww is None else D(ww))
+    r = rel_err(got.float().cpu().numpy().reshape(ref.shape), ref)
+    assert r <= tol, (op, red, r)
+    ref = oracle.spmm(arr.out_pointer, arr.out_node_indices, arr.out_edge_indices, x, w, op='u_mul_e', heads=heads)
+    got = ops.gspmm_dst_mul_e_sum(D(x, bf16), D(w), [1], False, None, g)
+    r = rel_err(got.float().cpu().numpy().reshape(ref.shape), ref)
+    assert r <= tol, ('dst_mul_e', r)
+    uu = rng.standard_normal((n, heads), dtype=np.float32)
+    vv = rng.standard_normal((n, heads), dtype=np.float32)
+    got = ops.gsddmm_u_add_v_mul_alpha(D(uu), D(vv), 1, g)
+    assert np.array_equal(got.cpu().numpy(), oracle.sddmm_u_add_v(src, dst, uu, vv)), 'u_add_v'
+    sop = str(rng.choice(['sub', 'mul', 'div']))
+    got = ops.gsddmm_u_op_v(sop, D(uu), D(vv + 3), g)
+    assert np.array_equal(got.cpu().numpy(), oracle.sddmm_u_op_v(sop, src, dst, uu, vv + 3)), 'u_op_v'
+    k3 = x.reshape(n, heads, dim)
+    got = ops.gsddmm_u_dot_v(D(k3, bf16), D(k3, bf16), g)
+    r = rel_err(got.cpu().numpy(), oracle.sddmm_u_dot_v(src, dst, k3, k3))
+    assert r <= 2e-05, ('dot', r)
+    lg = (rng.standard_normal((e, heads)) * 4).astype(np.float32)
+    got = ops.SegmentSoftmax(D(lg), 1, None, g)
+    r = rel_err(got.cpu().numpy(), oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, lg))
+    assert r <= 2e-05, ('softmax', r)
+    got = ops.BroadcastSrcNode(D(x, bf16), g)
+    assert np.array_equal(got.float().cpu().numpy(), x[src]), 'gather'
+    for (a, b) in ((g.in_pointer, arr.in_pointer), (g.in_node_indices, arr.in_node_indices), (g.in_edge_indices, arr.in_edge_indices), (g.out_pointer, arr.out_pointer), (g.out_node_indices, arr.out_node_indices), (g.out_edge_indices, arr.out_edge_indices)):
+        assert np.array_equal(a.cpu().numpy(), b), 'prep'
