@@ -5,25 +5,64 @@
 // examples/GAT/GAT.py:25-29 after the split / reorder passes) as one kernel, so
 // Z is written once and never re-read for the attention terms.
 //
-// Tall-skinny GEMM on v_mfma_f32_16x16x4_f32: a workgroup (4 waves) owns 128
-// rows, each wave 32 rows (2 tiles of 16) x 64 columns per pass.  Both operands
-// go global -> registers -> LDS in slices of 32 k: the MFMA operand layout puts
-// the 16 rows of a tile on 16 adjacent lanes, so loading X straight into that
-// layout makes every lane its own cache access (the address unit then bounds
-// the kernel at well under half the MFMA rate); staged through LDS, adjacent
-// lanes read adjacent addresses of a row and the layout change costs one
-// 16-byte LDS read per lane and 16 k.  Two register sets hold the slices one
-// and two ahead of the one being multiplied, two LDS buffers the current and
-// the next slice, so a slice costs one barrier and its global loads have two
-// slices of MFMAs to arrive.  Accumulators come out as D[row][col] with 16
-// adjacent lanes on 16 adjacent columns: Z stores coalesce, and the per-head
-// dot products need one 16-lane DPP sum per row and head.
+// Tall-skinny GEMM with fp32 operands and fp32 results on the bf16 matrix
+// instruction (v_mfma_f32_16x16x32_bf16, 16x the rate of the fp32 one): every
+// operand value is split exactly into three bf16 pieces, x = x0 + x1 + x2 (8
+// significant bits each, 24 in all), and the product is accumulated in fp32 from
+// the six piece products of weight >= 2^-16, x0w0 + x0w1 + x1w0 + x1w1 + x0w2 +
+// x2w0; each piece product is exact in fp32 and the three dropped ones are below
+// 2^-24 of |x||w|, i.e. below the rounding of an fp32 product.  Measured against
+// float64 the result is as close as the fp32 instruction's (max error / max |Z|
+// 8e-7 against 1.2e-6 at K = 602).  Non-finite inputs give NaN (inf - inf in the
+// split) where fp32 products may give inf.
+//
+// A workgroup (4 waves) owns up to 128 rows, each wave up to 32 rows (2 tiles of
+// 16) x 64 columns per pass.  Both operands go global -> registers -> LDS in
+// slices of 32 k: the MFMA operand layout puts the 16 rows of a tile on 16
+// adjacent lanes, so loading X straight into that layout makes every lane its
+// own cache access; staged through LDS, adjacent lanes read adjacent addresses
+// of a row.  X is staged as fp32 and split after the operand read (each value is
+// consumed by exactly one lane); W is split when it is committed to LDS, as three
+// [column][k] bf16 arrays, so an operand read is one 16-byte LDS read per piece.
+// Two register sets hold the slices one and two ahead of the one being
+// multiplied, two LDS buffers the current and the next slice, so a slice costs
+// one barrier and its global loads have two slices of work to arrive.
+// Accumulators come out as D[row][col] with 16 adjacent lanes on 16 adjacent
+// columns: Z stores coalesce, and the per-head dot products need one 16-lane DPP
+// sum per row and head.
+//
+// Rows per wave (<= 32) are chosen by the host so that the workgroups fill a
+// whole number of rounds over the device (two workgroups per CU): the kernel is
+// bound by memory, a wave with 29 of its 32 rows real reads 29/32 of the bytes,
+// and a last round that is half empty costs more than the idle tile rows.
 #include "common.h"
 
 namespace ga {
 namespace {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// x = p0 + p1 + p2 exactly, each piece a bf16 (the top 8 significant bits of
+// what the pieces before it leave); eight values -> three packed operands.
+__device__ __forceinline__ void split8(const float (&v)[8], uint4 &p0, uint4 &p1, uint4 &p2) {
+  uint32_t a[8], b[8], c[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    a[j] = __float_as_uint(v[j]);
+    const float r1 = v[j] - __uint_as_float(a[j] & 0xffff0000u);
+    b[j] = __float_as_uint(r1);
+    const float r2 = r1 - __uint_as_float(b[j] & 0xffff0000u);
+    c[j] = __float_as_uint(r2);
+  }
+  constexpr uint32_t hi = 0x07060302u;                   // high halves of (S1, S0)
+  p0 = uint4{__builtin_amdgcn_perm(a[1], a[0], hi), __builtin_amdgcn_perm(a[3], a[2], hi),
+             __builtin_amdgcn_perm(a[5], a[4], hi), __builtin_amdgcn_perm(a[7], a[6], hi)};
+  p1 = uint4{__builtin_amdgcn_perm(b[1], b[0], hi), __builtin_amdgcn_perm(b[3], b[2], hi),
+             __builtin_amdgcn_perm(b[5], b[4], hi), __builtin_amdgcn_perm(b[7], b[6], hi)};
+  p2 = uint4{__builtin_amdgcn_perm(c[1], c[0], hi), __builtin_amdgcn_perm(c[3], c[2], hi),
+             __builtin_amdgcn_perm(c[5], c[4], hi), __builtin_amdgcn_perm(c[7], c[6], hi)};
+}
 
 constexpr int kRT = 2;                                   // 16-row tiles per wave
 constexpr int kWaveRows = kRT * 16;                      // 32
@@ -32,7 +71,7 @@ constexpr int kCB = 4;                                   // 16-column blocks per
 constexpr int kPassCols = kCB * 16;                      // 64
 constexpr int kSliceK = 32;                              // k per LDS slice
 constexpr int kXs = kSliceK + 4;                         // LDS row stride of the X tile
-constexpr int kWs = kPassCols + 4;                       // LDS row stride of the W tile
+constexpr int kWb = kSliceK / 2 + 4;                      // LDS column stride of a W piece, in bf16 pairs
 
 template <int VK> struct XVec;
 template <> struct XVec<4> { using type = float4; };
@@ -55,17 +94,16 @@ linear_attn_kernel(
     const float *__restrict__ X, const float *__restrict__ W,
     const float *__restrict__ a_l, const float *__restrict__ a_r,
     float *__restrict__ Z, float *__restrict__ el, float *__restrict__ er,
-    int64_t rows, int K, int M, int heads) {
+    int64_t rows, int K, int M, int heads, int rpw) {
   using xvec_t = typename XVec<VK>::type;
   __shared__ __attribute__((aligned(16))) float xs[2][kWgRows * kXs];
-  __shared__ __attribute__((aligned(16))) float ws[2][kSliceK * kWs];
+  __shared__ __attribute__((aligned(16))) uint32_t wb[2][3][kPassCols * kWb];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int lr = lane & 15, lk = lane >> 4;
   const int col0 = blockIdx.y * kPassCols;               // first column of the pass
-  const int64_t wg_row0 = (int64_t)blockIdx.x * kWgRows;
-  const int64_t wrow0 = wg_row0 + wave * kWaveRows;
-  const bool vec_w = (M & 3) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0;
+  const int64_t wg_row0 = (int64_t)blockIdx.x * (kBlock / kWave) * rpw;   // rpw rows per wave
+  const int64_t wrow0 = wg_row0 + wave * rpw;
   const int n_slices = (K + kSliceK - 1) / kSliceK;
 
   // X slice: 128 rows x 32 k in vectors of VK floats, kVpr per row; thread i
@@ -75,37 +113,30 @@ linear_attn_kernel(
   constexpr int kVpr = kSliceK / VK;                     // vectors per row and slice
   constexpr int kXPieces = kWgRows * kVpr / kBlock;      // 4 / 8 / 16 per thread
   constexpr int kRowStep = kBlock / kVpr;                // rows between a thread's vectors
-  constexpr int kWPieces = kSliceK * (kPassCols / 4) / kBlock;  // float4 of W: 2
   struct Stage {
     xvec_t x[kXPieces];
-    float4 w[kWPieces];
+    float w[8];
   };
+  const int wc = threadIdx.x & 63, wkg = threadIdx.x >> 6;   // column, group of 8 k
   const int xr = threadIdx.x / kVpr, xc = (threadIdx.x % kVpr) * VK;
   const float *xbase[kXPieces];
 #pragma unroll
-  for (int j = 0; j < kXPieces; ++j)
-    xbase[j] = X + min(wg_row0 + xr + j * kRowStep, rows - 1) * K;
-  const bool w_cols_plain = vec_w && col0 + kPassCols <= M;     // uniform
+  for (int j = 0; j < kXPieces; ++j) {
+    // LDS row L holds row min(L % 32, rpw - 1) of wave L / 32 (idle tile rows repeat
+    // the wave's last row: a cache hit, never stored)
+    const int L = xr + j * kRowStep;
+    xbase[j] = X + min(wg_row0 + (L >> 5) * rpw + min(L & 31, rpw - 1), rows - 1) * K;
+  }
 
   auto fetch = [&](int sl, Stage &st) {
     const int kc = min(sl * kSliceK + xc, K - VK);
 #pragma unroll
     for (int j = 0; j < kXPieces; ++j)
       st.x[j] = *reinterpret_cast<const xvec_t *>(xbase[j] + kc);
+    const float *wsrc = W + min(col0 + wc, M - 1);
 #pragma unroll
-    for (int j = 0; j < kWPieces; ++j) {
-      const int i = threadIdx.x + j * kBlock;
-      const int kk = min(sl * kSliceK + (i >> 4), K - 1), cc = col0 + (i & 15) * 4;
-      const float *src = W + (int64_t)kk * M;
-      if (w_cols_plain) {
-        st.w[j] = *reinterpret_cast<const float4 *>(src + cc);
-      } else {
-        st.w[j].x = src[min(cc, M - 1)];
-        st.w[j].y = src[min(cc + 1, M - 1)];
-        st.w[j].z = src[min(cc + 2, M - 1)];
-        st.w[j].w = src[min(cc + 3, M - 1)];
-      }
-    }
+    for (int j = 0; j < 8; ++j)
+      st.w[j] = wsrc[(int64_t)min(sl * kSliceK + wkg * 8 + j, K - 1) * M];
   };
   auto commit = [&](int sl, const Stage &st) {
     const int buf = sl & 1;
@@ -116,18 +147,16 @@ linear_attn_kernel(
       if (!xin) v = xvec_t{};
       *reinterpret_cast<xvec_t *>(&xs[buf][(xr + j * kRowStep) * kXs + xc]) = v;
     }
+    float wv[8];
+    const bool cin = col0 + wc < M;
 #pragma unroll
-    for (int j = 0; j < kWPieces; ++j) {
-      const int i = threadIdx.x + j * kBlock;
-      float4 v = st.w[j];
-      const int cc = col0 + (i & 15) * 4;
-      const bool kin = sl * kSliceK + (i >> 4) < K;
-      v.x = kin && cc < M ? v.x : 0.0f;
-      v.y = kin && cc + 1 < M ? v.y : 0.0f;
-      v.z = kin && cc + 2 < M ? v.z : 0.0f;
-      v.w = kin && cc + 3 < M ? v.w : 0.0f;
-      *reinterpret_cast<float4 *>(&ws[buf][(i >> 4) * kWs + (i & 15) * 4]) = v;
-    }
+    for (int j = 0; j < 8; ++j)
+      wv[j] = cin && sl * kSliceK + wkg * 8 + j < K ? st.w[j] : 0.0f;
+    uint4 p0, p1, p2;
+    split8(wv, p0, p1, p2);
+    *reinterpret_cast<uint4 *>(&wb[buf][0][wc * kWb + wkg * 4]) = p0;
+    *reinterpret_cast<uint4 *>(&wb[buf][1][wc * kWb + wkg * 4]) = p1;
+    *reinterpret_cast<uint4 *>(&wb[buf][2][wc * kWb + wkg * 4]) = p2;
   };
 
   floatx4 acc[kRT][kCB];
@@ -136,55 +165,43 @@ linear_attn_kernel(
 #pragma unroll
     for (int cb = 0; cb < kCB; ++cb) acc[t][cb] = floatx4{0, 0, 0, 0};
 
-  // MFMA operands of the lane: X[row lr of tile t][k = kb*16 + lk*4 + q] against
-  // W[k = kb*16 + lk*4 + q][column cb*16 + lr], q = 0..3 (the k order inside a
-  // block of 16 is permuted identically for both operands)
-  const int xl_ofs = (wave * kWaveRows + lr) * kXs + lk * 4;
-  const int wl_ofs = lk * 4 * kWs + lr;
-  struct Frag {
-    float4 x[kRT];
-    float w[4][kCB];
-  };
-  auto read_frag = [&](int buf, int kb, Frag &f) {
-    const float *xl = &xs[buf][xl_ofs + kb * 16];
-    const float *wl = &ws[buf][wl_ofs + kb * 16 * kWs];
-#pragma unroll
-    for (int t = 0; t < kRT; ++t) f.x[t] = *reinterpret_cast<const float4 *>(xl + t * 16 * kXs);
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int cb = 0; cb < kCB; ++cb) f.w[q][cb] = wl[q * kWs + cb * 16];
-  };
-  auto mma = [&](const Frag &f) {
+  const int xl_ofs = (wave * kWaveRows + lr) * kXs + lk * 8;
+  const int wl_ofs = lr * kWb + lk * 4;                  // in uint32 (pairs of bf16)
+  auto step = [&](int sl, Stage &next) {
+    const int buf = sl & 1;
+    float4 xa[kRT][2];
+    uint4 wf[3][kCB];
 #pragma unroll
     for (int t = 0; t < kRT; ++t) {
-      const float xv[4] = {f.x[t].x, f.x[t].y, f.x[t].z, f.x[t].w};
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-#pragma unroll
-        for (int cb = 0; cb < kCB; ++cb)
-          acc[t][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[q], f.w[q][cb], acc[t][cb], 0, 0, 0);
+      xa[t][0] = *reinterpret_cast<const float4 *>(&xs[buf][xl_ofs + t * 16 * kXs]);
+      xa[t][1] = *reinterpret_cast<const float4 *>(&xs[buf][xl_ofs + t * 16 * kXs + 4]);
     }
-  };
-  // One slice.  Waves of one SIMD run this loop in step with each other, so a
-  // stall is not covered by another wave's MFMAs: each wave hides its own.  The
-  // fragments of a block are read from LDS while the block before it multiplies;
-  // the next slice's registers go to the other LDS buffer (last read a slice ago,
-  // before that slice's barrier) and the slice three ahead is fetched into the
-  // registers just freed, all under the first block's MFMAs.
-  Frag f0, f1;
-  auto step = [&](int sl, Stage &next) {
-    read_frag(sl & 1, 1, f1);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(f0);
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+#pragma unroll
+      for (int cb = 0; cb < kCB; ++cb)
+        wf[p][cb] = *reinterpret_cast<const uint4 *>(&wb[buf][p][wl_ofs + cb * 16 * kWb]);
     commit(sl + 1, next);
     fetch(sl + 3, next);
-    __builtin_amdgcn_sched_barrier(0);
+    uint4 xp[kRT][3];
+#pragma unroll
+    for (int t = 0; t < kRT; ++t) {
+      const float v[8] = {xa[t][0].x, xa[t][0].y, xa[t][0].z, xa[t][0].w,
+                          xa[t][1].x, xa[t][1].y, xa[t][1].z, xa[t][1].w};
+      split8(v, xp[t][0], xp[t][1], xp[t][2]);
+    }
+    // small terms first; eight independent accumulators between dependent MFMAs
+    constexpr int px[6] = {2, 0, 1, 1, 0, 0}, pw[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+    for (int q = 0; q < 6; ++q)
+#pragma unroll
+      for (int t = 0; t < kRT; ++t)
+#pragma unroll
+        for (int cb = 0; cb < kCB; ++cb)
+          acc[t][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(bf16x8, xp[t][px[q]]), __builtin_bit_cast(bf16x8, wf[pw[q]][cb]),
+              acc[t][cb], 0, 0, 0);
     __syncthreads();
-    read_frag((sl + 1) & 1, 0, f0);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(f1);
-    __builtin_amdgcn_sched_barrier(0);
   };
 
   Stage sa, sb;                                          // even / odd slices
@@ -193,10 +210,6 @@ linear_attn_kernel(
   commit(0, sa);
   fetch(2, sa);
   __syncthreads();
-  read_frag(0, 0, f0);
-  // slices in pairs (the register sets alternate), an odd last one on its own:
-  // a conditional second half inside the loop would make the allocator copy
-  // the accumulators around on every trip
   int sl = 0;
   for (; sl + 1 < n_slices; sl += 2) {
     step(sl, sb);
@@ -220,8 +233,9 @@ linear_attn_kernel(
   for (int t = 0; t < kRT; ++t) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int64_t row = wrow0 + t * 16 + lk * 4 + r;
-      const bool live = row < rows;
+      const int wr = t * 16 + lk * 4 + r;                // row of the wave
+      const int64_t row = wrow0 + wr;
+      const bool live = wr < rpw && row < rows;
 #pragma unroll
       for (int cb = 0; cb < kCB; ++cb) {
         const int c = col0 + cb * 16 + lr;
@@ -256,6 +270,20 @@ linear_attn_kernel(
   }
 }
 
+// compute units of the current device (queried once per device)
+int device_cus() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+  }
+  return n;
+}
+
 }  // namespace
 }  // namespace ga
 
@@ -274,14 +302,24 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
   const int vk = (K % 4 == 0 && aligned(X, 16)) ? 4 : ((K % 2 == 0 && aligned(X, 8)) ? 2 : 1);
   const int64_t dph = M / heads;
   if (attn && !(dph == 16 || dph == 32 || dph == 64)) return GA_EUNSUPPORTED;
-  const int64_t gx = (rows + kWgRows - 1) / kWgRows;
+  // rows per wave: 32, or fewer when that fills the last round of workgroups (two
+  // per CU) instead of leaving it part empty
+  int64_t rpw = kWaveRows;
+  constexpr int64_t kWaves = kBlock / kWave;
+  const int64_t slots = 2 * (int64_t)device_cus();
+  const int64_t full = (rows + kWgRows - 1) / kWgRows;
+  if (full > slots) {
+    const int64_t rounds = (full + slots - 1) / slots;
+    rpw = (rows + rounds * slots * kWaves - 1) / (rounds * slots * kWaves);
+  }
+  const int64_t gx = (rows + kWaves * rpw - 1) / (kWaves * rpw);
   const int64_t gy = (M + kPassCols - 1) / kPassCols;
   if (gx > 0x7fffffff || gy > 65535) return GA_EUNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
 #define GA_LAUNCH_LINEAR(ATTN, VK)                                                 \
   hipLaunchKernelGGL((linear_attn_kernel<ATTN, VK>), dim3((unsigned)gx, (unsigned)gy), \
                      dim3(kBlock), 0, s, X, W, a_l, a_r, Z, el, er, rows, (int)K,   \
-                     (int)M, (int)heads)
+                     (int)M, (int)heads, (int)rpw)
   if (attn) {
     if (vk == 4) GA_LAUNCH_LINEAR(true, 4);
     else if (vk == 2) GA_LAUNCH_LINEAR(true, 2);

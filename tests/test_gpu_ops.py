@@ -697,7 +697,10 @@ def test_e_mul_e_sum(device):
 @pytest.mark.parametrize("rows,K,M,heads", [(1000, 602, 64, 1), (333, 77, 64, 2),
                                             (777, 64, 64, 4),
                                             (300, 100, 256, 4), (5000, 16, 32, 2),
-                                            (50, 8, 16, 1), (1, 4, 64, 1)])
+                                            (50, 8, 16, 1), (1, 4, 64, 1),
+                                            # more than one round of workgroups: fewer
+                                            # than 32 rows per wave (18 and 25 here)
+                                            (70001, 40, 64, 2), (200000, 33, 32, 1)])
 def test_linear_attn(device, rows, K, M, heads):
     rng = np.random.default_rng(K + M)
     x = rng.standard_normal((rows, K), dtype=np.float32)
