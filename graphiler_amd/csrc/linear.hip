@@ -16,8 +16,8 @@
 // 8e-7 against 1.2e-6 at K = 602).  Non-finite inputs give NaN (inf - inf in the
 // split) where fp32 products may give inf.
 //
-// A workgroup (4 waves) owns up to 128 rows, each wave up to 32 rows (2 tiles of
-// 16) x 64 columns per pass.  Both operands go global -> registers -> LDS in
+// A workgroup (4 waves) owns 128 rows, each wave 32 rows (2 tiles of 16) x 64
+// columns per pass.  Both operands go global -> registers -> LDS in
 // slices of 32 k: the MFMA operand layout puts the 16 rows of a tile on 16
 // adjacent lanes, so loading X straight into that layout makes every lane its
 // own cache access; staged through LDS, adjacent lanes read adjacent addresses
@@ -30,11 +30,6 @@
 // Accumulators come out as D[row][col] with 16 adjacent lanes on 16 adjacent
 // columns: Z stores coalesce, and the per-head dot products need one 16-lane DPP
 // sum per row and head.
-//
-// Rows per wave (<= 32) are chosen by the host so that the workgroups fill a
-// whole number of rounds over the device (two workgroups per CU): the kernel is
-// bound by memory, a wave with 29 of its 32 rows real reads 29/32 of the bytes,
-// and a last round that is half empty costs more than the idle tile rows.
 #include "common.h"
 
 namespace ga {
@@ -94,7 +89,7 @@ linear_attn_kernel(
     const float *__restrict__ X, const float *__restrict__ W,
     const float *__restrict__ a_l, const float *__restrict__ a_r,
     float *__restrict__ Z, float *__restrict__ el, float *__restrict__ er,
-    int64_t rows, int K, int M, int heads, int rpw) {
+    int64_t rows, int K, int M, int heads) {
   using xvec_t = typename XVec<VK>::type;
   __shared__ __attribute__((aligned(16))) float xs[2][kWgRows * kXs];
   __shared__ __attribute__((aligned(16))) uint32_t wb[2][3][kPassCols * kWb];
@@ -102,8 +97,8 @@ linear_attn_kernel(
   const int wave = threadIdx.x / kWave;
   const int lr = lane & 15, lk = lane >> 4;
   const int col0 = blockIdx.y * kPassCols;               // first column of the pass
-  const int64_t wg_row0 = (int64_t)blockIdx.x * (kBlock / kWave) * rpw;   // rpw rows per wave
-  const int64_t wrow0 = wg_row0 + wave * rpw;
+  const int64_t wg_row0 = (int64_t)blockIdx.x * kWgRows;
+  const int64_t wrow0 = wg_row0 + wave * kWaveRows;
   const int n_slices = (K + kSliceK - 1) / kSliceK;
 
   // X slice: 128 rows x 32 k in vectors of VK floats, kVpr per row; thread i
@@ -121,12 +116,8 @@ linear_attn_kernel(
   const int xr = threadIdx.x / kVpr, xc = (threadIdx.x % kVpr) * VK;
   const float *xbase[kXPieces];
 #pragma unroll
-  for (int j = 0; j < kXPieces; ++j) {
-    // LDS row L holds row min(L % 32, rpw - 1) of wave L / 32 (idle tile rows repeat
-    // the wave's last row: a cache hit, never stored)
-    const int L = xr + j * kRowStep;
-    xbase[j] = X + min(wg_row0 + (L >> 5) * rpw + min(L & 31, rpw - 1), rows - 1) * K;
-  }
+  for (int j = 0; j < kXPieces; ++j)
+    xbase[j] = X + min(wg_row0 + xr + j * kRowStep, rows - 1) * K;
 
   auto fetch = [&](int sl, Stage &st) {
     const int kc = min(sl * kSliceK + xc, K - VK);
@@ -233,9 +224,8 @@ linear_attn_kernel(
   for (int t = 0; t < kRT; ++t) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int wr = t * 16 + lk * 4 + r;                // row of the wave
-      const int64_t row = wrow0 + wr;
-      const bool live = wr < rpw && row < rows;
+      const int64_t row = wrow0 + t * 16 + lk * 4 + r;
+      const bool live = row < rows;
 #pragma unroll
       for (int cb = 0; cb < kCB; ++cb) {
         const int c = col0 + cb * 16 + lr;
@@ -270,20 +260,6 @@ linear_attn_kernel(
   }
 }
 
-// compute units of the current device (queried once per device)
-int device_cus() {
-  static int cached[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
-  if (n == 0) {
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
-  }
-  return n;
-}
-
 }  // namespace
 }  // namespace ga
 
@@ -302,24 +278,14 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
   const int vk = (K % 4 == 0 && aligned(X, 16)) ? 4 : ((K % 2 == 0 && aligned(X, 8)) ? 2 : 1);
   const int64_t dph = M / heads;
   if (attn && !(dph == 16 || dph == 32 || dph == 64)) return GA_EUNSUPPORTED;
-  // rows per wave: 32, or fewer when that fills the last round of workgroups (two
-  // per CU) instead of leaving it part empty
-  int64_t rpw = kWaveRows;
-  constexpr int64_t kWaves = kBlock / kWave;
-  const int64_t slots = 2 * (int64_t)device_cus();
-  const int64_t full = (rows + kWgRows - 1) / kWgRows;
-  if (full > slots) {
-    const int64_t rounds = (full + slots - 1) / slots;
-    rpw = (rows + rounds * slots * kWaves - 1) / (rounds * slots * kWaves);
-  }
-  const int64_t gx = (rows + kWaves * rpw - 1) / (kWaves * rpw);
+  const int64_t gx = (rows + kWgRows - 1) / kWgRows;
   const int64_t gy = (M + kPassCols - 1) / kPassCols;
   if (gx > 0x7fffffff || gy > 65535) return GA_EUNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
 #define GA_LAUNCH_LINEAR(ATTN, VK)                                                 \
   hipLaunchKernelGGL((linear_attn_kernel<ATTN, VK>), dim3((unsigned)gx, (unsigned)gy), \
                      dim3(kBlock), 0, s, X, W, a_l, a_r, Z, el, er, rows, (int)K,   \
-                     (int)M, (int)heads, (int)rpw)
+                     (int)M, (int)heads)
   if (attn) {
     if (vk == 4) GA_LAUNCH_LINEAR(true, 4);
     else if (vk == 2) GA_LAUNCH_LINEAR(true, 2);

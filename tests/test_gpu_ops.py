@@ -698,9 +698,11 @@ def test_e_mul_e_sum(device):
                                             (777, 64, 64, 4),
                                             (300, 100, 256, 4), (5000, 16, 32, 2),
                                             (50, 8, 16, 1), (1, 4, 64, 1),
-                                            # more than one round of workgroups: fewer
-                                            # than 32 rows per wave (18 and 25 here)
-                                            (70001, 40, 64, 2), (200000, 33, 32, 1)])
+                                            (70001, 40, 64, 2), (200000, 33, 32, 1),
+                                            # K % 4 == 2: rows start 0 or 8 bytes past a
+                                            # 16-byte boundary, alternately (8-byte vectors)
+                                            (257, 6, 16, 1), (300, 34, 64, 2),
+                                            (513, 98, 64, 4), (131, 30, 32, 1)])
 def test_linear_attn(device, rows, K, M, heads):
     rng = np.random.default_rng(K + M)
     x = rng.standard_normal((rows, K), dtype=np.float32)
@@ -715,6 +717,28 @@ def test_linear_attn(device, rows, K, M, heads):
     assert_close(er.cpu().numpy(), (zh * a[1]).sum(-1), 2 * TOL_F32, "linear er")
     z2 = ops.linear_attn(_dev(x, device), _dev(w, device))
     assert np.array_equal(z2.cpu().numpy(), z.cpu().numpy())
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3, 4])
+@pytest.mark.parametrize("K", [66, 602, 64, 37])
+def test_linear_attn_row_alignment(device, K, offset):
+    """The feature matrix at every 4-byte offset from a 16-byte boundary (a view
+    into a larger buffer): each offset selects another vector width of the row
+    loads."""
+    rows, M = 300, 64
+    rng = np.random.default_rng(K + offset)
+    x = rng.standard_normal((rows, K), dtype=np.float32)
+    w = datasets.glorot(rng, (K, M))
+    a = rng.standard_normal((2, 1, M), dtype=np.float32)
+    buf = torch.zeros(rows * K + 8, device=device)
+    xd = buf[offset:offset + rows * K].view(rows, K)
+    xd.copy_(_dev(x, device))
+    assert xd.data_ptr() % 16 == (4 * offset) % 16
+    z, el, er = ops.linear_attn(xd, _dev(w, device), _dev(a[0], device), _dev(a[1], device))
+    zr = x.astype(np.float64) @ w.astype(np.float64)
+    assert_close(z.cpu().numpy(), zr, TOL_F32, "linear z")
+    assert_close(el.cpu().numpy(), (zr * a[0]).sum(-1, keepdims=True), 2 * TOL_F32, "linear el")
+    assert_close(er.cpu().numpy(), (zr * a[1]).sum(-1, keepdims=True), 2 * TOL_F32, "linear er")
 
 
 @pytest.mark.parametrize("rows,K,M,heads,bf16", [
