@@ -23,6 +23,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
+from .. import ops
 from ..mpdfg import GraphData, mpdfg_builder, update_all
 from . import udf
 
@@ -88,7 +89,7 @@ class GCN:
         self.w2 = _param(rng, (hidden_dim, out_dim), device)
 
     def _layer(self, g, x, w, mode):
-        g.ndata['h'] = torch.mm(x, w)
+        g.ndata['h'] = torch.mm(x, w) if mode in EAGER else ops.linear(x, w)
         if mode in EAGER:
             src = g.graph.COO_src
             m = g.ndata['h'][src] * torch.pow(g.ndata['degree'][src], -0.5)

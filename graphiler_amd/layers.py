@@ -6,8 +6,8 @@ src/optimizer/fusion.cpp:15-145) and executes it in ``update_all``
 (python/graphiler/update_all.py:1-5).  The functions below are those
 opt-level-2 operator sequences written out by hand for the four example models,
 calling :mod:`graphiler_amd.ops`; the GAT projection uses the kernel that also
-produces the attention terms, other dense per-node linears stay on ``torch.mm``
-as in the reference plans.
+produces the attention terms, the GCN projection :func:`graphiler_amd.ops.linear`
+(the library's kernel at tall-and-narrow fp32 shapes, ``torch.mm`` otherwise).
 """
 from __future__ import annotations
 
@@ -23,7 +23,7 @@ def gcn_layer(g: DGLGraph, h: torch.Tensor, weight: torch.Tensor,
               relu: bool = True) -> torch.Tensor:
     """examples/GCN/GCN.py:21-27,39: h' = act(SpMMSrc((h @ W) * norm_src)),
     optionally scaled by ``norm_dst`` for the symmetric normalisation."""
-    m = torch.mm(h, weight) * norm_src
+    m = ops.linear(h, weight) * norm_src
     out = ops.SpMMSrc(m, [1], False, None, g)
     if norm_dst is not None:
         out = out * norm_dst

@@ -719,6 +719,21 @@ def test_linear_attn(device, rows, K, M, heads):
     assert np.array_equal(z2.cpu().numpy(), z.cpu().numpy())
 
 
+@pytest.mark.parametrize("rows,K,M", [(20000, 50, 64), (16384, 128, 41), (40000, 602, 16),
+                                      (1000, 50, 64), (20000, 50, 128)])
+def test_linear_dispatch(device, rows, K, M):
+    """ops.linear: own kernel at tall-and-narrow fp32 shapes, the vendor GEMM
+    elsewhere; the same product either way."""
+    rng = np.random.default_rng(rows + K + M)
+    x = rng.standard_normal((rows, K), dtype=np.float32)
+    w = datasets.glorot(rng, (K, M))
+    got = ops.linear(_dev(x, device), _dev(w, device))
+    assert_close(got.cpu().numpy(), x.astype(np.float64) @ w.astype(np.float64), TOL_F32, "linear")
+    own = rows >= ops.LINEAR_MIN_ROWS and M <= ops.LINEAR_MAX_COLS
+    same = np.array_equal(got.cpu().numpy(), ops.linear_attn(_dev(x, device), _dev(w, device)).cpu().numpy())
+    assert same or not own
+
+
 @pytest.mark.parametrize("offset", [1, 2, 3, 4])
 @pytest.mark.parametrize("K", [66, 602, 64, 37])
 def test_linear_attn_row_alignment(device, K, offset):
