@@ -24,8 +24,9 @@
 // of a row.  X is staged as fp32 and split after the operand read (each value is
 // consumed by exactly one lane); W is split when it is committed to LDS, as three
 // [column][k] bf16 arrays, so an operand read is one 16-byte LDS read per piece.
-// Two register sets hold the slices one and two ahead of the one being
-// multiplied, two LDS buffers the current and the next slice, so a slice costs
+// Loads go through buffer descriptors (fixed lane offsets, the slice as the scalar
+// offset), so the loop has no address arithmetic.  Two register sets hold the slices
+// one and two ahead of the one being multiplied, two LDS buffers the current and the next slice, so a slice costs
 // one barrier and its global loads have two slices of work to arrive.
 // Accumulators come out as D[row][col] with 16 adjacent lanes on 16 adjacent
 // columns: Z stores coalesce, and the per-head dot products need one 16-lane DPP
@@ -58,6 +59,34 @@ __device__ __forceinline__ void split8(const float (&v)[8], uint4 &p0, uint4 &p1
   p2 = uint4{__builtin_amdgcn_perm(c[1], c[0], hi), __builtin_amdgcn_perm(c[3], c[2], hi),
              __builtin_amdgcn_perm(c[5], c[4], hi), __builtin_amdgcn_perm(c[7], c[6], hi)};
 }
+
+// Loads through a buffer descriptor: address = descriptor base + 32-bit lane offset
+// + 32-bit scalar offset, formed by the load unit.  The lane offsets are fixed for
+// the whole kernel and the scalar offset advances with the slice, so a load costs no
+// address arithmetic (plain pointers cost a 64-bit vector add per load here).  The
+// scalar offset takes no part in the descriptor's range check, so the code keeps
+// every address valid itself.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint64_t bytes) {
+  const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+}
+template <int VK> struct BufLoad;
+template <> struct BufLoad<4> {
+  static __device__ __forceinline__ float4 at(rsrc_t r, uint32_t lane_off, uint32_t scalar_off) {
+    return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, scalar_off, 0));
+  }
+};
+template <> struct BufLoad<2> {
+  static __device__ __forceinline__ float2 at(rsrc_t r, uint32_t lane_off, uint32_t scalar_off) {
+    return __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, scalar_off, 0));
+  }
+};
+template <> struct BufLoad<1> {
+  static __device__ __forceinline__ float at(rsrc_t r, uint32_t lane_off, uint32_t scalar_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, scalar_off, 0));
+  }
+};
 
 constexpr int kRT = 2;                                   // 16-row tiles per wave
 constexpr int kWaveRows = kRT * 16;                      // 32
@@ -94,7 +123,7 @@ linear_attn_kernel(
   __shared__ __attribute__((aligned(16))) float xs[2][kWgRows * kXs];
   __shared__ __attribute__((aligned(16))) uint32_t wb[2][3][kPassCols * kWb];
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // in a scalar register
   const int lr = lane & 15, lk = lane >> 4;
   const int col0 = blockIdx.y * kPassCols;               // first column of the pass
   const int64_t wg_row0 = (int64_t)blockIdx.x * kWgRows;
@@ -112,37 +141,61 @@ linear_attn_kernel(
     xvec_t x[kXPieces];
     float w[8];
   };
-  const int wc = threadIdx.x & 63, wkg = threadIdx.x >> 6;   // column, group of 8 k
+  // Lane offsets (bytes) never change; the slice / the row of W is the scalar offset.
+  // Slices that lie wholly inside the rows (all but the last, and that one too when
+  // K % 32 == 0) take paths without clamps and selects.
+  const int wc = threadIdx.x & 63, wkg = wave;               // column, group of 8 k
   const int xr = threadIdx.x / kVpr, xc = (threadIdx.x % kVpr) * VK;
-  const float *xbase[kXPieces];
+  const rsrc_t xrs = make_rsrc(X + wg_row0 * K, (uint64_t)(rows - wg_row0) * K * 4);
+  const rsrc_t wrs = make_rsrc(W, (uint64_t)K * M * 4);
+  uint32_t xoff[kXPieces];                               // the piece in slice 0
 #pragma unroll
   for (int j = 0; j < kXPieces; ++j)
-    xbase[j] = X + min(wg_row0 + xr + j * kRowStep, rows - 1) * K;
+    xoff[j] = (uint32_t)((min(wg_row0 + xr + j * kRowStep, rows - 1) - wg_row0) * K + xc) * 4u;
+  const uint32_t woff = (uint32_t)min(col0 + wc, M - 1) * 4u;
+  const bool w_cols_full = col0 + kPassCols <= M;        // uniform
 
   auto fetch = [&](int sl, Stage &st) {
-    const int kc = min(sl * kSliceK + xc, K - VK);
+    if (sl * kSliceK + kSliceK <= K) {
 #pragma unroll
-    for (int j = 0; j < kXPieces; ++j)
-      st.x[j] = *reinterpret_cast<const xvec_t *>(xbase[j] + kc);
-    const float *wsrc = W + min(col0 + wc, M - 1);
+      for (int j = 0; j < kXPieces; ++j)
+        st.x[j] = BufLoad<VK>::at(xrs, xoff[j], (uint32_t)sl * (kSliceK * 4));
+    } else {
+      // clamped to the row's last vector (a valid address); zeroed at commit
+      const uint32_t dk = (uint32_t)(min(sl * kSliceK + xc, K - VK) - xc) * 4u;
+#pragma unroll
+      for (int j = 0; j < kXPieces; ++j) st.x[j] = BufLoad<VK>::at(xrs, xoff[j] + dk, 0);
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      st.w[j] = wsrc[(int64_t)min(sl * kSliceK + wkg * 8 + j, K - 1) * M];
+      st.w[j] = BufLoad<1>::at(wrs, woff, (uint32_t)min(sl * kSliceK + wkg * 8 + j, K - 1) * (uint32_t)M * 4u);
   };
   auto commit = [&](int sl, const Stage &st) {
     const int buf = sl & 1;
-    const bool xin = sl * kSliceK + xc < K;
+    const bool inside = sl * kSliceK + kSliceK <= K;     // uniform
+    if (inside) {
 #pragma unroll
-    for (int j = 0; j < kXPieces; ++j) {
-      xvec_t v = st.x[j];
-      if (!xin) v = xvec_t{};
-      *reinterpret_cast<xvec_t *>(&xs[buf][(xr + j * kRowStep) * kXs + xc]) = v;
+      for (int j = 0; j < kXPieces; ++j)
+        *reinterpret_cast<xvec_t *>(&xs[buf][(xr + j * kRowStep) * kXs + xc]) = st.x[j];
+    } else {
+      const bool xin = sl * kSliceK + xc < K;
+#pragma unroll
+      for (int j = 0; j < kXPieces; ++j) {
+        xvec_t v = st.x[j];
+        if (!xin) v = xvec_t{};
+        *reinterpret_cast<xvec_t *>(&xs[buf][(xr + j * kRowStep) * kXs + xc]) = v;
+      }
     }
     float wv[8];
-    const bool cin = col0 + wc < M;
+    if (inside && w_cols_full) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      wv[j] = cin && sl * kSliceK + wkg * 8 + j < K ? st.w[j] : 0.0f;
+      for (int j = 0; j < 8; ++j) wv[j] = st.w[j];
+    } else {
+      const bool cin = col0 + wc < M;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        wv[j] = cin && sl * kSliceK + wkg * 8 + j < K ? st.w[j] : 0.0f;
+    }
     uint4 p0, p1, p2;
     split8(wv, p0, p1, p2);
     *reinterpret_cast<uint4 *>(&wb[buf][0][wc * kWb + wkg * 4]) = p0;
@@ -272,6 +325,8 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
   if (rows > 0x7fffffff || K > 0x7fffffff || M > 0x7fffffff) return GA_EINVAL;
   if (rows == 0) return GA_OK;
   if (!X || !W || !Z) return GA_EINVAL;
+  // 32-bit byte offsets: 128 rows of K floats, and all of W
+  if (K > (1 << 22) || K * M >= ((int64_t)1 << 30)) return GA_EUNSUPPORTED;
   const bool attn = el != nullptr || er != nullptr;
   if (attn && (!el || !er || !a_l || !a_r)) return GA_EINVAL;
   if (!aligned(X, 4) || !aligned(W, 4) || !aligned(Z, 4)) return GA_EALIGN;
