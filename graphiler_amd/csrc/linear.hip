@@ -26,8 +26,9 @@
 // [column][k] bf16 arrays, so an operand read is one 16-byte LDS read per piece.
 // Loads go through buffer descriptors (fixed lane offsets, the slice as the scalar
 // offset), so the loop has no address arithmetic.  Two register sets hold the slices
-// one and two ahead of the one being multiplied, two LDS buffers the current and the next slice, so a slice costs
-// one barrier and its global loads have two slices of work to arrive.
+// one and two ahead of the one being multiplied, two LDS buffers the current and
+// the next slice, so a slice costs one barrier and its global loads have two slices
+// of work to arrive.
 // Accumulators come out as D[row][col] with 16 adjacent lanes on 16 adjacent
 // columns: Z stores coalesce, and the per-head dot products need one 16-lane DPP
 // sum per row and head.
