@@ -111,6 +111,34 @@ struct Frag<bf16_t, 1> {
   }
 };
 
+// Loads through a buffer descriptor: address = descriptor base + 32-bit lane offset
+// + 32-bit scalar offset, formed by the load unit.  The lane offsets are fixed for
+// the whole kernel and the scalar offset advances with the slice, so a load costs no
+// address arithmetic (plain pointers cost a 64-bit vector add per load here).  The
+// scalar offset takes no part in the descriptor's range check, so the code keeps
+// every address valid itself.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint64_t bytes) {
+  const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+}
+template <int VK> struct BufLoad;
+template <> struct BufLoad<4> {
+  static __device__ __forceinline__ float4 at(rsrc_t r, uint32_t lane_off, uint32_t scalar_off) {
+    return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, scalar_off, 0));
+  }
+};
+template <> struct BufLoad<2> {
+  static __device__ __forceinline__ float2 at(rsrc_t r, uint32_t lane_off, uint32_t scalar_off) {
+    return __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, scalar_off, 0));
+  }
+};
+template <> struct BufLoad<1> {
+  static __device__ __forceinline__ float at(rsrc_t r, uint32_t lane_off, uint32_t scalar_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, scalar_off, 0));
+  }
+};
+
 // ---- host side -----------------------------------------------------------
 
 inline int ilog2_floor(uint64_t x) {
