@@ -289,8 +289,11 @@ int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,
  * src/optimizer/split.cpp:5-34); with el == er == NULL it is the plain node
  * projection of examples/GCN/GCN.py:39.  X (rows, K), W (K, M), Z (rows, M),
  * a_l / a_r (heads, M/heads), el / er (rows, heads), all fp32.
+ * Every fp32 product is formed exactly, from bf16 pieces of its operands on the
+ * matrix unit, and summed in fp32: the result is as close to the exact product
+ * as plain fp32 arithmetic gets; a non-finite input gives NaN.
  * GA_EUNSUPPORTED when the attention terms are requested with M/heads not in
- * {16, 32, 64}.
+ * {16, 32, 64}, when K > 2^22 or when K * M >= 2^30.
  */
 int ga_linear_attn(const float *X, const float *W, const float *a_l,
                    const float *a_r, float *Z, float *el, float *er,
