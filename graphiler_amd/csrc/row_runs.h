@@ -256,8 +256,22 @@ __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
     const float *p = partial + ((q_lo * 2 + 1) * geo.lanes_total + flane) * SF;
 #pragma unroll
     for (int i = 0; i < SF; ++i) acc[i] = p[i];
-    for (int64_t w = q_lo + 1; w <= q; ++w)
-      Policy::merge(acc, partial + ((w * 2) * geo.lanes_total + flane) * SF);
+    // the chain is combined in workgroup order; four states are fetched at a time
+    // so that the loads of a long chain (a hub row) overlap instead of queueing up
+    // one latency after the other
+    const int64_t stride = (int64_t)2 * geo.lanes_total * SF;
+    const float *src = partial + (((q_lo + 1) * 2) * geo.lanes_total + flane) * SF;
+    int64_t w = q_lo + 1;
+    for (; w + 3 <= q; w += 4, src += 4 * stride) {
+      float nxt[4][SF];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int i = 0; i < SF; ++i) nxt[u][i] = src[u * stride + i];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) Policy::merge(acc, nxt[u]);
+    }
+    for (; w <= q; ++w, src += stride) Policy::merge(acc, src);
     Policy::emit(args, out, row, geo.feat, f0, acc);
     (void)G;
   } else {
