@@ -26,9 +26,14 @@
 // [column][k] bf16 arrays, so an operand read is one 16-byte LDS read per piece.
 // Loads go through buffer descriptors (fixed lane offsets, the slice as the scalar
 // offset), so the loop has no address arithmetic.  Two register sets hold the slices
-// one and two ahead of the one being multiplied, two LDS buffers the current and
-// the next slice, so a slice costs one barrier and its global loads have two slices
-// of work to arrive.
+// one and two ahead of the one being multiplied.  Every wave stages the rows it
+// multiplies itself, so the X tile needs one LDS buffer and no barrier (a wave's LDS
+// accesses execute in order: the next slice is written after the current one has
+// been read); the W pieces, shared by the four waves, have two buffers and cost the
+// one barrier per slice.  The W operands of a column block are read while the block
+// before it multiplies.  49 KB of LDS and under 168 registers: three workgroups per
+// CU when the grid has at least one per CU; smaller grids are latency-bound and run
+// the build with the two-per-CU register budget, which is faster there.
 // Accumulators come out as D[row][col] with 16 adjacent lanes on 16 adjacent
 // columns: Z stores coalesce, and the per-head dot products need one 16-lane DPP
 // sum per row and head.
@@ -82,18 +87,16 @@ template <> struct XVec<1> { using type = float; };
 // wholly outside a row: ragged edges clamp the address at fetch time (a valid
 // one, the row's last vector) and zero by select at commit time, where the
 // value is consumed anyway; no lane is ever predicated off in the k loop.
-template <bool HAS_ATTN, int VK>
-// two waves per SIMD: with that register budget the accumulators stay in place
-// across the loop (left to itself the allocator splits them over both register
-// files and copies 48 of them every trip)
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2, 2))) void
+// WAVES: waves per SIMD the register allocation aims at (3 or 2)
+template <bool HAS_ATTN, int VK, int WAVES>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void
 linear_attn_kernel(
     const float *__restrict__ X, const float *__restrict__ W,
     const float *__restrict__ a_l, const float *__restrict__ a_r,
     float *__restrict__ Z, float *__restrict__ el, float *__restrict__ er,
     int64_t rows, int K, int M, int heads) {
   using xvec_t = typename XVec<VK>::type;
-  __shared__ __attribute__((aligned(16))) float xs[2][kWgRows * kXs];
+  __shared__ __attribute__((aligned(16))) float xs[kWgRows * kXs];   // wave-private rows, one buffer
   __shared__ __attribute__((aligned(16))) uint32_t wb[2][3][kPassCols * kWb];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // in a scalar register
@@ -103,13 +106,13 @@ linear_attn_kernel(
   const int64_t wrow0 = wg_row0 + wave * kWaveRows;
   const int n_slices = (K + kSliceK - 1) / kSliceK;
 
-  // X slice: 128 rows x 32 k in vectors of VK floats, kVpr per row; thread i
-  // owns vectors i, i + 256, ...: a wave instruction reads 64 * VK * 4
-  // contiguous-by-row bytes (8 * VK rows of 128 bytes).  Slices past the last
+  // X slice of a wave: its 32 rows x 32 k in vectors of VK floats, kVpr per row; lane
+  // i owns vectors i, i + 64, ...: a wave instruction reads 64 * VK * 4
+  // contiguous-by-row bytes (2 * VK rows of 128 bytes).  Slices past the last
   // are fetched too (from the clamped address) and never multiplied.
   constexpr int kVpr = kSliceK / VK;                     // vectors per row and slice
-  constexpr int kXPieces = kWgRows * kVpr / kBlock;      // 4 / 8 / 16 per thread
-  constexpr int kRowStep = kBlock / kVpr;                // rows between a thread's vectors
+  constexpr int kXPieces = kWaveRows * kVpr / kWave;     // 4 / 8 / 16 per thread
+  constexpr int kRowStep = kWave / kVpr;                 // rows between a thread's vectors
   struct Stage {
     xvec_t x[kXPieces];
     float w[8];
@@ -118,7 +121,7 @@ linear_attn_kernel(
   // Slices that lie wholly inside the rows (all but the last, and that one too when
   // K % 32 == 0) take paths without clamps and selects.
   const int wc = threadIdx.x & 63, wkg = wave;               // column, group of 8 k
-  const int xr = threadIdx.x / kVpr, xc = (threadIdx.x % kVpr) * VK;
+  const int xr = wave * kWaveRows + lane / kVpr, xc = (lane % kVpr) * VK;   // each wave stages its own rows
   const rsrc_t xrs = make_rsrc(X + wg_row0 * K, (uint64_t)(rows - wg_row0) * K * 4);
   const rsrc_t wrs = make_rsrc(W, (uint64_t)K * M * 4);
   uint32_t xoff[kXPieces];                               // the piece in slice 0
@@ -149,14 +152,14 @@ linear_attn_kernel(
     if (inside) {
 #pragma unroll
       for (int j = 0; j < kXPieces; ++j)
-        *reinterpret_cast<xvec_t *>(&xs[buf][(xr + j * kRowStep) * kXs + xc]) = st.x[j];
+        *reinterpret_cast<xvec_t *>(&xs[(xr + j * kRowStep) * kXs + xc]) = st.x[j];
     } else {
       const bool xin = sl * kSliceK + xc < K;
 #pragma unroll
       for (int j = 0; j < kXPieces; ++j) {
         xvec_t v = st.x[j];
         if (!xin) v = xvec_t{};
-        *reinterpret_cast<xvec_t *>(&xs[buf][(xr + j * kRowStep) * kXs + xc]) = v;
+        *reinterpret_cast<xvec_t *>(&xs[(xr + j * kRowStep) * kXs + xc]) = v;
       }
     }
     float wv[8];
@@ -187,17 +190,18 @@ linear_attn_kernel(
   auto step = [&](int sl, Stage &next) {
     const int buf = sl & 1;
     float4 xa[kRT][2];
-    uint4 wf[3][kCB];
+    uint4 wf[2][3];
 #pragma unroll
     for (int t = 0; t < kRT; ++t) {
-      xa[t][0] = *reinterpret_cast<const float4 *>(&xs[buf][xl_ofs + t * 16 * kXs]);
-      xa[t][1] = *reinterpret_cast<const float4 *>(&xs[buf][xl_ofs + t * 16 * kXs + 4]);
+      xa[t][0] = *reinterpret_cast<const float4 *>(&xs[xl_ofs + t * 16 * kXs]);
+      xa[t][1] = *reinterpret_cast<const float4 *>(&xs[xl_ofs + t * 16 * kXs + 4]);
     }
+    auto read_w = [&](int cb, uint4 (&f)[3]) {
 #pragma unroll
-    for (int p = 0; p < 3; ++p)
-#pragma unroll
-      for (int cb = 0; cb < kCB; ++cb)
-        wf[p][cb] = *reinterpret_cast<const uint4 *>(&wb[buf][p][wl_ofs + cb * 16 * kWb]);
+      for (int p = 0; p < 3; ++p)
+        f[p] = *reinterpret_cast<const uint4 *>(&wb[buf][p][wl_ofs + cb * 16 * kWb]);
+    };
+    read_w(0, wf[0]);
     commit(sl + 1, next);
     fetch(sl + 3, next);
     uint4 xp[kRT][3];
@@ -207,17 +211,18 @@ linear_attn_kernel(
                           xa[t][1].x, xa[t][1].y, xa[t][1].z, xa[t][1].w};
       split8(v, xp[t][0], xp[t][1], xp[t][2]);
     }
-    // small terms first; eight independent accumulators between dependent MFMAs
     constexpr int px[6] = {2, 0, 1, 1, 0, 0}, pw[6] = {0, 2, 1, 0, 1, 0};
 #pragma unroll
-    for (int q = 0; q < 6; ++q)
+    for (int cb = 0; cb < kCB; ++cb) {
+      if (cb + 1 < kCB) read_w(cb + 1, wf[(cb + 1) & 1]);
 #pragma unroll
-      for (int t = 0; t < kRT; ++t)
+      for (int q = 0; q < 6; ++q)
 #pragma unroll
-        for (int cb = 0; cb < kCB; ++cb)
+        for (int t = 0; t < kRT; ++t)
           acc[t][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              __builtin_bit_cast(bf16x8, xp[t][px[q]]), __builtin_bit_cast(bf16x8, wf[pw[q]][cb]),
+              __builtin_bit_cast(bf16x8, xp[t][px[q]]), __builtin_bit_cast(bf16x8, wf[cb & 1][pw[q]]),
               acc[t][cb], 0, 0, 0);
+    }
     __syncthreads();
   };
 
@@ -310,19 +315,28 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
   const int64_t gy = (M + kPassCols - 1) / kPassCols;
   if (gx > 0x7fffffff || gy > 65535) return GA_EUNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
-#define GA_LAUNCH_LINEAR(ATTN, VK)                                                 \
-  hipLaunchKernelGGL((linear_attn_kernel<ATTN, VK>), dim3((unsigned)gx, (unsigned)gy), \
+#define GA_LAUNCH_LINEAR(ATTN, VK, WAVES)                                          \
+  hipLaunchKernelGGL((linear_attn_kernel<ATTN, VK, WAVES>), dim3((unsigned)gx, (unsigned)gy), \
                      dim3(kBlock), 0, s, X, W, a_l, a_r, Z, el, er, rows, (int)K,   \
                      (int)M, (int)heads)
+#define GA_LAUNCH_LINEAR_VK(ATTN, WAVES)                 \
+  do {                                                   \
+    if (vk == 4) GA_LAUNCH_LINEAR(ATTN, 4, WAVES);       \
+    else if (vk == 2) GA_LAUNCH_LINEAR(ATTN, 2, WAVES);  \
+    else GA_LAUNCH_LINEAR(ATTN, 1, WAVES);               \
+  } while (0)
+  // three workgroups per CU once there is at least one per CU to start with; below
+  // that the kernel is latency-bound and the build with the larger register budget
+  // (two per CU) has the shorter dependent chain per slice
+  const bool dense_grid = gx * gy >= 256;
   if (attn) {
-    if (vk == 4) GA_LAUNCH_LINEAR(true, 4);
-    else if (vk == 2) GA_LAUNCH_LINEAR(true, 2);
-    else GA_LAUNCH_LINEAR(true, 1);
+    if (dense_grid) GA_LAUNCH_LINEAR_VK(true, 3);
+    else GA_LAUNCH_LINEAR_VK(true, 2);
   } else {
-    if (vk == 4) GA_LAUNCH_LINEAR(false, 4);
-    else if (vk == 2) GA_LAUNCH_LINEAR(false, 2);
-    else GA_LAUNCH_LINEAR(false, 1);
+    if (dense_grid) GA_LAUNCH_LINEAR_VK(false, 3);
+    else GA_LAUNCH_LINEAR_VK(false, 2);
   }
+#undef GA_LAUNCH_LINEAR_VK
 #undef GA_LAUNCH_LINEAR
   return launch_status();
 }
