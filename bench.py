@@ -23,9 +23,9 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 # HBM bytes per dominant-kernel launch measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); the summary
 # lives under profiles/.  None until measured for the kernel named below.
-MEASURED_TRAFFIC_BYTES = {"plan": 1_519_190_735, "fused": 1_526_745_856,
-                          "compiled": 1_526_745_856}
-DENSE_TRAFFIC_BYTES = 661_808_853   # the projection kernel, same two counter runs
+MEASURED_TRAFFIC_BYTES = {"plan": 1_518_404_824, "fused": 1_513_481_691,
+                          "compiled": 1_513_481_691}
+DENSE_TRAFFIC_BYTES = 695_050_095   # the projection kernel, same two counter runs
 
 
 def main():
