@@ -328,7 +328,8 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
   // three workgroups per CU once there is at least one per CU to start with; below
   // that the kernel is latency-bound and the build with the larger register budget
   // (two per CU) has the shorter dependent chain per slice
-  const bool dense_grid = gx * gy >= 256;
+  constexpr int64_t kDeviceCUs = 256;                    // MI355X
+  const bool dense_grid = gx * gy >= kDeviceCUs;
   if (attn) {
     if (dense_grid) GA_LAUNCH_LINEAR_VK(true, 3);
     else GA_LAUNCH_LINEAR_VK(true, 2);
