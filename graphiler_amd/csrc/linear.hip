@@ -323,11 +323,14 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
   do {                                                   \
     if (vk == 4) GA_LAUNCH_LINEAR(ATTN, 4, WAVES);       \
     else if (vk == 2) GA_LAUNCH_LINEAR(ATTN, 2, WAVES);  \
-    else GA_LAUNCH_LINEAR(ATTN, 1, WAVES);               \
+    else GA_LAUNCH_LINEAR(ATTN, 1, 2);                   \
   } while (0)
   // three workgroups per CU once there is at least one per CU to start with; below
   // that the kernel is latency-bound and the build with the larger register budget
-  // (two per CU) has the shorter dependent chain per slice
+  // (two per CU) has the shorter dependent chain per slice.  Rows that are only
+  // 4-byte aligned (odd K) are staged one float per load: that build holds 32 staged
+  // registers per lane, does not fit the three-workgroup budget without spilling
+  // (measured 4x slower there), and always runs two per CU.
   constexpr int64_t kDeviceCUs = 256;                    // MI355X
   const bool dense_grid = gx * gy >= kDeviceCUs;
   if (attn) {
