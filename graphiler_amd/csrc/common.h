@@ -111,6 +111,71 @@ struct Frag<bf16_t, 1> {
   }
 };
 
+// Row access of the row-reduction kernels.  RowIO<T, VEC, false> is Frag: the lane's
+// VEC features are consecutive and move with one 16-byte access.  RowIO<T, VEC, true>
+// is for rows that such accesses do not tile (feature count not a multiple of the
+// vector, or unaligned storage): the lane's features lie one lane-group width apart
+// (f0, f0 + stride, f0 + 2 stride, ...), so the lanes of a group read consecutive
+// elements with each of their VEC element loads.  Features past the end of the row
+// are read from the lane's first feature instead and never stored.
+__device__ __forceinline__ float elem_to_f32(float x) { return x; }
+__device__ __forceinline__ float elem_to_f32(bf16_t x) { return bf16_lo(x); }
+__device__ __forceinline__ void f32_to_elem(float f, float &o) { o = f; }
+__device__ __forceinline__ void f32_to_elem(float f, bf16_t &o) { o = (bf16_t)f32_to_bf16_bits(f); }
+
+template <typename T, int VEC, bool SPREAD>
+struct RowIO;
+
+template <typename T, int VEC>
+struct RowIO<T, VEC, false> {
+  typedef typename Frag<T, VEC>::raw_t raw_t;
+  struct lane_t {};
+  static __device__ __forceinline__ lane_t lane(int, int) { return lane_t(); }
+  static __device__ __forceinline__ raw_t load(const T *p, const lane_t &) {
+    return Frag<T, VEC>::load(p);
+  }
+  static __device__ __forceinline__ void widen(const raw_t &r, float (&f)[VEC]) {
+    Frag<T, VEC>::widen(r, f);
+  }
+  static __device__ __forceinline__ void store(T *p, const float (&f)[VEC], const lane_t &) {
+    Frag<T, VEC>::store(p, f);
+  }
+};
+
+template <typename T, int VEC>
+struct RowIO<T, VEC, true> {
+  struct raw_t { T e[VEC]; };
+  struct lane_t {
+    int off[VEC];   // element offset of feature v from the lane's first feature
+    int live;       // features of this lane that lie inside the row
+  };
+  // stride = 1 << stride_shift features between a lane's features; `left` = features
+  // from the lane's first one to the end of the row (> 0 for a live lane)
+  static __device__ __forceinline__ lane_t lane(int stride_shift, int left) {
+    lane_t l;
+    const int n = (left + (1 << stride_shift) - 1) >> stride_shift;
+    l.live = n < VEC ? n : VEC;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) l.off[v] = v < l.live ? v << stride_shift : 0;
+    return l;
+  }
+  static __device__ __forceinline__ raw_t load(const T *p, const lane_t &l) {
+    raw_t r;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) r.e[v] = p[l.off[v]];
+    return r;
+  }
+  static __device__ __forceinline__ void widen(const raw_t &r, float (&f)[VEC]) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) f[v] = elem_to_f32(r.e[v]);
+  }
+  static __device__ __forceinline__ void store(T *p, const float (&f)[VEC], const lane_t &l) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v)
+      if (v < l.live) f32_to_elem(f[v], p[l.off[v]]);
+  }
+};
+
 // Loads through a buffer descriptor: address = descriptor base + 32-bit lane offset
 // + 32-bit scalar offset, formed by the load unit.  The lane offsets are fixed for
 // the whole kernel and the scalar offset advances with the slice, so a load costs no

@@ -42,12 +42,15 @@ __device__ __forceinline__ float lanes_sum(float v, int lanes) {
   return v;
 }
 
-template <typename T, int VEC, int MODE = kGatNode>
+// SPREAD: the lane's features lie a lane-group width apart (rows that 16-byte
+// accesses do not tile); they share the lane's one (m, l) pair, i.e. one head.
+template <typename T, int VEC, int MODE = kGatNode, bool SPREAD = false>
 struct GatPolicy {
   static constexpr bool EDGE = MODE == kGatEdge;
   typedef T out_t;
   static constexpr int kVec = VEC;
   static constexpr int kState = VEC + 2;
+  static constexpr bool kSpread = SPREAD;
   struct Args {
     const int32_t *nbr;   // kGatEdge: the edge-id column, or null when slot = edge id
     const float *el;      // kGatEdge: per-edge logits (E, heads); kGatFromZ: a_l (heads*dph)
@@ -58,6 +61,7 @@ struct GatPolicy {
     float slope;
     bool ids_vec;   // row_of_slot and nbr are 16-byte aligned
     int head_lanes; // kGatFromZ: lanes that share a head (dph / VEC)
+    int stride_shift;   // SPREAD: log2 of the lanes per group, set by the launcher
   };
   static __device__ __forceinline__ void init(float (&st)[VEC + 2]) {
 #pragma unroll
@@ -82,13 +86,13 @@ struct GatPolicy {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) o[v] = 0.0f;
   }
-  static __device__ __forceinline__ void emit(const Args &, out_t *out, int64_t row, int feat,
+  static __device__ __forceinline__ void emit(const Args &A, out_t *out, int64_t row, int feat,
                                               int f0, const float (&st)[kState]) {
-    emit_row<GatPolicy>(out, row, feat, f0, st);
+    emit_row<GatPolicy>(out, row, feat, f0, st, A.stride_shift);
   }
-  static __device__ __forceinline__ void emit_empty(const Args &, out_t *out, int64_t row,
+  static __device__ __forceinline__ void emit_empty(const Args &A, out_t *out, int64_t row,
                                                     int feat, int f0) {
-    emit_empty_row<GatPolicy>(out, row, feat, f0);
+    emit_empty_row<GatPolicy>(out, row, feat, f0, A.stride_shift);
   }
 
   template <class Close>
@@ -97,8 +101,10 @@ struct GatPolicy {
                                               int64_t a, int64_t b, int f0, int feat,
                                               float (&st)[VEC + 2], int &cur,
                                               Close &&close_segment) {
-    typedef Frag<T, VEC> IO;
-    const int h = f0 / A.dph;
+    static_assert(!(SPREAD && MODE == kGatFromZ), "the per-head dot product needs consecutive features");
+    typedef RowIO<T, VEC, SPREAD> IO;
+    const typename IO::lane_t ln = IO::lane(A.stride_shift, feat - f0);
+    const int h = SPREAD ? 0 : f0 / A.dph;
     float al[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) al[v] = MODE == kGatFromZ ? A.el[f0 + v] : 0.0f;
@@ -115,7 +121,7 @@ struct GatPolicy {
       }
 #pragma unroll
       for (int t = 0; t < kUnroll; ++t) {
-        x[t] = IO::load(A.z + (int64_t)g[t] * feat + f0);
+        x[t] = IO::load(A.z + (int64_t)g[t] * feat + f0, ln);
         if constexpr (MODE == kGatEdge)
           s[t] = A.el[(int64_t)g[t] * A.heads + h];
         else if constexpr (MODE == kGatNode)
@@ -182,18 +188,18 @@ struct GatPolicy {
   }
 };
 
-template <typename T, int VEC, int MODE = kGatNode>
+template <typename T, int VEC, int MODE = kGatNode, bool SPREAD = false>
 int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const int32_t *nbr, const float *el, const float *er,
                const void *z, void *out, int64_t n_rows, int64_t n_edges,
                int heads, int dim, float slope, float *ws, hipStream_t stream) {
-  typedef GatPolicy<T, VEC, MODE> P;
+  typedef GatPolicy<T, VEC, MODE, SPREAD> P;
   const bool ids_vec = aligned(row_of_slot, 16) && (!nbr || aligned(nbr, 16));
   const int head_lanes = dim / VEC;
   if (MODE == kGatFromZ &&
       (dim % VEC != 0 || head_lanes > 16 || (head_lanes & (head_lanes - 1)) != 0))
     return GA_EUNSUPPORTED;
-  typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec, head_lanes};
+  typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec, head_lanes, 0};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges,
                         heads * dim, ws, stream);
 }
@@ -241,6 +247,10 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
       return ga::launch_gat<float, 4>(pointer, row_of_slot, nbr, el, er, z, out,
                                       n_rows, n_edges, (int)heads, (int)dim,
                                       slope, ws, s);
+    if (heads == 1 && dim >= 3 && dim <= 256)   // rows that 16-byte accesses do not tile
+      return ga::launch_gat<float, 4, ga::kGatNode, true>(pointer, row_of_slot, nbr, el, er, z,
+                                                          out, n_rows, n_edges, 1, (int)dim,
+                                                          slope, ws, s);
     return ga::launch_gat<float, 1>(pointer, row_of_slot, nbr, el, er, z, out,
                                     n_rows, n_edges, (int)heads, (int)dim, slope,
                                     ws, s);
@@ -249,6 +259,10 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
     return ga::launch_gat<ga::bf16_t, 8>(pointer, row_of_slot, nbr, el, er, z,
                                          out, n_rows, n_edges, (int)heads,
                                          (int)dim, slope, ws, s);
+  if (heads == 1 && dim >= 3 && dim <= 256)
+    return ga::launch_gat<ga::bf16_t, 4, ga::kGatNode, true>(pointer, row_of_slot, nbr, el, er, z,
+                                                             out, n_rows, n_edges, 1, (int)dim,
+                                                             slope, ws, s);
   return ga::launch_gat<ga::bf16_t, 1>(pointer, row_of_slot, nbr, el, er, z, out,
                                        n_rows, n_edges, (int)heads, (int)dim,
                                        slope, ws, s);
@@ -284,12 +298,18 @@ int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,
     if (vec_ok && dim % 4 == 0)
       return ga::launch_gat<float, 4, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m,
                                             out, n_rows, n_edges, h, d, 0.0f, ws, s);
+    if (heads == 1 && dim >= 3 && dim <= 256)   // rows that 16-byte accesses do not tile
+      return ga::launch_gat<float, 4, ga::kGatEdge, true>(pointer, row_of_slot, eid, logit, nullptr,
+                                                          m, out, n_rows, n_edges, 1, d, 0.0f, ws, s);
     return ga::launch_gat<float, 1, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m, out,
                                           n_rows, n_edges, h, d, 0.0f, ws, s);
   }
   if (vec_ok && dim % 8 == 0)
     return ga::launch_gat<ga::bf16_t, 8, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m,
                                                out, n_rows, n_edges, h, d, 0.0f, ws, s);
+  if (heads == 1 && dim >= 3 && dim <= 256)
+    return ga::launch_gat<ga::bf16_t, 4, ga::kGatEdge, true>(pointer, row_of_slot, eid, logit, nullptr,
+                                                             m, out, n_rows, n_edges, 1, d, 0.0f, ws, s);
   return ga::launch_gat<ga::bf16_t, 1, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m,
                                              out, n_rows, n_edges, h, d, 0.0f, ws, s);
 }

@@ -2,8 +2,9 @@
 // the fused GAT aggregation).
 //
 // Schedule.  The slots [0, E) are cut into equal runs of 2^run_shift slots.  A
-// group of `tpr` adjacent lanes (tpr * VEC features = one feature-row tile,
-// 16 bytes per lane when VEC > 1) owns one run and walks it in slot order with
+// group of `tpr` adjacent lanes (tpr * VEC features = one feature-row tile;
+// a lane holds VEC consecutive features, 16 bytes, or -- Policy::kSpread -- VEC
+// features tpr apart, see RowIO) owns one run and walks it in slot order with
 // eight gathers in flight per lane; a workgroup of 256 lanes owns G = 256 / tpr
 // consecutive runs.  Rows that lie inside one run are written straight to the
 // output.  A row shared by neighbouring runs leaves partial states, which the
@@ -25,6 +26,8 @@
 //                               write a finished / an edgeless row's tile; the
 //                               usual ones are emit_row / emit_empty_row below,
 //                               a policy with further outputs writes them here
+//   kSpread                     lane layout (see above); such a policy's Args carry
+//                               `stride_shift`, which the launcher sets to log2(tpr)
 #pragma once
 
 #include "common.h"
@@ -75,17 +78,27 @@ struct RunFlags {
 
 template <class Policy>
 __device__ __forceinline__ void emit_row(typename Policy::out_t *out, int64_t row, int feat,
-                                         int f0, const float (&st)[Policy::kState]) {
+                                         int f0, const float (&st)[Policy::kState],
+                                         int stride_shift = 0) {
+  typedef RowIO<typename Policy::out_t, Policy::kVec, Policy::kSpread> IO;
   float o[Policy::kVec];
   Policy::finish(st, o);
-  Frag<typename Policy::out_t, Policy::kVec>::store(out + row * feat + f0, o);
+  IO::store(out + row * feat + f0, o, IO::lane(stride_shift, feat - f0));
 }
 template <class Policy>
 __device__ __forceinline__ void emit_empty_row(typename Policy::out_t *out, int64_t row,
-                                               int feat, int f0) {
+                                               int feat, int f0, int stride_shift = 0) {
+  typedef RowIO<typename Policy::out_t, Policy::kVec, Policy::kSpread> IO;
   float o[Policy::kVec];
   Policy::empty_row(o);
-  Frag<typename Policy::out_t, Policy::kVec>::store(out + row * feat + f0, o);
+  IO::store(out + row * feat + f0, o, IO::lane(stride_shift, feat - f0));
+}
+
+// First feature of lane `lane` of a group in feature tile `tile`.
+template <class Policy>
+__device__ __forceinline__ int lane_first_feature(int tile, int lane, int tpr_shift) {
+  return Policy::kSpread ? ((tile * Policy::kVec) << tpr_shift) + lane
+                         : ((tile << tpr_shift) + lane) * Policy::kVec;
 }
 
 template <class Policy>
@@ -93,14 +106,13 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
     typename Policy::Args args, const int32_t *__restrict__ pointer,
     const int32_t *__restrict__ row_of_slot, typename Policy::out_t *__restrict__ out,
     float *__restrict__ partial, RunGeom geo) {
-  constexpr int VEC = Policy::kVec;
   constexpr int SF = Policy::kState;
   if ((int64_t)blockIdx.x >= geo.n_wg) {
     // Trailing blocks: one lane group per row, rows without edges get the empty
     // value.  They share the launch with the gathers, so this small amount of
     // streaming work hides behind them instead of costing a pass of its own.
     const int tpr_ = 1 << geo.tpr_shift;
-    const int f0_ = ((int)blockIdx.y * tpr_ + (threadIdx.x & (tpr_ - 1))) * VEC;
+    const int f0_ = lane_first_feature<Policy>((int)blockIdx.y, threadIdx.x & (tpr_ - 1), geo.tpr_shift);
     const int64_t row = (((int64_t)blockIdx.x - geo.n_wg) * kBlock + threadIdx.x) >> geo.tpr_shift;
     if (f0_ < geo.feat && row < geo.n_rows && pointer[row] == pointer[row + 1])
       Policy::emit_empty(args, out, row, geo.feat, f0_);
@@ -116,7 +128,7 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
   const int lane = threadIdx.x & (tpr - 1);
   const int64_t k = (int64_t)blockIdx.x * G + grp;
   const int flane = (int)blockIdx.y * tpr + lane;   // feature lane index
-  const int f0 = flane * VEC;
+  const int f0 = lane_first_feature<Policy>((int)blockIdx.y, lane, geo.tpr_shift);
   const bool live = k < geo.n_runs && f0 < geo.feat;
 
   float *my_a = lds_state + ((grp * 2 + 0) * tpr + lane) * SF;
@@ -235,12 +247,11 @@ __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
     const int32_t *__restrict__ row_of_slot,
     const float *__restrict__ partial, typename Policy::out_t *__restrict__ out,
     RunGeom geo, int64_t n_wg, int fix_blocks) {
-  constexpr int VEC = Policy::kVec;
   constexpr int SF = Policy::kState;
   const int tpr = 1 << geo.tpr_shift;
   const int G = kBlock >> geo.tpr_shift;
   const int flane = (int)blockIdx.y * tpr + (threadIdx.x & (tpr - 1));
-  const int f0 = flane * VEC;
+  const int f0 = lane_first_feature<Policy>((int)blockIdx.y, threadIdx.x & (tpr - 1), geo.tpr_shift);
   if (f0 >= geo.feat) return;
   if ((int)blockIdx.x < fix_blocks) {
     const int64_t q = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> geo.tpr_shift;
@@ -282,15 +293,20 @@ __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
   }
 }
 
-// Workspace bound that holds for every element type / vector width: at most
-// ceil(n_runs / 4) workgroups (tpr <= 64), two partial rows each.
+// Workspace bound that holds for every element type, vector width and lane layout:
+// at most ceil(n_runs / 4) workgroups (tpr <= 64), two partial rows each.  A partial
+// row has a state per lane of every feature tile, dead lanes included; the widest
+// case is the spread layout of four features per lane, whose tiles are counted here.
 inline size_t runs_workspace_bytes(int64_t n_edges, int64_t feat,
                                    int state_floats_per_feature) {
   if (n_edges <= 0 || feat <= 0) return 0;
   const int run_shift = run_shift_for(n_edges, feat);
   const int64_t n_runs = (n_edges + ((int64_t)1 << run_shift) - 1) >> run_shift;
   const int64_t n_wg = (n_runs + 3) / 4;
-  return (size_t)n_wg * 2 * (size_t)feat * state_floats_per_feature * sizeof(float);
+  const int64_t lanes = (feat + 3) / 4;
+  const int64_t tpr = (int64_t)1 << ilog2_ceil((uint64_t)(lanes > kWave ? kWave : lanes));
+  const int64_t slots = (lanes + tpr - 1) / tpr * tpr * 4;
+  return (size_t)n_wg * 2 * (size_t)slots * state_floats_per_feature * sizeof(float);
 }
 
 template <class Policy>
@@ -309,7 +325,8 @@ int launch_runs(typename Policy::Args args, const int32_t *pointer,
   geo.n_edges = n_edges;
   geo.n_rows = n_rows;
   geo.feat = feat;
-  geo.lanes_total = lanes;
+  geo.lanes_total = Policy::kSpread ? ftiles * tpr : lanes;
+  if constexpr (Policy::kSpread) args.stride_shift = geo.tpr_shift;
   const int G = kBlock >> geo.tpr_shift;
   const int64_t n_wg = (geo.n_runs + G - 1) / G;
   const int64_t row_blocks = (n_rows + G - 1) / G;

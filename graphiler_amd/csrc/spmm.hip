@@ -42,12 +42,15 @@ __device__ __forceinline__ float bin_apply(float x, float w) {
 }
 
 // Row-reduction policy of the SpMM: the state is the VEC running reductions.
-template <typename T, int VEC, int RED, int BOP>
+// SPREAD: the lane's features lie a lane-group width apart (rows that 16-byte
+// accesses do not tile); all of them must share the edge datum, i.e. one head.
+template <typename T, int VEC, int RED, int BOP, bool SPREAD = false>
 struct SpmmPolicy {
   static constexpr bool HASW = BOP != 0;
   typedef T out_t;
   static constexpr int kVec = VEC;
   static constexpr int kState = VEC;
+  static constexpr bool kSpread = SPREAD;
   struct Args {
     const int32_t *gidx;  // row of `u` gathered per slot (neighbour id, or edge
                           // id for copy_e); nullptr: the slot index itself
@@ -57,6 +60,7 @@ struct SpmmPolicy {
     int heads;
     int dph;
     bool ids_vec;   // row_of_slot, gidx and eid (where given) are 16-byte aligned
+    int stride_shift;   // SPREAD: log2 of the lanes per group, set by the launcher
   };
   static __device__ __forceinline__ void init(float (&st)[VEC]) {
 #pragma unroll
@@ -71,13 +75,13 @@ struct SpmmPolicy {
     for (int v = 0; v < VEC; ++v) o[v] = st[v];
   }
   static __device__ __forceinline__ void empty_row(float (&o)[VEC]) { init(o); }
-  static __device__ __forceinline__ void emit(const Args &, out_t *out, int64_t row, int feat,
+  static __device__ __forceinline__ void emit(const Args &A, out_t *out, int64_t row, int feat,
                                               int f0, const float (&st)[kState]) {
-    emit_row<SpmmPolicy>(out, row, feat, f0, st);
+    emit_row<SpmmPolicy>(out, row, feat, f0, st, A.stride_shift);
   }
-  static __device__ __forceinline__ void emit_empty(const Args &, out_t *out, int64_t row,
+  static __device__ __forceinline__ void emit_empty(const Args &A, out_t *out, int64_t row,
                                                     int feat, int f0) {
-    emit_empty_row<SpmmPolicy>(out, row, feat, f0);
+    emit_empty_row<SpmmPolicy>(out, row, feat, f0, A.stride_shift);
   }
 
   template <class Close>
@@ -86,8 +90,9 @@ struct SpmmPolicy {
                                               int64_t a, int64_t b, int f0, int feat,
                                               float (&st)[VEC], int &cur,
                                               Close &&close_segment) {
-    typedef Frag<T, VEC> IO;
-    const int h = HASW ? f0 / A.dph : 0;
+    typedef RowIO<T, VEC, SPREAD> IO;
+    const typename IO::lane_t ln = IO::lane(A.stride_shift, feat - f0);
+    const int h = HASW && !SPREAD ? f0 / A.dph : 0;
     for (int64_t j = a; j < b; j += kUnroll) {
       int r[kUnroll], g[kUnroll], e[kUnroll];
       float ww[kUnroll];
@@ -110,7 +115,7 @@ struct SpmmPolicy {
         for (int t = 0; t < kUnroll; ++t) ww[t] = A.w[(int64_t)e[t] * A.heads + h];
       }
 #pragma unroll
-      for (int t = 0; t < kUnroll; ++t) x[t] = IO::load(A.u + (int64_t)g[t] * feat + f0);
+      for (int t = 0; t < kUnroll; ++t) x[t] = IO::load(A.u + (int64_t)g[t] * feat + f0, ln);
 #pragma unroll
       for (int t = 0; t < kUnroll; ++t) {
         if (j + t < b) {
@@ -130,15 +135,15 @@ struct SpmmPolicy {
   }
 };
 
-template <typename T, int VEC, int RED, int BOP>
+template <typename T, int VEC, int RED, int BOP, bool SPREAD>
 int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
                 const int32_t *gidx, const int32_t *eid, const void *u,
                 const float *w, void *out, int64_t n_rows, int64_t n_edges,
                 int feat, int heads, float *partial, hipStream_t stream) {
-  typedef SpmmPolicy<T, VEC, RED, BOP> P;
+  typedef SpmmPolicy<T, VEC, RED, BOP, SPREAD> P;
   const bool ids_vec = aligned(row_of_slot, 16) && (!gidx || aligned(gidx, 16)) &&
                        (!eid || aligned(eid, 16));
-  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads, ids_vec};
+  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads, ids_vec, 0};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, feat,
                         partial, stream);
 }
@@ -158,6 +163,7 @@ struct SpmmArgPolicy {
   typedef T out_t;
   static constexpr int kVec = VEC;
   static constexpr int kState = 2 * VEC;
+  static constexpr bool kSpread = false;
   struct Args {
     const int32_t *gidx;  // row of `u` gathered per slot; nullptr: the slot index
     const int32_t *eid;   // edge id per slot; nullptr: the slot index
@@ -295,14 +301,14 @@ int launch_spmm_arg(int reduce, int bop, const int32_t *pointer,
 #undef GA_SPMM_ARG
 }
 
-template <typename T, int VEC, int RED>
+template <typename T, int VEC, int RED, bool SPREAD>
 int pick_w(int bop, const int32_t *pointer, const int32_t *row_of_slot,
            const int32_t *gidx, const int32_t *eid, const void *u,
            const float *w, void *out, int64_t n_rows, int64_t n_edges, int feat,
            int heads, float *partial, hipStream_t stream) {
 #define GA_SPMM_BOP(B)                                                             \
-  return launch_spmm<T, VEC, RED, B>(pointer, row_of_slot, gidx, eid, u, w, out,   \
-                                     n_rows, n_edges, feat, heads, partial, stream)
+  return launch_spmm<T, VEC, RED, B, SPREAD>(pointer, row_of_slot, gidx, eid, u, w, out, \
+                                             n_rows, n_edges, feat, heads, partial, stream)
   switch (bop) {
     case GA_U_MUL_E: GA_SPMM_BOP(GA_U_MUL_E);
     case GA_U_ADD_E: GA_SPMM_BOP(GA_U_ADD_E);
@@ -313,7 +319,7 @@ int pick_w(int bop, const int32_t *pointer, const int32_t *row_of_slot,
 #undef GA_SPMM_BOP
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool SPREAD = false>
 int pick_red(int reduce, int bop, const int32_t *pointer,
              const int32_t *row_of_slot, const int32_t *gidx,
              const int32_t *eid, const void *u, const float *w, void *out,
@@ -321,15 +327,15 @@ int pick_red(int reduce, int bop, const int32_t *pointer,
              float *partial, hipStream_t stream) {
   switch (reduce) {
     case GA_SUM:
-      return pick_w<T, VEC, GA_SUM>(bop, pointer, row_of_slot, gidx, eid, u, w,
+      return pick_w<T, VEC, GA_SUM, SPREAD>(bop, pointer, row_of_slot, gidx, eid, u, w,
                                     out, n_rows, n_edges, feat, heads, partial,
                                     stream);
     case GA_MAX:
-      return pick_w<T, VEC, GA_MAX>(bop, pointer, row_of_slot, gidx, eid, u, w,
+      return pick_w<T, VEC, GA_MAX, SPREAD>(bop, pointer, row_of_slot, gidx, eid, u, w,
                                     out, n_rows, n_edges, feat, heads, partial,
                                     stream);
     default:
-      return pick_w<T, VEC, GA_MIN>(bop, pointer, row_of_slot, gidx, eid, u, w,
+      return pick_w<T, VEC, GA_MIN, SPREAD>(bop, pointer, row_of_slot, gidx, eid, u, w,
                                     out, n_rows, n_edges, feat, heads, partial,
                                     stream);
   }
@@ -405,11 +411,18 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
   const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
   hipStream_t s = (hipStream_t)stream;
   float *partial = (float *)workspace;
+  // rows that 16-byte accesses do not tile: four features per lane, a lane-group
+  // width apart, when all of a row shares the edge datum (one head, or none read)
+  const bool spread_ok = (!hasw || heads == 1) && feat >= 3 && feat <= 256;
   if (dtype == GA_F32) {
     if (vec_ok && feat % 4 == 0 && (!hasw || dph % 4 == 0))
       return ga::pick_red<float, 4>(reduce, bop, pointer, row_of_slot, gidx,
                                     eid, u, w, out, n_rows, n_edges, (int)feat,
                                     (int)heads, partial, s);
+    if (spread_ok)
+      return ga::pick_red<float, 4, true>(reduce, bop, pointer, row_of_slot, gidx,
+                                          eid, u, w, out, n_rows, n_edges, (int)feat,
+                                          (int)heads, partial, s);
     return ga::pick_red<float, 1>(reduce, bop, pointer, row_of_slot, gidx, eid,
                                   u, w, out, n_rows, n_edges, (int)feat,
                                   (int)heads, partial, s);
@@ -418,6 +431,10 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
     return ga::pick_red<ga::bf16_t, 8>(reduce, bop, pointer, row_of_slot, gidx,
                                        eid, u, w, out, n_rows, n_edges,
                                        (int)feat, (int)heads, partial, s);
+  if (spread_ok)
+    return ga::pick_red<ga::bf16_t, 4, true>(reduce, bop, pointer, row_of_slot, gidx,
+                                             eid, u, w, out, n_rows, n_edges, (int)feat,
+                                             (int)heads, partial, s);
   return ga::pick_red<ga::bf16_t, 1>(reduce, bop, pointer, row_of_slot, gidx,
                                      eid, u, w, out, n_rows, n_edges, (int)feat,
                                      (int)heads, partial, s);

@@ -369,6 +369,59 @@ def test_gat_aggregate_fused(graph, device, heads, dim, bf16):
     assert not got.float().cpu().numpy()[np.diff(arr.in_pointer) == 0].any()
 
 
+@pytest.mark.parametrize("feat", [3, 7, 17, 41, 65, 130, 255])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_one_head_rows_without_16_byte_tiles(graph, device, feat, bf16):
+    """Feature rows that 16-byte accesses do not tile (odd widths, bf16 widths that
+    are not multiples of 8), one head: the row reductions then give each lane four
+    features a lane-group width apart.  Copy and weighted sums, a max, the fused GAT
+    chain and the per-edge softmax sum against the oracle; the unaligned-base case
+    takes the same kernels from a view that starts one element into a buffer."""
+    name, g, arr = graph
+    rng = np.random.default_rng(feat * 3 + bf16)
+    n, e = arr.num_nodes, arr.COO_src.shape[0]
+    tol = TOL_BF16 if bf16 else TOL_F32
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    m = rng.standard_normal((e, feat), dtype=np.float32)
+    w = rng.standard_normal((e, 1), dtype=np.float32)
+    if bf16:
+        x, m = to_bf16_f32(x), to_bf16_f32(m)
+    xd, md, wd = _dev(x, device, bf16), _dev(m, device, bf16), _dev(w, device)
+    adj = (arr.in_pointer, arr.in_node_indices, arr.in_edge_indices)
+    empty = np.diff(arr.in_pointer) == 0
+
+    got = ops.SpMMSrc(xd, [1], False, None, g).float().cpu().numpy()
+    assert_close(got, oracle.spmm(*adj, x, op="copy_u"), tol, f"copy_u {name} F={feat}")
+    assert not got[empty].any()
+    shifted = torch.empty(n * feat + 1, dtype=xd.dtype, device=device)[1:].view(n, feat)
+    shifted.copy_(xd)
+    got = ops.SpMMSrc(shifted, [1], False, None, g).float().cpu().numpy()
+    assert_close(got, oracle.spmm(*adj, x, op="copy_u"), tol, f"copy_u shifted {name} F={feat}")
+    got = ops.SpMMEdge(md, [1], False, None, g).float().cpu().numpy()
+    assert_close(got, oracle.spmm(*adj, m, op="copy_e"), tol, f"copy_e {name} F={feat}")
+    got = ops.gspmm_src_mul_e_sum(xd, wd, [1], False, None, g).float().cpu().numpy()
+    assert_close(got, oracle.spmm(*adj, x, w, op="u_mul_e", heads=1), tol,
+                 f"u_mul_e {name} F={feat}")
+    got = ops.spmm(g, "copy_u", "max", xd).float().cpu().numpy()
+    ref = oracle.spmm(*adj, x, op="copy_u", reduce="max")
+    assert np.array_equal(np.isfinite(got), np.isfinite(ref))
+    assert np.array_equal(got[~empty], ref[~empty]), f"max {name} F={feat}"
+
+    el = rng.standard_normal((n, 1), dtype=np.float32) * 2
+    er = rng.standard_normal((n, 1), dtype=np.float32) * 2
+    got = ops.gat_aggregate(_dev(el, device), _dev(er, device), xd, g, 0.2).float().cpu().numpy()
+    ref = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er, x, heads=1, slope=0.2)
+    assert_close(got, ref, tol, f"fused GAT {name} D={feat}")
+    assert not got[empty].any()
+
+    logit = (rng.standard_normal((e, 1)) * 3).astype(np.float32)
+    att = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, logit)
+    prod = (m.astype(np.float64) * att).astype(np.float32)
+    got = ops.edge_softmax_sum(_dev(logit, device), md, g).float().cpu().numpy()
+    assert_close(got, oracle.spmm(*adj, prod, op="copy_e"), TOL_BF16 if bf16 else 2 * TOL_F32,
+                 f"edge_softmax_sum {name} D={feat}")
+
+
 @pytest.mark.parametrize("heads,dim,bf16", [(1, 64, False), (4, 64, True), (8, 16, True),
                                             (2, 8, False), (3, 32, False), (1, 16, True)])
 def test_gat_aggregate_from_z(graph, device, heads, dim, bf16):
