@@ -12,7 +12,8 @@
 //      logits are read exactly once;
 //   4. the (at most two) rows a chunk shares with its neighbours leave their
 //      per-head (max, sum-exp) in the workspace; a second launch merges the
-//      partials of such a row in chunk order and writes its elements.
+//      partials of every such row once (one workgroup per row, so a row of any
+//      length costs one pass over its partials), a third writes the elements.
 // Other head counts use a lane-group kernel that runs the heads one after the
 // other, with chunked two-pass handling of rows longer than 1024 slots.
 // No atomics; the order of every reduction is fixed by the graph and sizes.
@@ -304,9 +305,128 @@ __global__ __launch_bounds__(kBlock) void softmax_chunks_kernel(
                                       head_shift, chunk_id, c0, c1, lds_v);
 }
 
-// Pass 2: the rows a chunk shares with its neighbours (A = first row, begun in
-// an earlier chunk; B = last row, started here and continuing).  Both rows are
-// handled side by side so their dependent loads overlap.
+// Pass 2: every row that starts in one chunk and continues into later ones gets its
+// partials -- B of its first chunk, A of the following ones -- merged once, as
+// (max, sum-exp) pairs: the chunk list is split over the lanes of a head, each lane
+// folds its chunks in ascending order (four loads in flight), and a fixed tree
+// combines the lanes.  The row's pair is left in the A slot of the row's second
+// chunk, which nothing else reads.  Rows of up to kWaveMergeChunks chunks are merged
+// by the wavefront of their first chunk (softmax_row_totals_kernel, same grid as
+// pass 1); longer rows by a workgroup of 1024 lanes each (softmax_long_row_totals_
+// kernel), so that a row of any length costs one parallel pass over its partials.
+constexpr int kWaveMergeShift = 9;
+constexpr int kWaveMergeChunks = 1 << kWaveMergeShift;
+constexpr int kTotalsBlock = 1024;
+
+// (m, l) <- (m, l) (+) (sm, sl).  The side that holds the maximum keeps its sum
+// unscaled (also when both maxima are -inf: the sums are then 0 or NaN and stay
+// so); the empty state (-inf, 0) scales by 0 (exp_fast has no value at -inf).
+__device__ __forceinline__ void pair_merge(float &m, float &l, float sm, float sl) {
+  const float nm = fmaxf(m, sm);
+  const float a = m == nm ? 1.0f : (m == -INFINITY ? 0.0f : exp_fast(m - nm));
+  const float b = sm == nm ? 1.0f : (sm == -INFINITY ? 0.0f : exp_fast(sm - nm));
+  l = l * a + sl * b;
+  m = nm;
+}
+
+// Lane (g, h) of G lane groups folds chunks k_lo + g, k_lo + g + G, ... <= k_hi of head h.
+__device__ __forceinline__ void fold_row_partials(const float *__restrict__ stats, int64_t k_lo,
+                                                  int64_t k_hi, int g, int G, int H, int h,
+                                                  float &m, float &l) {
+  m = -INFINITY;
+  l = 0.0f;
+  int64_t c = k_lo + g;
+  if (g == 0) {                               // the B partial of the row's first chunk
+    const float *st = stats + ((k_lo * 2 + 1) * H + h) * 2;
+    m = st[0];
+    l = st[1];
+    c += G;
+  }
+  const int64_t step = (int64_t)2 * H * 2;    // floats from one chunk's A slot to the next
+  const float *p = stats + ((c * 2) * H + h) * 2;
+  for (; c + 3 * (int64_t)G <= k_hi; c += 4 * (int64_t)G, p += 4 * G * step) {
+    float2 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const float2 *>(p + u * G * step);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) pair_merge(m, l, v[u].x, v[u].y);
+  }
+  for (; c <= k_hi; c += G, p += G * step) {
+    const float2 v = *reinterpret_cast<const float2 *>(p);
+    pair_merge(m, l, v.x, v.y);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void softmax_row_totals_kernel(
+    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
+    float *__restrict__ stats, int64_t n_edges, int head_shift) {
+  ChunkInfo ci;
+  if (!chunk_info(row_of_slot, n_edges, head_shift, ci)) return;
+  if (!ci.continues) return;
+  const int cs_shift = 10 - head_shift;       // chunk_slots = 1024 >> head_shift
+  const int64_t s = pointer[ci.row_last], e = pointer[ci.row_last + 1];
+  if (s < ci.c0) return;                      // the row started in an earlier chunk
+  const int64_t chunk = ci.c0 >> cs_shift, k_hi = (e - 1) >> cs_shift;
+  if (k_hi - chunk >= kWaveMergeChunks) return;   // left to the workgroup kernel
+  const int H = 1 << head_shift;
+  const int lane = threadIdx.x & (kWave - 1);
+  float m, l;
+  fold_row_partials(stats, chunk, k_hi, lane >> head_shift, kWave >> head_shift, H,
+                    lane & (H - 1), m, l);
+  // butterfly over the lane groups; partner pairs are merged lower group first
+  for (int o = H; o < kWave; o <<= 1) {
+    const float pm = __shfl_xor(m, o), pl = __shfl_xor(l, o);
+    if (lane & o) {
+      float qm = pm, ql = pl;
+      pair_merge(qm, ql, m, l);
+      m = qm;
+      l = ql;
+    } else {
+      pair_merge(m, l, pm, pl);
+    }
+  }
+  if (lane < H) *reinterpret_cast<float2 *>(stat_ptr(stats, chunk + 1, 0, H, lane)) = make_float2(m, l);
+}
+
+// Workgroup j (>= 1) looks at the row that covers the first slot of chunk
+// j * kWaveMergeChunks and merges it when it is longer than kWaveMergeChunks chunks
+// and that chunk is the first multiple of kWaveMergeChunks after the row's first
+// chunk -- every such row contains exactly one.
+__global__ __launch_bounds__(kTotalsBlock) void softmax_long_row_totals_kernel(
+    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
+    float *__restrict__ stats, int head_shift) {
+  __shared__ float2 red[kTotalsBlock];
+  const int cs_shift = 10 - head_shift;
+  const int64_t mark = ((int64_t)blockIdx.x + 1) << kWaveMergeShift;
+  const int row = row_of_slot[mark << cs_shift];
+  const int64_t s = pointer[row], e = pointer[row + 1];
+  const int64_t k_lo = s >> cs_shift, k_hi = (e - 1) >> cs_shift;
+  if (k_hi - k_lo < kWaveMergeChunks) return;
+  if (((k_lo >> kWaveMergeShift) + 1) << kWaveMergeShift != mark) return;
+  const int H = 1 << head_shift;
+  const int h = threadIdx.x & (H - 1);
+  float m, l;
+  fold_row_partials(stats, k_lo, k_hi, threadIdx.x >> head_shift, kTotalsBlock >> head_shift,
+                    H, h, m, l);
+  red[threadIdx.x] = make_float2(m, l);
+  __syncthreads();                            // also: every partial has been read
+  for (int o = kTotalsBlock >> 1; o >= H; o >>= 1) {
+    if ((int)threadIdx.x < o) {
+      float2 p = red[threadIdx.x];
+      const float2 q = red[threadIdx.x + o];
+      pair_merge(p.x, p.y, q.x, q.y);
+      red[threadIdx.x] = p;
+    }
+    __syncthreads();
+  }
+  if ((int)threadIdx.x < H)
+    *reinterpret_cast<float2 *>(stat_ptr(stats, k_lo + 1, 0, H, h)) = red[h];
+}
+
+// Pass 3: the rows a chunk shares with its neighbours (A = first row, begun in
+// an earlier chunk; B = last row, started here and continuing) are normalised with
+// their merged statistics.  Both rows are handled side by side so their dependent
+// loads overlap.
 __global__ __launch_bounds__(kBlock) void softmax_boundary_kernel(
     const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
     const int32_t *__restrict__ eid, const float *__restrict__ x,
@@ -343,23 +463,13 @@ __global__ __launch_bounds__(kBlock) void softmax_boundary_kernel(
   float m[2], rcp_l[2];
 #pragma unroll
   for (int w = 0; w < 2; ++w) {
-    // merge the row's partials (B of its first chunk, then A's): the lanes of
-    // a head split the chunk list, then combine with a fixed shuffle tree
-    const int64_t k_lo = s[w] >> cs_shift, k_hi = (e[w] - 1) >> cs_shift;
-    float mm = -INFINITY;
-    if (e[w] > s[w])
-      for (int64_t c = k_lo + g; c <= k_hi; c += G)
-        mm = fmaxf(mm, stat_ptr(stats, c, c == k_lo ? 1 : 0, H, h)[0]);
-    for (int o = kWave >> 1; o >= H; o >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o));
-    float l = 0.0f;
-    if (e[w] > s[w])
-      for (int64_t c = k_lo + g; c <= k_hi; c += G) {
-        const float *st = stat_ptr(stats, c, c == k_lo ? 1 : 0, H, h);
-        l += st[1] * exp_fast(st[0] - mm);
-      }
-    for (int o = kWave >> 1; o >= H; o >>= 1) l += __shfl_xor(l, o);
-    m[w] = mm;
-    rcp_l[w] = __builtin_amdgcn_rcpf(l);
+    m[w] = 0.0f;
+    rcp_l[w] = 0.0f;
+    if (e[w] > s[w]) {      // totals of the row: A slot of its second chunk
+      const float *t = stat_ptr(stats, (s[w] >> cs_shift) + 1, 0, H, h);
+      m[w] = t[0];
+      rcp_l[w] = __builtin_amdgcn_rcpf(t[1]);
+    }
   }
 #pragma unroll
   for (int w = 0; w < 2; ++w) {
@@ -483,6 +593,33 @@ __global__ __launch_bounds__(kBlock) void softmax_long_stats_generic_kernel(
   }
 }
 
+// One workgroup per long row (the one that owns the row's first chunk) merges the
+// row's per-chunk statistics and leaves the totals in the first chunk's place.
+__global__ __launch_bounds__(kBlock) void softmax_long_totals_generic_kernel(
+    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
+    float *__restrict__ stats, int heads) {
+  __shared__ float lds[kBlock / kWave];
+  int64_t lo, hi, c_first, c_last;
+  if (!long_chunk(pointer, row_of_slot, kLongRow, kLongRow + 1, lo, hi, c_first,
+                  c_last))
+    return;
+  if ((int64_t)blockIdx.x != c_first) return;
+  for (int h = 0; h < heads; ++h) {
+    float m = -INFINITY;
+    for (int64_t c = c_first + threadIdx.x; c <= c_last; c += kBlock)
+      m = fmaxf(m, stats[(c * heads + h) * 2]);
+    m = block_reduce<true>(m, lds);
+    float l = 0.0f;
+    for (int64_t c = c_first + threadIdx.x; c <= c_last; c += kBlock)
+      l += stats[(c * heads + h) * 2 + 1] * expf(stats[(c * heads + h) * 2] - m);
+    l = block_reduce<false>(l, lds);   // its barriers: every partial has been read
+    if (threadIdx.x == 0) {
+      stats[(c_first * heads + h) * 2] = m;
+      stats[(c_first * heads + h) * 2 + 1] = l;
+    }
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void softmax_long_write_generic_kernel(
     const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
     const int32_t *__restrict__ eid, const float *__restrict__ x,
@@ -492,12 +629,8 @@ __global__ __launch_bounds__(kBlock) void softmax_long_write_generic_kernel(
                   c_last))
     return;
   for (int h = 0; h < heads; ++h) {
-    float m = -INFINITY;
-    for (int64_t c = c_first; c <= c_last; ++c)
-      m = fmaxf(m, stats[(c * heads + h) * 2]);
-    float l = 0.0f;
-    for (int64_t c = c_first; c <= c_last; ++c)
-      l += stats[(c * heads + h) * 2 + 1] * expf(stats[(c * heads + h) * 2] - m);
+    const float m = stats[(c_first * heads + h) * 2];
+    const float l = stats[(c_first * heads + h) * 2 + 1];
     for (int64_t q = lo + threadIdx.x; q < hi; q += kBlock) {
       const int64_t e = eid ? (int64_t)eid[q] : q;
       y[e * heads + h] = expf(x[e * heads + h] - m) / l;
@@ -559,10 +692,17 @@ int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
       hipLaunchKernelGGL(softmax_chunks_kernel<false>, dim3((unsigned)blocks),
                          dim3(kBlock), 0, s, row_of_slot, eid, x, y, stats,
                          n_edges, head_shift);
-    if (chunks > 1)
+    if (chunks > 1) {
+      hipLaunchKernelGGL(softmax_row_totals_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                         pointer, row_of_slot, stats, n_edges, head_shift);
+      const int64_t marks = (chunks - 1) >> kWaveMergeShift;   // multiples of the limit below `chunks`
+      if (marks > 0)
+        hipLaunchKernelGGL(softmax_long_row_totals_kernel, dim3((unsigned)marks),
+                           dim3(kTotalsBlock), 0, s, pointer, row_of_slot, stats, head_shift);
       hipLaunchKernelGGL(softmax_boundary_kernel, dim3((unsigned)blocks),
                          dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, y, stats,
                          n_edges, head_shift);
+    }
     return launch_status();
   }
 
@@ -582,6 +722,8 @@ int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
     hipLaunchKernelGGL(softmax_long_stats_generic_kernel, dim3((unsigned)lchunks),
                        dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, stats,
                        (int)heads);
+    hipLaunchKernelGGL(softmax_long_totals_generic_kernel, dim3((unsigned)lchunks),
+                       dim3(kBlock), 0, s, pointer, row_of_slot, stats, (int)heads);
     hipLaunchKernelGGL(softmax_long_write_generic_kernel, dim3((unsigned)lchunks),
                        dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, stats, y,
                        (int)heads);

@@ -309,6 +309,28 @@ def test_segment_softmax(graph, device, heads):
         assert np.abs(sums[nonempty] - 1.0).max() < 1e-5
 
 
+@pytest.mark.parametrize("heads", [1, 8, 32, 3])
+def test_segment_softmax_rows_over_many_chunks(device, heads):
+    """A row of 150,000 edges next to ordinary ones: its statistics are merged from
+    hundreds to thousands of per-chunk partials (once per row), and two more long
+    rows share chunks with it.  Edge ids shuffled against the adjacency order."""
+    rng = np.random.default_rng(heads + 77)
+    n = 400
+    dst = np.concatenate([np.full(150_000, 7), np.full(5_000, 8), np.full(2_500, 300),
+                          rng.integers(0, n, 3_000)]).astype(np.int64)
+    dst = dst[rng.permutation(dst.shape[0])]
+    src = rng.integers(0, n, dst.shape[0], dtype=np.int64)
+    g = prepare_graph(src, dst, n, device=device)
+    arr = build_graph_arrays(src, dst, n)
+    x = (rng.standard_normal((dst.shape[0], heads)) * 4.0).astype(np.float32)
+    got = ops.SegmentSoftmax(_dev(x, device), 1, None, g).cpu().numpy()
+    ref = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, x)
+    assert_close(got, ref, TOL_F32, f"softmax long rows H={heads}")
+    sums = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                       got.astype(np.float32), op="copy_e")
+    assert np.abs(sums[np.diff(arr.in_pointer) > 0] - 1.0).max() < 2e-5
+
+
 def test_segment_softmax_1d_input(graph, device):
     name, g, arr = graph
     rng = np.random.default_rng(0)
