@@ -16,6 +16,13 @@ __device__ __forceinline__ float load_f32<bf16_t>(const bf16_t *p) {
   return bf16_lo(*p);
 }
 
+// a / b for 0 <= a, 0 < b: the 32-bit division when the numerator fits, which is
+// several times shorter than the 64-bit one the flat indexings would otherwise pay
+// per element.
+__device__ __forceinline__ int64_t div_pos(int64_t a, int b) {
+  return (a >> 32) == 0 ? (int64_t)((uint32_t)a / (uint32_t)b) : a / b;
+}
+
 // ---- u (op) v --------------------------------------------------------------
 // One thread per output element; FEAT1 specialisation handles four consecutive
 // edges per thread so index and output accesses are 16 bytes wide.  OP is the
@@ -35,7 +42,7 @@ __global__ __launch_bounds__(kBlock) void u_add_v_kernel(
     int64_t n_edges, int feat) {
   const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (t >= n_edges * feat) return;
-  const int64_t i = t / feat;
+  const int64_t i = div_pos(t, feat);
   const int k = (int)(t - i * feat);
   out[t] = edge_op<OP>(load_f32(u + (int64_t)lhs[i] * feat + k),
                        load_f32(v + (int64_t)rhs[i] * feat + k));
@@ -90,20 +97,37 @@ __global__ __launch_bounds__(kBlock) void u_dot_v_vec_kernel(
   if (live && (lane & (lph - 1)) == 0) out[i * heads + lane / lph] = s;
 }
 
-template <typename IdxT, typename T>
-__global__ __launch_bounds__(kBlock) void u_dot_v_scalar_kernel(
+// Shapes the kernel above does not take (a row wider than a wavefront's 16-byte
+// loads, a head width that is not a power-of-two number of such loads, unaligned
+// storage): a group of 2^lpu_shift lanes per (edge, head) walks the head's `dim`
+// elements, VEC at a time (VEC > 1: dim % VEC == 0 and 16-byte aligned rows), the
+// lanes reading consecutive pieces; combined with xor shuffles (fixed tree).
+template <typename IdxT, typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void u_dot_v_group_kernel(
     const IdxT *__restrict__ lhs, const IdxT *__restrict__ rhs,
     const T *__restrict__ u, const T *__restrict__ v, float *__restrict__ out,
-    int64_t n_edges, int heads, int dim) {
-  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (t >= n_edges * heads) return;
-  const int64_t i = t / heads;
-  const int h = (int)(t - i * heads);
-  const T *a = u + ((int64_t)lhs[i] * heads + h) * dim;
-  const T *b = v + ((int64_t)rhs[i] * heads + h) * dim;
+    int64_t n_units, int heads, int dim, int lpu_shift) {
+  typedef Frag<T, VEC> IO;
+  const int lpu = 1 << lpu_shift;
+  const int lane = threadIdx.x & (lpu - 1);
+  const int64_t unit = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> lpu_shift;
+  const bool live = unit < n_units;
   float s = 0.0f;
-  for (int q = 0; q < dim; ++q) s = fmaf(load_f32(a + q), load_f32(b + q), s);
-  out[t] = s;
+  if (live) {
+    const int64_t i = div_pos(unit, heads);
+    const int h = (int)(unit - i * heads);
+    const T *a = u + ((int64_t)lhs[i] * heads + h) * dim;
+    const T *b = v + ((int64_t)rhs[i] * heads + h) * dim;
+    for (int q = lane * VEC; q < dim; q += lpu * VEC) {
+      float af[VEC], bf[VEC];
+      IO::widen(IO::load(a + q), af);
+      IO::widen(IO::load(b + q), bf);
+#pragma unroll
+      for (int t = 0; t < VEC; ++t) s = fmaf(af[t], bf[t], s);
+    }
+  }
+  for (int off = lpu >> 1; off > 0; off >>= 1) s += __shfl_xor(s, off);
+  if (live && lane == 0) out[unit] = s;
 }
 
 // ---- row gather --------------------------------------------------------------
@@ -120,10 +144,37 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(
   for (int64_t q = lane; q < units; q += gl) dst[q] = src[q];
 }
 
+// Rows whose unit count leaves many lanes of a power-of-two lane group idle: one
+// thread per output unit instead, so reads and writes are contiguous over the
+// whole wavefront whatever the row length.
+template <typename IdxT, typename UnitT>
+__global__ __launch_bounds__(kBlock) void gather_units_kernel(
+    const IdxT *__restrict__ idx, const UnitT *__restrict__ x,
+    UnitT *__restrict__ y, int64_t n_units_total, int units) {
+  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t >= n_units_total) return;
+  const int64_t i = div_pos(t, units);
+  const int k = (int)(t - i * units);
+  y[t] = x[(int64_t)idx[i] * units + k];
+}
+
 template <typename IdxT, typename UnitT>
 int launch_gather(const void *idx, const void *x, void *y, int64_t n_out,
                   int64_t units, hipStream_t s) {
   const int gl_shift = ilog2_ceil((uint64_t)(units > kWave ? kWave : units));
+  const int64_t gl = (int64_t)1 << gl_shift;
+  const int64_t lane_slots = (units + gl - 1) / gl * gl;   // lanes x iterations per row
+  // more than 1/9 of them idle; longer rows amortise the idle tail and lose more to
+  // the per-element index arithmetic (measured: 129 units 15 % slower this way)
+  if (lane_slots * 8 > units * 9 && units < kWave) {
+    const int64_t total = n_out * units;
+    const int64_t fblocks = (total + kBlock - 1) / kBlock;
+    if (fblocks > 0x7fffffff) return GA_EUNSUPPORTED;
+    hipLaunchKernelGGL((gather_units_kernel<IdxT, UnitT>), dim3((unsigned)fblocks),
+                       dim3(kBlock), 0, s, (const IdxT *)idx, (const UnitT *)x,
+                       (UnitT *)y, total, (int)units);
+    return launch_status();
+  }
   const int64_t per_block = kBlock >> gl_shift;
   const int64_t blocks = (n_out + per_block - 1) / per_block;
   if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
@@ -170,6 +221,26 @@ int launch_u_op_v(const void *lhs, const void *rhs, const void *u,
 }
 
 template <typename IdxT, typename T, int VEC>
+int launch_u_dot_v_group(const void *lhs, const void *rhs, const void *u, const void *v,
+                         float *out, int64_t n_edges, int heads, int dim, hipStream_t s) {
+  // 16-byte pieces: one per lane and step, so a step reads the head's row contiguously;
+  // single elements: about four steps per lane (measured: one lane per element loses to
+  // a single lane per head at dim 5 and 17)
+  const int64_t pieces = (dim + VEC - 1) / VEC;
+  const int lpu_shift = VEC > 1 ? ilog2_ceil((uint64_t)(pieces > kWave ? kWave : pieces))
+                                : ilog2_floor((uint64_t)(pieces >= 4 * kWave ? kWave
+                                                         : (pieces >= 4 ? pieces / 4 : 1)));
+  const int64_t n_units = n_edges * heads;
+  const int64_t per_block = kBlock >> lpu_shift;
+  const int64_t blocks = (n_units + per_block - 1) / per_block;
+  if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
+  hipLaunchKernelGGL((u_dot_v_group_kernel<IdxT, T, VEC>), dim3((unsigned)blocks),
+                     dim3(kBlock), 0, s, (const IdxT *)lhs, (const IdxT *)rhs,
+                     (const T *)u, (const T *)v, out, n_units, heads, dim, lpu_shift);
+  return launch_status();
+}
+
+template <typename IdxT, typename T, int VEC>
 int launch_u_dot_v(const void *lhs, const void *rhs, const void *u,
                    const void *v, float *out, int64_t n_edges, int heads,
                    int dim, hipStream_t s) {
@@ -186,12 +257,10 @@ int launch_u_dot_v(const void *lhs, const void *rhs, const void *u,
                        dim3((unsigned)blocks), dim3(kBlock), 0, s,
                        (const IdxT *)lhs, (const IdxT *)rhs, (const T *)u,
                        (const T *)v, out, n_edges, heads, dim, gl_shift, lph);
+  } else if (VEC > 1 && dim % VEC == 0 && aligned(u, 16) && aligned(v, 16)) {
+    return launch_u_dot_v_group<IdxT, T, VEC>(lhs, rhs, u, v, out, n_edges, heads, dim, s);
   } else {
-    const int64_t blocks = (n_edges * heads + kBlock - 1) / kBlock;
-    if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-    hipLaunchKernelGGL((u_dot_v_scalar_kernel<IdxT, T>), dim3((unsigned)blocks),
-                       dim3(kBlock), 0, s, (const IdxT *)lhs, (const IdxT *)rhs,
-                       (const T *)u, (const T *)v, out, n_edges, heads, dim);
+    return launch_u_dot_v_group<IdxT, T, 1>(lhs, rhs, u, v, out, n_edges, heads, dim, s);
   }
   return launch_status();
 }

@@ -276,7 +276,8 @@ def test_sddmm_u_op_v_bit_exact(graph, device, op, feat):
 
 
 @pytest.mark.parametrize("heads,dim", [(1, 64), (8, 16), (4, 64), (3, 5),
-                                       (1, 1), (2, 256)])
+                                       (1, 1), (2, 256), (8, 64), (1, 17), (2, 24),
+                                       (1, 300), (5, 129)])
 @pytest.mark.parametrize("bf16", [False, True])
 def test_sddmm_u_dot_v(graph, device, heads, dim, bf16):
     name, g, arr = graph
@@ -343,7 +344,10 @@ def test_segment_softmax_1d_input(graph, device):
 
 @pytest.mark.parametrize("shape,dtype", [((64,), np.float32), ((1,), np.float32),
                                          ((3, 5), np.float32), ((7,), np.int64),
-                                         ((128,), np.float16), ((3,), np.uint8)])
+                                         ((128,), np.float16), ((3,), np.uint8),
+                                         ((17,), np.float32), ((129,), np.float32),
+                                         ((18,), np.float32), ((33,), np.float16),
+                                         ((5,), np.uint8), ((100,), np.float64)])
 def test_broadcast_bit_exact(graph, device, shape, dtype):
     name, g, arr = graph
     rng = np.random.default_rng(1)
