@@ -823,10 +823,14 @@ __global__ __launch_bounds__(kBlock) void segment_mm_scalar_kernel(
 }
 
 template <typename T, int KBLK, int CG>
-void launch_cg(const int32_t *tp, const T *X, const T *W, T *Y, const MmGeom &g,
-               int64_t grid, size_t lds, hipStream_t s) {
+int launch_cg(const int32_t *tp, const T *X, const T *W, T *Y, const MmGeom &g,
+              int64_t grid, size_t lds, hipStream_t s) {
+  // weight tiles above the default 64 KB (fp32 K = 256 x M = 64 and up) opt in to
+  // the CU's full LDS
+  if (!allow_lds((const void *)segment_mm_kernel<T, KBLK, CG>, lds)) return GA_EUNSUPPORTED;
   hipLaunchKernelGGL((segment_mm_kernel<T, KBLK, CG>), dim3((unsigned)grid),
                      dim3(kBlock), lds, s, tp, X, W, Y, g);
+  return launch_status();
 }
 
 template <typename T, int KBLK, int NF, int CG, int EPI>
@@ -935,18 +939,16 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
   }
   if (fused) return GA_EUNSUPPORTED;   // only the exact-shape kernel gathers
   const size_t lds = (size_t)MM::tile_elems(g.KB, g.MB) * sizeof(T);
-  if (lds > (size_t)kMaxLds) return GA_EUNSUPPORTED;
+  if (lds > (size_t)kMaxLdsOptIn) return GA_EUNSUPPORTED;
   const int mbp = MM::mb_pad(g.MB);
   if (MM::kPaired) {
-    if (mbp <= 2) launch_cg<T, KBLK, 2>(tp, Xh, Wh, Yh, g, grid, lds, s);
-    else if (mbp <= 4) launch_cg<T, KBLK, 4>(tp, Xh, Wh, Yh, g, grid, lds, s);
-    else launch_cg<T, KBLK, 8>(tp, Xh, Wh, Yh, g, grid, lds, s);
-  } else {
-    if (mbp <= 1) launch_cg<T, KBLK, 1>(tp, Xh, Wh, Yh, g, grid, lds, s);
-    else if (mbp <= 2) launch_cg<T, KBLK, 2>(tp, Xh, Wh, Yh, g, grid, lds, s);
-    else launch_cg<T, KBLK, 4>(tp, Xh, Wh, Yh, g, grid, lds, s);
+    if (mbp <= 2) return launch_cg<T, KBLK, 2>(tp, Xh, Wh, Yh, g, grid, lds, s);
+    if (mbp <= 4) return launch_cg<T, KBLK, 4>(tp, Xh, Wh, Yh, g, grid, lds, s);
+    return launch_cg<T, KBLK, 8>(tp, Xh, Wh, Yh, g, grid, lds, s);
   }
-  return launch_status();
+  if (mbp <= 1) return launch_cg<T, KBLK, 1>(tp, Xh, Wh, Yh, g, grid, lds, s);
+  if (mbp <= 2) return launch_cg<T, KBLK, 2>(tp, Xh, Wh, Yh, g, grid, lds, s);
+  return launch_cg<T, KBLK, 4>(tp, Xh, Wh, Yh, g, grid, lds, s);
 }
 
 template <typename T, int KBLK>

@@ -498,7 +498,8 @@ def _typed_rows(rng, counts):
 @pytest.mark.parametrize("K,M,heads", [(16, 64, 1), (64, 8, 1), (64, 64, 1),
                                        (128, 128, 1), (20, 12, 1), (6, 5, 1),
                                        (16, 16, 8), (32, 48, 2), (8, 3, 3),
-                                       (256, 32, 1), (128, 200, 1)])
+                                       (256, 32, 1), (128, 200, 1), (256, 64, 1),
+                                       (512, 64, 1), (256, 128, 1), (132, 16, 2)])
 @pytest.mark.parametrize("bf16", [False, True])
 def test_segment_mm(device, K, M, heads, bf16):
     rng = np.random.default_rng(K * 1000 + M + heads)
