@@ -238,9 +238,35 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
 
 // Blocks [0, fix_blocks): one lane group per main-kernel workgroup q; the group
 // whose slot range holds the END of a row that began in an earlier workgroup
-// combines that row's global partial states in workgroup order.  Remaining
-// blocks (only for a graph without edges, where the main kernel does not run):
-// one lane group per row, every row gets Policy::empty_row.
+// combines that row's global partial states in workgroup order.  A chain of more
+// than kLongChain states (a row over that many workgroups) is combined by the whole
+// block instead: every lane group folds a contiguous piece of the chain, in order,
+// and the owning group combines the pieces in order -- so a row of any length costs
+// chain / groups sequential steps, not chain.  Remaining blocks (only for a graph
+// without edges, where the main kernel does not run): one lane group per row, every
+// row gets Policy::empty_row.
+constexpr int kLongChain = 64;
+
+// acc <- acc (+) states w0 .. w1-1 of a chain (stride floats apart, `src` at w0), four
+// fetched at a time so that the loads overlap instead of queueing up one latency
+// after the other.
+template <class Policy>
+__device__ __forceinline__ void fold_chain(float (&acc)[Policy::kState], const float *src,
+                                           int64_t stride, int64_t w0, int64_t w1) {
+  constexpr int SF = Policy::kState;
+  int64_t w = w0;
+  for (; w + 4 <= w1; w += 4, src += 4 * stride) {
+    float nxt[4][SF];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < SF; ++i) nxt[u][i] = src[u * stride + i];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) Policy::merge(acc, nxt[u]);
+  }
+  for (; w < w1; ++w, src += stride) Policy::merge(acc, src);
+}
+
 template <class Policy>
 __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
     typename Policy::Args args, const int32_t *__restrict__ pointer,
@@ -248,48 +274,78 @@ __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
     const float *__restrict__ partial, typename Policy::out_t *__restrict__ out,
     RunGeom geo, int64_t n_wg, int fix_blocks) {
   constexpr int SF = Policy::kState;
+  extern __shared__ float piece_state[];      // [thread][SF]: pieces of a long chain
+  __shared__ int64_t long_first[kBlock];      // per lane group: first workgroup of its long chain, or -1
   const int tpr = 1 << geo.tpr_shift;
   const int G = kBlock >> geo.tpr_shift;
-  const int flane = (int)blockIdx.y * tpr + (threadIdx.x & (tpr - 1));
-  const int f0 = lane_first_feature<Policy>((int)blockIdx.y, threadIdx.x & (tpr - 1), geo.tpr_shift);
-  if (f0 >= geo.feat) return;
-  if ((int)blockIdx.x < fix_blocks) {
-    const int64_t q = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> geo.tpr_shift;
-    if (q >= n_wg) return;
-    const int wg_shift = geo.run_shift + (8 - geo.tpr_shift);  // log2(G * run)
+  const int lane = threadIdx.x & (tpr - 1);
+  const int grp = threadIdx.x >> geo.tpr_shift;
+  const int flane = (int)blockIdx.y * tpr + lane;
+  const int f0 = lane_first_feature<Policy>((int)blockIdx.y, lane, geo.tpr_shift);
+  const bool lane_live = f0 < geo.feat;
+  if ((int)blockIdx.x >= fix_blocks) {
+    const int64_t row =
+        ((int64_t)(blockIdx.x - fix_blocks) * kBlock + threadIdx.x) >> geo.tpr_shift;
+    if (!lane_live || row >= geo.n_rows || pointer[row] != pointer[row + 1]) return;
+    Policy::emit_empty(args, out, row, geo.feat, f0);
+    return;
+  }
+  const int64_t q = (int64_t)blockIdx.x * G + grp;
+  const int wg_shift = geo.run_shift + (8 - geo.tpr_shift);  // log2(G * run)
+  const int64_t stride = (int64_t)2 * geo.lanes_total * SF;  // floats between workgroups' states
+  bool mine = false;     // a row that began in an earlier workgroup ends in workgroup q
+  int row = 0;
+  int64_t q_lo = 0;
+  if (q < n_wg) {
     const int64_t a = q << wg_shift;
     const int64_t b = min(a + ((int64_t)1 << wg_shift), geo.n_edges);
-    const int row = row_of_slot[a];
+    row = row_of_slot[a];
     const int64_t s = pointer[row], e = pointer[row + 1];
-    if (!(s < a && e <= b)) return;
-    const int64_t q_lo = s >> wg_shift;
+    mine = s < a && e <= b;
+    q_lo = s >> wg_shift;
+  }
+  // the chain: slot 1 of workgroup q_lo, then slot 0 of workgroups q_lo + 1 .. q
+  const bool is_long = mine && q - q_lo > kLongChain;
+  if (lane == 0) long_first[grp] = is_long ? q_lo : -1;
+  if (mine && !is_long && lane_live) {
     float acc[SF];
     const float *p = partial + ((q_lo * 2 + 1) * geo.lanes_total + flane) * SF;
 #pragma unroll
     for (int i = 0; i < SF; ++i) acc[i] = p[i];
-    // the chain is combined in workgroup order; four states are fetched at a time
-    // so that the loads of a long chain (a hub row) overlap instead of queueing up
-    // one latency after the other
-    const int64_t stride = (int64_t)2 * geo.lanes_total * SF;
-    const float *src = partial + (((q_lo + 1) * 2) * geo.lanes_total + flane) * SF;
-    int64_t w = q_lo + 1;
-    for (; w + 3 <= q; w += 4, src += 4 * stride) {
-      float nxt[4][SF];
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int i = 0; i < SF; ++i) nxt[u][i] = src[u * stride + i];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) Policy::merge(acc, nxt[u]);
-    }
-    for (; w <= q; ++w, src += stride) Policy::merge(acc, src);
+    fold_chain<Policy>(acc, partial + (((q_lo + 1) * 2) * geo.lanes_total + flane) * SF, stride,
+                       q_lo + 1, q + 1);
     Policy::emit(args, out, row, geo.feat, f0, acc);
-    (void)G;
-  } else {
-    const int64_t row =
-        ((int64_t)(blockIdx.x - fix_blocks) * kBlock + threadIdx.x) >> geo.tpr_shift;
-    if (row >= geo.n_rows || pointer[row] != pointer[row + 1]) return;
-    Policy::emit_empty(args, out, row, geo.feat, f0);
+  }
+  if (!__syncthreads_or(is_long)) return;     // the usual case: no long chain in this block
+  // pieces: the first min(G, 64) lane groups take one each
+  const int p_shift = min(8 - geo.tpr_shift, 6);
+  for (int gg = 0; gg < G; ++gg) {
+    const int64_t c_lo = long_first[gg];      // the same for the whole block
+    if (c_lo < 0) continue;
+    const int64_t first = c_lo + 1;           // slot-0 states of workgroups first .. first + len - 1
+    const int64_t len = (int64_t)blockIdx.x * G + gg - c_lo;
+    const int64_t w0 = first + ((len * grp) >> p_shift), w1 = first + ((len * (grp + 1)) >> p_shift);
+    if (lane_live && (grp >> p_shift) == 0 && w0 < w1) {
+      float acc[SF];
+      const float *src = partial + ((w0 * 2) * geo.lanes_total + flane) * SF;
+#pragma unroll
+      for (int i = 0; i < SF; ++i) acc[i] = src[i];
+      fold_chain<Policy>(acc, src + stride, stride, w0 + 1, w1);
+#pragma unroll
+      for (int i = 0; i < SF; ++i) piece_state[threadIdx.x * SF + i] = acc[i];
+    }
+    __syncthreads();
+    if (grp == gg && lane_live) {             // the chain's own group: pieces in order
+      float acc[SF];
+      const float *p = partial + ((c_lo * 2 + 1) * geo.lanes_total + flane) * SF;
+#pragma unroll
+      for (int i = 0; i < SF; ++i) acc[i] = p[i];
+      for (int j = 0; j < (1 << p_shift); ++j)
+        if (((len * j) >> p_shift) < ((len * (j + 1)) >> p_shift))
+          Policy::merge(acc, piece_state + ((j << geo.tpr_shift) + lane) * SF);
+      Policy::emit(args, out, row, geo.feat, f0, acc);
+    }
+    __syncthreads();
   }
 }
 
@@ -345,8 +401,8 @@ int launch_runs(typename Policy::Args args, const int32_t *pointer,
   if (fix_blocks + fill_blocks > 0)
     hipLaunchKernelGGL((runs_fixup_kernel<Policy>),
                        dim3((unsigned)(fix_blocks + fill_blocks), ftiles),
-                       dim3(kBlock), 0, stream, args, pointer, row_of_slot, partial,
-                       (out_t *)out, geo, n_wg, (int)fix_blocks);
+                       dim3(kBlock), (size_t)kBlock * SF * sizeof(float), stream, args, pointer,
+                       row_of_slot, partial, (out_t *)out, geo, n_wg, (int)fix_blocks);
   return launch_status();
 }
 

@@ -310,17 +310,74 @@ def test_segment_softmax(graph, device, heads):
         assert np.abs(sums[nonempty] - 1.0).max() < 1e-5
 
 
+def _hub_graph(seed):
+    """400 nodes; node 7 has 150,000 in-edges, nodes 8 and 300 have 5,000 and 2,500,
+    3,000 more fall anywhere; edge ids shuffled against the adjacency order."""
+    rng = np.random.default_rng(seed)
+    n = 400
+    dst = np.concatenate([np.full(150_000, 7), np.full(5_000, 8), np.full(2_500, 300),
+                          rng.integers(0, n, 3_000)]).astype(np.int64)
+    dst = dst[rng.permutation(dst.shape[0])]
+    src = rng.integers(0, n, dst.shape[0], dtype=np.int64)
+    return src, dst, n
+
+
+@pytest.mark.parametrize("feat,heads,bf16", [(64, 1, False), (256, 4, True), (17, 1, False),
+                                             (1, 1, False), (128, 8, False)])
+def test_row_reductions_over_many_workgroups(device, feat, heads, bf16):
+    """A 150,000-edge row spans hundreds to thousands of workgroups of the row
+    reductions, so its partial states are combined by whole blocks (pieces of the
+    chain in parallel, then in order); the 5,000- and 2,500-edge rows take the
+    sequential chain.  Sums, extrema with their positions (small integers: exact, many
+    ties), the fused GAT chain and the per-edge softmax sum against the oracle."""
+    src, dst, n = _hub_graph(feat + heads)
+    rng = np.random.default_rng(feat)
+    e = src.shape[0]
+    g = prepare_graph(src, dst, n, device=device)
+    arr = build_graph_arrays(src, dst, n)
+    adj = (arr.in_pointer, arr.in_node_indices, arr.in_edge_indices)
+    tol = TOL_BF16 if bf16 else TOL_F32
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    w = rng.standard_normal((e, heads), dtype=np.float32)
+    if bf16:
+        x = to_bf16_f32(x)
+    xd = _dev(x, device, bf16)
+    got = ops.SpMMSrc(xd, [1], False, None, g).float().cpu().numpy()
+    assert_close(got, oracle.spmm(*adj, x, op="copy_u"), tol, f"copy_u F={feat}")
+    got = ops.gspmm_src_mul_e_sum(xd, _dev(w, device), [1], False, None, g).float().cpu().numpy()
+    assert_close(got, oracle.spmm(*adj, x, w, op="u_mul_e", heads=heads), tol, f"u_mul_e F={feat}")
+
+    xi = rng.integers(-3, 4, size=(n, feat)).astype(np.float32)
+    out, arg_u, _ = ops.spmm(g, "copy_u", "max", _dev(xi, device, bf16), None, return_arg=True)
+    ref, ref_u, _ = oracle.spmm(*adj, xi, None, op="copy_u", reduce="max", heads=1, want_arg=True)
+    np.testing.assert_array_equal(out.float().cpu().numpy(), ref)
+    np.testing.assert_array_equal(arg_u.cpu().numpy(), ref_u)
+
+    dim = feat // heads
+    el = rng.standard_normal((n, heads), dtype=np.float32) * 2
+    er = rng.standard_normal((n, heads), dtype=np.float32) * 2
+    got = ops.gat_aggregate(_dev(el, device), _dev(er, device), xd, g, 0.2).float().cpu().numpy()
+    ref = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er, x, heads=heads, slope=0.2)
+    assert_close(got, ref, tol, f"fused GAT {heads}x{dim}")
+
+    logit = (rng.standard_normal((e, heads)) * 3).astype(np.float32)
+    m = rng.standard_normal((e, feat), dtype=np.float32)
+    if bf16:
+        m = to_bf16_f32(m)
+    att = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, logit)
+    prod = (m.reshape(e, heads, dim).astype(np.float64) * att[:, :, None]).reshape(e, -1)
+    got = ops.edge_softmax_sum(_dev(logit, device), _dev(m, device, bf16), g).float().cpu().numpy()
+    assert_close(got, oracle.spmm(*adj, prod.astype(np.float32), op="copy_e"),
+                 TOL_BF16 if bf16 else 2 * TOL_F32, f"edge_softmax_sum {heads}x{dim}")
+
+
 @pytest.mark.parametrize("heads", [1, 8, 32, 3])
 def test_segment_softmax_rows_over_many_chunks(device, heads):
     """A row of 150,000 edges next to ordinary ones: its statistics are merged from
     hundreds to thousands of per-chunk partials (once per row), and two more long
     rows share chunks with it.  Edge ids shuffled against the adjacency order."""
     rng = np.random.default_rng(heads + 77)
-    n = 400
-    dst = np.concatenate([np.full(150_000, 7), np.full(5_000, 8), np.full(2_500, 300),
-                          rng.integers(0, n, 3_000)]).astype(np.int64)
-    dst = dst[rng.permutation(dst.shape[0])]
-    src = rng.integers(0, n, dst.shape[0], dtype=np.int64)
+    src, dst, n = _hub_graph(heads + 77)
     g = prepare_graph(src, dst, n, device=device)
     arr = build_graph_arrays(src, dst, n)
     x = (rng.standard_normal((dst.shape[0], heads)) * 4.0).astype(np.float32)
