@@ -1,9 +1,10 @@
 // Edge segment softmax for gfx950 (any number of heads), fp32.
 //
-// Power-of-two head counts (<= 64) run a chunked, load-balanced scheme: the
-// (slot, head) elements are cut into chunks of 1024 elements, one wavefront per
-// chunk whatever the degree distribution.  Lane = (slot group g, head h); a lane
-// owns 16 consecutive slots of its head, so
+// Up to 64 heads run a chunked, load-balanced scheme: the (slot, head) elements
+// are cut into chunks of 1024 lane elements, one wavefront per chunk whatever the
+// degree distribution.  Lane = (slot group g, head h) with the heads rounded up to a
+// power of two (lanes of the padding heads idle); a lane owns 16 consecutive slots
+// of its head, so
 //   1. segments that lie inside one lane are reduced sequentially in registers;
 //   2. segments shared by neighbouring lanes are combined with two segmented
 //      shuffle scans over the lanes of a head (rows are sorted, so equal keys at
@@ -14,7 +15,7 @@
 //      per-head (max, sum-exp) in the workspace; a second launch merges the
 //      partials of every such row once (one workgroup per row, so a row of any
 //      length costs one pass over its partials), a third writes the elements.
-// Other head counts use a lane-group kernel that runs the heads one after the
+// More than 64 heads use a lane-group kernel that runs the heads one after the
 // other, with chunked two-pass handling of rows longer than 1024 slots.
 // No atomics; the order of every reduction is fixed by the graph and sizes.
 #include "common.h"
@@ -119,9 +120,9 @@ template <bool DIRECT, bool FULL>
 __device__ __forceinline__ void softmax_chunk_body(
     const int32_t *__restrict__ row_of_slot, const int32_t *__restrict__ eid,
     const float *__restrict__ x, float *__restrict__ y, float *__restrict__ stats,
-    int64_t n_edges, int head_shift, int64_t chunk_id, int64_t c0, int64_t c1,
+    int64_t n_edges, int head_shift, int heads, int64_t chunk_id, int64_t c0, int64_t c1,
     float (*lds_v)[kChunkElems + kChunkElems / kT]) {
-  const int H = 1 << head_shift;
+  const int H = 1 << head_shift;              // lanes per slot; heads <= H of them are live
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int g = lane >> head_shift, h = lane & (H - 1);
@@ -199,10 +200,10 @@ __device__ __forceinline__ void softmax_chunk_body(
 #pragma unroll
     for (int j = 0; j < kT; ++j) {
       const int64_t slot = s0 + j;
-      const bool valid = FULL || slot < c1;
+      const bool valid = FULL || (slot < c1 && h < heads);
       key[j] = valid ? row_of_slot[slot] : -1;
       const int64_t e = (valid && eid) ? (int64_t)eid[slot] : slot;
-      off[j] = (e << head_shift) + h;
+      off[j] = e * heads + h;
       v[j] = valid ? x[off[j]] : -INFINITY;
     }
   }
@@ -288,7 +289,7 @@ template <bool DIRECT>
 __global__ __launch_bounds__(kBlock) void softmax_chunks_kernel(
     const int32_t *__restrict__ row_of_slot, const int32_t *__restrict__ eid,
     const float *__restrict__ x, float *__restrict__ y, float *__restrict__ stats,
-    int64_t n_edges, int head_shift) {
+    int64_t n_edges, int head_shift, int heads) {
   // per wave: one tile of 1024 words (+ one pad word per 16), used in turn for
   // the keys, the logits and the results
   __shared__ float lds_v[kBlock / kWave][kChunkElems + kChunkElems / kT];
@@ -297,12 +298,14 @@ __global__ __launch_bounds__(kBlock) void softmax_chunks_kernel(
   const int64_t c0 = chunk_id * chunk_slots;
   if (c0 >= n_edges) return;                                        // whole wave
   const int64_t c1 = min(c0 + (int64_t)chunk_slots, n_edges);
-  if (c1 - c0 == chunk_slots)
+  // the variant without validity tests needs every lane live: a whole chunk and as
+  // many heads as lanes per slot
+  if (c1 - c0 == chunk_slots && heads == (1 << head_shift))
     softmax_chunk_body<DIRECT, true>(row_of_slot, eid, x, y, stats, n_edges,
-                                     head_shift, chunk_id, c0, c1, lds_v);
+                                     head_shift, heads, chunk_id, c0, c1, lds_v);
   else
     softmax_chunk_body<DIRECT, false>(row_of_slot, eid, x, y, stats, n_edges,
-                                      head_shift, chunk_id, c0, c1, lds_v);
+                                      head_shift, heads, chunk_id, c0, c1, lds_v);
 }
 
 // Pass 2: every row that starts in one chunk and continues into later ones gets its
@@ -431,7 +434,7 @@ __global__ __launch_bounds__(kBlock) void softmax_boundary_kernel(
     const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
     const int32_t *__restrict__ eid, const float *__restrict__ x,
     float *__restrict__ y, float *__restrict__ stats, int64_t n_edges,
-    int head_shift) {
+    int head_shift, int heads) {
   ChunkInfo ci;
   if (!chunk_info(row_of_slot, n_edges, head_shift, ci)) return;
   const bool has_b = ci.continues && !(ci.began_before && ci.row_first == ci.row_last);
@@ -453,10 +456,10 @@ __global__ __launch_bounds__(kBlock) void softmax_boundary_kernel(
     hi[w] = min(e[w], ci.c1);
     o0[w] = -1;
     x0[w] = 0.0f;
-    if (lo[w] + g < hi[w]) {
+    if (lo[w] + g < hi[w] && h < heads) {
       const int64_t slot = lo[w] + g;
       const int64_t ed = eid ? (int64_t)eid[slot] : slot;
-      o0[w] = (ed << head_shift) + h;
+      o0[w] = ed * heads + h;
       x0[w] = x[o0[w]];
     }
   }
@@ -483,9 +486,9 @@ __global__ __launch_bounds__(kBlock) void softmax_boundary_kernel(
         const int64_t slot = base + (int64_t)t * G;
         o[t] = -1;
         xv[t] = 0.0f;
-        if (slot < hi[w]) {
+        if (slot < hi[w] && h < heads) {
           const int64_t ed = eid ? (int64_t)eid[slot] : slot;
-          o[t] = (ed << head_shift) + h;
+          o[t] = ed * heads + h;
           xv[t] = x[o[t]];
         }
       }
@@ -638,9 +641,11 @@ __global__ __launch_bounds__(kBlock) void softmax_long_write_generic_kernel(
   }
 }
 
-inline bool pow2_heads(int64_t heads) {
-  return (heads & (heads - 1)) == 0 && heads <= kWave;
-}
+// Head counts up to a wavefront run the chunked scheme with the lanes per slot
+// rounded up to a power of two (3 heads: 4 lanes, one idle); more heads the generic
+// kernels.
+inline bool chunked_heads(int64_t heads) { return heads <= kWave; }
+inline int lanes_per_slot_shift(int64_t heads) { return ilog2_ceil((uint64_t)heads); }
 
 }  // namespace
 }  // namespace ga
@@ -649,11 +654,12 @@ extern "C" {
 
 size_t ga_softmax_workspace_bytes(int64_t n_edges, int64_t heads) {
   if (n_edges <= 0 || heads <= 0) return 0;
-  if (ga::pow2_heads(heads)) {
-    // two partial (max, sum) pairs per head for every 1024-element chunk
-    const int64_t chunk_slots = ga::kChunkElems / heads;
+  if (ga::chunked_heads(heads)) {
+    // two partial (max, sum) pairs per lane of a slot for every chunk of 1024 lanes' elements
+    const int shift = ga::lanes_per_slot_shift(heads);
+    const int64_t chunk_slots = ga::kChunkElems >> shift;
     const int64_t chunks = (n_edges + chunk_slots - 1) / chunk_slots;
-    return (size_t)chunks * 2 * (size_t)heads * 2 * sizeof(float);
+    return (size_t)chunks * 2 * ((size_t)1 << shift) * 2 * sizeof(float);
   }
   if (n_edges <= ga::kLongRow) return 0;
   const int64_t chunks = (n_edges + ga::kLongRow - 1) / ga::kLongRow;
@@ -678,20 +684,21 @@ int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
   hipStream_t s = (hipStream_t)stream;
   float *stats = (float *)workspace;
 
-  if (pow2_heads(heads)) {
-    const int head_shift = ilog2_floor((uint64_t)heads);
+  if (chunked_heads(heads)) {
+    const int head_shift = lanes_per_slot_shift(heads);
+    const bool every_lane_live = heads == ((int64_t)1 << head_shift);
     const int64_t chunk_slots = kChunkElems >> head_shift;
     const int64_t chunks = (n_edges + chunk_slots - 1) / chunk_slots;
     const int64_t blocks = (chunks + kBlock / kWave - 1) / (kBlock / kWave);
     if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-    if (!eid && aligned(x, 16) && aligned(y, 16) && aligned(row_of_slot, 16))
+    if (every_lane_live && !eid && aligned(x, 16) && aligned(y, 16) && aligned(row_of_slot, 16))
       hipLaunchKernelGGL(softmax_chunks_kernel<true>, dim3((unsigned)blocks),
                          dim3(kBlock), 0, s, row_of_slot, eid, x, y, stats,
-                         n_edges, head_shift);
+                         n_edges, head_shift, (int)heads);
     else
       hipLaunchKernelGGL(softmax_chunks_kernel<false>, dim3((unsigned)blocks),
                          dim3(kBlock), 0, s, row_of_slot, eid, x, y, stats,
-                         n_edges, head_shift);
+                         n_edges, head_shift, (int)heads);
     if (chunks > 1) {
       hipLaunchKernelGGL(softmax_row_totals_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s,
                          pointer, row_of_slot, stats, n_edges, head_shift);
@@ -701,7 +708,7 @@ int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
                            dim3(kTotalsBlock), 0, s, pointer, row_of_slot, stats, head_shift);
       hipLaunchKernelGGL(softmax_boundary_kernel, dim3((unsigned)blocks),
                          dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, y, stats,
-                         n_edges, head_shift);
+                         n_edges, head_shift, (int)heads);
     }
     return launch_status();
   }

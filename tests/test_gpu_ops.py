@@ -292,7 +292,7 @@ def test_sddmm_u_dot_v(graph, device, heads, dim, bf16):
     assert_close(got.cpu().numpy(), ref, TOL_F32, f"u_dot_v {name} {heads}x{dim}")
 
 
-@pytest.mark.parametrize("heads", [1, 4, 8, 3, 64])
+@pytest.mark.parametrize("heads", [1, 4, 8, 3, 64, 5, 6, 12, 33, 65, 100])
 def test_segment_softmax(graph, device, heads):
     name, g, arr = graph
     rng = np.random.default_rng(heads)
@@ -371,7 +371,7 @@ def test_row_reductions_over_many_workgroups(device, feat, heads, bf16):
                  TOL_BF16 if bf16 else 2 * TOL_F32, f"edge_softmax_sum {heads}x{dim}")
 
 
-@pytest.mark.parametrize("heads", [1, 8, 32, 3])
+@pytest.mark.parametrize("heads", [1, 8, 32, 3, 12, 100])
 def test_segment_softmax_rows_over_many_chunks(device, heads):
     """A row of 150,000 edges next to ordinary ones: its statistics are merged from
     hundreds to thousands of per-chunk partials (once per row), and two more long
