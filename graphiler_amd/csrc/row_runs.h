@@ -239,7 +239,7 @@ __global__ __launch_bounds__(kBlock) void runs_kernel(
 // Blocks [0, fix_blocks): one lane group per main-kernel workgroup q; the group
 // whose slot range holds the END of a row that began in an earlier workgroup
 // combines that row's global partial states in workgroup order.  A chain of more
-// than kLongChain states (a row over that many workgroups) is combined by the whole
+// than max(kLongChain, lane groups per block) states is combined by the whole
 // block instead: every lane group folds a contiguous piece of the chain, in order,
 // and the owning group combines the pieces in order -- so a row of any length costs
 // chain / groups sequential steps, not chain.  Remaining blocks (only for a graph
@@ -305,7 +305,9 @@ __global__ __launch_bounds__(kBlock) void runs_fixup_kernel(
     q_lo = s >> wg_shift;
   }
   // the chain: slot 1 of workgroup q_lo, then slot 0 of workgroups q_lo + 1 .. q
-  const bool is_long = mine && q - q_lo > kLongChain;
+  // with many narrow lane groups per block the cooperative form starts later: its
+  // barriers and the scan over the groups cost more than a chain of that length
+  const bool is_long = mine && q - q_lo > max(kLongChain, G);
   if (lane == 0) long_first[grp] = is_long ? q_lo : -1;
   if (mine && !is_long && lane_live) {
     float acc[SF];
