@@ -158,6 +158,48 @@ __global__ __launch_bounds__(kBlock) void gather_units_kernel(
   y[t] = x[(int64_t)idx[i] * units + k];
 }
 
+// Rows of 256 bytes or more that are only 4- or 2-byte aligned (129 floats, 129 bf16
+// values): 16-byte pieces moved through a type of that alignment -- the load / store
+// unit takes such addresses, and a fraction of the accesses beats aligned narrow ones
+// -- and the few units left over at the end of the row by the group's first lanes.
+template <typename UnitT>
+struct __attribute__((packed, aligned(sizeof(UnitT)))) Piece16 {
+  UnitT u[16 / sizeof(UnitT)];
+};
+
+template <typename IdxT, typename UnitT>
+__global__ __launch_bounds__(kBlock) void gather_rows_pieces_kernel(
+    const IdxT *__restrict__ idx, const UnitT *__restrict__ x,
+    UnitT *__restrict__ y, int64_t n_out, int64_t units, int gl_shift) {
+  constexpr int kPer = 16 / sizeof(UnitT);    // units per piece; the tail is shorter
+  const int gl = 1 << gl_shift;               // >= 16 lanes: rows have >= 16 pieces
+  const int lane = threadIdx.x & (gl - 1);
+  const int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> gl_shift;
+  if (i >= n_out) return;
+  const UnitT *src = x + (int64_t)idx[i] * units;
+  UnitT *dst = y + i * units;
+  const int64_t pieces = units / kPer;
+  for (int64_t q = lane; q < pieces; q += gl)
+    *reinterpret_cast<Piece16<UnitT> *>(dst + kPer * q) =
+        *reinterpret_cast<const Piece16<UnitT> *>(src + kPer * q);
+  const int64_t t = kPer * pieces + lane;
+  if (t < units) dst[t] = src[t];
+}
+
+template <typename IdxT, typename UnitT>
+int launch_gather_pieces(const void *idx, const void *x, void *y, int64_t n_out,
+                         int64_t row_bytes, hipStream_t s) {
+  const int64_t units = row_bytes / (int64_t)sizeof(UnitT), pieces = row_bytes / 16;
+  const int gl_shift = ilog2_ceil((uint64_t)(pieces > kWave ? kWave : pieces));
+  const int64_t per_block = kBlock >> gl_shift;
+  const int64_t blocks = (n_out + per_block - 1) / per_block;
+  if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
+  hipLaunchKernelGGL((gather_rows_pieces_kernel<IdxT, UnitT>), dim3((unsigned)blocks),
+                     dim3(kBlock), 0, s, (const IdxT *)idx, (const UnitT *)x, (UnitT *)y, n_out,
+                     units, gl_shift);
+  return launch_status();
+}
+
 template <typename IdxT, typename UnitT>
 int launch_gather(const void *idx, const void *x, void *y, int64_t n_out,
                   int64_t units, hipStream_t s) {
@@ -193,10 +235,14 @@ int pick_gather_unit(const void *idx, const void *x, void *y, int64_t n_out,
     return launch_gather<IdxT, uint4>(idx, x, y, n_out, row_bytes / 16, s);
   if ((bits & 7) == 0)
     return launch_gather<IdxT, uint2>(idx, x, y, n_out, row_bytes / 8, s);
-  if ((bits & 3) == 0)
+  if ((bits & 3) == 0) {
+    if (row_bytes >= 256) return launch_gather_pieces<IdxT, uint32_t>(idx, x, y, n_out, row_bytes, s);
     return launch_gather<IdxT, uint32_t>(idx, x, y, n_out, row_bytes / 4, s);
-  if ((bits & 1) == 0)
+  }
+  if ((bits & 1) == 0) {
+    if (row_bytes >= 256) return launch_gather_pieces<IdxT, uint16_t>(idx, x, y, n_out, row_bytes, s);
     return launch_gather<IdxT, uint16_t>(idx, x, y, n_out, row_bytes / 2, s);
+  }
   return launch_gather<IdxT, uint8_t>(idx, x, y, n_out, row_bytes, s);
 }
 

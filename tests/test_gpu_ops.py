@@ -404,7 +404,9 @@ def test_segment_softmax_1d_input(graph, device):
                                          ((128,), np.float16), ((3,), np.uint8),
                                          ((17,), np.float32), ((129,), np.float32),
                                          ((18,), np.float32), ((33,), np.float16),
-                                         ((5,), np.uint8), ((100,), np.float64)])
+                                         ((5,), np.uint8), ((100,), np.float64),
+                                         ((67,), np.float32), ((258,), np.float16),
+                                         ((1025,), np.float32)])
 def test_broadcast_bit_exact(graph, device, shape, dtype):
     name, g, arr = graph
     rng = np.random.default_rng(1)
