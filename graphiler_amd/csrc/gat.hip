@@ -22,6 +22,16 @@ __device__ __forceinline__ float leaky(float t, float slope) {
   return t >= 0.0f ? t : t * slope;
 }
 
+// The running maximum as the point the exponentials are taken from: while every
+// logit seen so far is -inf (masked edges) the maximum is -inf too and
+// exp(-inf - -inf) would be NaN; taken from 0 instead, such edges weigh 0 and a
+// later finite logit rescales the (empty) state by exp(-inf) = 0.  A row whose
+// logits are all -inf ends with a zero denominator and yields NaN, as the
+// reference's softmax does (segment_softmax_kernel.cu:9-49).
+__device__ __forceinline__ float finite_or_zero(float m) {
+  return m == -INFINITY ? 0.0f : m;
+}
+
 // State per lane: VEC un-normalised weighted sums, then the running maximum m
 // and the running denominator l of the lane's head.
 // MODE selects where the logits come from:
@@ -71,7 +81,8 @@ struct GatPolicy {
   }
   static __device__ __forceinline__ void merge(float (&dst)[VEC + 2], const float *src) {
     const float nm = fmaxf(dst[VEC], src[VEC]);
-    const float sa = __expf(dst[VEC] - nm), sb = __expf(src[VEC] - nm);
+    const float ref = finite_or_zero(nm);
+    const float sa = __expf(dst[VEC] - ref), sb = __expf(src[VEC] - ref);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) dst[v] = dst[v] * sa + src[v] * sb;
     dst[VEC + 1] = dst[VEC + 1] * sa + src[VEC + 1] * sb;
@@ -149,14 +160,15 @@ struct GatPolicy {
 #pragma unroll
         for (int t = 1; t < kUnroll; ++t) bm = fmaxf(bm, s[t]);
         const float nm = fmaxf(st[VEC], bm);
-        const float sc = __expf(st[VEC] - nm);
+        const float ref = finite_or_zero(nm);
+        const float sc = __expf(st[VEC] - ref);
         st[VEC + 1] *= sc;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) st[v] *= sc;
         st[VEC] = nm;
 #pragma unroll
         for (int t = 0; t < kUnroll; ++t) {
-          const float p = __expf(s[t] - nm);
+          const float p = __expf(s[t] - ref);
           st[VEC + 1] += p;
           float xf[VEC];
           IO::widen(x[t], xf);
@@ -173,8 +185,9 @@ struct GatPolicy {
               init(st);
             }
             const float nm = fmaxf(st[VEC], s[t]);
-            const float sc = __expf(st[VEC] - nm);
-            const float p = __expf(s[t] - nm);
+            const float ref = finite_or_zero(nm);
+            const float sc = __expf(st[VEC] - ref);
+            const float p = __expf(s[t] - ref);
             st[VEC + 1] = st[VEC + 1] * sc + p;
             float xf[VEC];
             IO::widen(x[t], xf);

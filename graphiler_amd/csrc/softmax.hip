@@ -28,12 +28,23 @@ constexpr int kChunkElems = kWave * kT;   // 1024 elements per wavefront
 constexpr int kLongRow = 1024;            // generic path: slots per long-row chunk
 
 // exp(x) as exp2(x * log2 e) with the rounding error of the product fed back
-// (x*log2e = t + r, exp2(t + r) ~ exp2(t) * (1 + r ln 2)): about 2 ulp, six
-// instructions instead of the library routine's thirty.
+// (x*log2e = t + r, exp2(t + r) ~ exp2(t) * (1 + r ln 2)): about 2 ulp, eight
+// instructions instead of the library routine's thirty.  Arguments below -126
+// (-inf included: a masked logit) are moved to -126, where the result is already
+// 0 in fp32 -- the error term would be inf - inf there; NaN stays NaN.
 __device__ __forceinline__ float exp_fast(float x) {
+  x = x < -126.0f ? -126.0f : x;
   const float t = x * 1.44269502162933349609375f;
   const float r = fmaf(x, 1.44269502162933349609375f, -t) + x * 1.925963033e-8f;
   return __builtin_amdgcn_exp2f(t) * fmaf(r, 0.693147182464599609375f, 1.0f);
+}
+
+// The maximum of a piece of a row as the point its exponentials are taken from:
+// a piece whose logits are all -inf (masked edges) has the maximum -inf, and
+// exp(-inf - -inf) would be NaN; taken from 0 its elements weigh 0, and the
+// piece's (max, sum) = (-inf, 0) merges as the empty state.
+__device__ __forceinline__ float finite_or_zero(float m) {
+  return m == -INFINITY ? 0.0f : m;
 }
 
 // Per-chunk partial statistics: [chunk][A|B][head][max, sum].  A = the chunk's
@@ -228,7 +239,7 @@ __device__ __forceinline__ void softmax_chunk_body(
   float p[kT], l[kT];
 #pragma unroll
   for (int j = 0; j < kT; ++j)
-    p[j] = (FULL || key[j] >= 0) ? exp_fast(v[j] - m[j]) : 0.0f;
+    p[j] = (FULL || key[j] >= 0) ? exp_fast(v[j] - finite_or_zero(m[j])) : 0.0f;
   l[0] = p[0];
 #pragma unroll
   for (int j = 1; j < kT; ++j) l[j] = key[j] == key[j - 1] ? l[j - 1] + p[j] : p[j];
@@ -583,10 +594,11 @@ __global__ __launch_bounds__(kBlock) void softmax_long_stats_generic_kernel(
       m = fmaxf(m, x[e * heads + h]);
     }
     m = block_reduce<true>(m, lds);
+    const float ref = finite_or_zero(m);
     float l = 0.0f;
     for (int64_t q = lo + threadIdx.x; q < hi; q += kBlock) {
       const int64_t e = eid ? (int64_t)eid[q] : q;
-      l += expf(x[e * heads + h] - m);
+      l += expf(x[e * heads + h] - ref);
     }
     l = block_reduce<false>(l, lds);
     if (threadIdx.x == 0) {

@@ -389,6 +389,71 @@ def test_segment_softmax_rows_over_many_chunks(device, heads):
     assert np.abs(sums[np.diff(arr.in_pointer) > 0] - 1.0).max() < 2e-5
 
 
+def _mask_some_logits(rng, ptr, eid, x):
+    """-inf on about a third of the logits, keeping one finite logit per row and head."""
+    x = x.copy()
+    mask = rng.random(x.shape) < 0.35
+    for v in range(len(ptr) - 1):
+        if ptr[v + 1] > ptr[v]:
+            mask[eid[ptr[v] + rng.integers(0, ptr[v + 1] - ptr[v])]] = False
+    x[mask] = -np.inf
+    return x
+
+
+@pytest.mark.parametrize("heads", [1, 8, 100])
+def test_segment_softmax_masked_logits(device, heads):
+    """-inf logits (masked edges) weigh exactly 0 and leave the other edges of their
+    row untouched, as expf(-inf - max) = 0 does in segment_softmax_kernel.cu:22-45;
+    rows of every length incl. the 150,000-edge one, leading -inf runs included."""
+    rng = np.random.default_rng(heads + 5)
+    src, dst, n = _hub_graph(heads + 5)
+    g = prepare_graph(src, dst, n, device=device)
+    arr = build_graph_arrays(src, dst, n)
+    x = (rng.standard_normal((dst.shape[0], heads)) * 4.0).astype(np.float32)
+    x = _mask_some_logits(rng, arr.in_pointer, arr.in_edge_indices, x)
+    got = ops.SegmentSoftmax(_dev(x, device), 1, None, g).cpu().numpy()
+    ref = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, x)
+    assert np.isfinite(got).all()
+    assert not got[np.isneginf(x)].any()
+    assert_close(got, ref, TOL_F32, f"softmax with -inf logits H={heads}")
+
+
+@pytest.mark.parametrize("feat,heads", [(64, 1), (128, 8), (17, 1)])
+def test_fused_softmax_sums_masked_logits(device, feat, heads):
+    """The fused GAT pass and the per-edge softmax sum with -inf logits: a source whose
+    attention term is -inf contributes nothing, also when the -inf edges come first in
+    a row (the running maximum is then still -inf)."""
+    rng = np.random.default_rng(feat + heads)
+    src, dst, n = _hub_graph(feat)
+    src[:] = rng.integers(1, n, src.shape[0])      # node 0 is never the only source ...
+    g = prepare_graph(src, dst, n, device=device)
+    arr = build_graph_arrays(src, dst, n)
+    e = src.shape[0]
+    z = rng.standard_normal((n, feat), dtype=np.float32)
+    el = rng.standard_normal((n, heads), dtype=np.float32) * 2
+    er = rng.standard_normal((n, heads), dtype=np.float32) * 2
+    el[rng.random(n) < 0.3] = -np.inf
+    has_finite = np.zeros(n, bool)
+    has_finite[dst[np.isfinite(el[src, 0])]] = True
+    extra = np.flatnonzero(~has_finite & (np.diff(arr.in_pointer) > 0))
+    el[src[arr.in_edge_indices[arr.in_pointer[extra]]]] = 0.5   # ... every row keeps a finite logit
+    got = ops.gat_aggregate(_dev(el, device), _dev(er, device), _dev(z, device), g, 0.2).cpu().numpy()
+    ref = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er, z, heads=heads, slope=0.2)
+    assert np.isfinite(got).all()
+    assert_close(got, ref, TOL_F32, f"fused GAT with -inf terms {heads}x{feat // heads}")
+
+    logit = (rng.standard_normal((e, heads)) * 3).astype(np.float32)
+    logit = _mask_some_logits(rng, arr.in_pointer, arr.in_edge_indices, logit)
+    m = rng.standard_normal((e, feat), dtype=np.float32)
+    att = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, logit)
+    prod = (m.reshape(e, heads, -1).astype(np.float64) * att[:, :, None]).reshape(e, -1)
+    got = ops.edge_softmax_sum(_dev(logit, device), _dev(m, device), g).cpu().numpy()
+    assert np.isfinite(got).all()
+    assert_close(got, oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                                  prod.astype(np.float32), op="copy_e"),
+                 2 * TOL_F32, f"edge_softmax_sum with -inf logits {heads}x{feat // heads}")
+
+
 def test_segment_softmax_1d_input(graph, device):
     name, g, arr = graph
     rng = np.random.default_rng(0)
