@@ -14,7 +14,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libgraphiler_hip.so")
 
 GA_OK = 0
-GA_EINVAL, GA_EUNSUPPORTED, GA_EWORKSPACE, GA_EALIGN = -1, -2, -3, -4
+GA_EINVAL, GA_EUNSUPPORTED, GA_EWORKSPACE, GA_EALIGN, GA_ESCRATCH = -1, -2, -3, -4, -5
+GA_STATIC_SCRATCH_BYTES = 32 << 20
 GA_F32, GA_BF16 = 0, 1
 GA_COPY_U, GA_COPY_E, GA_U_MUL_E, GA_U_ADD_E, GA_U_SUB_E, GA_U_DIV_E = 0, 1, 2, 3, 4, 5
 GA_SDDMM_ADD, GA_SDDMM_SUB, GA_SDDMM_MUL, GA_SDDMM_DIV = 0, 1, 2, 3
@@ -58,6 +59,8 @@ SIGNATURES = {
                                        _i64, _i64, ctypes.c_float, _int, _vp, _sz, _vp]),
     "ga_edge_softmax_sum": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                    _int, _vp, _sz, _vp]),
+    "ga_gat_aggregate_static": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+                                       _i64, _i64, ctypes.c_float, _int, _vp]),
     "ga_gat_aggregate": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
                                 _i64, _i64, ctypes.c_float, _int, _vp, _sz,
                                 _vp]),

@@ -13,6 +13,8 @@
 // and the weighted rows are per-edge rows, both read through the edge-id
 // column: out[v] = sum_e softmax_v(logit)[e] * m[e], the SegmentSoftmax ->
 // mul -> SpMMEdge tail of examples/HGT/HGT.py:50-53 with no attention tensor.
+#include <mutex>
+
 #include "row_runs.h"
 
 namespace ga {
@@ -205,7 +207,8 @@ template <typename T, int VEC, int MODE = kGatNode, bool SPREAD = false>
 int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const int32_t *nbr, const float *el, const float *er,
                const void *z, void *out, int64_t n_rows, int64_t n_edges,
-               int heads, int dim, float slope, float *ws, hipStream_t stream) {
+               int heads, int dim, float slope, float *ws, hipStream_t stream,
+               size_t ws_bytes = SIZE_MAX) {
   typedef GatPolicy<T, VEC, MODE, SPREAD> P;
   const bool ids_vec = aligned(row_of_slot, 16) && (!nbr || aligned(nbr, 16));
   const int head_lanes = dim / VEC;
@@ -214,7 +217,87 @@ int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
     return GA_EUNSUPPORTED;
   typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec, head_lanes, 0};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges,
-                        heads * dim, ws, stream);
+                        heads * dim, ws, stream, ws_bytes);
+}
+
+// The element type and lane layout ga_gat_aggregate runs for a shape, launched
+// with `ws` (capacity `ws_bytes`) as the partial-row scratch.
+int gat_aggregate_dispatch(const int32_t *pointer, const int32_t *row_of_slot,
+                           const int32_t *nbr, const float *el, const float *er,
+                           const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                           int heads, int dim, float slope, int dtype, float *ws,
+                           size_t ws_bytes, hipStream_t s) {
+  const bool vec_ok = aligned(out, 16) && (!z || aligned(z, 16));
+  if (dtype == GA_F32) {
+    if (vec_ok && dim % 4 == 0)
+      return launch_gat<float, 4>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
+                                  heads, dim, slope, ws, s, ws_bytes);
+    if (heads == 1 && dim >= 3 && dim <= 256)   // rows that 16-byte accesses do not tile
+      return launch_gat<float, 4, kGatNode, true>(pointer, row_of_slot, nbr, el, er, z, out,
+                                                  n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes);
+    return launch_gat<float, 1>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
+                                heads, dim, slope, ws, s, ws_bytes);
+  }
+  if (vec_ok && dim % 8 == 0)
+    return launch_gat<bf16_t, 8>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
+                                 heads, dim, slope, ws, s, ws_bytes);
+  if (heads == 1 && dim >= 3 && dim <= 256)
+    return launch_gat<bf16_t, 4, kGatNode, true>(pointer, row_of_slot, nbr, el, er, z, out,
+                                                 n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes);
+  return launch_gat<bf16_t, 1>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
+                               heads, dim, slope, ws, s, ws_bytes);
+}
+
+// Argument checks shared by ga_gat_aggregate and ga_gat_aggregate_static
+// (everything but the workspace).  GA_OK with *nothing_to_do set for n_rows == 0.
+int gat_aggregate_check(const int32_t *pointer, const int32_t *row_of_slot,
+                        const int32_t *nbr, const float *el, const float *er,
+                        const void *z, const void *out, int64_t n_rows, int64_t n_edges,
+                        int64_t heads, int64_t dim, int dtype, bool *nothing_to_do) {
+  *nothing_to_do = false;
+  if (n_rows < 0 || n_edges < 0 || heads <= 0 || dim <= 0) return GA_EINVAL;
+  if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || heads * dim > 0x7fffffff)
+    return GA_EINVAL;
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  if (n_rows == 0) {
+    *nothing_to_do = true;
+    return GA_OK;
+  }
+  if (!pointer || !out) return GA_EINVAL;
+  if (n_edges > 0 && (!row_of_slot || !nbr || !el || !er || !z)) return GA_EINVAL;
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!aligned(out, esz) || (z && !aligned(z, esz)) || (el && !aligned(el, 4)) ||
+      (er && !aligned(er, 4)))
+    return GA_EALIGN;
+  return GA_OK;
+}
+
+// Scratch of ga_gat_aggregate_static: the partial rows that ga_gat_aggregate
+// takes as its workspace, held by the library itself.  Every device the library
+// runs on has its own copy of this array at its own address; host code never
+// uses the array's name as an address, only the pointer that
+// hipGetSymbolAddress returned for the current device (static_scratch_for).
+static __device__ __align__(256) unsigned char scratch[GA_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void *scratch_ptr[kMaxDevices];   // per device, filled on the first call there
+
+int static_scratch_for_current_device(void **ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return GA_EUNSUPPORTED;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return GA_EINVAL;
+    scratch_ptr[dev] = p;
+  }
+  *ptr = scratch_ptr[dev];
+  return GA_OK;
 }
 
 }  // namespace
@@ -234,51 +317,38 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
                      int64_t heads, int64_t dim, float slope, int dtype,
                      void *workspace, size_t workspace_bytes,
                      ga_stream_t stream) {
-  if (n_rows < 0 || n_edges < 0 || heads <= 0 || dim <= 0) return GA_EINVAL;
-  if (n_rows > 0x7fffffff || n_edges > 0x7fffffff ||
-      heads * dim > 0x7fffffff)
-    return GA_EINVAL;
-  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
-  if (n_rows == 0) return GA_OK;
-  if (!pointer || !out) return GA_EINVAL;
-  const int64_t feat = heads * dim;
-  if (n_edges > 0) {
-    if (!row_of_slot || !nbr || !el || !er || !z) return GA_EINVAL;
-    if (!workspace || !ga::aligned(workspace, 16) ||
-        ga_gat_workspace_bytes(n_edges, feat, heads) > workspace_bytes)
-      return GA_EWORKSPACE;
-  }
-  const size_t esz = dtype == GA_F32 ? 4 : 2;
-  if (!ga::aligned(out, esz) || (z && !ga::aligned(z, esz)) ||
-      (el && !ga::aligned(el, 4)) || (er && !ga::aligned(er, 4)))
-    return GA_EALIGN;
-  const bool vec_ok = ga::aligned(out, 16) && (!z || ga::aligned(z, 16));
-  hipStream_t s = (hipStream_t)stream;
-  float *ws = (float *)workspace;
-  if (dtype == GA_F32) {
-    if (vec_ok && dim % 4 == 0)
-      return ga::launch_gat<float, 4>(pointer, row_of_slot, nbr, el, er, z, out,
-                                      n_rows, n_edges, (int)heads, (int)dim,
-                                      slope, ws, s);
-    if (heads == 1 && dim >= 3 && dim <= 256)   // rows that 16-byte accesses do not tile
-      return ga::launch_gat<float, 4, ga::kGatNode, true>(pointer, row_of_slot, nbr, el, er, z,
-                                                          out, n_rows, n_edges, 1, (int)dim,
-                                                          slope, ws, s);
-    return ga::launch_gat<float, 1>(pointer, row_of_slot, nbr, el, er, z, out,
-                                    n_rows, n_edges, (int)heads, (int)dim, slope,
-                                    ws, s);
-  }
-  if (vec_ok && dim % 8 == 0)
-    return ga::launch_gat<ga::bf16_t, 8>(pointer, row_of_slot, nbr, el, er, z,
-                                         out, n_rows, n_edges, (int)heads,
-                                         (int)dim, slope, ws, s);
-  if (heads == 1 && dim >= 3 && dim <= 256)
-    return ga::launch_gat<ga::bf16_t, 4, ga::kGatNode, true>(pointer, row_of_slot, nbr, el, er, z,
-                                                             out, n_rows, n_edges, 1, (int)dim,
-                                                             slope, ws, s);
-  return ga::launch_gat<ga::bf16_t, 1>(pointer, row_of_slot, nbr, el, er, z, out,
-                                       n_rows, n_edges, (int)heads, (int)dim,
-                                       slope, ws, s);
+  bool nothing = false;
+  const int rc = ga::gat_aggregate_check(pointer, row_of_slot, nbr, el, er, z, out, n_rows,
+                                         n_edges, heads, dim, dtype, &nothing);
+  if (rc != GA_OK || nothing) return rc;
+  if (n_edges > 0 &&
+      (!workspace || !ga::aligned(workspace, 16) ||
+       ga_gat_workspace_bytes(n_edges, heads * dim, heads) > workspace_bytes))
+    return GA_EWORKSPACE;
+  return ga::gat_aggregate_dispatch(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
+                                    (int)heads, (int)dim, slope, dtype, (float *)workspace,
+                                    workspace_bytes, (hipStream_t)stream);
+}
+
+int ga_gat_aggregate_static(const int32_t *pointer, const int32_t *row_of_slot,
+                            const int32_t *nbr, const float *el, const float *er,
+                            const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                            int64_t heads, int64_t dim, float slope, int dtype,
+                            ga_stream_t stream) {
+  bool nothing = false;
+  const int rc = ga::gat_aggregate_check(pointer, row_of_slot, nbr, el, er, z, out, n_rows,
+                                         n_edges, heads, dim, dtype, &nothing);
+  if (rc != GA_OK || nothing) return rc;
+  void *ws = nullptr;
+  const int sc = ga::static_scratch_for_current_device(&ws);
+  if (sc != GA_OK) return sc;
+  // The kernels write every partial row before the fix-up pass reads it, so the
+  // previous call's contents need no clearing.
+  const int lr = ga::gat_aggregate_dispatch(pointer, row_of_slot, nbr, el, er, z, out, n_rows,
+                                            n_edges, (int)heads, (int)dim, slope, dtype,
+                                            (float *)ws, (size_t)GA_STATIC_SCRATCH_BYTES,
+                                            (hipStream_t)stream);
+  return lr == GA_EWORKSPACE ? GA_ESCRATCH : lr;
 }
 
 int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,

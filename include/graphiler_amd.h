@@ -36,6 +36,7 @@ extern "C" {
 #define GA_EUNSUPPORTED (-2) /* valid request this build has no kernel for   */
 #define GA_EWORKSPACE (-3)   /* workspace missing, too small or misaligned   */
 #define GA_EALIGN (-4)       /* pointer not aligned to its element size      */
+#define GA_ESCRATCH (-5)     /* problem needs more than the library's static scratch */
 
 typedef void *ga_stream_t;
 
@@ -244,6 +245,31 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
                      int64_t heads, int64_t dim, float slope, int dtype,
                      void *workspace, size_t workspace_bytes,
                      ga_stream_t stream);
+
+/* ga_gat_aggregate for callers that cannot allocate device memory or hand over
+ * a workspace: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  Same arguments,
+ * kernels and results (bit for bit) as ga_gat_aggregate, but the partial rows of
+ * destination rows that span workgroups go to a buffer of
+ * GA_STATIC_SCRATCH_BYTES that the library holds in device memory itself (a
+ * file-scope array: every GPU the library runs on keeps it until the process
+ * ends).  The call allocates nothing and calls no allocating routine.
+ *   - GA_ESCRATCH (nothing launched) when the graph and width need more partial
+ *     rows than the buffer holds: 2 rows of heads*dim features (x 1.25 - 1.5 for
+ *     the softmax state) per workgroup; 64.3 M edges x 256 bf16 features need
+ *     20 MB, 11.6 M edges x 64 fp32 features 4.3 MB.
+ *   - All calls on one GPU share that GPU's buffer: calls that overlap on one
+ *     GPU (two streams, two threads) race; calls on one stream are ordered.
+ *   - The first call on a device looks the buffer's address up
+ *     (hipGetSymbolAddress, once per device); make that call outside a stream
+ *     capture.
+ */
+#define GA_STATIC_SCRATCH_BYTES (32u << 20)
+int ga_gat_aggregate_static(const int32_t *pointer, const int32_t *row_of_slot,
+                            const int32_t *nbr, const float *el, const float *er,
+                            const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                            int64_t heads, int64_t dim, float slope, int dtype,
+                            ga_stream_t stream);
 
 /* The same chain with the source term recomputed from the gathered row:
  *   s_i = leaky_relu(<z[nbr[i], h, :], a_l[h, :]> + er[v, h], slope)
