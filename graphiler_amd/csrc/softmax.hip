@@ -1,20 +1,25 @@
 // Edge segment softmax for gfx950 (any number of heads), fp32.
 //
-// Up to 64 heads run a chunked, load-balanced scheme: the (slot, head) elements
-// are cut into chunks of 1024 lane elements, one wavefront per chunk whatever the
-// degree distribution.  Lane = (slot group g, head h) with the heads rounded up to a
-// power of two (lanes of the padding heads idle); a lane owns 16 consecutive slots
-// of its head, so
+// Up to 64 heads run a tiled, load-balanced scheme: the (slot, head) elements are
+// cut into chunks of 1024 lane elements, one wavefront per chunk whatever the
+// degree distribution, and kTileWaves consecutive chunks form the tile of one
+// workgroup.  Lane = (slot group g, head h) with the heads rounded up to a power of
+// two (lanes of the padding heads idle); a lane owns 16 consecutive slots of its
+// head, so
 //   1. segments that lie inside one lane are reduced sequentially in registers;
 //   2. segments shared by neighbouring lanes are combined with two segmented
 //      shuffle scans over the lanes of a head (rows are sorted, so equal keys at
 //      distance d imply equal keys in between);
-//   3. rows that lie inside the chunk are normalised and written at once: their
-//      logits are read exactly once;
-//   4. the (at most two) rows a chunk shares with its neighbours leave their
-//      per-head (max, sum-exp) in the workspace; a second launch merges the
-//      partials of every such row once (one workgroup per row, so a row of any
-//      length costs one pass over its partials), a third writes the elements.
+//   3. segments shared by neighbouring wavefronts of the tile are combined as
+//      (max, sum-exp) pairs through LDS, after one workgroup barrier;
+//   4. rows that lie inside the tile are normalised and written at once: their
+//      logits are read exactly once and stay in registers meanwhile;
+//   5. the (at most two) rows a tile shares with its neighbours leave their
+//      per-head pair in the workspace; a second launch folds every such row's
+//      pairs and writes the row's elements, tile by tile.
+// The rows of a chunk's slots come from the row pointer (the row starts inside
+// the chunk), not from the slot -> row column, which is read at the two ends of a
+// chunk only: 4 bytes per row instead of 4 bytes per slot.
 // More than 64 heads use a lane-group kernel that runs the heads one after the
 // other, with chunked two-pass handling of rows longer than 1024 slots.
 // No atomics; the order of every reduction is fixed by the graph and sizes.
@@ -47,34 +52,12 @@ __device__ __forceinline__ float finite_or_zero(float m) {
   return m == -INFINITY ? 0.0f : m;
 }
 
-// Per-chunk partial statistics: [chunk][A|B][head][max, sum].  A = the chunk's
-// first row when it began in an earlier chunk; B = its last row when that row
-// started inside the chunk and continues in the next one.
-__device__ __forceinline__ float *stat_ptr(float *stats, int64_t chunk, int which,
+// Partial statistics of rows that leave a tile: [tile][A|B][head][max, sum].
+// A = the tile's first row when it began in an earlier tile; B = its last row
+// when that row started inside the tile and continues in the next one.
+__device__ __forceinline__ float *stat_ptr(float *stats, int64_t tile, int which,
                                            int H, int h) {
-  return stats + ((chunk * 2 + which) * H + h) * 2;
-}
-
-struct ChunkInfo {
-  int64_t c0, c1;       // slot range of the chunk
-  int row_first, row_last;
-  bool began_before;    // first row started in an earlier chunk
-  bool continues;       // last row goes on in the next chunk
-};
-
-__device__ __forceinline__ bool chunk_info(const int32_t *__restrict__ row_of_slot,
-                                           int64_t n_edges, int head_shift,
-                                           ChunkInfo &ci) {
-  const int64_t chunk = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
-  const int chunk_slots = kChunkElems >> head_shift;
-  ci.c0 = chunk * chunk_slots;
-  if (ci.c0 >= n_edges) return false;
-  ci.c1 = min(ci.c0 + (int64_t)chunk_slots, n_edges);
-  ci.row_first = row_of_slot[ci.c0];
-  ci.row_last = row_of_slot[ci.c1 - 1];
-  ci.began_before = ci.c0 > 0 && row_of_slot[ci.c0 - 1] == ci.row_first;
-  ci.continues = ci.c1 < n_edges && row_of_slot[ci.c1] == ci.row_last;
-  return true;
+  return stats + ((tile * 2 + which) * H + h) * 2;
 }
 
 // Segmented scans over the lanes of one head (lanes at distance `step`
@@ -121,58 +104,123 @@ __device__ __forceinline__ void chunk_totals(float vf, float vl, int kf, int kl,
   tl = IS_MAX ? fmaxf(P, next) : P + next;
 }
 
-// Pass 1: one wavefront per chunk.  DIRECT: edge ids are slot numbers, so the
-// chunk is one contiguous piece of x / y; it is moved with fully coalesced
-// 16-byte accesses and re-distributed to the owning lanes through a padded,
+// (m, l) <- (m, l) (+) (sm, sl).  The side that holds the maximum keeps its sum
+// unscaled (also when both maxima are -inf: the sums are then 0 or NaN and stay
+// so); the empty state (-inf, 0) scales by 0.
+__device__ __forceinline__ void pair_merge(float &m, float &l, float sm, float sl) {
+  const float nm = fmaxf(m, sm);
+  const float a = m == nm ? 1.0f : (m == -INFINITY ? 0.0f : exp_fast(m - nm));
+  const float b = sm == nm ? 1.0f : (sm == -INFINITY ? 0.0f : exp_fast(sm - nm));
+  l = l * a + sl * b;
+  m = nm;
+}
+
+// ---- pass 1: tiles ----------------------------------------------------------
+// A workgroup of W wavefronts owns a tile of W chunks; wavefront w owns chunk
+// tile * W + w (1024 lane elements) and keeps it in registers from the load of the
+// logits to the store of the results.
+constexpr int kTileWaves = 8;                              // wavefronts (chunks) per tile
+constexpr int kTilePad = kChunkElems + kChunkElems / kT;   // LDS words per wavefront
+
+// What a wavefront tells the other wavefronts of its tile about its chunk.
+constexpr int kActive = 1;      // the chunk holds slots
+constexpr int kBegan = 2;       // its first row began before the chunk
+constexpr int kContinues = 4;   // its last row continues past the chunk
+constexpr int kSingle = 8;      // first row == last row
+// a row passes straight through a chunk: began before, fills it, continues
+__device__ __forceinline__ bool passes_through(int flags) {
+  return (flags & (kBegan | kContinues | kSingle)) == (kBegan | kContinues | kSingle);
+}
+
+struct ChunkRows {
+  int64_t c0, c1;       // slot range
+  int row_first, row_last;
+  bool began_before, continues, has_b;
+};
+
+// Per-lane state that lives from the reduction (before the workgroup barrier) to
+// the store (after it).
+template <bool DIRECT>
+struct LaneRows {
+  int key[kT];          // row of each of the lane's slots, -1 for none
+  float p[kT];          // exp(logit - maximum of the segment inside this chunk)
+  float l[kT];          // sum of p over the lane's part of the segment
+  float raw[DIRECT ? kT : 1];        // DIRECT: the logits (written back for rows that leave the tile)
+  int64_t off[DIRECT ? 1 : kT];      // gathered: element offsets
+  float mf, ml, lf, ll; // chunk-wide (max, sum) of the lane's first / last segment
+};
+
+// Rows of the lane's 16 slots without reading the slot -> row column: the row
+// that holds the chunk's first slot and the one that holds its last come from
+// that column (two reads per chunk), the row starts in between from the row
+// pointer -- each row that starts inside the chunk marks its first slot in a
+// wave-private LDS tile, a lane reads its 16 marks, and what lies before a
+// lane's first mark is the largest mark of the lanes before it (rows ascend
+// with the slot), found with a scan over the lanes.
+__device__ __forceinline__ void rows_of_chunk(const int32_t *__restrict__ pointer,
+                                              const ChunkRows &cr, int head_shift, int lane,
+                                              int *tile, int (&key)[kT]) {
+  const int H = 1 << head_shift;
+  const int g = lane >> head_shift;
+  const int chunk_slots = kChunkElems >> head_shift;
+#pragma unroll
+  for (int i = 0; i < kT; ++i) {
+    const int q = i * kWave + lane;
+    if (q < chunk_slots) tile[q + (q >> 4)] = -1;
+  }
+  __builtin_amdgcn_wave_barrier();
+  for (int r = cr.row_first + 1 + lane; r <= cr.row_last; r += kWave) {
+    const int s = pointer[r], e = pointer[r + 1];
+    if (e > s) {                                  // rows without edges own no slot
+      const int q = (int)(s - cr.c0);
+      tile[q + (q >> 4)] = r;
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  int last = -1;
+#pragma unroll
+  for (int j = 0; j < kT; ++j) {
+    key[j] = tile[g * (kT + 1) + j];
+    last = max(last, key[j]);
+  }
+  __builtin_amdgcn_wave_barrier();
+  int inc = last;                                 // largest mark of lanes <= me (same head)
+  for (int off = H; off < kWave; off <<= 1) {
+    const int t = __shfl_up(inc, off);
+    if (lane >= off) inc = max(inc, t);
+  }
+  int before = __shfl_up(inc, H);
+  before = lane >= H ? max(before, cr.row_first) : cr.row_first;
+#pragma unroll
+  for (int j = 0; j < kT; ++j) {
+    if (key[j] < 0) key[j] = before;
+    before = key[j];
+  }
+}
+
+// Reduction of one chunk.  DIRECT: edge ids are slot numbers, so the chunk is
+// one contiguous piece of x / y; it is moved with fully coalesced 16-byte
+// accesses and re-distributed to the owning lanes through the padded,
 // wave-private LDS tile.  Otherwise every element is gathered through eid.
-// FULL: the chunk holds all 1024 elements (every chunk but the last), so no
-// element needs a validity test.
+// FULL: the chunk holds all 1024 elements and every lane is live, so no element
+// needs a validity test.
 template <bool DIRECT, bool FULL>
-__device__ __forceinline__ void softmax_chunk_body(
-    const int32_t *__restrict__ row_of_slot, const int32_t *__restrict__ eid,
-    const float *__restrict__ x, float *__restrict__ y, float *__restrict__ stats,
-    int64_t n_edges, int head_shift, int heads, int64_t chunk_id, int64_t c0, int64_t c1,
-    float (*lds_v)[kChunkElems + kChunkElems / kT]) {
+__device__ __forceinline__ void chunk_reduce(
+    const int32_t *__restrict__ pointer, const int32_t *__restrict__ eid,
+    const float *__restrict__ x, const ChunkRows &cr, int head_shift, int heads,
+    float *tile, LaneRows<DIRECT> &S) {
   const int H = 1 << head_shift;              // lanes per slot; heads <= H of them are live
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
   const int g = lane >> head_shift, h = lane & (H - 1);
-  const int64_t s0 = c0 + (int64_t)g * kT;   // first slot of this lane
-
-  int key[kT];
-  int64_t off[kT];
+  const int64_t s0 = cr.c0 + (int64_t)g * kT;   // first slot of this lane
+  const int64_t base_elem = cr.c0 << head_shift;
+  const int n_elem = (int)((cr.c1 - cr.c0) << head_shift);
   float v[kT];
-  const int64_t base_elem = c0 << head_shift;
-  const int n_elem = (int)((c1 - c0) << head_shift);
-  // LDS word of element q = (i*64 + lane)*4 + c of the chunk, as seen by the
-  // lane that loads / stores it from global memory
-  int lds_at[kChunkElems / (kWave * 4)][4];
-  if (DIRECT) {
-#pragma unroll
-    for (int i = 0; i < kChunkElems / (kWave * 4); ++i)
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const int q = (i * kWave + lane) * 4 + c;
-        const int slot = q >> head_shift, hd = q & (H - 1);
-        lds_at[i][c] = (((slot >> 4) << head_shift) + hd) * (kT + 1) + (slot & 15);
-      }
-    float *tv = lds_v[wave];
-    int *tk = reinterpret_cast<int *>(lds_v[wave]);
-    const int n_slots = (int)(c1 - c0);
-    // all global loads first (keys and logits), then the two redistributions
-    int4 kk[kChunkElems / (kWave * 4)];
-    float4 xv[kChunkElems / (kWave * 4)];
+  float4 xv[kChunkElems / (kWave * 4)];
+  if (DIRECT) {                               // the logits first: they depend on nothing
 #pragma unroll
     for (int i = 0; i < kChunkElems / (kWave * 4); ++i) {
       const int q = (i * kWave + lane) * 4;
-      kk[i] = make_int4(-1, -1, -1, -1);
-      if (FULL ? q < n_slots : q + 3 < n_slots) {
-        kk[i] = *reinterpret_cast<const int4 *>(row_of_slot + c0 + q);
-      } else if (!FULL && q < n_slots) {
-        kk[i].x = row_of_slot[c0 + q];
-        if (q + 1 < n_slots) kk[i].y = row_of_slot[c0 + q + 1];
-        if (q + 2 < n_slots) kk[i].z = row_of_slot[c0 + q + 2];
-      }
       xv[i] = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
       if (FULL || q + 3 < n_elem) {
         xv[i] = *reinterpret_cast<const float4 *>(x + base_elem + q);
@@ -182,330 +230,345 @@ __device__ __forceinline__ void softmax_chunk_body(
         if (q + 2 < n_elem) xv[i].z = x[base_elem + q + 2];
       }
     }
-#pragma unroll
-    for (int i = 0; i < kChunkElems / (kWave * 4); ++i) {
-      const int q = (i * kWave + lane) * 4;
-      if (q < n_slots) {          // keys: one per slot, word slot + slot/16
-        const int w = q + (q >> 4);
-        tk[w] = kk[i].x; tk[w + 1] = kk[i].y; tk[w + 2] = kk[i].z; tk[w + 3] = kk[i].w;
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int j = 0; j < kT; ++j)
-      key[j] = (FULL || s0 + j < c1) ? tk[g * (kT + 1) + j] : -1;
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int i = 0; i < kChunkElems / (kWave * 4); ++i) {
-      tv[lds_at[i][0]] = xv[i].x; tv[lds_at[i][1]] = xv[i].y;
-      tv[lds_at[i][2]] = xv[i].z; tv[lds_at[i][3]] = xv[i].w;
-    }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int j = 0; j < kT; ++j) {
-      v[j] = (FULL || key[j] >= 0) ? tv[lane * (kT + 1) + j] : -INFINITY;
-      off[j] = 0;
-    }
-    __builtin_amdgcn_wave_barrier();
   } else {
 #pragma unroll
     for (int j = 0; j < kT; ++j) {
       const int64_t slot = s0 + j;
-      const bool valid = FULL || (slot < c1 && h < heads);
-      key[j] = valid ? row_of_slot[slot] : -1;
+      const bool valid = FULL || (slot < cr.c1 && h < heads);
       const int64_t e = (valid && eid) ? (int64_t)eid[slot] : slot;
-      off[j] = e * heads + h;
-      v[j] = valid ? x[off[j]] : -INFINITY;
+      S.off[j] = e * heads + h;
+      v[j] = valid ? x[S.off[j]] : -INFINITY;
     }
   }
-  // which rows does the chunk share with its neighbours?  (needed last)
-  ChunkInfo ci;
-  chunk_info(row_of_slot, n_edges, head_shift, ci);
+  rows_of_chunk(pointer, cr, head_shift, lane, reinterpret_cast<int *>(tile), S.key);
+  if (!FULL) {
+#pragma unroll
+    for (int j = 0; j < kT; ++j)
+      if (!(s0 + j < cr.c1 && h < heads)) S.key[j] = -1;
+  }
+  if (DIRECT) {
+#pragma unroll
+    for (int i = 0; i < kChunkElems / (kWave * 4); ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int q = (i * kWave + lane) * 4 + c;
+        const int slot = q >> head_shift, hd = q & (H - 1);
+        const float xe = c == 0 ? xv[i].x : (c == 1 ? xv[i].y : (c == 2 ? xv[i].z : xv[i].w));
+        tile[(((slot >> 4) << head_shift) + hd) * (kT + 1) + (slot & 15)] = xe;
+      }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int j = 0; j < kT; ++j) {
+      v[j] = (FULL || S.key[j] >= 0) ? tile[lane * (kT + 1) + j] : -INFINITY;
+      S.raw[j] = v[j];
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
   // ---- maxima ------------------------------------------------------------
   float m[kT];
   m[0] = v[0];
 #pragma unroll
   for (int j = 1; j < kT; ++j)
-    m[j] = key[j] == key[j - 1] ? fmaxf(m[j - 1], v[j]) : v[j];
+    m[j] = S.key[j] == S.key[j - 1] ? fmaxf(m[j - 1], v[j]) : v[j];
 #pragma unroll
   for (int j = kT - 2; j >= 0; --j)
-    if (key[j] == key[j + 1]) m[j] = m[j + 1];
-  const int kf = key[0], kl = key[kT - 1];
-  float mf, ml;
-  chunk_totals<true>(m[0], m[kT - 1], kf, kl, lane, H, mf, ml);
+    if (S.key[j] == S.key[j + 1]) m[j] = m[j + 1];
+  const int kf = S.key[0], kl = S.key[kT - 1];
+  chunk_totals<true>(m[0], m[kT - 1], kf, kl, lane, H, S.mf, S.ml);
 #pragma unroll
-  for (int j = 0; j < kT; ++j) m[j] = key[j] == kf ? mf : (key[j] == kl ? ml : m[j]);
+  for (int j = 0; j < kT; ++j) m[j] = S.key[j] == kf ? S.mf : (S.key[j] == kl ? S.ml : m[j]);
   // ---- sums of exponentials ------------------------------------------------
-  float p[kT], l[kT];
 #pragma unroll
   for (int j = 0; j < kT; ++j)
-    p[j] = (FULL || key[j] >= 0) ? exp_fast(v[j] - finite_or_zero(m[j])) : 0.0f;
-  l[0] = p[0];
+    S.p[j] = (FULL || S.key[j] >= 0) ? exp_fast(v[j] - finite_or_zero(m[j])) : 0.0f;
+  S.l[0] = S.p[0];
 #pragma unroll
-  for (int j = 1; j < kT; ++j) l[j] = key[j] == key[j - 1] ? l[j - 1] + p[j] : p[j];
+  for (int j = 1; j < kT; ++j) S.l[j] = S.key[j] == S.key[j - 1] ? S.l[j - 1] + S.p[j] : S.p[j];
 #pragma unroll
   for (int j = kT - 2; j >= 0; --j)
-    if (key[j] == key[j + 1]) l[j] = l[j + 1];
-  float lf, ll;
-  chunk_totals<false>(l[0], l[kT - 1], kf, kl, lane, H, lf, ll);
-  // ---- rows inside the chunk: done; boundary rows: leave their statistics --
-  // (pass 2 rewrites every element of a boundary row, so DIRECT stores all)
-  const float rf = __builtin_amdgcn_rcpf(lf), rl = __builtin_amdgcn_rcpf(ll);
-  if (DIRECT) {
-    float *tv = lds_v[wave];
-#pragma unroll
-    for (int j = 0; j < kT; ++j) {
-      const float rt = key[j] == kf ? rf : (key[j] == kl ? rl : __builtin_amdgcn_rcpf(l[j]));
-      tv[lane * (kT + 1) + j] = p[j] * rt;
+    if (S.key[j] == S.key[j + 1]) S.l[j] = S.l[j + 1];
+  chunk_totals<false>(S.l[0], S.l[kT - 1], kf, kl, lane, H, S.lf, S.ll);
+}
+
+// After the workgroup barrier: the (max, sum) pairs of the rows a chunk shares
+// with other chunks of the tile are in LDS (pair_a / pair_b per wavefront, with
+// each wavefront's flags).  Rows that end up complete are normalised and stored;
+// rows that leave the tile leave their pair for the tile in `stats` and keep
+// their logits (DIRECT: written back unchanged, so that y may be x; gathered:
+// not written) for the second pass.
+template <bool DIRECT, bool FULL, int W>
+__device__ __forceinline__ void chunk_store(
+    const ChunkRows &cr, float *__restrict__ y, float *__restrict__ stats, int head_shift,
+    int heads, int wave, const int *wflags, const float2 *pair_a, const float2 *pair_b,
+    float *tile, const LaneRows<DIRECT> &S) {
+  const int H = 1 << head_shift;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int g = lane >> head_shift, h = lane & (H - 1);
+  const int64_t tile_id = blockIdx.x;
+  // pairs are stored [wavefront][head] with 64 heads per wavefront
+  auto pa = [&](int w) { return pair_a[w * kWave + h]; };
+  auto pb = [&](int w) { return pair_b[w * kWave + h]; };
+  float scale_a = 0.0f, scale_b = 0.0f;
+  bool open_a = false, open_b = false;
+  if (cr.began_before) {                    // the chunk's first row
+    int j = wave - 1;
+    while (j >= 0 && passes_through(wflags[j])) --j;
+    const bool open_left = j < 0;           // it began before the tile
+    int k = wave;
+    if (passes_through(wflags[wave])) {
+      k = wave + 1;
+      while (k < W && passes_through(wflags[k])) ++k;
     }
+    const bool open_right = k >= W;         // it continues past the tile
+    const int end = open_right ? W - 1 : k;
+    float M = -INFINITY, L = 0.0f;
+    if (!open_left) {
+      const float2 t = pb(j);
+      M = t.x;
+      L = t.y;
+    }
+    for (int q = open_left ? 0 : j + 1; q <= end; ++q) {
+      const float2 t = pa(q);
+      pair_merge(M, L, t.x, t.y);
+    }
+    open_a = open_left || open_right;
+    if (open_a && g == 0) {
+      if (open_left && wave == 0)
+        *reinterpret_cast<float2 *>(stat_ptr(stats, tile_id, 0, H, h)) = make_float2(M, L);
+      if (!open_left && wave == W - 1)
+        *reinterpret_cast<float2 *>(stat_ptr(stats, tile_id, 1, H, h)) = make_float2(M, L);
+    }
+    scale_a = S.mf == -INFINITY ? 0.0f : exp_fast(S.mf - M) * __builtin_amdgcn_rcpf(L);
+  }
+  if (cr.has_b) {                           // the chunk's last row, begun in this chunk
+    int k = wave + 1;
+    while (k < W && passes_through(wflags[k])) ++k;
+    open_b = k >= W;
+    const int end = open_b ? W - 1 : k;
+    const float2 t0 = pb(wave);
+    float M = t0.x, L = t0.y;
+    for (int q = wave + 1; q <= end; ++q) {
+      const float2 t = pa(q);
+      pair_merge(M, L, t.x, t.y);
+    }
+    if (open_b && g == 0 && wave == W - 1)
+      *reinterpret_cast<float2 *>(stat_ptr(stats, tile_id, 1, H, h)) = make_float2(M, L);
+    scale_b = S.ml == -INFINITY ? 0.0f : exp_fast(S.ml - M) * __builtin_amdgcn_rcpf(L);
+  }
+  const int kf = S.key[0], kl = S.key[kT - 1];
+  const float rf = __builtin_amdgcn_rcpf(S.lf), rl = __builtin_amdgcn_rcpf(S.ll);
+  const int key_a = cr.began_before ? cr.row_first : -2;
+  const int key_b = cr.has_b ? cr.row_last : -2;
+  float o[kT];
+  bool keep[kT];
+#pragma unroll
+  for (int j = 0; j < kT; ++j) {
+    const int kj = S.key[j];
+    float rt = kj == kf ? rf : (kj == kl ? rl : __builtin_amdgcn_rcpf(S.l[j]));
+    bool open = false;
+    if (kj == key_a) {
+      rt = scale_a;
+      open = open_a;
+    } else if (kj == key_b) {
+      rt = scale_b;
+      open = open_b;
+    }
+    o[j] = S.p[j] * rt;
+    keep[j] = open;
+    if (DIRECT && open) o[j] = S.raw[j];
+  }
+  if (DIRECT) {
+    const int64_t base_elem = cr.c0 << head_shift;
+    const int n_elem = (int)((cr.c1 - cr.c0) << head_shift);
+#pragma unroll
+    for (int j = 0; j < kT; ++j) tile[lane * (kT + 1) + j] = o[j];
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int i = 0; i < kChunkElems / (kWave * 4); ++i) {
       const int q = (i * kWave + lane) * 4;
-      const float4 o = make_float4(tv[lds_at[i][0]], tv[lds_at[i][1]],
-                                   tv[lds_at[i][2]], tv[lds_at[i][3]]);
+      float e[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int qq = q + c;
+        const int slot = qq >> head_shift, hd = qq & (H - 1);
+        e[c] = tile[(((slot >> 4) << head_shift) + hd) * (kT + 1) + (slot & 15)];
+      }
       if (FULL || q + 3 < n_elem) {
-        *reinterpret_cast<float4 *>(y + base_elem + q) = o;
+        *reinterpret_cast<float4 *>(y + base_elem + q) = make_float4(e[0], e[1], e[2], e[3]);
       } else if (q < n_elem) {
-        y[base_elem + q] = o.x;
-        if (q + 1 < n_elem) y[base_elem + q + 1] = o.y;
-        if (q + 2 < n_elem) y[base_elem + q + 2] = o.z;
+        y[base_elem + q] = e[0];
+        if (q + 1 < n_elem) y[base_elem + q + 1] = e[1];
+        if (q + 2 < n_elem) y[base_elem + q + 2] = e[2];
       }
     }
   } else {
-    const int skip_a = ci.began_before ? ci.row_first : -2;
-    const int skip_b = ci.continues ? ci.row_last : -2;
 #pragma unroll
-    for (int j = 0; j < kT; ++j) {
-      const float rt = key[j] == kf ? rf : (key[j] == kl ? rl : __builtin_amdgcn_rcpf(l[j]));
-      if ((FULL || key[j] >= 0) && key[j] != skip_a && key[j] != skip_b)
-        y[off[j]] = p[j] * rt;
-    }
-  }
-  const int64_t chunk = chunk_id;
-  if (ci.began_before && g == 0) {           // lanes 0..H-1 start with row_first
-    float *st = stat_ptr(stats, chunk, 0, H, h);
-    st[0] = mf;
-    st[1] = lf;
-  }
-  if (ci.continues && !(ci.began_before && ci.row_first == ci.row_last) &&
-      g == (kWave >> head_shift) - 1) {      // a continuing chunk is full
-    float *st = stat_ptr(stats, chunk, 1, H, h);
-    st[0] = ml;
-    st[1] = ll;
+    for (int j = 0; j < kT; ++j)
+      if ((FULL || S.key[j] >= 0) && !keep[j]) y[S.off[j]] = o[j];
   }
 }
 
-template <bool DIRECT>
-__global__ __launch_bounds__(kBlock) void softmax_chunks_kernel(
-    const int32_t *__restrict__ row_of_slot, const int32_t *__restrict__ eid,
-    const float *__restrict__ x, float *__restrict__ y, float *__restrict__ stats,
-    int64_t n_edges, int head_shift, int heads) {
-  // per wave: one tile of 1024 words (+ one pad word per 16), used in turn for
-  // the keys, the logits and the results
-  __shared__ float lds_v[kBlock / kWave][kChunkElems + kChunkElems / kT];
+template <bool DIRECT, int W>
+__global__ __launch_bounds__(W *kWave) void softmax_tiles_kernel(
+    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
+    const int32_t *__restrict__ eid, const float *__restrict__ x, float *__restrict__ y,
+    float *__restrict__ stats, int64_t n_edges, int head_shift, int heads) {
+  // per wavefront: one tile of 1024 words (+ one pad word per 16), used in turn for
+  // the row marks, the logits and the results
+  __shared__ float lds_tile[W][kTilePad];
+  __shared__ float2 pair_a[W * kWave], pair_b[W * kWave];
+  __shared__ int wflags[W];
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int H = 1 << head_shift;
   const int chunk_slots = kChunkElems >> head_shift;
-  const int64_t chunk_id = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
-  const int64_t c0 = chunk_id * chunk_slots;
-  if (c0 >= n_edges) return;                                        // whole wave
-  const int64_t c1 = min(c0 + (int64_t)chunk_slots, n_edges);
+  const int64_t chunk_id = (int64_t)blockIdx.x * W + wave;
+  ChunkRows cr;
+  cr.c0 = chunk_id * chunk_slots;
+  const bool active = cr.c0 < n_edges;                                // whole wavefront
+  cr.c1 = min(cr.c0 + (int64_t)chunk_slots, n_edges);
   // the variant without validity tests needs every lane live: a whole chunk and as
   // many heads as lanes per slot
-  if (c1 - c0 == chunk_slots && heads == (1 << head_shift))
-    softmax_chunk_body<DIRECT, true>(row_of_slot, eid, x, y, stats, n_edges,
-                                     head_shift, heads, chunk_id, c0, c1, lds_v);
+  const bool full = active && cr.c1 - cr.c0 == chunk_slots && heads == H;
+  LaneRows<DIRECT> S;
+  int flags = 0;
+  if (active) {
+    cr.row_first = row_of_slot[cr.c0];
+    cr.row_last = row_of_slot[cr.c1 - 1];
+    cr.began_before = pointer[cr.row_first] < cr.c0;
+    cr.continues = pointer[cr.row_last + 1] > cr.c1;
+    cr.has_b = cr.continues && !(cr.began_before && cr.row_first == cr.row_last);
+    if (full)
+      chunk_reduce<DIRECT, true>(pointer, eid, x, cr, head_shift, heads, lds_tile[wave], S);
+    else
+      chunk_reduce<DIRECT, false>(pointer, eid, x, cr, head_shift, heads, lds_tile[wave], S);
+    flags = kActive | (cr.began_before ? kBegan : 0) | (cr.continues ? kContinues : 0) |
+            (cr.row_first == cr.row_last ? kSingle : 0);
+    const int g = lane >> head_shift, h = lane & (H - 1);
+    if (cr.began_before && g == 0)            // lanes 0..H-1 start with row_first
+      pair_a[wave * kWave + h] = make_float2(S.mf, S.lf);
+    if (cr.has_b && g == (kWave >> head_shift) - 1)   // a continuing chunk is full
+      pair_b[wave * kWave + h] = make_float2(S.ml, S.ll);
+  }
+  if (lane == 0) wflags[wave] = flags;
+  __syncthreads();
+  if (!active) return;
+  if (full)
+    chunk_store<DIRECT, true, W>(cr, y, stats, head_shift, heads, wave, wflags, pair_a, pair_b,
+                                 lds_tile[wave], S);
   else
-    softmax_chunk_body<DIRECT, false>(row_of_slot, eid, x, y, stats, n_edges,
-                                      head_shift, heads, chunk_id, c0, c1, lds_v);
+    chunk_store<DIRECT, false, W>(cr, y, stats, head_shift, heads, wave, wflags, pair_a, pair_b,
+                                  lds_tile[wave], S);
 }
 
-// Pass 2: every row that starts in one chunk and continues into later ones gets its
-// partials -- B of its first chunk, A of the following ones -- merged once, as
-// (max, sum-exp) pairs: the chunk list is split over the lanes of a head, each lane
-// folds its chunks in ascending order (four loads in flight), and a fixed tree
-// combines the lanes.  The row's pair is left in the A slot of the row's second
-// chunk, which nothing else reads.  Rows of up to kWaveMergeChunks chunks are merged
-// by the wavefront of their first chunk (softmax_row_totals_kernel, same grid as
-// pass 1); longer rows by a workgroup of 1024 lanes each (softmax_long_row_totals_
-// kernel), so that a row of any length costs one parallel pass over its partials.
-constexpr int kWaveMergeShift = 9;
-constexpr int kWaveMergeChunks = 1 << kWaveMergeShift;
-constexpr int kTotalsBlock = 1024;
+// ---- pass 2: rows that leave a tile -------------------------------------------
+// One workgroup per tile.  For the (at most two) rows the tile shares with its
+// neighbours -- A: its first row, begun in an earlier tile; B: its last row,
+// started here and continuing -- the row's pair is folded from the tiles' partials
+// (B of the row's first tile, then A of the following ones, in tile order: every
+// tile of a row folds the same chain and gets the same pair), and the row's
+// elements inside this tile are normalised with it.  Chains of up to kShortChain
+// tiles are folded by every lane of a head for itself; longer ones are cut into a
+// piece per lane group, folded in parallel and combined in order.
+constexpr int kFixBlock = 256;
+constexpr int kShortChain = 16;
 
-// (m, l) <- (m, l) (+) (sm, sl).  The side that holds the maximum keeps its sum
-// unscaled (also when both maxima are -inf: the sums are then 0 or NaN and stay
-// so); the empty state (-inf, 0) scales by 0 (exp_fast has no value at -inf).
-__device__ __forceinline__ void pair_merge(float &m, float &l, float sm, float sl) {
-  const float nm = fmaxf(m, sm);
-  const float a = m == nm ? 1.0f : (m == -INFINITY ? 0.0f : exp_fast(m - nm));
-  const float b = sm == nm ? 1.0f : (sm == -INFINITY ? 0.0f : exp_fast(sm - nm));
-  l = l * a + sl * b;
-  m = nm;
-}
-
-// Lane (g, h) of G lane groups folds chunks k_lo + g, k_lo + g + G, ... <= k_hi of head h.
-__device__ __forceinline__ void fold_row_partials(const float *__restrict__ stats, int64_t k_lo,
-                                                  int64_t k_hi, int g, int G, int H, int h,
-                                                  float &m, float &l) {
-  m = -INFINITY;
-  l = 0.0f;
-  int64_t c = k_lo + g;
-  if (g == 0) {                               // the B partial of the row's first chunk
-    const float *st = stats + ((k_lo * 2 + 1) * H + h) * 2;
-    m = st[0];
-    l = st[1];
-    c += G;
-  }
-  const int64_t step = (int64_t)2 * H * 2;    // floats from one chunk's A slot to the next
-  const float *p = stats + ((c * 2) * H + h) * 2;
-  for (; c + 3 * (int64_t)G <= k_hi; c += 4 * (int64_t)G, p += 4 * G * step) {
-    float2 v[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const float2 *>(p + u * G * step);
-#pragma unroll
-    for (int u = 0; u < 4; ++u) pair_merge(m, l, v[u].x, v[u].y);
-  }
-  for (; c <= k_hi; c += G, p += G * step) {
-    const float2 v = *reinterpret_cast<const float2 *>(p);
-    pair_merge(m, l, v.x, v.y);
-  }
-}
-
-__global__ __launch_bounds__(kBlock) void softmax_row_totals_kernel(
+__global__ __launch_bounds__(kFixBlock) void softmax_tile_rows_kernel(
     const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
-    float *__restrict__ stats, int64_t n_edges, int head_shift) {
-  ChunkInfo ci;
-  if (!chunk_info(row_of_slot, n_edges, head_shift, ci)) return;
-  if (!ci.continues) return;
-  const int cs_shift = 10 - head_shift;       // chunk_slots = 1024 >> head_shift
-  const int64_t s = pointer[ci.row_last], e = pointer[ci.row_last + 1];
-  if (s < ci.c0) return;                      // the row started in an earlier chunk
-  const int64_t chunk = ci.c0 >> cs_shift, k_hi = (e - 1) >> cs_shift;
-  if (k_hi - chunk >= kWaveMergeChunks) return;   // left to the workgroup kernel
+    const int32_t *__restrict__ eid, const float *__restrict__ x, float *__restrict__ y,
+    const float *__restrict__ stats, int64_t n_edges, int head_shift, int heads,
+    int tile_shift) {
+  __shared__ float2 piece[kFixBlock];
+  __shared__ float2 total[kWave];
+  const int64_t t0 = (int64_t)blockIdx.x << tile_shift;
+  const int64_t t1 = min(t0 + ((int64_t)1 << tile_shift), n_edges);
+  const int row_first = row_of_slot[t0], row_last = row_of_slot[t1 - 1];
+  const bool began_before = pointer[row_first] < t0;
+  const bool continues = pointer[row_last + 1] > t1;
+  const bool has_b = continues && !(began_before && row_first == row_last);
+  if (!began_before && !has_b) return;                      // whole workgroup
   const int H = 1 << head_shift;
-  const int lane = threadIdx.x & (kWave - 1);
-  float m, l;
-  fold_row_partials(stats, chunk, k_hi, lane >> head_shift, kWave >> head_shift, H,
-                    lane & (H - 1), m, l);
-  // butterfly over the lane groups; partner pairs are merged lower group first
-  for (int o = H; o < kWave; o <<= 1) {
-    const float pm = __shfl_xor(m, o), pl = __shfl_xor(l, o);
-    if (lane & o) {
-      float qm = pm, ql = pl;
-      pair_merge(qm, ql, m, l);
-      m = qm;
-      l = ql;
+  const int G = kFixBlock >> head_shift;
+  const int g = threadIdx.x >> head_shift, h = threadIdx.x & (H - 1);
+  for (int which = 0; which < 2; ++which) {
+    if (which == 0 ? !began_before : !has_b) continue;      // whole workgroup
+    const int row = which == 0 ? row_first : row_last;
+    const int64_t s = pointer[row], e = pointer[row + 1];
+    const int64_t k_lo = s >> tile_shift, k_hi = (e - 1) >> tile_shift;
+    const int64_t len = k_hi - k_lo + 1;                    // states: B of k_lo, A of k_lo+1 .. k_hi
+    const float *a_of = stats + (size_t)h * 2;              // A pair of tile k: a_of[k * 4H]
+    const size_t step = (size_t)4 * H;
+    float M, L;
+    if (len <= kShortChain) {
+      const float2 b0 = *reinterpret_cast<const float2 *>(a_of + k_lo * step + 2 * H);
+      M = b0.x;
+      L = b0.y;
+      for (int64_t k = k_lo + 1; k <= k_hi; ++k) {
+        const float2 t = *reinterpret_cast<const float2 *>(a_of + k * step);
+        pair_merge(M, L, t.x, t.y);
+      }
     } else {
-      pair_merge(m, l, pm, pl);
+      // piece g: states [len*g/G, len*(g+1)/G) of the chain
+      const int64_t w0 = len * g / G, w1 = len * (g + 1) / G;
+      M = -INFINITY;
+      L = 0.0f;
+      int64_t w = w0;
+      if (w == 0 && w1 > 0) {
+        const float2 b0 = *reinterpret_cast<const float2 *>(a_of + k_lo * step + 2 * H);
+        M = b0.x;
+        L = b0.y;
+        w = 1;
+      }
+      for (; w + 4 <= w1; w += 4) {
+        float2 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          t[u] = *reinterpret_cast<const float2 *>(a_of + (k_lo + w + u) * step);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) pair_merge(M, L, t[u].x, t[u].y);
+      }
+      for (; w < w1; ++w) {
+        const float2 t = *reinterpret_cast<const float2 *>(a_of + (k_lo + w) * step);
+        pair_merge(M, L, t.x, t.y);
+      }
+      __syncthreads();                                      // `piece` free again
+      piece[threadIdx.x] = make_float2(M, L);
+      __syncthreads();
+      M = -INFINITY;
+      L = 0.0f;
+      for (int q = 0; q < G; ++q) {
+        const float2 t = piece[(q << head_shift) + h];
+        pair_merge(M, L, t.x, t.y);
+      }
     }
-  }
-  if (lane < H) *reinterpret_cast<float2 *>(stat_ptr(stats, chunk + 1, 0, H, lane)) = make_float2(m, l);
-}
-
-// Workgroup j (>= 1) looks at the row that covers the first slot of chunk
-// j * kWaveMergeChunks and merges it when it is longer than kWaveMergeChunks chunks
-// and that chunk is the first multiple of kWaveMergeChunks after the row's first
-// chunk -- every such row contains exactly one.
-__global__ __launch_bounds__(kTotalsBlock) void softmax_long_row_totals_kernel(
-    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
-    float *__restrict__ stats, int head_shift) {
-  __shared__ float2 red[kTotalsBlock];
-  const int cs_shift = 10 - head_shift;
-  const int64_t mark = ((int64_t)blockIdx.x + 1) << kWaveMergeShift;
-  const int row = row_of_slot[mark << cs_shift];
-  const int64_t s = pointer[row], e = pointer[row + 1];
-  const int64_t k_lo = s >> cs_shift, k_hi = (e - 1) >> cs_shift;
-  if (k_hi - k_lo < kWaveMergeChunks) return;
-  if (((k_lo >> kWaveMergeShift) + 1) << kWaveMergeShift != mark) return;
-  const int H = 1 << head_shift;
-  const int h = threadIdx.x & (H - 1);
-  float m, l;
-  fold_row_partials(stats, k_lo, k_hi, threadIdx.x >> head_shift, kTotalsBlock >> head_shift,
-                    H, h, m, l);
-  red[threadIdx.x] = make_float2(m, l);
-  __syncthreads();                            // also: every partial has been read
-  for (int o = kTotalsBlock >> 1; o >= H; o >>= 1) {
-    if ((int)threadIdx.x < o) {
-      float2 p = red[threadIdx.x];
-      const float2 q = red[threadIdx.x + o];
-      pair_merge(p.x, p.y, q.x, q.y);
-      red[threadIdx.x] = p;
-    }
+    __syncthreads();                                        // `total` free again
+    if (g == 0) total[h] = make_float2(M, __builtin_amdgcn_rcpf(L));
     __syncthreads();
-  }
-  if ((int)threadIdx.x < H)
-    *reinterpret_cast<float2 *>(stat_ptr(stats, k_lo + 1, 0, H, h)) = red[h];
-}
-
-// Pass 3: the rows a chunk shares with its neighbours (A = first row, begun in
-// an earlier chunk; B = last row, started here and continuing) are normalised with
-// their merged statistics.  Both rows are handled side by side so their dependent
-// loads overlap.
-__global__ __launch_bounds__(kBlock) void softmax_boundary_kernel(
-    const int32_t *__restrict__ pointer, const int32_t *__restrict__ row_of_slot,
-    const int32_t *__restrict__ eid, const float *__restrict__ x,
-    float *__restrict__ y, float *__restrict__ stats, int64_t n_edges,
-    int head_shift, int heads) {
-  ChunkInfo ci;
-  if (!chunk_info(row_of_slot, n_edges, head_shift, ci)) return;
-  const bool has_b = ci.continues && !(ci.began_before && ci.row_first == ci.row_last);
-  if (!ci.began_before && !has_b) return;
-  const int H = 1 << head_shift;
-  const int G = kWave >> head_shift;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int g = lane >> head_shift, h = lane & (H - 1);
-  const int cs_shift = 10 - head_shift;       // chunk_slots = 1024 >> head_shift
-
-  int64_t s[2] = {0, 0}, e[2] = {0, 0};
-  if (ci.began_before) { s[0] = pointer[ci.row_first]; e[0] = pointer[ci.row_first + 1]; }
-  if (has_b) { s[1] = pointer[ci.row_last]; e[1] = pointer[ci.row_last + 1]; }
-  int64_t lo[2], hi[2], o0[2];
-  float x0[2];
+    // the row's elements inside this tile
+    const int64_t lo = max(s, t0), hi = min(e, t1);
+    const int64_t n = (hi - lo) * heads;
+    for (int64_t base = 0; base < n; base += 4 * kFixBlock) {
+      int64_t o[4];
+      float xv[4];
+      float2 t[4];
 #pragma unroll
-  for (int w = 0; w < 2; ++w) {            // first element of each row, early
-    lo[w] = max(s[w], ci.c0);
-    hi[w] = min(e[w], ci.c1);
-    o0[w] = -1;
-    x0[w] = 0.0f;
-    if (lo[w] + g < hi[w] && h < heads) {
-      const int64_t slot = lo[w] + g;
-      const int64_t ed = eid ? (int64_t)eid[slot] : slot;
-      o0[w] = ed * heads + h;
-      x0[w] = x[o0[w]];
-    }
-  }
-  float m[2], rcp_l[2];
-#pragma unroll
-  for (int w = 0; w < 2; ++w) {
-    m[w] = 0.0f;
-    rcp_l[w] = 0.0f;
-    if (e[w] > s[w]) {      // totals of the row: A slot of its second chunk
-      const float *t = stat_ptr(stats, (s[w] >> cs_shift) + 1, 0, H, h);
-      m[w] = t[0];
-      rcp_l[w] = __builtin_amdgcn_rcpf(t[1]);
-    }
-  }
-#pragma unroll
-  for (int w = 0; w < 2; ++w) {
-    if (o0[w] >= 0) y[o0[w]] = exp_fast(x0[w] - m[w]) * rcp_l[w];
-    // the rest of the row's slots in this chunk, eight loads in flight
-    for (int64_t base = lo[w] + g + G; base < hi[w]; base += 8 * (int64_t)G) {
-      int64_t o[8];
-      float xv[8];
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const int64_t slot = base + (int64_t)t * G;
-        o[t] = -1;
-        xv[t] = 0.0f;
-        if (slot < hi[w] && h < heads) {
+      for (int u = 0; u < 4; ++u) {
+        const int64_t i = base + u * kFixBlock + threadIdx.x;
+        o[u] = -1;
+        xv[u] = 0.0f;
+        t[u] = make_float2(0.0f, 0.0f);
+        if (i < n) {
+          const int64_t slot = lo + i / heads;
+          const int hd = (int)(i % heads);
           const int64_t ed = eid ? (int64_t)eid[slot] : slot;
-          o[t] = ed * heads + h;
-          xv[t] = x[o[t]];
+          o[u] = ed * heads + hd;
+          xv[u] = x[o[u]];
+          t[u] = total[hd];
         }
       }
 #pragma unroll
-      for (int t = 0; t < 8; ++t)
-        if (o[t] >= 0) y[o[t]] = exp_fast(xv[t] - m[w]) * rcp_l[w];
+      for (int u = 0; u < 4; ++u)
+        if (o[u] >= 0) y[o[u]] = exp_fast(xv[u] - t[u].x) * t[u].y;
     }
   }
 }
@@ -667,11 +730,11 @@ extern "C" {
 size_t ga_softmax_workspace_bytes(int64_t n_edges, int64_t heads) {
   if (n_edges <= 0 || heads <= 0) return 0;
   if (ga::chunked_heads(heads)) {
-    // two partial (max, sum) pairs per lane of a slot for every chunk of 1024 lanes' elements
+    // two partial (max, sum) pairs per lane of a slot for every tile
     const int shift = ga::lanes_per_slot_shift(heads);
-    const int64_t chunk_slots = ga::kChunkElems >> shift;
-    const int64_t chunks = (n_edges + chunk_slots - 1) / chunk_slots;
-    return (size_t)chunks * 2 * ((size_t)1 << shift) * 2 * sizeof(float);
+    const int64_t tile_slots = (int64_t)ga::kTileWaves * (ga::kChunkElems >> shift);
+    const int64_t tiles = (n_edges + tile_slots - 1) / tile_slots;
+    return (size_t)tiles * 2 * ((size_t)1 << shift) * 2 * sizeof(float);
   }
   if (n_edges <= ga::kLongRow) return 0;
   const int64_t chunks = (n_edges + ga::kLongRow - 1) / ga::kLongRow;
@@ -690,6 +753,11 @@ int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
   if (n_rows == 0 || n_edges == 0) return GA_OK;
   if (!pointer || !row_of_slot || !x || !y) return GA_EINVAL;
   if (!aligned(x, 4) || !aligned(y, 4)) return GA_EALIGN;
+  if (x != y) {     // y may be x itself; any other overlap would read results as logits
+    const uintptr_t xa = reinterpret_cast<uintptr_t>(x), ya = reinterpret_cast<uintptr_t>(y);
+    const uintptr_t bytes = (uintptr_t)n_edges * (uintptr_t)heads * sizeof(float);
+    if (xa < ya + bytes && ya < xa + bytes) return GA_EINVAL;
+  }
   const size_t need = ga_softmax_workspace_bytes(n_edges, heads);
   if (need && (!workspace || workspace_bytes < need || !aligned(workspace, 16)))
     return GA_EWORKSPACE;
@@ -699,29 +767,21 @@ int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
   if (chunked_heads(heads)) {
     const int head_shift = lanes_per_slot_shift(heads);
     const bool every_lane_live = heads == ((int64_t)1 << head_shift);
-    const int64_t chunk_slots = kChunkElems >> head_shift;
-    const int64_t chunks = (n_edges + chunk_slots - 1) / chunk_slots;
-    const int64_t blocks = (chunks + kBlock / kWave - 1) / (kBlock / kWave);
-    if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-    if (every_lane_live && !eid && aligned(x, 16) && aligned(y, 16) && aligned(row_of_slot, 16))
-      hipLaunchKernelGGL(softmax_chunks_kernel<true>, dim3((unsigned)blocks),
-                         dim3(kBlock), 0, s, row_of_slot, eid, x, y, stats,
+    const int tile_shift = ilog2_floor((uint64_t)kTileWaves) + ilog2_floor((uint64_t)kChunkElems) - head_shift;
+    const int64_t tiles = (n_edges + ((int64_t)1 << tile_shift) - 1) >> tile_shift;
+    if (tiles > 0x7fffffff) return GA_EUNSUPPORTED;
+    if (every_lane_live && !eid && aligned(x, 16) && aligned(y, 16))
+      hipLaunchKernelGGL((softmax_tiles_kernel<true, kTileWaves>), dim3((unsigned)tiles),
+                         dim3(kTileWaves * kWave), 0, s, pointer, row_of_slot, eid, x, y, stats,
                          n_edges, head_shift, (int)heads);
     else
-      hipLaunchKernelGGL(softmax_chunks_kernel<false>, dim3((unsigned)blocks),
-                         dim3(kBlock), 0, s, row_of_slot, eid, x, y, stats,
+      hipLaunchKernelGGL((softmax_tiles_kernel<false, kTileWaves>), dim3((unsigned)tiles),
+                         dim3(kTileWaves * kWave), 0, s, pointer, row_of_slot, eid, x, y, stats,
                          n_edges, head_shift, (int)heads);
-    if (chunks > 1) {
-      hipLaunchKernelGGL(softmax_row_totals_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s,
-                         pointer, row_of_slot, stats, n_edges, head_shift);
-      const int64_t marks = (chunks - 1) >> kWaveMergeShift;   // multiples of the limit below `chunks`
-      if (marks > 0)
-        hipLaunchKernelGGL(softmax_long_row_totals_kernel, dim3((unsigned)marks),
-                           dim3(kTotalsBlock), 0, s, pointer, row_of_slot, stats, head_shift);
-      hipLaunchKernelGGL(softmax_boundary_kernel, dim3((unsigned)blocks),
-                         dim3(kBlock), 0, s, pointer, row_of_slot, eid, x, y, stats,
-                         n_edges, head_shift, (int)heads);
-    }
+    if (tiles > 1)
+      hipLaunchKernelGGL(softmax_tile_rows_kernel, dim3((unsigned)tiles), dim3(kFixBlock), 0, s,
+                         pointer, row_of_slot, eid, x, y, stats, n_edges, head_shift, (int)heads,
+                         tile_shift);
     return launch_status();
   }
 
