@@ -40,6 +40,7 @@ SIGNATURES = {
                                 _vp]),
     "ga_sddmm_u_op_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _int, _int,
                                _vp]),
+    "ga_sddmm_u_op_v_adj": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "ga_sddmm_u_dot_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64,
                                 _int, _vp]),
     "ga_softmax_workspace_bytes": (_sz, [_i64, _i64]),

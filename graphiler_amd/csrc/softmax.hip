@@ -124,7 +124,6 @@ constexpr int kTilePad = kChunkElems;                      // LDS words per wave
 constexpr int kQuads = kChunkElems / (kWave * 4);          // 16-byte pieces per lane
 // logits of a chunk that span more than this use per-row maxima as the reference
 // point of their exponentials; a narrower chunk uses its own maximum for all rows
-constexpr float kFlatRange = 60.0f;
 constexpr float kFlatMinExp = 8.7565108e-27f;   // e^-60
 
 // How a chunk's logits reach the lanes:
@@ -203,7 +202,7 @@ __device__ __forceinline__ void segment_max(float (&m)[kT], const float (&c)[kT]
   }
 }
 
-// exp(x) for x in [-kFlatRange, 0] (and 0 for -inf): exp2 of the rounded product.  The
+// exp(x) for x in [-60, 0] (and 0 for -inf): exp2 of the rounded product.  The
 // product's rounding (|x| log2 e 2^-24 in the exponent) costs at most 3.6e-6 of the
 // result at x = -60 and 3e-7 at x = -5, where exp_fast's correction term would cost
 // five more instructions per element.

@@ -95,6 +95,13 @@ struct DGLGraph : torch::CustomClassHolder {
                 "edge columns must all have num_edges entries");
     SetNtypePointer(ntype_pointer);
     SetEtypePointer(etype_pointer);
+    // what the kernels schedule with, once, here: the slot -> row maps and whether
+    // edge ids are slot numbers (a device-to-host read: not something an operator
+    // call should wait for)
+    if (in_pointer.is_cuda()) {
+      side(false);
+      side(true);
+    }
   }
   void SetNtypePointer(at::optional<torch::Tensor> pointer) {
     if (pointer.has_value()) check_index(pointer.value(), at::kInt, "ntype_pointer");
@@ -145,11 +152,17 @@ struct DGLGraph : torch::CustomClassHolder {
     }
     return s;
   }
+  // Scratch shared by the operators called on this graph: calls that use it must be
+  // ordered on one stream (two streams working on one graph object race on it).  It
+  // grows on demand; a buffer that was handed out is never freed while the graph
+  // lives, because a recorded HIP graph may still replay launches that write to it.
   torch::Tensor workspace(size_t bytes) {
     std::lock_guard<std::mutex> lock(mu_);
-    if (!ws_.defined() || (size_t)ws_.numel() < bytes)
+    if (!ws_.defined() || (size_t)ws_.numel() < bytes) {
+      if (ws_.defined()) retired_ws_.push_back(ws_);
       ws_ = torch::empty({(int64_t)std::max<size_t>(bytes, 256)},
                          in_pointer.options().dtype(at::kByte));
+    }
     return ws_;
   }
 
@@ -157,6 +170,7 @@ struct DGLGraph : torch::CustomClassHolder {
   std::mutex mu_;
   Side in_side_, out_side_;
   torch::Tensor ws_;
+  std::vector<torch::Tensor> retired_ws_;
 };
 
 using GraphPtr = c10::intrusive_ptr<DGLGraph>;
@@ -279,6 +293,20 @@ torch::Tensor u_add_v_mul_alpha(torch::Tensor src_feature, torch::Tensor dst_fea
               "src_feature and dst_feature must share a width");
   torch::Tensor out = torch::empty(out_shape(graph->num_edges, src_feature),
                                    src_feature.options().dtype(at::kFloat));
+  // two or four fp32 values per node on a graph stored by destination: walk the
+  // adjacency (rows from the row pointer, one index column instead of two)
+  if (dt == GA_F32 && (feat == 2 || feat == 4) && graph->num_edges > 0 &&
+      graph->side(false).identity) {
+    const int rc = ga_sddmm_u_op_v_adj(
+        graph->in_pointer.data_ptr<int>(), graph->side(false).rows.data_ptr<int>(),
+        graph->in_node_indices.data_ptr<int>(), src_feature.data_ptr<float>(),
+        dst_feature.data_ptr<float>(), out.data_ptr<float>(), graph->num_nodes,
+        graph->num_edges, feat, GA_SDDMM_ADD, current_stream(out));
+    if (rc != GA_EALIGN && rc != GA_EUNSUPPORTED) {
+      check_ga(rc, "ga_sddmm_u_op_v_adj");
+      return out;
+    }
+  }
   const EdgeColumns c = edge_columns(graph);
   check_ga(ga_sddmm_u_add_v(c.lhs, c.rhs, c.bits, src_feature.data_ptr(),
                             dst_feature.data_ptr(), out.data_ptr<float>(),
@@ -524,8 +552,11 @@ torch::Tensor gat_aggregate(torch::Tensor el, torch::Tensor er, torch::Tensor z,
   check_input(er, "er");
   check_input(z, "z");
   const int dt = feat_dtype(z, "z");
-  TORCH_CHECK(el.scalar_type() == at::kFloat && er.scalar_type() == at::kFloat,
-              "el and er must be float32");
+  // the attention terms of a bf16 plan may arrive as bf16 (mm(z, attn_weight) on the
+  // stored z): the logits are formed in fp32 either way
+  TORCH_CHECK(el.is_floating_point() && er.is_floating_point(), "el and er must be floating point");
+  el = el.to(at::kFloat).contiguous();
+  er = er.to(at::kFloat).contiguous();
   const int64_t heads = feat_dim(el), feat = feat_dim(z);
   TORCH_CHECK(feat_dim(er) == heads && heads > 0 && feat % heads == 0,
               "inconsistent head count");
@@ -557,7 +588,8 @@ torch::Tensor gat_aggregate_al(torch::Tensor a_l, torch::Tensor el, torch::Tenso
   check_input(z, "z");
   TORCH_CHECK(a_l.is_cuda(), "a_l must be a CUDA tensor");
   const int dt = feat_dtype(z, "z");
-  TORCH_CHECK(er.scalar_type() == at::kFloat, "er must be float32");
+  TORCH_CHECK(er.is_floating_point(), "er must be floating point");
+  er = er.to(at::kFloat).contiguous();
   const int64_t heads = feat_dim(er), feat = feat_dim(z);
   TORCH_CHECK(heads > 0 && feat % heads == 0 && a_l.numel() == feat, "inconsistent head count");
   TORCH_CHECK(er.size(0) == graph->num_nodes && z.size(0) == graph->num_nodes,

@@ -196,10 +196,15 @@ class DGLGraph:
         return self._identity("out_ident", self.out_edge_indices)
 
     def workspace(self, nbytes: int) -> torch.Tensor:
-        """Scratch buffer reused across calls on this graph (grows on demand).
-        Calls that use it are ordered on the current stream."""
+        """Scratch buffer shared by the operators called on this graph (grows on
+        demand).  Calls that use it must be ordered on one stream: two streams
+        working on one graph object race on it.  A buffer that was handed out is
+        kept alive as long as the graph, because a recorded HIP graph may still
+        replay launches that write to it."""
         ws = self._cache.get("ws")
         if ws is None or ws.numel() < nbytes:
+            if ws is not None:
+                self._cache.setdefault("retired_ws", []).append(ws)
             ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8,
                              device=self.device)
             self._cache["ws"] = ws

@@ -79,6 +79,10 @@ def dedup(graph: torch._C.Graph) -> None:
                 n.destroy()
                 changed = True
                 continue
+            # a result that an in-place operator (leaky_relu_, relu_, ...) later
+            # overwrites, or an operand that one does, is not the same value twice
+            if ours and (any(mutated(o) for o in n.outputs()) or any(mutated(i) for i in n.inputs())):
+                continue
             key = (n.kind(), tuple(i.unique() for i in n.inputs()))
             if key in seen:
                 n.replaceAllUsesWith(seen[key])
@@ -531,6 +535,18 @@ class _Rewriter:
             mm, bc = a.node(), b.node()
             if mm.kind() == "my_ops::SegmentMMEdgeGather" and self.single_use(a) and \
                     bc.kind() in ("my_ops::BroadcastSrcNode", "my_ops::BroadcastDstNode"):
+                # only the product this docstring describes: no per-row factor (the
+                # dot has no place for one) and one head -- with (T, H, K, M) weights
+                # the sum over dim 1 runs over heads * M, not per head
+                scale = mm.inputsAt(3)
+                if scale.node().kind() != "prim::Constant" or \
+                        not isinstance(scale.type(), torch._C.NoneType):
+                    continue
+                # (typed products in a plan come from bmm, whose operands are 3-D; a
+                # weight whose rank is known must say the same)
+                w_type = mm.inputsAt(1).type()
+                if isinstance(w_type, torch._C.TensorType) and w_type.dim() not in (None, 3):
+                    continue
                 which = self.const(0 if bc.kind().endswith("SrcNode") else 1, n)
                 out = self.make("my_ops::SegmentMMEdgeDot",
                                 [mm.inputsAt(0), mm.inputsAt(1), mm.inputsAt(2),

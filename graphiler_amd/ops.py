@@ -195,34 +195,46 @@ def _edge_columns(g: DGLGraph):
     return g.COO_src, g.COO_dst, 64
 
 
+# Operand widths (fp32 values per node) at which the SDDMM that walks the adjacency
+# beats the two-column kernel on an MI355X: with one value per node both are bound by
+# the rate of the 4-byte gathers of the source term (about two cycles per gather and
+# compute unit: 44 us against 61 us for 11.6 M edges); from two values on the walk
+# wins (4 values, 64.3 M edges: 0.78 against 0.90 ms).
+_ADJ_SDDMM_WIDTHS = (2, 4)
+
+
 def gsddmm_u_add_v_mul_alpha(src_feature, dst_feature, alpha: int,
                              graph: DGLGraph) -> torch.Tensor:
     """sddmm.cu:118-129: out[e] = src_feature[src[e]] + dst_feature[dst[e]]
     in edge-id order, fp32 (E, feat).  ``alpha`` is ignored, as in the reference."""
-    _check_input(src_feature, "src_feature")
-    _check_input(dst_feature, "dst_feature")
-    dt = _feat_dtype(src_feature, "src_feature")
-    if dst_feature.dtype != src_feature.dtype:
-        raise RuntimeError("src_feature and dst_feature must share a dtype")
-    feat = get_feat_dim(src_feature)
-    if get_feat_dim(dst_feature) != feat:
-        raise RuntimeError("src_feature and dst_feature must share a width")
-    out = torch.empty(_out_shape(graph.num_edges, src_feature),
-                      dtype=torch.float32, device=src_feature.device)
-    lhs, rhs, bits = _edge_columns(graph)
-    capi.check(capi.load().ga_sddmm_u_add_v(
-        lhs.data_ptr(), rhs.data_ptr(), bits, src_feature.data_ptr(),
-        dst_feature.data_ptr(), out.data_ptr(), graph.num_edges, feat, dt,
-        _stream(out)), "ga_sddmm_u_add_v")
-    return out
+    return gsddmm_u_op_v("add", src_feature, dst_feature, graph)
 
 
 def gsddmm_u_op_v(op: str, src_feature, dst_feature, graph: DGLGraph) -> torch.Tensor:
     """Generic SDDMM of the reference (sddmm.cuh:34-71 with the add / sub / mul /
     div functors, functor.cuh:19-72): out[e] = src_feature[src[e]] (op)
-    dst_feature[dst[e]] in edge-id order, fp32 (E, feat)."""
+    dst_feature[dst[e]] in edge-id order, fp32 (E, feat).  fp32 operands of width
+    2 or 4 on a graph whose edge ids are in-adjacency slots walk the adjacency
+    (rows from the row pointer: one index column read instead of two)."""
     code = {"add": capi.GA_SDDMM_ADD, "sub": capi.GA_SDDMM_SUB, "mul": capi.GA_SDDMM_MUL,
             "div": capi.GA_SDDMM_DIV}[op]
+    if (src_feature.dtype == torch.float32 and dst_feature.dtype == torch.float32
+            and src_feature.is_cuda and dst_feature.is_cuda
+            and src_feature.is_contiguous() and dst_feature.is_contiguous()
+            and get_feat_dim(src_feature) == get_feat_dim(dst_feature)
+            and get_feat_dim(src_feature) in _ADJ_SDDMM_WIDTHS and graph.num_edges > 0
+            and graph.in_eid_is_identity):
+        feat = get_feat_dim(src_feature)
+        out = torch.empty(_out_shape(graph.num_edges, src_feature),
+                          dtype=torch.float32, device=src_feature.device)
+        rc = capi.load().ga_sddmm_u_op_v_adj(
+            graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
+            graph.in_node_indices.data_ptr(), src_feature.data_ptr(),
+            dst_feature.data_ptr(), out.data_ptr(), graph.num_nodes, graph.num_edges,
+            feat, code, _stream(out))
+        if rc not in (capi.GA_EALIGN, capi.GA_EUNSUPPORTED):   # else: the two-column kernel
+            capi.check(rc, "ga_sddmm_u_op_v_adj")
+            return out
     _check_input(src_feature, "src_feature")
     _check_input(dst_feature, "dst_feature")
     dt = _feat_dtype(src_feature, "src_feature")
@@ -479,8 +491,10 @@ def gat_aggregate(el, er, z, graph: DGLGraph, negative_slope: float = 0.01):
     _check_input(er, "er")
     _check_input(z, "z")
     dt = _feat_dtype(z, "z")
-    if el.dtype != torch.float32 or er.dtype != torch.float32:
-        raise RuntimeError("el and er must be float32")
+    if not (el.is_floating_point() and er.is_floating_point()):
+        raise RuntimeError("el and er must be floating point")
+    # bf16 attention terms (a bf16 plan's mm(z, attn_weight)): the logits are fp32 either way
+    el, er = el.float().contiguous(), er.float().contiguous()
     heads = get_feat_dim(el)
     feat = get_feat_dim(z)
     if get_feat_dim(er) != heads or feat % heads:

@@ -149,6 +149,21 @@ int ga_sddmm_u_op_v(const void *lhs, const void *rhs, int idx_bits,
                     const void *u, const void *v, float *out, int64_t n_edges,
                     int64_t feat, int op, int dtype, ga_stream_t stream);
 
+/* The same operators over a grouped adjacency, for graphs whose edge ids are slot
+ * numbers (eid[i] == i, e.g. edges stored by destination): out[i, k] =
+ * u[nbr[i], k] (op) v[row(i), k] for every slot i, i.e. the reference's
+ * SDDMMCoo_u_add_v_mul_alpha (sddmm.cu:118-129) with lhs target = the neighbour
+ * column, rhs target = the row (selector.h:30-60).  The row of a slot comes from the
+ * row pointer, so no second index column is read and v is read once per row:
+ * 4 + 8 feat bytes per edge instead of 8 + 12 feat.  fp32, feat 1, 2 or 4
+ * (GA_EUNSUPPORTED otherwise: use ga_sddmm_u_op_v); nbr and out 16-byte aligned,
+ * u and v aligned to a row (GA_EALIGN otherwise).  row_of_slot is read at two
+ * slots per 256 - 1024 only.  Bit-exact with ga_sddmm_u_op_v. */
+int ga_sddmm_u_op_v_adj(const int32_t *pointer, const int32_t *row_of_slot,
+                        const int32_t *nbr, const float *u, const float *v, float *out,
+                        int64_t n_rows, int64_t n_edges, int64_t feat, int op,
+                        ga_stream_t stream);
+
 /* out[i, h] = sum_d u[lhs[i], h, d] * v[rhs[i], h, d], fp32 output (E, heads).
  * The Dot functor (functor.cuh:103-116) with the reduction over the last
  * dimension (bcast.cc:37-39,57-60; kernel sddmm.cuh:80-120), which the

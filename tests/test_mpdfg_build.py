@@ -108,6 +108,31 @@ def test_inplace_activation_chain_is_fused_and_removed():
     assert "my_ops::gsddmm_u_add_v_mul_alpha" not in k
 
 
+def reads_one_field_twice_message(edges: EdgeBatchDummy):
+    x = edges.src['h']
+    y = torch.relu_(edges.src['h'] + 0.0)      # a second read, overwritten in place afterwards
+    z = torch.relu_(edges.src['h'])            # in place on the broadcast itself
+    return {'m': x + y + z}
+
+
+def test_value_numbering_keeps_reads_that_are_overwritten_apart():
+    """Two equal graph operators are one value only while nothing writes to either
+    result: the read that relu_ overwrites must not become the read that is used
+    unchanged (level 0 runs only the value numbering)."""
+    plan = mpdfg_builder(reads_one_field_twice_message, U.gcn_reduce, opt_level=0)
+    plan.forward
+    nodes = list(plan.graph.nodes())
+    reads = [n for n in nodes if n.kind() == "my_ops::BroadcastSrcNode"]
+    inplace = [n for n in nodes if n.kind() == "aten::relu_"]
+    for r in inplace:
+        target = r.inputsAt(0).node()
+        if target.kind() == "my_ops::BroadcastSrcNode":
+            # the overwritten read feeds the in-place operator only
+            assert [u.user.kind() for u in target.output().uses()] == ["aten::relu_"]
+    assert len(reads) >= 2 or not any(r.inputsAt(0).node().kind() == "my_ops::BroadcastSrcNode"
+                                      for r in inplace)
+
+
 def bad_reduce(nodes: NodeBatchDummy):
     return {'h': torch.sum(nodes.mailbox['missing'], dim=1)}
 
