@@ -77,7 +77,19 @@ def test_config3_rgcn_full(device, bf16):
     msg = oracle.segment_mm(etp, oracle.gather_rows(wl.src, x), w1) * norm
     ref = oracle.spmm(ptr, nbr, eid, msg.astype(np.float32), op="copy_e")
     assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
-                 "config 3 RGCN layer")
+                 "config 3 RGCN layer 1 (16 -> 64)")
+    # second layer (64 -> 8) on the device's own first-layer output after relu, so that
+    # the check is of this layer alone
+    w2 = datasets.glorot(rng, (60, 64, 8))
+    if bf16:
+        w2 = to_bf16_f32(w2)
+    h1 = torch.relu(got)
+    got2 = layers.rgcn_layer(g, h1, _t(w2, device, bf16), _t(norm, device))
+    h1_h = h1.float().cpu().numpy()
+    msg = oracle.segment_mm(etp, oracle.gather_rows(wl.src, h1_h), w2) * norm
+    ref2 = oracle.spmm(ptr, nbr, eid, msg.astype(np.float32), op="copy_e")
+    assert_close(got2.float().cpu().numpy(), ref2, TOL_BF16 if bf16 else TOL_F32,
+                 "config 3 RGCN layer 2 (64 -> 8)")
 
 
 def test_config4_hgt_operators_full(device):
@@ -190,3 +202,36 @@ def test_config5_large_gat_sampled_and_properties(device):
     want = (x32.double() * _t(np.bincount(wl.src, minlength=n).astype(np.float64),
                               device)[:, None]).sum(0).cpu().numpy()
     np.testing.assert_allclose(col, want, rtol=1e-6, atol=1e-3 * np.abs(want).max())
+
+
+@pytest.mark.timeout(600)
+def test_config5_three_layer_network_layer_by_layer(device):
+    """The 3-layer network of configuration 5 (100 -> 256 -> 256 -> 256, 4 heads x 64,
+    bf16 storage, elu between layers) at full size.  Each layer is checked on its own:
+    the oracle gets the device's input to that layer and is evaluated on sampled
+    destination rows plus the three heaviest ones (their in-edges reach most of the
+    graph's nodes, so the projection is computed for every node, in fp32 on the host)."""
+    wl = datasets.gat_rmat_large()
+    n, heads, d = wl.num_nodes, 4, 64
+    deg = np.bincount(wl.dst, minlength=n)
+    g = prepare_graph(wl.src, wl.dst, n, device=device)
+    ptr = g.in_pointer.cpu().numpy()
+    rng = np.random.default_rng(45)
+    sample = np.unique(np.concatenate([rng.integers(0, n, 2000), np.argsort(deg)[-3:], [0, n - 1]]))
+    sub_ptr = np.concatenate([[0], np.cumsum(deg[sample])]).astype(np.int32)
+    sub_nbr = np.concatenate([wl.src[ptr[v]:ptr[v + 1]] for v in sample]).astype(np.int32)
+    x = _t(to_bf16_f32(rng.standard_normal((n, 100), dtype=np.float32)), device, True)
+    for layer, k in enumerate((100, 256, 256)):
+        w = to_bf16_f32(datasets.glorot(rng, (k, heads * d)))
+        a = datasets.glorot(rng, (2, heads, d), fan_in=2 * d, fan_out=1)
+        out = layers.gat_layer(g, x, _t(w, device, True), _t(a, device), heads, 0.2, fused=True)
+        x_h = x.float().cpu().numpy()
+        z32 = x_h @ w                                        # fp32 accumulate, like the device
+        zh = z32.reshape(n, heads, d)
+        el = (zh * a[0]).sum(-1).astype(np.float32)
+        er = (zh * a[1]).sum(-1).astype(np.float32)
+        z = to_bf16_f32(z32)                                 # the rows the aggregation reads are stored bf16
+        ref = oracle.gat_aggregate(sub_ptr, sub_nbr, el, er[sample], z, heads=heads, slope=0.2)
+        assert_close(out.float().cpu().numpy()[sample], ref, TOL_BF16,
+                     f"config 5 network, layer {layer + 1} ({k} -> 256), sampled rows")
+        x = torch.nn.functional.elu(out)
