@@ -20,6 +20,8 @@ GA_F32, GA_BF16 = 0, 1
 GA_COPY_U, GA_COPY_E, GA_U_MUL_E, GA_U_ADD_E, GA_U_SUB_E, GA_U_DIV_E = 0, 1, 2, 3, 4, 5
 GA_SDDMM_ADD, GA_SDDMM_SUB, GA_SDDMM_MUL, GA_SDDMM_DIV = 0, 1, 2, 3
 GA_SUM, GA_MAX, GA_MIN = 0, 1, 2
+(GA_BCAST_ADD, GA_BCAST_SUB, GA_BCAST_MUL, GA_BCAST_DIV, GA_BCAST_COPY_LHS, GA_BCAST_COPY_RHS,
+ GA_BCAST_DOT) = range(7)
 
 _vp, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
 
@@ -40,6 +42,10 @@ SIGNATURES = {
                                 _vp]),
     "ga_sddmm_u_op_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _int, _int,
                                _vp]),
+    "ga_spmm_csr_bcast": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp,
+                                 _i64, _i64, _i64, _int, _int, _vp]),
+    "ga_sddmm_bcast": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp, _vp, _i64, _i64,
+                              _i64, _i64, _int, _vp]),
     "ga_sddmm_u_op_v_adj": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "ga_sddmm_u_dot_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64,
                                 _int, _vp]),

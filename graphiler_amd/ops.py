@@ -100,17 +100,21 @@ def spmm(g: DGLGraph, op: str, reduce: str, u: torch.Tensor,
         if w.shape[0] != g.num_edges:
             raise RuntimeError("edge weights must have one row per edge")
         heads = get_feat_dim(w)
-        if feat % heads:
+        shaped = w.dim() == u.dim() and u.dim() >= 3
+        if feat % heads and not shaped:
             raise RuntimeError("feature width is not a multiple of the heads")
-        if w.dim() == u.dim() and u.dim() >= 3:
-            # shaped operands, e.g. (N, H, D) * (E, H, 1): accept exactly the
-            # broadcasts that are "one weight per head" (bcast.cc:19-71 tables)
+        if shaped:
+            # shaped operands, e.g. (N, H, D) * (E, H, 1): the row-reduction kernels
+            # take exactly the broadcasts that are "one weight per head" (tables of
+            # bcast.cc:19-71); any other shape pair goes to the general kernel
             b = calc_bcast_off("mul", tuple(u.shape), tuple(w.shape))
-            per_head = np.arange(feat, dtype=np.int64) // (feat // heads)
-            if b.out_len != feat or not np.array_equal(b.lhs_offset, np.arange(feat)) \
+            per_head = np.arange(feat, dtype=np.int64) // max(feat // heads, 1)
+            if feat % heads or b.out_len != feat \
+                    or not np.array_equal(b.lhs_offset, np.arange(feat)) \
                     or not np.array_equal(b.rhs_offset, per_head):
-                raise RuntimeError("unsupported broadcast between features "
-                                   f"{tuple(u.shape)} and edge weights {tuple(w.shape)}")
+                return gspmm(g, {"u_mul_e": "mul", "e_mul_e": "mul", "u_add_e": "add",
+                                 "u_sub_e": "sub", "u_div_e": "div"}[op], reduce, u, w,
+                             reverse=reverse, return_arg=return_arg, edge_rows=edge_rows)
     n_src = g.num_edges if edge_rows else g.num_nodes
     if u.shape[0] != n_src:
         raise RuntimeError("features have the wrong number of rows")
@@ -275,6 +279,123 @@ def gsddmm_u_dot_v(src_feature, dst_feature, graph: DGLGraph) -> torch.Tensor:
         lhs.data_ptr(), rhs.data_ptr(), bits, src_feature.data_ptr(),
         dst_feature.data_ptr(), out.data_ptr(), graph.num_edges, heads, dim, dt,
         _stream(out)), "ga_sddmm_u_dot_v")
+    return out
+
+
+# ------------------------------------------------- general (broadcasting) forms ----
+_BCAST_OPS = {"add": capi.GA_BCAST_ADD, "sub": capi.GA_BCAST_SUB, "mul": capi.GA_BCAST_MUL,
+              "div": capi.GA_BCAST_DIV, "copy_lhs": capi.GA_BCAST_COPY_LHS,
+              "copy_rhs": capi.GA_BCAST_COPY_RHS, "dot": capi.GA_BCAST_DOT}
+
+
+def _bcast_shape(lhs_shape, rhs_shape, drop_last: bool):
+    """Feature shape of op(lhs, rhs) under numpy broadcasting of the dimensions after
+    the first (``drop_last``: the dot product consumes the last one)."""
+    ls = tuple(lhs_shape[1:-1] if drop_last else lhs_shape[1:])
+    rs = tuple(rhs_shape[1:-1] if drop_last else rhs_shape[1:])
+    return tuple(np.broadcast_shapes(ls, rs))
+
+
+def _offsets(table: np.ndarray, device) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(table, dtype=np.int64)).to(device)
+
+
+def gspmm(g: DGLGraph, op: str, reduce: str, u: Optional[torch.Tensor],
+          e: Optional[torch.Tensor], reverse: bool = False, return_arg: bool = False,
+          edge_rows: bool = False):
+    """The reference's general SpMM (SpMMCsrKernel with UseBcast, spmm.cuh:30-71):
+    out[v] = reduce over the in-edges i of v of ``op(u[src_i], e[edge_i])`` where the
+    feature shapes of ``u`` (N, ...) and ``e`` (E, ...) broadcast against each other by
+    numpy's rules (offset tables: :func:`graphiler_amd.bcast.calc_bcast_off`, the
+    reference's CalcBcastOff, bcast.cc:19-71).  op: add | sub | mul | div | copy_lhs |
+    copy_rhs; reduce: sum | max | min; fp32.  ``reverse``: over the out-adjacency.
+    ``edge_rows``: ``u`` is per-edge too (read through the edge-id column).
+    The general path: one thread per output element, no tuning; shapes the benchmark
+    models use (equal shapes, one weight per head) are served by :func:`spmm`."""
+    code = _BCAST_OPS[op]
+    if op == "dot":
+        raise RuntimeError("dot is an SDDMM operator")
+    use_u, use_e = op != "copy_rhs", op != "copy_lhs"
+    for t, name, used in ((u, "u", use_u), (e, "e", use_e)):
+        if used:
+            _check_input(t, name)
+            if t.dtype != torch.float32:
+                raise RuntimeError("the general SpMM is float32 only")
+    if reverse:
+        pointer, nbr, eid, ident = g.out_pointer, g.out_node_indices, g.out_edge_indices, \
+            g.out_eid_is_identity
+    else:
+        pointer, nbr, eid, ident = g.in_pointer, g.in_node_indices, g.in_edge_indices, \
+            g.in_eid_is_identity
+    if edge_rows:
+        nbr = eid
+    if use_u and u.shape[0] != (g.num_edges if edge_rows else g.num_nodes):
+        raise RuntimeError("u has the wrong number of rows")
+    if use_e and e.shape[0] != g.num_edges:
+        raise RuntimeError("e must have one row per edge")
+    ref = u if use_u else e
+    lhs_shape = tuple(u.shape) if use_u else (1,) + tuple(e.shape[1:])
+    rhs_shape = tuple(e.shape) if use_e else (1,) + tuple(u.shape[1:])
+    b = calc_bcast_off(op, lhs_shape, rhs_shape)
+    feat_shape = _bcast_shape(lhs_shape, rhs_shape, False) if b.use_bcast else \
+        tuple((e if op == "copy_rhs" else u).shape[1:])
+    out = torch.empty((g.num_nodes,) + feat_shape, dtype=torch.float32, device=ref.device)
+    arg_u = arg_e = None
+    if return_arg:
+        if reduce not in ("max", "min"):
+            raise RuntimeError("return_arg needs the max or the min reducer")
+        if use_u:
+            arg_u = torch.empty(out.shape, dtype=torch.int32, device=ref.device)
+        if use_e:
+            arg_e = torch.empty(out.shape, dtype=torch.int32, device=ref.device)
+    u_off = _offsets(b.lhs_offset, ref.device) if b.use_bcast else None
+    e_off = _offsets(b.rhs_offset, ref.device) if b.use_bcast else None
+    capi.check(capi.load().ga_spmm_csr_bcast(
+        pointer.data_ptr(), nbr.data_ptr(), None if ident else eid.data_ptr(), _ptr(u), _ptr(e),
+        out.data_ptr(), _ptr(arg_u), _ptr(arg_e), g.num_nodes, g.num_edges, _ptr(u_off),
+        _ptr(e_off), max(b.lhs_len, 1), max(b.rhs_len, 1), b.out_len, code, _REDUCE[reduce],
+        _stream(ref)), "ga_spmm_csr_bcast")
+    return (out, arg_u, arg_e) if return_arg else out
+
+
+_TARGETS = {"u": 0, "e": 1, "v": 2}
+
+
+def gsddmm(g: DGLGraph, op: str, lhs: torch.Tensor, rhs: torch.Tensor,
+           lhs_target: str = "u", rhs_target: str = "v") -> torch.Tensor:
+    """The reference's general SDDMM (SDDMMCooKernel / the dot-product kernel,
+    sddmm.cuh:34-120): out[e] = ``op(lhs[id_l(e)], rhs[id_r(e)])`` in edge-id order with
+    each operand on the source nodes ("u"), on the edges ("e") or on the destination
+    nodes ("v") (selector.h:30-60) and feature shapes that broadcast by numpy's rules
+    (bcast.cc:19-71); ``dot`` sums the products over the last dimension.  fp32.
+    The general path; ``u (op) v`` on equal shapes and ``u_dot_v`` per head are served
+    by :func:`gsddmm_u_op_v` / :func:`gsddmm_u_dot_v`."""
+    code = _BCAST_OPS[op]
+    _check_input(lhs, "lhs")
+    _check_input(rhs, "rhs")
+    if lhs.dtype != torch.float32 or rhs.dtype != torch.float32:
+        raise RuntimeError("the general SDDMM is float32 only")
+    for t, target, name in ((lhs, lhs_target, "lhs"), (rhs, rhs_target, "rhs")):
+        if target not in _TARGETS:
+            raise RuntimeError("targets are 'u' (source), 'e' (edge) or 'v' (destination)")
+        if t.shape[0] != (g.num_edges if target == "e" else g.num_nodes):
+            raise RuntimeError(f"{name} has the wrong number of rows for target {target!r}")
+    if op == "dot" and lhs.shape[-1] != rhs.shape[-1]:
+        raise RuntimeError("dot needs operands with the same last dimension")
+    b = calc_bcast_off(op, tuple(lhs.shape), tuple(rhs.shape))
+    if b.use_bcast:
+        feat_shape = _bcast_shape(lhs.shape, rhs.shape, op == "dot")
+    else:
+        src = rhs if op == "copy_rhs" else lhs
+        feat_shape = tuple(src.shape[1:-1] if op == "dot" else src.shape[1:])
+    out = torch.empty((g.num_edges,) + (feat_shape or (1,)), dtype=torch.float32, device=lhs.device)
+    l_off = _offsets(b.lhs_offset, lhs.device) if b.use_bcast else None
+    r_off = _offsets(b.rhs_offset, lhs.device) if b.use_bcast else None
+    capi.check(capi.load().ga_sddmm_bcast(
+        g.COO_src.data_ptr(), g.COO_dst.data_ptr(), lhs.data_ptr(), rhs.data_ptr(),
+        out.data_ptr(), g.num_edges, _TARGETS[lhs_target], _TARGETS[rhs_target], _ptr(l_off),
+        _ptr(r_off), max(b.lhs_len, 1), max(b.rhs_len, 1), b.out_len, b.reduce_size, code,
+        _stream(out)), "ga_sddmm_bcast")
     return out
 
 

@@ -47,6 +47,11 @@ enum ga_spmm_op {
   GA_COPY_U = 0, GA_COPY_E = 1,
   GA_U_MUL_E = 2, GA_U_ADD_E = 3, GA_U_SUB_E = 4, GA_U_DIV_E = 5 /* u[src] (op) w[edge] */
 };
+/* binary operators of the general (broadcasting) forms, functor.cuh:19-116 */
+enum ga_bcast_op {
+  GA_BCAST_ADD = 0, GA_BCAST_SUB = 1, GA_BCAST_MUL = 2, GA_BCAST_DIV = 3,
+  GA_BCAST_COPY_LHS = 4, GA_BCAST_COPY_RHS = 5, GA_BCAST_DOT = 6 /* SDDMM only */
+};
 /* functor.cuh:125-213: sum starts at 0, max at -inf, min at +inf             */
 enum ga_reduce { GA_SUM = 0, GA_MAX = 1, GA_MIN = 2 };
 
@@ -128,6 +133,22 @@ int ga_spmm_csr_arg(const int32_t *pointer, const int32_t *row_of_slot,
                     int op, int reduce, int dtype, void *workspace,
                     size_t workspace_bytes, ga_stream_t stream);
 
+/* SpMM whose operands broadcast against each other: the UseBcast = true form of
+ * the reference's generic kernel (SpMMCsrKernel, spmm.cuh:30-71) fed by the offset
+ * tables of CalcBcastOff (bcast.cc:19-71):
+ *   out[v, k] = reduce_{i in row v} op(u[nbr[i], u_off[k]], w[eid[i], w_off[k]])
+ * u (n_src, u_len), w (n_edges, w_len), out (n_rows, out_len), all fp32;
+ * u_off / w_off (out_len) int64 on the device, NULL = the identity (k).
+ * op: ga_bcast_op without DOT; reduce: ga_reduce; arg_u / arg_e as in
+ * ga_spmm_csr_arg (NULL when not wanted; max / min only).  Edges of a row are
+ * folded in adjacency order by one thread per output element: the general path,
+ * not a tuned one.  eid NULL when eid[i] == i. */
+int ga_spmm_csr_bcast(const int32_t *pointer, const int32_t *nbr, const int32_t *eid,
+                      const float *u, const float *w, float *out, int32_t *arg_u,
+                      int32_t *arg_e, int64_t n_rows, int64_t n_edges, const int64_t *u_off,
+                      const int64_t *w_off, int64_t u_len, int64_t w_len, int64_t out_len,
+                      int op, int reduce, ga_stream_t stream);
+
 /* ------------------------------------------------------------------ SDDMM --
  * out[i, k] = u[lhs[i], k] + v[rhs[i], k], fp32 output (E, feat).
  * Replaces SDDMMCoo_u_add_v_mul_alpha (sddmm.cu:118-129, kernel
@@ -163,6 +184,23 @@ int ga_sddmm_u_op_v_adj(const int32_t *pointer, const int32_t *row_of_slot,
                         const int32_t *nbr, const float *u, const float *v, float *out,
                         int64_t n_rows, int64_t n_edges, int64_t feat, int op,
                         ga_stream_t stream);
+
+/* The general SDDMM of the reference (SDDMMCooKernel / SDDMMCooTreeReduceKernel,
+ * sddmm.cuh:34-120): operands on the source nodes (target 0), on the edges (1) or on
+ * the destination nodes (2) in any combination (selector.h:30-60), feature shapes
+ * that broadcast (offset tables of CalcBcastOff, bcast.cc:19-71), and the dot
+ * product over the last dimension:
+ *   out[e, k] = op(lhs[id_l(e), lhs_off[k] * reduce_size ...],
+ *                  rhs[id_r(e), rhs_off[k] * reduce_size ...])
+ * with id = src[e] | e | dst[e] by target; GA_BCAST_DOT sums reduce_size products,
+ * every other operator needs reduce_size == 1.  src / dst int64 (the COO columns),
+ * lhs (*, lhs_len), rhs (*, rhs_len), out (n_edges, out_len) fp32 in edge-id order;
+ * lhs_off / rhs_off (out_len) int64 on the device, NULL = the identity. */
+int ga_sddmm_bcast(const int64_t *src, const int64_t *dst, const float *lhs, const float *rhs,
+                   float *out, int64_t n_edges, int lhs_target, int rhs_target,
+                   const int64_t *lhs_off, const int64_t *rhs_off, int64_t lhs_len,
+                   int64_t rhs_len, int64_t out_len, int64_t reduce_size, int op,
+                   ga_stream_t stream);
 
 /* out[i, h] = sum_d u[lhs[i], h, d] * v[rhs[i], h, d], fp32 output (E, heads).
  * The Dot functor (functor.cuh:103-116) with the reduction over the last

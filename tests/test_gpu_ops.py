@@ -148,7 +148,8 @@ def test_spmm_add_sub_div(graph, device, op, reduce, feat, heads, bf16):
 
 def test_spmm_u_mul_e_shaped_operands(graph, device):
     """(N, H, D) features with (E, H, 1) weights: the per-head broadcast of the
-    reference's shape tables; any other broadcast is rejected."""
+    reference's shape tables, served by the row-reduction kernel; any other broadcast
+    takes the general kernel (bcast.cc:19-71 tables consumed on the device)."""
     name, g, arr = graph
     rng = np.random.default_rng(11)
     e = arr.COO_src.shape[0]
@@ -159,9 +160,11 @@ def test_spmm_u_mul_e_shaped_operands(graph, device):
     ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
                       x.reshape(arr.num_nodes, 32), w.reshape(e, 4), op="u_mul_e", heads=4)
     assert_close(got.cpu().numpy().reshape(arr.num_nodes, 32), ref, TOL_F32, f"shaped {name}")
-    bad = rng.standard_normal((e, 1, 8), dtype=np.float32)      # per-feature, not per-head
-    with pytest.raises(RuntimeError, match="unsupported broadcast"):
-        ops.gspmm_src_mul_e_sum(_dev(x, device), _dev(bad, device), [1], False, None, g)
+    per_feat = rng.standard_normal((e, 1, 8), dtype=np.float32)      # per feature, not per head
+    got = ops.gspmm_src_mul_e_sum(_dev(x, device), _dev(per_feat, device), [1], False, None, g)
+    want = np.zeros((arr.num_nodes, 4, 8))
+    np.add.at(want, arr.COO_dst, x[arr.COO_src].astype(np.float64) * per_feat)
+    assert_close(got.cpu().numpy(), want, TOL_F32, f"shaped, per-feature weights {name}")
 
 
 @pytest.mark.parametrize("reduce", ["max", "min"])
