@@ -519,6 +519,78 @@ def SegmentMMEdgeGather(features, weights, endpoint: int, graph: DGLGraph,
     return out
 
 
+def _typed_tiles(graph: DGLGraph):
+    """The (destination tile, relation) ordering of the in-edges that TypedSpMMEdge
+    walks; built on the device at first use and kept with the graph."""
+    t = graph._cache.get("typed_tiles")
+    if t is None:
+        lib = capi.load()
+        n, e, r = graph.num_nodes, graph.num_edges, graph.num_etypes
+        cap = int(lib.ga_typed_tiles_chunk_capacity(n, e, r))
+        tiles = -(-n // capi.GA_TYPED_TILE_ROWS)
+        dev = graph.device
+        i32 = dict(dtype=torch.int32, device=dev)
+        t = (torch.empty(tiles + 1, **i32), torch.empty(max(cap, 1), **i32),
+             torch.empty(max(16 * cap, 1), **i32),
+             torch.empty(max(16 * cap, 4), dtype=torch.uint8, device=dev),
+             torch.empty(max(16 * cap, 4), **i32))
+        nbytes = int(lib.ga_typed_tiles_workspace_bytes(n, e, r))
+        if nbytes == 0:
+            raise RuntimeError("graph too large for the typed tile layout")
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        ident = graph.in_eid_is_identity
+        capi.check(lib.ga_typed_tiles_build(
+            graph.in_row_of_slot.data_ptr(), graph.in_node_indices.data_ptr(),
+            None if ident else graph.in_edge_indices.data_ptr(),
+            graph.etype_pointer.data_ptr(), n, e, r, t[0].data_ptr(), t[1].data_ptr(),
+            t[2].data_ptr(), t[3].data_ptr(), t[4].data_ptr(), ws.data_ptr(), ws.numel(),
+            torch.cuda.current_stream(dev).cuda_stream), "ga_typed_tiles_build")
+        graph._cache["typed_tiles"] = t
+    return t
+
+
+def typed_spmm_supported(features, weights) -> bool:
+    """Shapes TypedSpMMEdge takes: 64 output features, 16 / 32 / 48 / 64 input features."""
+    return weights.dim() == 3 and int(weights.shape[2]) == 64 \
+        and int(weights.shape[1]) in (16, 32, 48, 64) \
+        and get_feat_dim(features) == int(weights.shape[1])
+
+
+def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None) -> torch.Tensor:
+    """``SpMMEdge(SegmentMMEdge(BroadcastSrcNode(features), weights) * row_scale)``
+    in one pass (examples/RGCN/RGCN.py:25-33; broadcast.cu:58-63, segment_mm.cu:29-33,
+    spmm.cu:359-373): out[v] = sum over the in-edges e of v of
+    row_scale[e] * features[src(e)] @ weights[type(e)].  No per-edge tensor is written.
+    features (N, K), weights (R, K, 64) with K in 16, 32, 48, 64; ``row_scale`` (E,) or
+    (E, 1) fp32.  The additions of a row happen in the order of the prepared layout
+    (by relation, then adjacency order), the same in every call."""
+    _check_input(features, "features")
+    _check_input(weights, "weights")
+    dt = _feat_dtype(features, "features")
+    if weights.dtype != features.dtype:
+        raise RuntimeError("features and weights must have one dtype")
+    if graph.etype_pointer is None:
+        raise RuntimeError("the graph has no edge type pointer")
+    if weights.dim() != 3 or int(weights.shape[0]) != graph.num_etypes \
+            or get_feat_dim(features) != int(weights.shape[1]):
+        raise RuntimeError("weights must be (edge types, K, M) with K the feature width")
+    if int(features.shape[0]) != graph.num_nodes:
+        raise RuntimeError("features must have one row per node")
+    if row_scale is not None:
+        _check_input(row_scale, "row_scale")
+        if row_scale.dtype != torch.float32 or row_scale.numel() != graph.num_edges:
+            raise RuntimeError("row_scale must be one float32 per edge")
+    K, M = int(weights.shape[1]), int(weights.shape[2])
+    tcp, ctype, ssrc, sdst, sedge = _typed_tiles(graph)
+    out = torch.empty((graph.num_nodes, M), dtype=features.dtype, device=features.device)
+    capi.check(capi.load().ga_typed_spmm(
+        tcp.data_ptr(), ctype.data_ptr(), ssrc.data_ptr(), sdst.data_ptr(), sedge.data_ptr(),
+        features.data_ptr(), weights.data_ptr(), _ptr(row_scale), out.data_ptr(),
+        graph.num_nodes, int(features.shape[0]), graph.num_edges, graph.num_etypes, K, M,
+        dt, _stream(out)), "ga_typed_spmm")
+    return out
+
+
 def SegmentMMEdgeDot(features, weights, endpoint: int, other, other_endpoint: int,
                      graph: DGLGraph, scale=None) -> torch.Tensor:
     """out[e, h] = <features[endpoint(e)] @ weights[type(e)], other[other_endpoint(e)]>

@@ -185,6 +185,47 @@ int ga_sddmm_u_op_v_adj(const int32_t *pointer, const int32_t *row_of_slot,
                         int64_t n_rows, int64_t n_edges, int64_t feat, int op,
                         ga_stream_t stream);
 
+/* Typed neighbour sum: out[v, :] = sum over in-edges e of v of
+ * row_scale[e] * (x[src(e), :] @ W[type(e)]), the operator chain BroadcastSrcNode ->
+ * SegmentMMEdge -> mul -> SpMMEdge of an RGCN layer (broadcast.cu:58-63,
+ * segment_mm.cu:29-33, spmm.cu:359-373; examples/RGCN/RGCN.py:25-33) in one pass, with
+ * no (E, M) message tensor.
+ *
+ * ga_typed_tiles_build prepares the graph once: the slots of the in-adjacency
+ * (row_of_slot = destination, nbr = source, eid = edge id or null when slot = edge id;
+ * type_pointer: n_types + 1 entries over the edge ids, include/dglgraph.h:24-27) are
+ * ordered by (destination / GA_TYPED_TILE_ROWS, relation) and every such group is
+ * padded to chunks of 16 slots.  Outputs: tile_chunk_pointer (tiles + 1, tiles =
+ * ceil(n_rows / GA_TYPED_TILE_ROWS)), chunk_type (capacity), slot_src and slot_edge
+ * (16 * capacity, -1 in pad slots), slot_dst (16 * capacity bytes: destination - tile
+ * start, 255 in pad slots; 4-byte aligned), capacity =
+ * ga_typed_tiles_chunk_capacity(...).  Everything runs on `stream`; nothing is read
+ * back.
+ *
+ * ga_typed_spmm: x (n_src, K), W (n_types, K, M), out (n_rows, M) of `dtype`;
+ * row_scale (n_edges,) fp32 in edge-id order or null.  M must be 64, K one of 16, 32,
+ * 48, 64, and x and row_scale smaller than 4 GiB (GA_EUNSUPPORTED otherwise: use
+ * ga_segment_mm_gather + ga_spmm_csr).  The sum over the in-edges runs on the matrix
+ * cores with fp32 accumulation: bf16 messages enter as the two-operator chain rounds
+ * them, fp32 messages as three bf16 terms that carry 24 bits.  The order of the
+ * additions is fixed by the prepared layout, so repeated calls give identical bits;
+ * against the chain only that order differs.  Messages that are not finite reach
+ * exactly the rows the chain would give them to. */
+#define GA_TYPED_TILE_ROWS 128
+int64_t ga_typed_tiles_chunk_capacity(int64_t n_rows, int64_t n_edges, int64_t n_types);
+size_t ga_typed_tiles_workspace_bytes(int64_t n_rows, int64_t n_edges, int64_t n_types);
+int ga_typed_tiles_build(const int32_t *row_of_slot, const int32_t *nbr, const int32_t *eid,
+                         const int32_t *type_pointer, int64_t n_rows, int64_t n_edges,
+                         int64_t n_types, int32_t *tile_chunk_pointer, int32_t *chunk_type,
+                         int32_t *slot_src, unsigned char *slot_dst, int32_t *slot_edge,
+                         void *workspace, size_t workspace_bytes, ga_stream_t stream);
+int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
+                  const int32_t *slot_src, const unsigned char *slot_dst,
+                  const int32_t *slot_edge, const void *x, const void *W,
+                  const float *row_scale, void *out, int64_t n_rows, int64_t n_src,
+                  int64_t n_edges, int64_t n_types, int64_t K, int64_t M, int dtype,
+                  ga_stream_t stream);
+
 /* The general SDDMM of the reference (SDDMMCooKernel / SDDMMCooTreeReduceKernel,
  * sddmm.cuh:34-120): operands on the source nodes (target 0), on the edges (1) or on
  * the destination nodes (2) in any combination (selector.h:30-60), feature shapes

@@ -1,0 +1,180 @@
+"""The one-pass RGCN aggregation (ops.TypedSpMMEdge, ga_typed_tiles_build + ga_typed_spmm)
+against the oracle's operator chain it replaces: gather_rows -> segment_mm -> * norm ->
+spmm(copy_e), i.e. BroadcastSrcNode -> SegmentMMEdge -> mul -> SpMMEdge of
+examples/RGCN/RGCN.py:25-33.  fp32 within 1e-5 (norm and element-wise against the sum
+of the absolute messages), bf16 within 2e-2; identical bits from call to call; messages
+that are not finite reach exactly the rows the chain gives them to."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from graphiler_amd import capi, layers, ops, prepare_graph
+from graphiler_amd.graph import build_graph_arrays, sort_edges_by_type
+from helpers import TOL_BF16, TOL_F32, assert_close, to_bf16_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def _typed_graph(rng, n, e, r, device, hub=False):
+    src = rng.integers(0, n, e, dtype=np.int64)
+    dst = rng.integers(0, n, e, dtype=np.int64)
+    if hub and e:
+        dst[: e // 3] = n // 2          # one destination with a third of the edges
+    p = np.arange(1, r + 1, dtype=np.float64) ** -1.1
+    etype = rng.choice(r, size=e, p=p / p.sum()).astype(np.int64)
+    src, dst, etype, _ = sort_edges_by_type(src, dst, etype)
+    g = prepare_graph(src, dst, n, device=device, etype_of=etype, num_etypes=r)
+    return g, build_graph_arrays(src, dst, n), src, dst, etype
+
+
+def _dev(a, device, bf16=False):
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    return t.bfloat16() if bf16 else t
+
+
+def _reference(arr, src, etype, r, x, w, norm):
+    etp = oracle.type_pointer(etype, r)
+    msg = oracle.segment_mm(etp, oracle.gather_rows(src, x), w)
+    if norm is not None:
+        msg = msg * norm[:, None]
+    msg = msg.astype(np.float32)
+    args = (arr.in_pointer, arr.in_node_indices, arr.in_edge_indices)
+    return (oracle.spmm(*args, msg, op="copy_e"), oracle.spmm(*args, np.abs(msg), op="copy_e"))
+
+
+CASES = [  # nodes, edges, relations, K, hub
+    (300, 4000, 7, 16, False),
+    (1000, 20000, 60, 16, True),
+    (130, 900, 3, 32, False),
+    (257, 5000, 11, 48, True),
+    (128, 3000, 5, 64, False),
+    (5, 40, 2, 16, False),
+    (700, 0, 4, 16, False),
+]
+
+
+@pytest.mark.parametrize("n,e,r,k,hub", CASES)
+@pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
+@pytest.mark.parametrize("scaled", [True, False], ids=["norm", "plain"])
+def test_typed_spmm_matches_operator_chain(device, n, e, r, k, hub, bf16, scaled):
+    rng = np.random.default_rng(n + e + k)
+    g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device, hub)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    w = (rng.standard_normal((r, k, 64)) / np.sqrt(k)).astype(np.float32)
+    norm = rng.uniform(0.1, 1.5, e).astype(np.float32) if scaled else None
+    if bf16:
+        x, w = to_bf16_f32(x), to_bf16_f32(w)
+    got = ops.TypedSpMMEdge(_dev(x, device, bf16), _dev(w, device, bf16), g,
+                            row_scale=_dev(norm, device) if scaled else None)
+    assert got.shape == (n, 64) and got.dtype == (torch.bfloat16 if bf16 else torch.float32)
+    ref, mag = _reference(arr, src, etype, r, x, w, norm)
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
+                 f"typed spmm n={n} e={e} r={r} k={k}", mag=mag)
+    again = ops.TypedSpMMEdge(_dev(x, device, bf16), _dev(w, device, bf16), g,
+                              row_scale=_dev(norm, device) if scaled else None)
+    assert torch.equal(got.view(torch.int16 if bf16 else torch.int32),
+                       again.view(torch.int16 if bf16 else torch.int32)), "bits differ between calls"
+
+
+def test_typed_tiles_layout(device):
+    """The prepared layout itself (integer work, exact): every edge appears once, in a
+    chunk of its relation inside the tile of its destination; pad slots say -1 / 255;
+    chunks of a tile are contiguous and ordered by relation, slots inside a (tile,
+    relation) group by adjacency position."""
+    rng = np.random.default_rng(9)
+    n, e, r = 700, 9000, 13
+    g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device, hub=True)
+    tcp, ctype, ssrc, sdst, sedge = (t.cpu().numpy() for t in ops._typed_tiles(g))
+    rows = capi.GA_TYPED_TILE_ROWS
+    tiles = -(-n // rows)
+    assert tcp.shape == (tiles + 1,) and tcp[0] == 0 and np.all(np.diff(tcp) >= 0)
+    total = int(tcp[-1])
+    used = slice(0, 16 * total)
+    live = sedge[used] >= 0
+    assert np.array_equal(np.sort(sedge[used][live]), np.arange(e)), "every edge once"
+    assert np.all(ssrc[used][~live] == -1) and np.all(sdst[used][~live] == 255)
+    ed = sedge[used][live]
+    assert np.array_equal(ssrc[used][live], src[ed])
+    chunk_of_slot = np.arange(16 * total) // 16
+    tile_of_chunk = np.searchsorted(tcp, np.arange(total), side="right") - 1
+    assert np.array_equal(dst[ed], tile_of_chunk[chunk_of_slot[live]] * rows + sdst[used][live])
+    assert np.array_equal(etype[ed], ctype[:total][chunk_of_slot[live]])
+    # order: relation ascending inside a tile; a group's slots in adjacency order
+    for t in range(tiles):
+        ct = ctype[tcp[t]:tcp[t + 1]]
+        assert np.all(np.diff(ct) >= 0)
+    slot_of_edge = np.empty(e, dtype=np.int64)
+    slot_of_edge[arr.in_edge_indices] = np.arange(e)
+    pos = slot_of_edge[ed]
+    key = tile_of_chunk[chunk_of_slot[live]] * r + etype[ed]
+    same = key[1:] == key[:-1]
+    assert np.all(pos[1:][same] > pos[:-1][same])
+    # every group wastes less than one chunk
+    groups = len(np.unique(key))
+    assert total <= -(-e // 16) + groups
+    assert total <= capi.load().ga_typed_tiles_chunk_capacity(n, e, r)
+
+
+@pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
+def test_typed_spmm_messages_that_are_not_finite(device, bf16):
+    """inf and NaN source features: the rows that receive such a message become what
+    the chain makes them (inf, -inf or NaN), every other row stays finite and exact to
+    tolerance -- the selection matrices of the kernel must not spread them."""
+    rng = np.random.default_rng(31)
+    n, e, r, k = 400, 6000, 6, 16
+    g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    w = np.abs(rng.standard_normal((r, k, 64)) / np.sqrt(k)).astype(np.float32) + 0.01
+    if bf16:
+        x, w = to_bf16_f32(x), to_bf16_f32(w)
+    x[0, :] = np.inf            # +inf messages (weights are positive); row 0 is also what pad slots read
+    x[77, :] = -np.inf
+    x[200, 5] = np.nan
+    norm = rng.uniform(0.1, 1.5, e).astype(np.float32)
+    got = ops.TypedSpMMEdge(_dev(x, device, bf16), _dev(w, device, bf16), g,
+                            row_scale=_dev(norm, device)).float().cpu().numpy()
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref, _ = _reference(arr, src, etype, r, x, w, norm)
+    touched = np.zeros(n, dtype=bool)
+    touched[dst[np.isin(src, [0, 77, 200])]] = True
+    assert touched.any() and not touched.all()
+    assert np.all(np.isfinite(got[~touched])), "a row without such a message is not finite"
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    assert np.array_equal(np.isposinf(got), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(got), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    tol = TOL_BF16 if bf16 else TOL_F32
+    assert np.abs(got[fin] - ref[fin]).max() <= tol * np.abs(ref[fin]).max()
+
+
+def test_rgcn_layer_paths_agree(device):
+    rng = np.random.default_rng(4)
+    n, e, r = 500, 8000, 9
+    g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device)
+    x = _dev(rng.standard_normal((n, 16), dtype=np.float32), device)
+    w = _dev((rng.standard_normal((r, 16, 64)) / 4).astype(np.float32), device)
+    norm = _dev(rng.uniform(0.1, 1.0, (e, 1)).astype(np.float32), device)
+    a = layers.rgcn_layer(g, x, w, norm, fused="tiles")
+    b = layers.rgcn_layer(g, x, w, norm, fused=False)
+    c = layers.rgcn_layer(g, x, w, norm, fused=True)
+    assert_close(a.cpu().numpy(), b.cpu().numpy(), 2 * TOL_F32, "tiles against unfused")
+    assert_close(c.cpu().numpy(), b.cpu().numpy(), 2 * TOL_F32, "default against unfused")
+
+
+def test_typed_spmm_rejects_what_it_does_not_cover(device):
+    rng = np.random.default_rng(6)
+    g, arr, src, dst, etype = _typed_graph(rng, 100, 500, 3, device)
+    x = torch.randn(100, 16, device=device)
+    with pytest.raises(capi.GraphilerError):          # M != 64
+        ops.TypedSpMMEdge(x, torch.randn(3, 16, 32, device=device), g)
+    with pytest.raises(capi.GraphilerError):          # K not a multiple of 16
+        ops.TypedSpMMEdge(torch.randn(100, 8, device=device), torch.randn(3, 8, 64, device=device), g)
+    with pytest.raises(RuntimeError):                 # one weight per relation
+        ops.TypedSpMMEdge(x, torch.randn(4, 16, 64, device=device), g)
+    with pytest.raises(RuntimeError):
+        ops.TypedSpMMEdge(x, torch.randn(3, 16, 64, device=device).bfloat16(), g)
+    with pytest.raises(RuntimeError):
+        ops.TypedSpMMEdge(x.cpu(), torch.randn(3, 16, 64), g)
+    assert not ops.typed_spmm_supported(x, torch.randn(3, 16, 32, device=device))
+    assert ops.typed_spmm_supported(x, torch.randn(3, 16, 64, device=device))
