@@ -437,6 +437,10 @@ def main():
             opsr["segment_mm_node_128_128"] = op_record(
                 "c4.segment_mm_node", lambda: ops.SegmentMMNode(X, wk, g),
                 N * 2 * hid * b + Tn * hid * hid * b, 2.0 * N * hid * hid, "bf16", reps=50)
+            wq, wv = rnd(Tn, hid, hid, dtype=dt) / hid ** 0.5, rnd(Tn, hid, hid, dtype=dt) / hid ** 0.5
+            opsr["segment_mm_node_qkv_128_3x128"] = op_record(
+                "c4.segment_mm_node_qkv", lambda: ops.SegmentMMNodeStacked(X, [wk, wq, wv], g),
+                N * 4 * hid * b + 3 * Tn * hid * hid * b, 3 * 2.0 * N * hid * hid, "bf16", reps=50)
             opsr["segment_mm_dot_8x16x16"] = op_record(
                 "c4.segment_mm_dot", lambda: ops.SegmentMMEdgeDot(X, ra, 0, X, 1, g),
                 E * (16 + 2 * hid * b + 4 * H) + Te * H * D * D * b, 2.0 * E * H * D * D, "bf16", reps=50)

@@ -61,6 +61,8 @@ SIGNATURES = {
                                   _vp, _sz, _vp]),
     "ga_segment_mm": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                              _int, _vp]),
+    "ga_segment_mm_stacked": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                                     _int, _vp]),
     "ga_segment_mm_gather": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                     _i64, _i64, _i64, _i64, _int, _vp]),
     "ga_gather_rows": (_int, [_vp, _int, _vp, _vp, _i64, _i64, _vp]),

@@ -31,6 +31,7 @@
 // against a second gathered row, out[e, h] = <Y[e, h, :], Q[q_index[e], h, :]>
 // (HGT's sum(k * q)), in which case Y never reaches memory.
 #include "common.h"
+#include "wide_mm.h"
 
 #include <type_traits>
 
@@ -980,11 +981,42 @@ int launch_mfma(const int32_t *tp, int n_types, const void *X, const void *W,
 namespace ga {
 namespace {
 
+// Wide bf16 outputs (whole groups of 128 columns, one head, few types): the kernel of
+// wide_mm.hip reads X once for all of `n_w` weight tensors.  GA_EUNSUPPORTED: not its shape.
+int wide_typed(const int32_t *type_pointer, int64_t n_types, const void *X,
+               const void *const *W, void *const *Y, int n_w, int64_t rows, int64_t K,
+               int64_t M, hipStream_t s) {
+  if (M % kWideGroupCols != 0 || n_types > 64) return GA_EUNSUPPORTED;
+  const int per_w = (int)(M / kWideGroupCols);
+  if (!wide_mm_fits((int)K, n_w * per_w)) return GA_EUNSUPPORTED;
+  WideMm p = {};
+  p.tp = type_pointer;
+  p.n_types = (int)n_types;
+  p.rows = rows;
+  p.X = (const bf16_t *)X;
+  p.K = (int)K;
+  p.n_groups = n_w * per_w;
+  for (int w = 0; w < n_w; ++w)
+    for (int c = 0; c < per_w; ++c) {
+      const int g = w * per_w + c;
+      p.W[g] = (const bf16_t *)W[w] + c * kWideGroupCols;
+      p.w_type_stride[g] = K * M;
+      p.ldw[g] = M;
+      p.Y[g] = (bf16_t *)Y[w] + c * kWideGroupCols;
+      p.ldy[g] = M;
+    }
+  return wide_mm_launch(p, s);
+}
+
 int segment_mm_any(const int32_t *type_pointer, int64_t n_types, const void *X,
                    const void *W, void *Y, int64_t rows, int64_t heads, int64_t K,
                    int64_t M, int dtype, const MmExt &ext, hipStream_t s) {
   const bool fused = ext.x_index || ext.Q;
   int rc = GA_EUNSUPPORTED;
+  if (dtype == GA_BF16 && heads == 1 && !fused && !ext.row_scale && Y) {
+    rc = wide_typed(type_pointer, n_types, X, &W, &Y, 1, rows, K, M, s);
+    if (rc != GA_EUNSUPPORTED) return rc;
+  }
   if (aligned(X, 16) && (!Y || aligned(Y, 16)) && (!ext.Q || aligned(ext.Q, 16))) {
     if (dtype == GA_F32 && K % 4 == 0)
       rc = launch_mfma<float, 16>(type_pointer, (int)n_types, X, W, Y, rows,
@@ -1115,6 +1147,33 @@ extern "C" int ga_project_attn(const void *X, const void *W, const float *a_l,
     return GA_EUNSUPPORTED;
   }
   if ((M & 1) || !aligned(Z, 4)) return GA_EUNSUPPORTED;      // packed bf16 pair stores
+  {
+    // whole groups of 128 columns holding whole heads: one pass over X for all of them
+    const int64_t dph = M / heads;
+    if (M % kWideGroupCols == 0 && (dph == 32 || dph == 64 || dph == 128) &&
+        wide_mm_fits((int)K, (int)(M / kWideGroupCols))) {
+      WideMm p = {};
+      p.n_types = 1;
+      p.rows = rows;
+      p.X = (const bf16_t *)X;
+      p.K = (int)K;
+      p.n_groups = (int)(M / kWideGroupCols);
+      p.ldd = heads;
+      p.dph = (int)dph;
+      for (int g = 0; g < p.n_groups; ++g) {
+        p.W[g] = (const bf16_t *)W + g * kWideGroupCols;
+        p.ldw[g] = M;
+        p.Y[g] = (bf16_t *)Z + g * kWideGroupCols;
+        p.ldy[g] = M;
+        p.a_l[g] = a_l + g * kWideGroupCols;
+        p.a_r[g] = a_r + g * kWideGroupCols;
+        p.el[g] = el + g * (kWideGroupCols / dph);
+        p.er[g] = er + g * (kWideGroupCols / dph);
+      }
+      const int rc = wide_mm_launch(p, s);
+      if (rc != GA_EUNSUPPORTED) return rc;
+    }
+  }
   if (aligned(X, 16) && K % 8 == 0)
     return launch_dense_attn<bf16_t, 32>((const bf16_t *)X, (const bf16_t *)W, (bf16_t *)Z,
                                          a_l, a_r, el, er, rows, (int)K, (int)M, (int)heads, s);
@@ -1138,6 +1197,36 @@ extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
   MmExt ext = {};
   return segment_mm_any(type_pointer, n_types, X, W, Y, rows, heads, K, M, dtype, ext,
                         (hipStream_t)stream);
+}
+
+extern "C" int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_types,
+                                     const void *X, const void *const *W, void *const *Y,
+                                     int64_t n_weights, int64_t rows, int64_t K, int64_t M,
+                                     int dtype, ga_stream_t stream) {
+  using namespace ga;
+  if (n_weights < 1 || n_weights > 4 || !W || !Y) return GA_EINVAL;
+  const int bad = check_mm_args(n_types, rows, 1, K, M, dtype);
+  if (bad != GA_OK) return bad;
+  if (rows == 0 || n_types == 0) return GA_OK;
+  if (!type_pointer || !X) return GA_EINVAL;
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!aligned(X, esz)) return GA_EALIGN;
+  for (int64_t i = 0; i < n_weights; ++i) {
+    if (!W[i] || !Y[i]) return GA_EINVAL;
+    if (!aligned(W[i], esz) || !aligned(Y[i], esz)) return GA_EALIGN;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == GA_BF16) {
+    const int rc = wide_typed(type_pointer, n_types, X, W, Y, (int)n_weights, rows, K, M, s);
+    if (rc != GA_EUNSUPPORTED) return rc;
+  }
+  // any other shape: one product per weight tensor
+  MmExt ext = {};
+  for (int64_t i = 0; i < n_weights; ++i) {
+    const int rc = segment_mm_any(type_pointer, n_types, X, W[i], Y[i], rows, 1, K, M, dtype, ext, s);
+    if (rc != GA_OK) return rc;
+  }
+  return GA_OK;
 }
 
 extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types,

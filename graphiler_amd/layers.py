@@ -120,7 +120,7 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
     """examples/HGT/HGT.py:28-60 as the operator sequence of its optimised plan,
     generalised from one head to ``heads`` heads of width D = hidden / heads:
 
-      K, V, Q   = SegmentMMNode(h, W_k | W_v | W_q)            per node type
+      K, V, Q   = SegmentMMNode(h, W_k | W_v | W_q)            per node type, h read once
       k_e, v_e  = BroadcastSrcNode(K | V);  q_e = BroadcastDstNode(Q)
       k_e, v_e  = SegmentMMEdge(k_e, relation_att | relation_msg)   per edge type,
                                                          one (D x D) block per head
@@ -139,9 +139,8 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
     n, hidden = h.shape
     d = hidden // heads
     e = g.num_edges
-    k = ops.SegmentMMNode(h, k_weight, g)
-    v = ops.SegmentMMNode(h, v_weight, g)
-    q = ops.SegmentMMNode(h, q_weight, g)
+    # the three projections of h in one pass over its rows
+    k, v, q = ops.SegmentMMNodeStacked(h, [k_weight, v_weight, q_weight], g)
     if fused:
         attn = ops.SegmentMMEdgeDot(k, relation_att, 0, q, 1, g,
                                     scale=relation_pri.float() / (d ** 0.5))

@@ -460,6 +460,40 @@ def SegmentMMNode(features, weights, graph: DGLGraph) -> torch.Tensor:
                        graph.num_ntypes, graph.num_nodes)
 
 
+def SegmentMMNodeStacked(features, weights: Sequence[torch.Tensor], graph: DGLGraph):
+    """``[SegmentMMNode(features, w, graph) for w in weights]`` (1 to 4 weight tensors
+    of one shape (T, K, M)) with the rows of ``features`` read once: the K, Q and V
+    projections of an HGT layer (examples/HGT/HGT.py:35-44).  Returns the list of
+    (N, M) results, the same values as separate calls."""
+    import ctypes
+    if not 1 <= len(weights) <= 4:
+        raise RuntimeError("one to four weight tensors")
+    _check_input(features, "features")
+    dt = _feat_dtype(features, "features")
+    if graph.ntype_pointer is None:
+        raise RuntimeError("the graph has no type pointer for this operator")
+    shape = tuple(weights[0].shape)
+    for w in weights:
+        _check_input(w, "weights")
+        if w.dtype != features.dtype or tuple(w.shape) != shape or w.dim() != 3:
+            raise RuntimeError("weights must be (T, K, M) tensors of one shape and the features' dtype")
+    K, M = int(shape[1]), int(shape[2])
+    if int(shape[0]) != graph.num_ntypes:
+        raise RuntimeError("weights must have one matrix per type")
+    rows = int(features.shape[0])
+    if rows != graph.num_nodes or get_feat_dim(features) != K:
+        raise RuntimeError("features must be (rows, K)")
+    outs = [torch.empty((rows, M), dtype=features.dtype, device=features.device)
+            for _ in weights]
+    n = len(weights)
+    wp = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
+    yp = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+    capi.check(capi.load().ga_segment_mm_stacked(
+        graph.ntype_pointer.data_ptr(), graph.num_ntypes, features.data_ptr(), wp, yp, n,
+        rows, K, M, dt, _stream(features)), "ga_segment_mm_stacked")
+    return outs
+
+
 def SegmentMMEdge(features, weights, graph: DGLGraph) -> torch.Tensor:
     """segment_mm.cu:29-33: per-edge-type linear, edges sorted by type."""
     return _segment_mm(features, weights, graph.etype_pointer,

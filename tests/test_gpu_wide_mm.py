@@ -1,0 +1,122 @@
+"""Wide bf16 typed products (csrc/wide_mm.hip): several weight tensors applied to the
+same rows in one pass (ga_segment_mm_stacked, the K | Q | V projections of
+examples/HGT/HGT.py:35-44) and the shapes of ga_segment_mm / ga_project_attn that the
+same kernel takes (whole groups of 128 output columns, K % 32 == 0, K <= 256).  Against
+the oracle's segment_mm and a float64 product; the stacked form must give the bits of
+separate calls."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from graphiler_amd import capi, datasets, ops
+from helpers import TOL_BF16, TOL_F32, assert_close, to_bf16_f32
+
+pytestmark = pytest.mark.gpu
+
+COUNTS = [700, 0, 1, 333, 0, 64, 15, 129, 3000, 0, 257]      # rows per type, some empty
+
+
+def _dev(a, device, bf16=False):
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    return t.bfloat16() if bf16 else t
+
+
+def _stacked(tp, X, Ws, M, dtype_code):
+    lib = capi.load()
+    rows, K = X.shape
+    outs = [torch.full((rows, M), float("nan"), dtype=X.dtype, device=X.device) for _ in Ws]
+    wp = (ctypes.c_void_p * len(Ws))(*[w.data_ptr() for w in Ws])
+    yp = (ctypes.c_void_p * len(Ws))(*[o.data_ptr() for o in outs])
+    rc = lib.ga_segment_mm_stacked(tp.data_ptr(), tp.numel() - 1, X.data_ptr(), wp, yp, len(Ws),
+                                   rows, K, M, dtype_code, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, rc
+    return outs
+
+
+@pytest.mark.parametrize("K,M,n_w", [(128, 128, 3), (128, 128, 1), (128, 128, 4), (64, 128, 2),
+                                     (32, 256, 2), (96, 128, 3), (160, 128, 2), (256, 128, 2),
+                                     (256, 256, 1), (128, 256, 2), (64, 384, 1)])
+def test_stacked_products_wide(device, K, M, n_w):
+    rng = np.random.default_rng(K + M + n_w)
+    tp = np.concatenate([[0], np.cumsum(COUNTS)]).astype(np.int32)
+    rows = int(tp[-1])
+    X = to_bf16_f32(rng.standard_normal((rows, K), dtype=np.float32))
+    Ws = [to_bf16_f32((rng.standard_normal((len(COUNTS), K, M)) / np.sqrt(K)).astype(np.float32))
+          for _ in range(n_w)]
+    dX, dtp = _dev(X, device, True), _dev(tp, device)
+    dWs = [_dev(w, device, True) for w in Ws]
+    outs = _stacked(dtp, dX, dWs, M, capi.GA_BF16)
+    lib = capi.load()
+    for w, dw, y in zip(Ws, dWs, outs):
+        ref = oracle.segment_mm(tp, X, w)
+        assert_close(y.float().cpu().numpy(), ref, TOL_BF16, f"stacked K={K} M={M} n={n_w}",
+                     mag=oracle.segment_mm(tp, np.abs(X), np.abs(w)))
+        one = torch.empty_like(y)
+        assert lib.ga_segment_mm(dtp.data_ptr(), len(COUNTS), dX.data_ptr(), dw.data_ptr(),
+                                 one.data_ptr(), rows, 1, K, M, capi.GA_BF16,
+                                 torch.cuda.current_stream().cuda_stream) == 0
+        assert torch.equal(one.view(torch.int16), y.view(torch.int16)), "stacked != separate calls"
+
+
+@pytest.mark.parametrize("K,M,bf16", [(20, 24, False), (128, 128, False), (100, 128, True),
+                                      (128, 64, True), (512, 128, True)])
+def test_stacked_products_other_shapes(device, K, M, bf16):
+    """Shapes outside the one-pass kernel run as one product per weight tensor."""
+    rng = np.random.default_rng(K * 7 + M)
+    counts = [70, 0, 333, 129]
+    tp = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(tp[-1])
+    X = rng.standard_normal((rows, K), dtype=np.float32)
+    Ws = [(rng.standard_normal((len(counts), K, M)) / np.sqrt(K)).astype(np.float32) for _ in range(2)]
+    if bf16:
+        X, Ws = to_bf16_f32(X), [to_bf16_f32(w) for w in Ws]
+    outs = _stacked(_dev(tp, device), _dev(X, device, bf16), [_dev(w, device, bf16) for w in Ws], M,
+                    capi.GA_BF16 if bf16 else capi.GA_F32)
+    for w, y in zip(Ws, outs):
+        assert_close(y.float().cpu().numpy(), oracle.segment_mm(tp, X, w),
+                     TOL_BF16 if bf16 else TOL_F32, f"stacked fallback K={K} M={M}")
+
+
+def test_stacked_operator_and_hgt_projections(device):
+    """ops.SegmentMMNodeStacked on a typed graph = three SegmentMMNode calls."""
+    from graphiler_amd import prepare_graph
+    rng = np.random.default_rng(8)
+    n, e, tn = 900, 4000, 4
+    ntype = np.sort(rng.integers(0, tn, n))
+    src, dst = rng.integers(0, n, e), rng.integers(0, n, e)
+    g = prepare_graph(src, dst, n, device=device, ntype_of=ntype, num_ntypes=tn)
+    h = _dev(to_bf16_f32(rng.standard_normal((n, 128), dtype=np.float32)), device, True)
+    ws = [_dev(to_bf16_f32(datasets.glorot(rng, (tn, 128, 128))), device, True) for _ in range(3)]
+    outs = ops.SegmentMMNodeStacked(h, ws, g)
+    for w, y in zip(ws, outs):
+        assert torch.equal(ops.SegmentMMNode(h, w, g).view(torch.int16), y.view(torch.int16))
+    with pytest.raises(RuntimeError):
+        ops.SegmentMMNodeStacked(h, [ws[0], ws[1][:, :, :64].contiguous()], g)
+    with pytest.raises(RuntimeError):
+        ops.SegmentMMNodeStacked(h, [], g)
+
+
+@pytest.mark.parametrize("rows,K,M,heads", [
+    (1500, 256, 256, 4), (1500, 256, 256, 2), (1500, 256, 256, 8),   # heads of 64, 128, 32 columns
+    (777, 128, 128, 1), (777, 128, 128, 4), (333, 64, 384, 3), (255, 32, 512, 8),
+    (1, 96, 128, 2), (4097, 160, 256, 4)])
+def test_project_attn_wide(device, rows, K, M, heads):
+    """The projection with attention terms at the widths of the one-pass kernel."""
+    rng = np.random.default_rng(rows + K + M + heads)
+    x = to_bf16_f32(rng.standard_normal((rows, K), dtype=np.float32))
+    w = to_bf16_f32(datasets.glorot(rng, (K, M)))
+    a = rng.standard_normal((2, heads, M // heads), dtype=np.float32)
+    z, el, er = ops.linear_attn(_dev(x, device, True), _dev(w, device, True),
+                                _dev(a[0], device), _dev(a[1], device))
+    assert z.dtype == torch.bfloat16 and el.dtype == torch.float32 and el.shape == (rows, heads)
+    zr = x.astype(np.float64) @ w.astype(np.float64)
+    assert_close(z.float().cpu().numpy(), zr, TOL_BF16, "wide project z")
+    zh = zr.reshape(rows, heads, -1)
+    mag_l = (np.abs(zh) * np.abs(a[0])).sum(-1)
+    mag_r = (np.abs(zh) * np.abs(a[1])).sum(-1)
+    # el / er come from the fp32 accumulators, not from the rounded z
+    assert_close(el.cpu().numpy(), (zh * a[0]).sum(-1), TOL_F32, "wide project el", mag=mag_l)
+    assert_close(er.cpu().numpy(), (zh * a[1]).sum(-1), TOL_F32, "wide project er", mag=mag_r)
