@@ -16,7 +16,7 @@ struct WideMm {
   int n_types;
   int64_t rows;
   const bf16_t *X;            // (rows, K), rows K elements apart
-  int K;                      // multiple of 32, at most 256
+  int K;                      // multiple of 8 up to 256, or of 4 up to 128 (two groups at most)
   int n_groups;
   const bf16_t *W[kWideMaxGroups];      // first column of the group in W[type 0]
   int64_t w_type_stride[kWideMaxGroups];

@@ -111,7 +111,7 @@ __device__ __forceinline__ void wide_stage(const bf16_t *__restrict__ w, int64_t
   }
 }
 
-template <int NF, int NG, bool ATTN, int TW>
+template <int NF, int NG, bool ATTN, int TW, bool X8>
 __global__ __launch_bounds__(kWideBlock) void wide_mm_kernel(WideMm p, int chunk_rows) {
   constexpr int kWaveRows = 16 * TW;                       // rows of a wavefront per step
   constexpr int kStepRows = (kWideBlock / kWave) * kWaveRows;
@@ -124,11 +124,13 @@ __global__ __launch_bounds__(kWideBlock) void wide_mm_kernel(WideMm p, int chunk
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int n = lane & 15, q = lane >> 4;
 
-  // k fragments of this lane that lie inside a row
+  // halves (4 elements) of this lane's k fragments that lie inside a row: bits 2 f, 2 f + 1
   unsigned kmask = 0;
 #pragma unroll
-  for (int f = 0; f < NF; ++f)
-    if (f * 32 + q * 8 < p.K) kmask |= 1u << f;
+  for (int f = 0; f < NF; ++f) {
+    if (f * 32 + q * 8 < p.K) kmask |= 1u << (2 * f);
+    if (f * 32 + q * 8 + 4 < p.K) kmask |= 2u << (2 * f);
+  }
   // Addresses inside the chunk are "uniform base + 32-bit lane offset" (the host keeps a
   // chunk below 4 GiB of X and of every Y): no 64-bit arithmetic per access.
   const char *xbase = reinterpret_cast<const char *>(p.X + (int64_t)row0 * p.K);
@@ -140,9 +142,18 @@ __global__ __launch_bounds__(kWideBlock) void wide_mm_kernel(WideMm p, int chunk
       const int r = rel + 16 * t + n;
       const uint32_t off = (uint32_t)(r < nrows ? r : nrows - 1) * xrow + (uint32_t)q * 16u;
 #pragma unroll
-      for (int f = 0; f < NF; ++f)
-        x[t][f] = (kmask >> f & 1) ? *reinterpret_cast<const uint4 *>(xbase + off + f * 64)
-                                   : make_uint4(0, 0, 0, 0);
+      for (int f = 0; f < NF; ++f) {
+        if (X8) {       // rows 8-byte aligned only (K % 8 == 4): two loads per fragment
+          const uint2 lo = (kmask >> (2 * f) & 1) ? *reinterpret_cast<const uint2 *>(xbase + off + f * 64)
+                                                  : make_uint2(0, 0);
+          const uint2 hi = (kmask >> (2 * f) & 2) ? *reinterpret_cast<const uint2 *>(xbase + off + f * 64 + 8)
+                                                  : make_uint2(0, 0);
+          x[t][f] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        } else {
+          x[t][f] = (kmask >> (2 * f) & 1) ? *reinterpret_cast<const uint4 *>(xbase + off + f * 64)
+                                           : make_uint4(0, 0, 0, 0);
+        }
+      }
     }
   };
   // the rows of the first step are on their way while the weights are staged
@@ -262,15 +273,15 @@ int wide_cu_count() {
   return cus;
 }
 
-template <int NF, int NG, bool ATTN>
-int wide_launch_as(const WideMm &p, hipStream_t s) {
+template <int NF, int NG, bool ATTN, bool X8>
+int wide_launch_x(const WideMm &p, hipStream_t s) {
   const size_t lds = (size_t)NG * wide_group_elems(NF) * sizeof(bf16_t);
   if (lds > (size_t)kWideMaxLds) return GA_EUNSUPPORTED;
   // two row tiles per wavefront where the registers allow it: every weight fragment read
   // from LDS then feeds two matrix instructions
   constexpr int TW = NF <= 4 ? 2 : 1;
   constexpr int kStepRows = (kWideBlock / kWave) * 16 * TW;
-  const void *kernel = (const void *)wide_mm_kernel<NF, NG, ATTN, TW>;
+  const void *kernel = (const void *)wide_mm_kernel<NF, NG, ATTN, TW, X8>;
   if (lds > 64 * 1024) {
     static bool granted = false;       // per instantiation
     if (!granted) {
@@ -294,9 +305,19 @@ int wide_launch_as(const WideMm &p, hipStream_t s) {
   for (int g = 0; g < p.n_groups; ++g) widest = p.ldy[g] > widest ? p.ldy[g] : widest;
   if (chunk * widest * 2 > 0xffffffffll) return GA_EUNSUPPORTED;    // 32-bit offsets in a chunk
   const int64_t grid = (p.rows + chunk - 1) / chunk + (p.tp ? p.n_types : 0);
-  hipLaunchKernelGGL((wide_mm_kernel<NF, NG, ATTN, TW>), dim3((unsigned)grid), dim3(kWideBlock), lds, s, p,
+  hipLaunchKernelGGL((wide_mm_kernel<NF, NG, ATTN, TW, X8>), dim3((unsigned)grid), dim3(kWideBlock), lds, s, p,
                      (int)chunk);
   return launch_status();
+}
+
+template <int NF, int NG, bool ATTN>
+int wide_launch_as(const WideMm &p, hipStream_t s) {
+  // the 8-byte form only where its shapes occur: K <= 128, at most two groups
+  if constexpr (NF <= 4 && NG <= 2) {
+    if (p.K % 8 != 0) return wide_launch_x<NF, NG, ATTN, true>(p, s);
+  }
+  if (p.K % 8 != 0) return GA_EUNSUPPORTED;
+  return wide_launch_x<NF, NG, ATTN, false>(p, s);
 }
 
 template <int NF, bool ATTN>
@@ -313,7 +334,8 @@ int wide_launch_groups(const WideMm &p, hipStream_t s) {
 }  // namespace
 
 bool wide_mm_fits(int K, int n_groups) {
-  if (K <= 0 || K % 32 != 0 || K > 256 || n_groups < 1 || n_groups > kWideMaxGroups) return false;
+  if (K <= 0 || K % 4 != 0 || K > 256 || n_groups < 1 || n_groups > kWideMaxGroups) return false;
+  if (K % 8 != 0 && (K > 128 || n_groups > 2)) return false;     // 8-byte row loads: see wide_launch_as
   const int nf = K <= 64 ? 2 : (K <= 128 ? 4 : 8);
   return (size_t)n_groups * wide_group_elems(nf) * sizeof(bf16_t) <= (size_t)kWideMaxLds;
 }
@@ -321,7 +343,7 @@ bool wide_mm_fits(int K, int n_groups) {
 int wide_mm_launch(const WideMm &p, hipStream_t s) {
   if (!wide_mm_fits(p.K, p.n_groups)) return GA_EUNSUPPORTED;
   if (p.rows <= 0) return GA_OK;
-  if (p.rows > 0x7fffffff || !aligned(p.X, 16)) return GA_EUNSUPPORTED;
+  if (p.rows > 0x7fffffff || !aligned(p.X, p.K % 8 == 0 ? 16 : 8)) return GA_EUNSUPPORTED;
   const bool attn = p.a_l[0] != nullptr;
   if (attn && p.dph != 32 && p.dph != 64 && p.dph != 128) return GA_EUNSUPPORTED;
   for (int g = 0; g < p.n_groups; ++g) {

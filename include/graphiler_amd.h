@@ -287,9 +287,10 @@ int ga_segment_mm(const int32_t *type_pointer, int64_t n_types, const void *X,
  * i < n_weights (1 .. 4), every W[i] (n_types, K, M) and Y[i] (rows, M); W and Y are
  * host arrays of device pointers.  The K | Q | V projections of an HGT layer
  * (examples/HGT/HGT.py:35-44, three calls of segment_mm.cu:29-33 on one input) read X
- * once this way.  bf16 with K % 32 == 0, K <= 256, M % 128 == 0 and n_weights * M / 128
- * groups within the LDS of a CU runs as one launch; every other shape ga_segment_mm
- * takes runs as n_weights launches with the same results. */
+ * once this way.  bf16 with K % 8 == 0, K <= 256 (or K % 4 == 0, K <= 128, two groups
+ * at most), M % 128 == 0 and n_weights * M / 128 groups of 128 columns within the LDS
+ * of a CU runs as one launch; every other shape ga_segment_mm takes runs as n_weights
+ * launches with the same results. */
 int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_types, const void *X,
                           const void *const *W, void *const *Y, int64_t n_weights,
                           int64_t rows, int64_t K, int64_t M, int dtype, ga_stream_t stream);

@@ -1,7 +1,8 @@
 """Wide bf16 typed products (csrc/wide_mm.hip): several weight tensors applied to the
 same rows in one pass (ga_segment_mm_stacked, the K | Q | V projections of
 examples/HGT/HGT.py:35-44) and the shapes of ga_segment_mm / ga_project_attn that the
-same kernel takes (whole groups of 128 output columns, K % 32 == 0, K <= 256).  Against
+same kernel takes (whole groups of 128 output columns; K % 8 == 0 up to 256, K % 4 == 0
+up to 128).  Against
 the oracle's segment_mm and a float64 product; the stacked form must give the bits of
 separate calls."""
 import ctypes
@@ -38,7 +39,10 @@ def _stacked(tp, X, Ws, M, dtype_code):
 
 @pytest.mark.parametrize("K,M,n_w", [(128, 128, 3), (128, 128, 1), (128, 128, 4), (64, 128, 2),
                                      (32, 256, 2), (96, 128, 3), (160, 128, 2), (256, 128, 2),
-                                     (256, 256, 1), (128, 256, 2), (64, 384, 1)])
+                                     (256, 256, 1), (128, 256, 2), (64, 384, 1),
+                                     # K % 32 != 0: padded fragments; K % 8 == 4: 8-byte row loads
+                                     (40, 128, 3), (200, 128, 2), (100, 128, 2), (100, 256, 1),
+                                     (36, 128, 1), (124, 256, 1)])
 def test_stacked_products_wide(device, K, M, n_w):
     rng = np.random.default_rng(K + M + n_w)
     tp = np.concatenate([[0], np.cumsum(COUNTS)]).astype(np.int32)
@@ -61,7 +65,7 @@ def test_stacked_products_wide(device, K, M, n_w):
         assert torch.equal(one.view(torch.int16), y.view(torch.int16)), "stacked != separate calls"
 
 
-@pytest.mark.parametrize("K,M,bf16", [(20, 24, False), (128, 128, False), (100, 128, True),
+@pytest.mark.parametrize("K,M,bf16", [(20, 24, False), (128, 128, False), (102, 128, True),
                                       (128, 64, True), (512, 128, True)])
 def test_stacked_products_other_shapes(device, K, M, bf16):
     """Shapes outside the one-pass kernel run as one product per weight tensor."""
@@ -102,7 +106,8 @@ def test_stacked_operator_and_hgt_projections(device):
 @pytest.mark.parametrize("rows,K,M,heads", [
     (1500, 256, 256, 4), (1500, 256, 256, 2), (1500, 256, 256, 8),   # heads of 64, 128, 32 columns
     (777, 128, 128, 1), (777, 128, 128, 4), (333, 64, 384, 3), (255, 32, 512, 8),
-    (1, 96, 128, 2), (4097, 160, 256, 4)])
+    (1, 96, 128, 2), (4097, 160, 256, 4),
+    (3001, 100, 256, 4), (515, 36, 128, 2), (90, 248, 256, 4), (777, 124, 128, 4)])
 def test_project_attn_wide(device, rows, K, M, heads):
     """The projection with attention terms at the widths of the one-pass kernel."""
     rng = np.random.default_rng(rows + K + M + heads)
