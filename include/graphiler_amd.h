@@ -261,8 +261,9 @@ int ga_sddmm_u_dot_v(const void *lhs, const void *rhs, int idx_bits,
  * changes results once every logit of a segment is below about -87).
  * y entries of edges that belong to no row are left untouched: pass y zeroed
  * to match the reference's zeros_like output when eid is not a permutation.
- * workspace: ga_softmax_workspace_bytes() bytes (per-chunk statistics of
- * segments longer than 1024 values; 0 for small graphs), 16-byte aligned.
+ * y may be x itself (in place); any other overlap of the two is GA_EINVAL.
+ * workspace: ga_softmax_workspace_bytes() bytes (partial maxima / sums and
+ * descriptors of the rows that leave a tile of 8192 values), 16-byte aligned.
  */
 size_t ga_softmax_workspace_bytes(int64_t n_edges, int64_t heads);
 int ga_segment_softmax(const int32_t *pointer, const int32_t *row_of_slot,
