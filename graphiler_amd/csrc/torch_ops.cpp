@@ -152,6 +152,41 @@ struct DGLGraph : torch::CustomClassHolder {
     }
     return s;
   }
+  // The (destination tile, relation) order of the in-edges that the one-pass typed
+  // neighbour sum walks (ga_typed_tiles_build): built on first use, kept with the graph.
+  struct TypedTiles {
+    torch::Tensor tile_chunk_pointer, chunk_type, slot_src, slot_dst, slot_edge;
+    bool ready = false;
+  };
+  const TypedTiles &typed_tiles() {
+    const Side &in = side(false);
+    std::lock_guard<std::mutex> lock(mu_);
+    if (!tiles_.ready) {
+      TORCH_CHECK(etype_pointer.has_value(), "the graph has no edge type pointer");
+      const int64_t cap = ga_typed_tiles_chunk_capacity(num_nodes, num_edges, num_etypes);
+      const int64_t tiles = (num_nodes + GA_TYPED_TILE_ROWS - 1) / GA_TYPED_TILE_ROWS;
+      const auto i32 = in_pointer.options();
+      tiles_.tile_chunk_pointer = torch::empty({tiles + 1}, i32);
+      tiles_.chunk_type = torch::empty({std::max<int64_t>(cap, 1)}, i32);
+      tiles_.slot_src = torch::empty({std::max<int64_t>(16 * cap, 1)}, i32);
+      tiles_.slot_dst = torch::empty({std::max<int64_t>(16 * cap, 4)}, i32.dtype(at::kByte));
+      tiles_.slot_edge = torch::empty({std::max<int64_t>(16 * cap, 4)}, i32);
+      const size_t bytes = ga_typed_tiles_workspace_bytes(num_nodes, num_edges, num_etypes);
+      TORCH_CHECK(bytes > 0, "graph too large for the typed tile layout");
+      torch::Tensor ws = torch::empty({(int64_t)bytes}, i32.dtype(at::kByte));
+      check_ga(ga_typed_tiles_build(
+                   in.rows.data_ptr<int>(), in_node_indices.data_ptr<int>(),
+                   in.identity ? nullptr : in_edge_indices.data_ptr<int>(),
+                   etype_pointer.value().data_ptr<int>(), num_nodes, num_edges, num_etypes,
+                   tiles_.tile_chunk_pointer.data_ptr<int>(), tiles_.chunk_type.data_ptr<int>(),
+                   tiles_.slot_src.data_ptr<int>(), tiles_.slot_dst.data_ptr<uint8_t>(),
+                   tiles_.slot_edge.data_ptr<int>(), ws.data_ptr(), bytes,
+                   current_stream(in_pointer)),
+               "ga_typed_tiles_build");
+      tiles_.ready = true;
+    }
+    return tiles_;
+  }
   // Scratch shared by the operators called on this graph: calls that use it must be
   // ordered on one stream (two streams working on one graph object race on it).  It
   // grows on demand; a buffer that was handed out is never freed while the graph
@@ -169,6 +204,7 @@ struct DGLGraph : torch::CustomClassHolder {
  private:
   std::mutex mu_;
   Side in_side_, out_side_;
+  TypedTiles tiles_;
   torch::Tensor ws_;
   std::vector<torch::Tensor> retired_ws_;
 };
@@ -399,6 +435,40 @@ torch::Tensor SegmentMMEdge(torch::Tensor features, torch::Tensor weights,
                     graph->num_edges);
 }
 
+// [SegmentMMNode(features, w, graph) for w in weights] with the rows of `features` read
+// once when the weights have one shape (HGT's K, Q, V: examples/HGT/HGT.py:35-44)
+std::vector<torch::Tensor> SegmentMMNodeStacked(torch::Tensor features,
+                                                std::vector<torch::Tensor> weights,
+                                                const GraphPtr &graph) {
+  bool same = !weights.empty() && weights.size() <= 4;
+  for (const torch::Tensor &w : weights)
+    same = same && w.dim() == 3 && w.sizes() == weights[0].sizes() && w.is_cuda() &&
+           w.is_contiguous() && w.scalar_type() == features.scalar_type();
+  std::vector<torch::Tensor> outs;
+  if (!same) {
+    for (const torch::Tensor &w : weights) outs.push_back(SegmentMMNode(features, w, graph));
+    return outs;
+  }
+  check_input(features, "features");
+  const int dt = feat_dtype(features, "features");
+  TORCH_CHECK(graph->ntype_pointer.has_value(), "the graph has no type pointer for this operator");
+  const int64_t K = weights[0].size(1), M = weights[0].size(2), rows = features.size(0);
+  TORCH_CHECK(weights[0].size(0) == graph->num_ntypes, "weights must have one matrix per type");
+  TORCH_CHECK(rows == graph->num_nodes && feat_dim(features) == K, "features must be (rows, K)");
+  std::vector<const void *> wp;
+  std::vector<void *> yp;
+  for (const torch::Tensor &w : weights) {
+    outs.push_back(torch::empty({rows, M}, features.options()));
+    wp.push_back(w.data_ptr());
+    yp.push_back(outs.back().data_ptr());
+  }
+  check_ga(ga_segment_mm_stacked(graph->ntype_pointer.value().data_ptr<int>(), graph->num_ntypes,
+                                 features.data_ptr(), wp.data(), yp.data(), (int64_t)wp.size(),
+                                 rows, K, M, dt, current_stream(features)),
+           "ga_segment_mm_stacked");
+  return outs;
+}
+
 torch::Tensor gather(const torch::Tensor &features, const torch::Tensor &index);
 
 struct MmShape { int64_t heads, K, M; int dt; };
@@ -460,6 +530,42 @@ torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
     check_ga(rc, "ga_segment_mm_gather");
   }
   return late.defined() ? out * late : out;
+}
+
+// SpMMEdge(SegmentMMEdgeGather(features, weights, 0, row_scale)): an RGCN layer's message
+// and reduce steps (examples/RGCN/RGCN.py:25-33).  One pass without the per-edge
+// messages where that kernel is the faster one (fp32, 16 -> 64), the two operators
+// elsewhere.
+torch::Tensor TypedSpMMEdge(torch::Tensor features, torch::Tensor weights,
+                            at::optional<torch::Tensor> row_scale, const GraphPtr &graph) {
+  const MmShape s = edge_mm_shape(features, weights, graph);
+  const float *rs = nullptr;
+  bool plain_scale = !row_scale.has_value();
+  if (row_scale.has_value()) {
+    const torch::Tensor &r = row_scale.value();
+    if (r.is_cuda() && r.is_contiguous() && r.scalar_type() == at::kFloat &&
+        r.numel() == graph->num_edges && r.dim() <= 2 && r.size(0) == graph->num_edges) {
+      rs = r.data_ptr<float>();
+      plain_scale = true;
+    }
+  }
+  if (plain_scale && weights.dim() == 3 && features.dim() == 2 && s.dt == GA_F32 && s.K == 16 &&
+      s.M == 64) {
+    const DGLGraph::TypedTiles &t = graph->typed_tiles();
+    torch::Tensor out = torch::empty({graph->num_nodes, s.M}, features.options());
+    const int rc = ga_typed_spmm(
+        t.tile_chunk_pointer.data_ptr<int>(), t.chunk_type.data_ptr<int>(),
+        t.slot_src.data_ptr<int>(), t.slot_dst.data_ptr<uint8_t>(), t.slot_edge.data_ptr<int>(),
+        features.data_ptr(), weights.data_ptr(), rs, out.data_ptr(), graph->num_nodes,
+        features.size(0), graph->num_edges, graph->num_etypes, s.K, s.M, s.dt,
+        current_stream(out));
+    if (rc != GA_EUNSUPPORTED) {
+      check_ga(rc, "ga_typed_spmm");
+      return out;
+    }
+  }
+  return spmm(graph, GA_COPY_E, GA_SUM, SegmentMMEdgeGather(features, weights, 0, row_scale, graph),
+              at::nullopt, false);
 }
 
 // out[e, h] = <features[endpoint(e)] @ weights[type(e)], other[other_endpoint(e)]>
@@ -793,6 +899,11 @@ static auto registry =
         .op("my_ops::SegmentMMEdgeGather(Tensor x, Tensor w, int endpoint, Tensor? row_scale, "
             GRAPH_T " g) -> Tensor z",
             &SegmentMMEdgeGather)
+        .op("my_ops::TypedSpMMEdge(Tensor x, Tensor w, Tensor? row_scale, " GRAPH_T
+            " g) -> Tensor z",
+            &TypedSpMMEdge)
+        .op("my_ops::SegmentMMNodeStacked(Tensor x, Tensor[] ws, " GRAPH_T " g) -> Tensor[] zs",
+            &SegmentMMNodeStacked)
         .op("my_ops::SegmentMMEdgeDot(Tensor x, Tensor w, int endpoint, Tensor q, "
             "int q_endpoint, Tensor? scale, " GRAPH_T " g) -> Tensor z",
             &SegmentMMEdgeDot)

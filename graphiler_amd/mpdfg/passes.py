@@ -501,6 +501,10 @@ class _Rewriter:
         for n in list(self.G.nodes()):
             if n.kind() == "my_ops::gspmm_e_mul_e_sum":
                 changed |= self._fuse_row_scale(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::SpMMEdge":
+                changed |= self._fuse_typed_spmm(n)
+        changed |= self._fuse_stacked_mm()
         return changed
 
     def _fuse_gather_mm(self, n) -> bool:
@@ -632,6 +636,62 @@ class _Rewriter:
         n.output().replaceAllUsesWith(out)
         n.destroy()
         return True
+
+
+    def _fuse_typed_spmm(self, n) -> bool:
+        """SpMMEdge(SegmentMMEdgeGather(x, w, 0, s)) -> TypedSpMMEdge(x, w, s): the
+        message and reduce steps of an RGCN layer as one operator, which runs them
+        in one pass over destination tiles where that is the faster kernel."""
+        mm = n.inputsAt(0).node()
+        if mm.kind() != "my_ops::SegmentMMEdgeGather" or not self.single_use(n.inputsAt(0)):
+            return False
+        if self.const_of(mm.inputsAt(2)) != 0:
+            return False
+        out = self.make("my_ops::TypedSpMMEdge",
+                        [mm.inputsAt(0), mm.inputsAt(1), mm.inputsAt(3), self.dglgraph], n, NODE)
+        n.output().replaceAllUsesWith(out)
+        n.destroy()
+        mm.destroy()
+        return True
+
+    def _fuse_stacked_mm(self) -> bool:
+        """Two to four SegmentMMNode(x, w_i) of one x -> SegmentMMNodeStacked(x, [w_i]):
+        the rows of x are read once (HGT's K, Q, V projections).  The stacked node
+        takes the place of the last product of the group (every weight is defined
+        by then), so a product joins only while nothing reads an earlier result
+        before that place."""
+        groups = {}
+        for n in self.G.nodes():
+            if n.kind() == "my_ops::SegmentMMNode":
+                groups.setdefault(n.inputsAt(0).unique(), []).append(n)
+        changed = False
+        for nodes in groups.values():
+            nodes = nodes[:4]
+            while len(nodes) >= 2:
+                last = nodes[-1]
+                if all(u.user.isAfter(last) for n in nodes[:-1] for u in n.output().uses()):
+                    break
+                nodes = nodes[:-1]
+            if len(nodes) < 2:
+                continue
+            last = nodes[-1]
+            tensor = torch._C.TensorType.get()
+            lst = self.G.create("prim::ListConstruct", [n.inputsAt(1) for n in nodes], 1)
+            lst.insertBefore(last)
+            lst.output().setType(torch._C.ListType(tensor))
+            st = self.G.create("my_ops::SegmentMMNodeStacked",
+                               [last.inputsAt(0), lst.output(), self.dglgraph], 1)
+            st.insertBefore(last)
+            st.output().setType(torch._C.ListType(tensor))
+            un = self.G.create("prim::ListUnpack", [st.output()], len(nodes))
+            un.insertBefore(last)
+            for n, o in zip(nodes, un.outputs()):
+                o.setType(n.output().type())
+                self.res[o.unique()] = NODE
+                n.output().replaceAllUsesWith(o)
+                n.destroy()
+            changed = True
+        return changed
 
 
 def split(plan: MPDFG) -> None:

@@ -130,3 +130,42 @@ def test_error_convention(setup, device):
         torch.ops.my_ops.SpMMSrc(xt, [1], False, None, sg)
     with pytest.raises(RuntimeError, match="node-type"):
         torch.ops.my_ops.BroadcastNodeType(torch.ones(2, 2, device=device), sg)
+
+
+def test_typed_sum_and_stacked_products_through_torchscript(device):
+    """my_ops::TypedSpMMEdge (= SpMMEdge(SegmentMMEdgeGather(x, w, 0, s))) and
+    my_ops::SegmentMMNodeStacked (= one SegmentMMNode per weight) against the python
+    operators, at a shape that takes the one-pass kernels and at ones that do not."""
+    from graphiler_amd import ops as pyops
+    from graphiler_amd.graph import sort_edges_by_type
+    torch_boundary.load()
+    rng = np.random.default_rng(33)
+    n, e, r, tn = 600, 7000, 5, 3
+    src, dst = rng.integers(0, n, e), rng.integers(0, n, e)
+    et = rng.integers(0, r, e)
+    src, dst, et, _ = sort_edges_by_type(src, dst, et)
+    nt = np.sort(rng.integers(0, tn, n))
+    g = prepare_graph(src, dst, n, device=device, ntype_of=nt, num_ntypes=tn, etype_of=et,
+                      num_etypes=r)
+    sg = torch_boundary.script_graph(g)
+    ops = torch.ops.my_ops
+    norm = _t(rng.uniform(0.1, 1.0, (e, 1)).astype(np.float32), device)
+    for k, m in ((16, 64), (32, 64), (16, 24)):
+        x = _t(rng.standard_normal((n, k), dtype=np.float32), device)
+        w = _t((rng.standard_normal((r, k, m)) / np.sqrt(k)).astype(np.float32), device)
+        want = pyops.SpMMEdge(pyops.SegmentMMEdgeGather(x, w, 0, g, row_scale=norm), [1], False, None, g)
+        got = ops.TypedSpMMEdge(x, w, norm, sg)
+        assert_close(got.cpu().numpy(), want.cpu().numpy(), 2 * TOL_F32, f"TypedSpMMEdge {k}->{m}")
+        got = ops.TypedSpMMEdge(x, w, None, sg)
+        want = pyops.SpMMEdge(pyops.SegmentMMEdgeGather(x, w, 0, g), [1], False, None, g)
+        assert_close(got.cpu().numpy(), want.cpu().numpy(), 2 * TOL_F32, f"TypedSpMMEdge {k}->{m} plain")
+    h = _t(rng.standard_normal((n, 128), dtype=np.float32), device).bfloat16()
+    ws = [_t(datasets.glorot(rng, (tn, 128, 128)), device).bfloat16() for _ in range(3)]
+    outs = ops.SegmentMMNodeStacked(h, ws, sg)
+    assert len(outs) == 3
+    for w, y in zip(ws, outs):
+        assert torch.equal(y.view(torch.int16), ops.SegmentMMNode(h, w, sg).view(torch.int16))
+    mixed = [ws[0], ws[1][:, :, :64].contiguous()]          # different shapes: one product each
+    outs = ops.SegmentMMNodeStacked(h, mixed, sg)
+    assert outs[1].shape == (n, 64)
+    assert torch.equal(outs[1].view(torch.int16), ops.SegmentMMNode(h, mixed[1], sg).view(torch.int16))

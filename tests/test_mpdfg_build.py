@@ -65,13 +65,15 @@ def test_level2_fuses_into_graph_operators():
     assert "aten::mm" not in k
     _, k = _kinds("rgcn", 2)
     ours = [x for x in k if x.startswith("my_ops::")]
-    # the source rows are read through the COO column by the typed product, which
-    # also applies the norm to the rows it writes: no per-edge copy, no product tensor
-    assert ours == ["my_ops::SegmentMMEdgeGather", "my_ops::SpMMEdge"]
+    # message and reduce as one operator: the source rows are read through the graph,
+    # the norm is applied to the messages, and (where that kernel is the faster one) no
+    # per-edge tensor is written at all
+    assert ours == ["my_ops::TypedSpMMEdge"]
     assert "aten::bmm" not in k and "aten::mul" not in k
     _, k = _kinds("hgt", 2)
     ours = [x for x in k if x.startswith("my_ops::")]
-    assert ours.count("my_ops::SegmentMMNode") == 4
+    # K, V, Q read the node rows once; the output projection stays on its own
+    assert ours.count("my_ops::SegmentMMNodeStacked") == 1 and ours.count("my_ops::SegmentMMNode") == 1
     assert "my_ops::SegmentMMEdgeDot" in ours            # sum(bmm(k, W_att) * q) in one pass
     assert "my_ops::SegmentMMEdgeGather" in ours and "my_ops::edge_softmax_sum" in ours
     assert "my_ops::SegmentSoftmax" not in ours and "my_ops::gspmm_e_mul_e_sum" not in ours
