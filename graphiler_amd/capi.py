@@ -16,7 +16,6 @@ LIB_PATH = os.path.join(_HERE, "lib", "libgraphiler_hip.so")
 GA_OK = 0
 GA_EINVAL, GA_EUNSUPPORTED, GA_EWORKSPACE, GA_EALIGN, GA_ESCRATCH = -1, -2, -3, -4, -5
 GA_STATIC_SCRATCH_BYTES = 32 << 20
-GA_TYPED_TILE_ROWS = 128
 GA_F32, GA_BF16 = 0, 1
 GA_COPY_U, GA_COPY_E, GA_U_MUL_E, GA_U_ADD_E, GA_U_SUB_E, GA_U_DIV_E = 0, 1, 2, 3, 4, 5
 GA_SDDMM_ADD, GA_SDDMM_SUB, GA_SDDMM_MUL, GA_SDDMM_DIV = 0, 1, 2, 3
@@ -48,12 +47,13 @@ SIGNATURES = {
     "ga_sddmm_bcast": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp, _vp, _i64, _i64,
                               _i64, _i64, _int, _vp]),
     "ga_sddmm_u_op_v_adj": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
-    "ga_typed_tiles_chunk_capacity": (_i64, [_i64, _i64, _i64]),
-    "ga_typed_tiles_workspace_bytes": (_sz, [_i64, _i64, _i64]),
-    "ga_typed_tiles_build": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp,
-                                    _vp, _vp, _sz, _vp]),
+    "ga_typed_tile_rows": (_i64, [_i64]),
+    "ga_typed_tiles_chunk_capacity": (_i64, [_i64, _i64, _i64, _i64]),
+    "ga_typed_tiles_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
+    "ga_typed_tiles_build": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp,
+                                    _vp, _vp, _vp, _sz, _vp]),
     "ga_typed_spmm": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
-                             _i64, _i64, _i64, _int, _vp]),
+                             _i64, _i64, _i64, _i64, _int, _vp]),
     "ga_sddmm_u_dot_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64,
                                 _int, _vp]),
     "ga_softmax_workspace_bytes": (_sz, [_i64, _i64]),

@@ -156,6 +156,7 @@ struct DGLGraph : torch::CustomClassHolder {
   // neighbour sum walks (ga_typed_tiles_build): built on first use, kept with the graph.
   struct TypedTiles {
     torch::Tensor tile_chunk_pointer, chunk_type, slot_src, slot_dst, slot_edge;
+    int64_t tile_rows = 128;
     bool ready = false;
   };
   const TypedTiles &typed_tiles() {
@@ -163,21 +164,23 @@ struct DGLGraph : torch::CustomClassHolder {
     std::lock_guard<std::mutex> lock(mu_);
     if (!tiles_.ready) {
       TORCH_CHECK(etype_pointer.has_value(), "the graph has no edge type pointer");
-      const int64_t cap = ga_typed_tiles_chunk_capacity(num_nodes, num_edges, num_etypes);
-      const int64_t tiles = (num_nodes + GA_TYPED_TILE_ROWS - 1) / GA_TYPED_TILE_ROWS;
+      const int64_t rows = ga_typed_tile_rows(num_nodes);
+      const int64_t cap = ga_typed_tiles_chunk_capacity(num_nodes, num_edges, num_etypes, rows);
+      const int64_t tiles = (num_nodes + rows - 1) / rows;
+      tiles_.tile_rows = rows;
       const auto i32 = in_pointer.options();
       tiles_.tile_chunk_pointer = torch::empty({tiles + 1}, i32);
       tiles_.chunk_type = torch::empty({std::max<int64_t>(cap, 1)}, i32);
       tiles_.slot_src = torch::empty({std::max<int64_t>(16 * cap, 1)}, i32);
       tiles_.slot_dst = torch::empty({std::max<int64_t>(16 * cap, 4)}, i32.dtype(at::kByte));
       tiles_.slot_edge = torch::empty({std::max<int64_t>(16 * cap, 4)}, i32);
-      const size_t bytes = ga_typed_tiles_workspace_bytes(num_nodes, num_edges, num_etypes);
+      const size_t bytes = ga_typed_tiles_workspace_bytes(num_nodes, num_edges, num_etypes, rows);
       TORCH_CHECK(bytes > 0, "graph too large for the typed tile layout");
       torch::Tensor ws = torch::empty({(int64_t)bytes}, i32.dtype(at::kByte));
       check_ga(ga_typed_tiles_build(
                    in.rows.data_ptr<int>(), in_node_indices.data_ptr<int>(),
                    in.identity ? nullptr : in_edge_indices.data_ptr<int>(),
-                   etype_pointer.value().data_ptr<int>(), num_nodes, num_edges, num_etypes,
+                   etype_pointer.value().data_ptr<int>(), num_nodes, num_edges, num_etypes, rows,
                    tiles_.tile_chunk_pointer.data_ptr<int>(), tiles_.chunk_type.data_ptr<int>(),
                    tiles_.slot_src.data_ptr<int>(), tiles_.slot_dst.data_ptr<uint8_t>(),
                    tiles_.slot_edge.data_ptr<int>(), ws.data_ptr(), bytes,
@@ -534,8 +537,7 @@ torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
 
 // SpMMEdge(SegmentMMEdgeGather(features, weights, 0, row_scale)): an RGCN layer's message
 // and reduce steps (examples/RGCN/RGCN.py:25-33).  One pass without the per-edge
-// messages where that kernel is the faster one (fp32, 16 -> 64), the two operators
-// elsewhere.
+// messages where that kernel is the faster one (16 -> 64), the two operators elsewhere.
 torch::Tensor TypedSpMMEdge(torch::Tensor features, torch::Tensor weights,
                             at::optional<torch::Tensor> row_scale, const GraphPtr &graph) {
   const MmShape s = edge_mm_shape(features, weights, graph);
@@ -549,15 +551,14 @@ torch::Tensor TypedSpMMEdge(torch::Tensor features, torch::Tensor weights,
       plain_scale = true;
     }
   }
-  if (plain_scale && weights.dim() == 3 && features.dim() == 2 && s.dt == GA_F32 && s.K == 16 &&
-      s.M == 64) {
+  if (plain_scale && weights.dim() == 3 && features.dim() == 2 && s.K == 16 && s.M == 64) {
     const DGLGraph::TypedTiles &t = graph->typed_tiles();
     torch::Tensor out = torch::empty({graph->num_nodes, s.M}, features.options());
     const int rc = ga_typed_spmm(
         t.tile_chunk_pointer.data_ptr<int>(), t.chunk_type.data_ptr<int>(),
         t.slot_src.data_ptr<int>(), t.slot_dst.data_ptr<uint8_t>(), t.slot_edge.data_ptr<int>(),
         features.data_ptr(), weights.data_ptr(), rs, out.data_ptr(), graph->num_nodes,
-        features.size(0), graph->num_edges, graph->num_etypes, s.K, s.M, s.dt,
+        features.size(0), graph->num_edges, graph->num_etypes, t.tile_rows, s.K, s.M, s.dt,
         current_stream(out));
     if (rc != GA_EUNSUPPORTED) {
       check_ga(rc, "ga_typed_spmm");

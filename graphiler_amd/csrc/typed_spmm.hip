@@ -6,17 +6,18 @@
 // back: 2 M b bytes per edge against the K b bytes of the source row.
 //
 // The matrix cores want edges of one relation side by side, the sum wants edges of
-// one destination side by side.  Both hold inside a tile of 128 destination nodes
-// whose edges are ordered by relation:
+// one destination side by side.  Both hold inside a tile of 128 (or 144) destination
+// nodes whose edges are ordered by relation:
 //
 //   preparation (once per graph)   slots of the in-adjacency are sorted, stably, by
-//     (destination / 128, relation); every (tile, relation) group is padded to whole
+//     (destination / tile height, relation); every (tile, relation) group is padded to whole
 //     chunks of 16 slots, and per padded slot the source node, the destination inside
 //     the tile and the edge id are written out, per chunk its relation, per tile its
 //     first chunk.  A pad slot has source and edge id -1.
-//   kernel   one workgroup of four wavefronts per tile; every wavefront walks all chunks
-//     of the tile and owns 16 of the 64 output columns, whose 128 x 16 fp32 sums it keeps
-//     in matrix-core accumulators (32 registers).  Per chunk it gathers the 16 source
+//   kernel   one workgroup of four wavefronts per tile; a wavefront owns 32 of the 64
+//     output columns and walks every second chunk of the tile (two wavefronts share a
+//     chunk, one per column half); its 128 x 32 fp32 partial sums stay in matrix-core
+//     accumulators (64 registers), and the partial tiles meet in LDS at the end.  Per chunk it gathers the 16 source
 //     rows (one 16- or 8-byte read per lane), multiplies them with its 16 columns of the
 //     relation's weights (K / 4 v_mfma_f32_16x16x4_f32, or K / 16
 //     v_mfma_f32_16x16x16_bf16) and scales the 16 x 16 result rows: the messages.  The
@@ -45,9 +46,10 @@ namespace {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kTileRows = GA_TYPED_TILE_ROWS;   // destination nodes per tile
-constexpr int kTileShift = 7;
-static_assert((1 << kTileShift) == kTileRows, "tile rows");
+// destination nodes per tile: 128 or 144 (8 or 9 blocks of 16), chosen per graph so that
+// the workgroups fill whole rounds of the chip (ga_typed_tile_rows)
+constexpr int kMaxTileRows = 144;
+inline bool tile_rows_ok(int64_t r) { return r == 128 || r == 144; }
 constexpr int kChunk = 16;                      // slots per chunk: rows of one MFMA
 constexpr int kTypedM = 64;                     // output columns: 4 wavefronts x 16
 constexpr int kTypedBlock = 4 * kWave;
@@ -56,7 +58,7 @@ constexpr int kTypedBlock = 4 * kWave;
 // key of a slot: tile * n_types + relation
 __global__ __launch_bounds__(kBlock) void typed_keys_kernel(
     const int32_t *__restrict__ row_of_slot, const int32_t *__restrict__ eid,
-    const int32_t *__restrict__ type_pointer, int n_types, int64_t n_edges,
+    const int32_t *__restrict__ type_pointer, int n_types, int64_t n_edges, int tile_rows,
     int32_t *__restrict__ key, int32_t *__restrict__ ids) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= n_edges) return;
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(kBlock) void typed_keys_kernel(
     const int mid = (lo + hi) >> 1;
     if (type_pointer[mid] <= e) lo = mid; else hi = mid;
   }
-  key[i] = (row_of_slot[i] >> kTileShift) * n_types + lo;
+  key[i] = (row_of_slot[i] / tile_rows) * n_types + lo;
   ids[i] = (int32_t)i;
 }
 
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(kBlock) void typed_fill_kernel(
     const int32_t *__restrict__ chunk_base, const int32_t *__restrict__ first,
     const int32_t *__restrict__ ids_sorted, const int32_t *__restrict__ row_of_slot,
     const int32_t *__restrict__ nbr, const int32_t *__restrict__ eid, int64_t n_groups,
-    int n_types, int64_t chunk_capacity, int32_t *__restrict__ chunk_type,
+    int n_types, int tile_rows, int64_t chunk_capacity, int32_t *__restrict__ chunk_type,
     int32_t *__restrict__ slot_src, unsigned char *__restrict__ slot_dst,
     int32_t *__restrict__ slot_edge) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void typed_fill_kernel(
       const int i = ids_sorted[first[k] + off];
       src = nbr[i];
       edge = eid ? eid[i] : i;
-      dst = row_of_slot[i] & (kTileRows - 1);
+      dst = row_of_slot[i] % tile_rows;
     }
   }
   slot_src[p] = src;
@@ -168,7 +170,9 @@ int tiles_layout(int64_t n_groups, int64_t n_edges, TilesLayout &L) {
   return GA_OK;
 }
 
-inline int64_t tiles_of(int64_t n_rows) { return (n_rows + kTileRows - 1) / kTileRows; }
+inline int64_t tiles_of(int64_t n_rows, int64_t tile_rows) {
+  return (n_rows + tile_rows - 1) / tile_rows;
+}
 
 // ------------------------------------------------------------------------ kernel ----
 // Byte offsets into x, W and row_scale are 32-bit (checked on the host): a load is then
@@ -178,13 +182,19 @@ __device__ __forceinline__ V load_at(const void *base, uint32_t byte_offset) {
   return *reinterpret_cast<const V *>(reinterpret_cast<const char *>(base) + byte_offset);
 }
 
+// A wavefront owns kCB of the four 16-column blocks of the tile and walks every kCB-th
+// chunk: 4 / kCB wavefronts share a chunk (one per column group), kCB take turns on the
+// chunks.  Two blocks = a 128 x 32 tile per wavefront (64 accumulator registers): three
+// wavefronts fit a SIMD and the whole grid is resident at once.
+constexpr int kCB = 2;
+constexpr int kColGroups = 4 / kCB;
 template <typename T, int KS>
 struct TypedFrag;
 
 template <int KS>
 struct TypedFrag<float, KS> {
   float4 x[KS];           // row n of the chunk: k = 16 j + 4 q .. + 3
-  float w[4][KS][4];      // column block cb: W[16 j + 4 q + s][16 cb + n]
+  float w[kCB][KS][4];    // my column block c: W[16 j + 4 q + s][16 (cb0 + c) + n]
   static __device__ __forceinline__ void load_x(TypedFrag &f, const float *x, uint32_t row, int q) {
 #pragma unroll
     for (int j = 0; j < KS; ++j)
@@ -193,7 +203,7 @@ struct TypedFrag<float, KS> {
   // wt: the relation's weights (uniform); lane_off: element (4 q, n) of them
   static __device__ __forceinline__ void load_w(TypedFrag &f, const float *wt, uint32_t lane_off) {
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb)
+    for (int cb = 0; cb < kCB; ++cb)
 #pragma unroll
       for (int j = 0; j < KS; ++j)
 #pragma unroll
@@ -216,7 +226,7 @@ struct TypedFrag<float, KS> {
 template <int KS>
 struct TypedFrag<bf16_t, KS> {
   uint2 x[KS];            // four bf16: k = 16 j + 4 q .. + 3
-  uint2 w[4][KS];         // column block cb: W[16 j + 4 q .. + 3][16 cb + n]
+  uint2 w[kCB][KS];       // my column block c: W[16 j + 4 q .. + 3][16 (cb0 + c) + n]
   static __device__ __forceinline__ void load_x(TypedFrag &f, const bf16_t *x, uint32_t row, int q) {
 #pragma unroll
     for (int j = 0; j < KS; ++j)
@@ -224,7 +234,7 @@ struct TypedFrag<bf16_t, KS> {
   }
   static __device__ __forceinline__ void load_w(TypedFrag &f, const bf16_t *wt, uint32_t lane_off) {
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb)
+    for (int cb = 0; cb < kCB; ++cb)
 #pragma unroll
       for (int j = 0; j < KS; ++j) {
         uint32_t h[4];
@@ -320,13 +330,12 @@ __device__ __forceinline__ void store_row4(bf16_t *p, const float4 &v) {
   *reinterpret_cast<uint2 *>(p) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
 }
 
-constexpr int kTileBlocks = kTileRows / 16;   // 16-row blocks of a tile
 constexpr int kMergeStride = kTypedM + 4;     // row stride of the LDS tile the waves meet in
 
 // Elements of a tile that received a message that is not finite, by kind: bit
-// 4 b + i of word cb is element (b, cb, i) of the lane.
+// 4 b + i of word cb is element (b, cb, i) of the lane (up to 9 blocks: 36 bits).
 struct Poison {
-  uint32_t pinf[4], ninf[4], nan[4];
+  uint64_t pinf[kCB], ninf[kCB], nan[kCB];
 };
 
 struct TypedArgs {
@@ -336,12 +345,13 @@ struct TypedArgs {
   const float *row_scale;
 };
 
-// The chunks first, first + 4, ... < c1 of a tile into the lane's share of a 128 x 64
-// tile: tile[b][cb][i] = row 16 b + 4 q + i, column 16 cb + n.  CHECKED: messages that
+// The chunks first, first + kCB, ... < c1 of a tile into the lane's share of the
+// wavefront's 128 x (16 kCB) tile: tile[b][c][i] = row 16 b + 4 q + i, column 16 c + n of
+// the wavefront's columns (w_lane already points at them).  CHECKED: messages that
 // are not finite are replaced by zero and recorded in `poison`.
-template <typename T, int KS, bool SCALED, bool CHECKED>
+template <typename T, int KS, bool SCALED, bool CHECKED, int NB>
 __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c1, int n, int q,
-                                            floatx4 (&tile)[kTileBlocks][4], Poison &poison) {
+                                            floatx4 (&tile)[NB][kCB], Poison &poison) {
   constexpr int kTerms = Terms<T>::kTerms;
   const uint32_t w_lane = (4u * q) * kTypedM + n;
   // Loads are issued without branches around them (a chunk index past the end reads the
@@ -353,11 +363,14 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
     I.src = A.slot_src[c * kChunk + n];
     I.dst4 = A.slot_dst4[c * 4 + q];
     I.edge = A.slot_edge[c * kChunk + 4 * q + (n & 3)];
-    I.type = A.chunk_type[c];
+    // A vector load on purpose: scalar loads return out of order, so waiting for the
+    // type of the chunk at hand would also wait for the one requested just now.
+    I.type = __hip_atomic_load(A.chunk_type + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
   auto load_data = [&](const ChunkIds &I, ChunkData<T, KS> &D) __attribute__((always_inline)) {
     TypedFrag<T, KS>::load_x(D.f, (const T *)A.x, (uint32_t)(I.src < 0 ? 0 : I.src), q);
-    TypedFrag<T, KS>::load_w(D.f, (const T *)A.W + (int64_t)I.type * (16 * KS * kTypedM), w_lane);
+    const int type = __builtin_amdgcn_readfirstlane(I.type);
+    TypedFrag<T, KS>::load_w(D.f, (const T *)A.W + (int64_t)type * (16 * KS * kTypedM), w_lane);
     D.sc = SCALED ? load_at<float>(A.row_scale, (uint32_t)(I.edge < 0 ? 0 : I.edge) * 4u) : 1.0f;
     D.dst4 = I.dst4;
   };
@@ -368,9 +381,9 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
       sc[0] = row_share<0>(d.sc); sc[1] = row_share<1>(d.sc);
       sc[2] = row_share<2>(d.sc); sc[3] = row_share<3>(d.sc);
     }
-    uint2 t[4][kTerms];
+    uint2 t[kCB][kTerms];
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb) {
+    for (int cb = 0; cb < kCB; ++cb) {
       const floatx4 acc = TypedFrag<T, KS>::mma(d.f, cb);
       float m[4] = {acc[0] * sc[0], acc[1] * sc[1], acc[2] * sc[2], acc[3] * sc[3]};
       if (CHECKED) {
@@ -385,11 +398,11 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
             const int dst =
                 (__builtin_amdgcn_readlane(d.dst4, 16 * (r >> 2)) >> (8 * (r & 3))) & 0xff;
             const float v = as_summed(__shfl(m[r & 3], 16 * (r >> 2) + n), T());
-            if (dst < kTileRows && q == ((dst & 15) >> 2) && !is_finite(v)) {
-              const uint32_t bit = 1u << ((dst >> 4) * 4 + (dst & 3));
-              poison.nan[cb] |= v != v ? bit : 0u;
-              poison.pinf[cb] |= v == INFINITY ? bit : 0u;
-              poison.ninf[cb] |= v == -INFINITY ? bit : 0u;
+            if (dst < 16 * NB && q == ((dst & 15) >> 2) && !is_finite(v)) {
+              const uint64_t bit = 1ull << ((dst >> 4) * 4 + (dst & 3));
+              poison.nan[cb] |= v != v ? bit : 0ull;
+              poison.pinf[cb] |= v == INFINITY ? bit : 0ull;
+              poison.ninf[cb] |= v == -INFINITY ? bit : 0ull;
             }
           }
 #pragma unroll
@@ -410,7 +423,7 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
     // tile[b] += S_b @ messages: S_b[i][r] = 1 where row r of the chunk goes to row
     // 16 b + i of the tile; lane (n, q) holds S_b[n][4 q .. 4 q + 3]
 #pragma unroll
-    for (int b = 0; b < kTileBlocks; ++b) {
+    for (int b = 0; b < NB; ++b) {
       if (hit >> b & 1u) {
         const uint32_t s0 = u[0] == 16 * b ? 0x3f80u : 0u, s1 = u[1] == 16 * b ? 0x3f800000u : 0u;
         const uint32_t s2 = u[2] == 16 * b ? 0x3f80u : 0u, s3 = u[3] == 16 * b ? 0x3f800000u : 0u;
@@ -418,7 +431,7 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
 #pragma unroll
         for (int k = 0; k < kTerms; ++k)
 #pragma unroll
-          for (int cb = 0; cb < 4; ++cb)      // four independent accumulators back to back
+          for (int cb = 0; cb < kCB; ++cb)    // independent accumulators back to back
             tile[b][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
                 sel, __builtin_bit_cast(shortx4, t[cb][k]), tile[b][cb], 0, 0, 0);
       }
@@ -426,83 +439,92 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
   };
 
   if (first >= c1) return;
-  // two sets of registers take turns (the loop is unrolled twice, so no copies)
+  // Two sets of registers take turns (the loop is unrolled twice, so no copies): the ids
+  // of one of my chunks are requested two, its rows and weights one of my chunks ahead of
+  // the arithmetic (a third set did not pay for its registers).  Ids are requested before
+  // the rows of the same step: the wait for them at the next step then leaves that step's
+  // rows and weights in flight (loads return in order).
   ChunkIds ia, ib;
   ChunkData<T, KS> d0, d1;
   load_ids(first, ia);
-  load_ids(first + 4, ib);
+  load_ids(first + kCB, ib);
   load_data(ia, d0);
-  for (int c = first; c < c1; c += 8) {
-    load_ids(c + 8, ia);
+  for (int c = first; c < c1; c += 2 * kCB) {
+    load_ids(c + 2 * kCB, ia);
     load_data(ib, d1);
     compute(d0);
-    load_ids(c + 12, ib);
+    load_ids(c + 3 * kCB, ib);
     load_data(ia, d0);
-    if (c + 4 < c1) compute(d1);
+    if (c + kCB < c1) compute(d1);
   }
 }
 
-template <typename T, int KS, bool SCALED>
-__global__ __launch_bounds__(kTypedBlock, KS == 1 ? 2 : 1) void typed_tiles_kernel(
+template <typename T, int KS, bool SCALED, int NB>
+__global__ __launch_bounds__(kTypedBlock, KS == 1 ? 3 : 1) void typed_tiles_kernel(
     const int32_t *__restrict__ tile_chunk_pointer, TypedArgs A, T *__restrict__ out,
     int64_t n_rows) {
+  constexpr int kTileRows = 16 * NB;
+  static_assert(4 * NB <= 64 && kTileRows <= kMaxTileRows, "one bit per tile element of a lane");
   __shared__ __attribute__((aligned(16))) float merged[kTileRows * kMergeStride];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int lane = threadIdx.x & (kWave - 1);
   const int n = lane & 15, q = lane >> 4;
   const int c0 = tile_chunk_pointer[blockIdx.x], c1 = tile_chunk_pointer[blockIdx.x + 1];
-  // every wavefront takes every fourth chunk of the tile, all 64 columns
-  floatx4 tile[kTileBlocks][4];
+  // my column group and my turn on the chunks
+  const int colgroup = wave % kColGroups, turn = wave / kColGroups;
+  A.W = static_cast<const T *>(A.W) + 16 * kCB * colgroup;
+  floatx4 tile[NB][kCB];
   Poison poison;
 #pragma unroll
-  for (int cb = 0; cb < 4; ++cb) poison.pinf[cb] = poison.ninf[cb] = poison.nan[cb] = 0u;
+  for (int cb = 0; cb < kCB; ++cb) poison.pinf[cb] = poison.ninf[cb] = poison.nan[cb] = 0ull;
   auto clear = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int b = 0; b < kTileBlocks; ++b)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
-      for (int cb = 0; cb < 4; ++cb) tile[b][cb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+      for (int cb = 0; cb < kCB; ++cb) tile[b][cb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
   };
   clear();
-  walk_chunks<T, KS, SCALED, false>(A, c0 + wave, c1, n, q, tile, poison);
+  walk_chunks<T, KS, SCALED, false, NB>(A, c0 + turn, c1, n, q, tile, poison);
   // A message that is not finite turns the zeros of the selection matrix into NaN for
   // the rows around it.  Such a message leaves something that is not finite in the tile:
   // then the wavefront walks its chunks again, keeping those messages out of the matrix
   // cores and adding them here instead.
   bool fin = true;
 #pragma unroll
-  for (int b = 0; b < kTileBlocks; ++b)
+  for (int b = 0; b < NB; ++b)
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb)
+    for (int cb = 0; cb < kCB; ++cb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) fin = fin && is_finite(tile[b][cb][i]);
   if (__builtin_amdgcn_ballot_w64(!fin) != 0) {
     clear();
-    walk_chunks<T, KS, SCALED, true>(A, c0 + wave, c1, n, q, tile, poison);
+    walk_chunks<T, KS, SCALED, true, NB>(A, c0 + turn, c1, n, q, tile, poison);
 #pragma unroll
-    for (int b = 0; b < kTileBlocks; ++b)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
-      for (int cb = 0; cb < 4; ++cb)
+      for (int cb = 0; cb < kCB; ++cb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int bit = 4 * b + i;
-          if (poison.pinf[cb] >> bit & 1u) tile[b][cb][i] += INFINITY;
-          if (poison.ninf[cb] >> bit & 1u) tile[b][cb][i] -= INFINITY;
-          if (poison.nan[cb] >> bit & 1u) tile[b][cb][i] = NAN;
+          if (poison.pinf[cb] >> bit & 1ull) tile[b][cb][i] += INFINITY;
+          if (poison.ninf[cb] >> bit & 1ull) tile[b][cb][i] -= INFINITY;
+          if (poison.nan[cb] >> bit & 1ull) tile[b][cb][i] = NAN;
         }
   }
-  // ---- the four partial tiles meet in LDS, in the order of the wavefronts ---------------
-  for (int w = 0; w < 4; ++w) {
-    if (wave == w) {
+  // ---- the partial tiles meet in LDS: the column groups side by side, the wavefronts of
+  // a group one after the other in a fixed order ------------------------------------------
+  for (int w = 0; w < kCB; ++w) {
+    if (turn == w) {
 #pragma unroll
-      for (int b = 0; b < kTileBlocks; ++b) {
+      for (int b = 0; b < NB; ++b) {
 #pragma unroll
-        for (int cb = 0; cb < 4; ++cb)
+        for (int cb = 0; cb < kCB; ++cb)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            float *p = merged + (16 * b + 4 * q + i) * kMergeStride + 16 * cb + n;
+            float *p = merged + (16 * b + 4 * q + i) * kMergeStride + 16 * (kCB * colgroup + cb) + n;
             *p = w == 0 ? tile[b][cb][i] : *p + tile[b][cb][i];
           }
-        // one block at a time: 16 values in flight, not the whole tile
+        // one block at a time: few values in flight, not the whole tile
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -518,16 +540,41 @@ __global__ __launch_bounds__(kTypedBlock, KS == 1 ? 2 : 1) void typed_tiles_kern
   }
 }
 
+template <typename T, int KS, int NB>
+int launch_typed_nb(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows,
+                    hipStream_t s) {
+  const dim3 grid((unsigned)tiles_of(n_rows, 16 * NB));
+  if (A.row_scale)
+    hipLaunchKernelGGL((typed_tiles_kernel<T, KS, true, NB>), grid, dim3(kTypedBlock), 0, s, tcp, A,
+                       (T *)out, n_rows);
+  else
+    hipLaunchKernelGGL((typed_tiles_kernel<T, KS, false, NB>), grid, dim3(kTypedBlock), 0, s, tcp, A,
+                       (T *)out, n_rows);
+  return launch_status();
+}
+
 template <typename T, int KS>
 int launch_typed(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows,
-                 hipStream_t s) {
-  if (A.row_scale)
-    hipLaunchKernelGGL((typed_tiles_kernel<T, KS, true>), dim3((unsigned)tiles_of(n_rows)),
-                       dim3(kTypedBlock), 0, s, tcp, A, (T *)out, n_rows);
-  else
-    hipLaunchKernelGGL((typed_tiles_kernel<T, KS, false>), dim3((unsigned)tiles_of(n_rows)),
-                       dim3(kTypedBlock), 0, s, tcp, A, (T *)out, n_rows);
-  return launch_status();
+                 int64_t tile_rows, hipStream_t s) {
+  if (tile_rows == 144) return launch_typed_nb<T, KS, 9>(tcp, A, out, n_rows, s);
+  return launch_typed_nb<T, KS, 8>(tcp, A, out, n_rows, s);
+}
+
+// Workgroups of the kernel that a CU holds at once (three wavefronts per SIMD by its
+// registers, four wavefronts per workgroup).
+constexpr int kTypedGroupsPerCu = 3;
+
+int typed_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      cus = v;
+    else
+      cus = 256;
+  }
+  return cus;
 }
 
 }  // namespace
@@ -535,16 +582,38 @@ int launch_typed(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_ro
 
 extern "C" {
 
-int64_t ga_typed_tiles_chunk_capacity(int64_t n_rows, int64_t n_edges, int64_t n_types) {
-  if (n_rows < 0 || n_edges < 0 || n_types <= 0) return 0;
+int64_t ga_typed_tile_rows(int64_t n_rows) {
+  // The kernel holds kTypedGroupsPerCu workgroups per CU at once, one workgroup per tile:
+  // of the two tile heights take the one whose tiles fill whole rounds of the chip best
+  // (a last round with a few workgroups costs as much as a full one); 128 on a tie.
+  const int64_t slots = (int64_t)ga::typed_cu_count() * ga::kTypedGroupsPerCu;
+  int64_t best = 128;
+  double best_fill = 0.0;
+  for (int64_t rows : {(int64_t)128, (int64_t)144}) {
+    const int64_t tiles = ga::tiles_of(n_rows < 1 ? 1 : n_rows, rows);
+    const int64_t rounds = (tiles + slots - 1) / slots;
+    const double fill = (double)tiles / (double)(rounds * slots);
+    if (fill > best_fill + 1e-9) {
+      best_fill = fill;
+      best = rows;
+    }
+  }
+  return best;
+}
+
+int64_t ga_typed_tiles_chunk_capacity(int64_t n_rows, int64_t n_edges, int64_t n_types,
+                                      int64_t tile_rows) {
+  if (n_rows < 0 || n_edges < 0 || n_types <= 0 || !ga::tile_rows_ok(tile_rows)) return 0;
   // every (tile, relation) group that has edges wastes less than one chunk
-  const int64_t groups = ga::tiles_of(n_rows) * n_types;
+  const int64_t groups = ga::tiles_of(n_rows, tile_rows) * n_types;
   return (n_edges + ga::kChunk - 1) / ga::kChunk + (groups < n_edges ? groups : n_edges);
 }
 
-size_t ga_typed_tiles_workspace_bytes(int64_t n_rows, int64_t n_edges, int64_t n_types) {
+size_t ga_typed_tiles_workspace_bytes(int64_t n_rows, int64_t n_edges, int64_t n_types,
+                                      int64_t tile_rows) {
   if (n_rows < 0 || n_edges < 0 || n_types <= 0 || n_edges > 0x7fffffff) return 0;
-  const int64_t groups = ga::tiles_of(n_rows) * n_types;
+  if (!ga::tile_rows_ok(tile_rows)) return 0;
+  const int64_t groups = ga::tiles_of(n_rows, tile_rows) * n_types;
   if (groups > 0x7ffffffe) return 0;
   ga::TilesLayout L;
   if (ga::tiles_layout(groups, n_edges, L) != GA_OK) return 0;
@@ -553,15 +622,17 @@ size_t ga_typed_tiles_workspace_bytes(int64_t n_rows, int64_t n_edges, int64_t n
 
 int ga_typed_tiles_build(const int32_t *row_of_slot, const int32_t *nbr, const int32_t *eid,
                          const int32_t *type_pointer, int64_t n_rows, int64_t n_edges,
-                         int64_t n_types, int32_t *tile_chunk_pointer, int32_t *chunk_type,
+                         int64_t n_types, int64_t tile_rows, int32_t *tile_chunk_pointer,
+                         int32_t *chunk_type,
                          int32_t *slot_src, unsigned char *slot_dst, int32_t *slot_edge,
                          void *workspace, size_t workspace_bytes, ga_stream_t stream) {
   using namespace ga;
   if (n_rows < 0 || n_edges < 0 || n_types <= 0) return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || n_types > 0x7fffffff) return GA_EINVAL;
-  const int64_t n_tiles = tiles_of(n_rows), n_groups = n_tiles * n_types;
+  if (!tile_rows_ok(tile_rows)) return GA_EINVAL;
+  const int64_t n_tiles = tiles_of(n_rows, tile_rows), n_groups = n_tiles * n_types;
   if (n_groups > 0x7ffffffe) return GA_EUNSUPPORTED;
-  const int64_t cap = ga_typed_tiles_chunk_capacity(n_rows, n_edges, n_types);
+  const int64_t cap = ga_typed_tiles_chunk_capacity(n_rows, n_edges, n_types, tile_rows);
   if (cap * kChunk > 0x7fffffff) return GA_EUNSUPPORTED;
   if (!tile_chunk_pointer || !type_pointer) return GA_EINVAL;
   if (n_edges > 0 && (!row_of_slot || !nbr || !chunk_type || !slot_src || !slot_dst || !slot_edge))
@@ -580,7 +651,7 @@ int ga_typed_tiles_build(const int32_t *row_of_slot, const int32_t *nbr, const i
   if (n_edges > 0) {
     const int64_t blocks = (n_edges + kBlock - 1) / kBlock;
     hipLaunchKernelGGL(typed_keys_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, row_of_slot,
-                       eid, type_pointer, (int)n_types, n_edges, key, ids);
+                       eid, type_pointer, (int)n_types, n_edges, (int)tile_rows, key, ids);
     size_t tb = L.sort_bytes;
     hipError_t e = rocprim::radix_sort_pairs(ws + L.temp, tb, key, key_sorted, ids, ids_sorted,
                                              (size_t)n_edges, 0, end_bit_for(n_groups), s);
@@ -601,7 +672,8 @@ int ga_typed_tiles_build(const int32_t *row_of_slot, const int32_t *nbr, const i
   if (cap > 0) {
     const int64_t blocks = (cap * kChunk + kBlock - 1) / kBlock;
     hipLaunchKernelGGL(typed_fill_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, base, first,
-                       ids_sorted, row_of_slot, nbr, eid, n_groups, (int)n_types, cap, chunk_type,
+                       ids_sorted, row_of_slot, nbr, eid, n_groups, (int)n_types, (int)tile_rows, cap,
+                       chunk_type,
                        slot_src, slot_dst, slot_edge);
   }
   return launch_status();
@@ -611,10 +683,11 @@ int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
                   const int32_t *slot_src, const unsigned char *slot_dst,
                   const int32_t *slot_edge, const void *x, const void *W,
                   const float *row_scale, void *out, int64_t n_rows, int64_t n_src,
-                  int64_t n_edges, int64_t n_types, int64_t K, int64_t M, int dtype,
-                  ga_stream_t stream) {
+                  int64_t n_edges, int64_t n_types, int64_t tile_rows, int64_t K, int64_t M,
+                  int dtype, ga_stream_t stream) {
   using namespace ga;
   if (n_rows < 0 || n_src < 0 || n_edges < 0 || n_types <= 0 || K <= 0 || M <= 0) return GA_EINVAL;
+  if (!tile_rows_ok(tile_rows)) return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff) return GA_EINVAL;
   if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
   if (M != kTypedM || K % 16 != 0 || K > 64) return GA_EUNSUPPORTED;
@@ -622,7 +695,7 @@ int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
   // the kernel addresses x, one relation of W and row_scale with 32-bit byte offsets,
   // the slot arrays with 32-bit indices
   if ((uint64_t)n_src * K * esz > 0xffffffffull || (uint64_t)n_edges * 4 > 0xffffffffull ||
-      ga_typed_tiles_chunk_capacity(n_rows, n_edges, n_types) * kChunk > 0x7fffffff)
+      ga_typed_tiles_chunk_capacity(n_rows, n_edges, n_types, tile_rows) * kChunk > 0x7fffffff)
     return GA_EUNSUPPORTED;
   if (n_rows == 0) return GA_OK;
   if (!tile_chunk_pointer || !out) return GA_EINVAL;
@@ -635,7 +708,7 @@ int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
   hipStream_t s = (hipStream_t)stream;
   const TypedArgs A{chunk_type, slot_src, slot_edge, (const uint32_t *)slot_dst, x, W, row_scale};
   const int ks = (int)(K / 16);
-#define GA_TYPED(T, KS) return launch_typed<T, KS>(tile_chunk_pointer, A, out, n_rows, s)
+#define GA_TYPED(T, KS) return launch_typed<T, KS>(tile_chunk_pointer, A, out, n_rows, tile_rows, s)
   if (dtype == GA_F32) {
     switch (ks) {
       case 1: GA_TYPED(float, 1);

@@ -555,20 +555,22 @@ def SegmentMMEdgeGather(features, weights, endpoint: int, graph: DGLGraph,
 
 def _typed_tiles(graph: DGLGraph):
     """The (destination tile, relation) ordering of the in-edges that TypedSpMMEdge
-    walks; built on the device at first use and kept with the graph."""
+    walks, and its tile height; built on the device at first use and kept with the
+    graph."""
     t = graph._cache.get("typed_tiles")
     if t is None:
         lib = capi.load()
         n, e, r = graph.num_nodes, graph.num_edges, graph.num_etypes
-        cap = int(lib.ga_typed_tiles_chunk_capacity(n, e, r))
-        tiles = -(-n // capi.GA_TYPED_TILE_ROWS)
+        rows = int(lib.ga_typed_tile_rows(n))
+        cap = int(lib.ga_typed_tiles_chunk_capacity(n, e, r, rows))
+        tiles = -(-n // rows)
         dev = graph.device
         i32 = dict(dtype=torch.int32, device=dev)
         t = (torch.empty(tiles + 1, **i32), torch.empty(max(cap, 1), **i32),
              torch.empty(max(16 * cap, 1), **i32),
              torch.empty(max(16 * cap, 4), dtype=torch.uint8, device=dev),
-             torch.empty(max(16 * cap, 4), **i32))
-        nbytes = int(lib.ga_typed_tiles_workspace_bytes(n, e, r))
+             torch.empty(max(16 * cap, 4), **i32), rows)
+        nbytes = int(lib.ga_typed_tiles_workspace_bytes(n, e, r, rows))
         if nbytes == 0:
             raise RuntimeError("graph too large for the typed tile layout")
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
@@ -576,7 +578,7 @@ def _typed_tiles(graph: DGLGraph):
         capi.check(lib.ga_typed_tiles_build(
             graph.in_row_of_slot.data_ptr(), graph.in_node_indices.data_ptr(),
             None if ident else graph.in_edge_indices.data_ptr(),
-            graph.etype_pointer.data_ptr(), n, e, r, t[0].data_ptr(), t[1].data_ptr(),
+            graph.etype_pointer.data_ptr(), n, e, r, rows, t[0].data_ptr(), t[1].data_ptr(),
             t[2].data_ptr(), t[3].data_ptr(), t[4].data_ptr(), ws.data_ptr(), ws.numel(),
             torch.cuda.current_stream(dev).cuda_stream), "ga_typed_tiles_build")
         graph._cache["typed_tiles"] = t
@@ -615,13 +617,13 @@ def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None) -> torch.T
         if row_scale.dtype != torch.float32 or row_scale.numel() != graph.num_edges:
             raise RuntimeError("row_scale must be one float32 per edge")
     K, M = int(weights.shape[1]), int(weights.shape[2])
-    tcp, ctype, ssrc, sdst, sedge = _typed_tiles(graph)
+    tcp, ctype, ssrc, sdst, sedge, tile_rows = _typed_tiles(graph)
     out = torch.empty((graph.num_nodes, M), dtype=features.dtype, device=features.device)
     capi.check(capi.load().ga_typed_spmm(
         tcp.data_ptr(), ctype.data_ptr(), ssrc.data_ptr(), sdst.data_ptr(), sedge.data_ptr(),
         features.data_ptr(), weights.data_ptr(), _ptr(row_scale), out.data_ptr(),
-        graph.num_nodes, int(features.shape[0]), graph.num_edges, graph.num_etypes, K, M,
-        dt, _stream(out)), "ga_typed_spmm")
+        graph.num_nodes, int(features.shape[0]), graph.num_edges, graph.num_etypes, tile_rows,
+        K, M, dt, _stream(out)), "ga_typed_spmm")
     return out
 
 

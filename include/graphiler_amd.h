@@ -194,9 +194,11 @@ int ga_sddmm_u_op_v_adj(const int32_t *pointer, const int32_t *row_of_slot,
  * ga_typed_tiles_build prepares the graph once: the slots of the in-adjacency
  * (row_of_slot = destination, nbr = source, eid = edge id or null when slot = edge id;
  * type_pointer: n_types + 1 entries over the edge ids, include/dglgraph.h:24-27) are
- * ordered by (destination / GA_TYPED_TILE_ROWS, relation) and every such group is
- * padded to chunks of 16 slots.  Outputs: tile_chunk_pointer (tiles + 1, tiles =
- * ceil(n_rows / GA_TYPED_TILE_ROWS)), chunk_type (capacity), slot_src and slot_edge
+ * ordered by (destination / tile_rows, relation) and every such group is padded to
+ * chunks of 16 slots.  tile_rows is 128 or 144: ga_typed_tile_rows(n_rows) names the one
+ * whose tiles fill whole rounds of this device's CUs best; the same value goes to every
+ * call for the graph.  Outputs: tile_chunk_pointer (tiles + 1, tiles =
+ * ceil(n_rows / tile_rows)), chunk_type (capacity), slot_src and slot_edge
  * (16 * capacity, -1 in pad slots), slot_dst (16 * capacity bytes: destination - tile
  * start, 255 in pad slots; 4-byte aligned), capacity =
  * ga_typed_tiles_chunk_capacity(...).  Everything runs on `stream`; nothing is read
@@ -211,20 +213,23 @@ int ga_sddmm_u_op_v_adj(const int32_t *pointer, const int32_t *row_of_slot,
  * additions is fixed by the prepared layout, so repeated calls give identical bits;
  * against the chain only that order differs.  Messages that are not finite reach
  * exactly the rows the chain would give them to. */
-#define GA_TYPED_TILE_ROWS 128
-int64_t ga_typed_tiles_chunk_capacity(int64_t n_rows, int64_t n_edges, int64_t n_types);
-size_t ga_typed_tiles_workspace_bytes(int64_t n_rows, int64_t n_edges, int64_t n_types);
+int64_t ga_typed_tile_rows(int64_t n_rows);
+int64_t ga_typed_tiles_chunk_capacity(int64_t n_rows, int64_t n_edges, int64_t n_types,
+                                      int64_t tile_rows);
+size_t ga_typed_tiles_workspace_bytes(int64_t n_rows, int64_t n_edges, int64_t n_types,
+                                      int64_t tile_rows);
 int ga_typed_tiles_build(const int32_t *row_of_slot, const int32_t *nbr, const int32_t *eid,
                          const int32_t *type_pointer, int64_t n_rows, int64_t n_edges,
-                         int64_t n_types, int32_t *tile_chunk_pointer, int32_t *chunk_type,
-                         int32_t *slot_src, unsigned char *slot_dst, int32_t *slot_edge,
-                         void *workspace, size_t workspace_bytes, ga_stream_t stream);
+                         int64_t n_types, int64_t tile_rows, int32_t *tile_chunk_pointer,
+                         int32_t *chunk_type, int32_t *slot_src, unsigned char *slot_dst,
+                         int32_t *slot_edge, void *workspace, size_t workspace_bytes,
+                         ga_stream_t stream);
 int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
                   const int32_t *slot_src, const unsigned char *slot_dst,
                   const int32_t *slot_edge, const void *x, const void *W,
                   const float *row_scale, void *out, int64_t n_rows, int64_t n_src,
-                  int64_t n_edges, int64_t n_types, int64_t K, int64_t M, int dtype,
-                  ga_stream_t stream);
+                  int64_t n_edges, int64_t n_types, int64_t tile_rows, int64_t K, int64_t M,
+                  int dtype, ga_stream_t stream);
 
 /* The general SDDMM of the reference (SDDMMCooKernel / SDDMMCooTreeReduceKernel,
  * sddmm.cuh:34-120): operands on the source nodes (target 0), on the edges (1) or on

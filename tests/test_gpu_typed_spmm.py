@@ -85,8 +85,9 @@ def test_typed_tiles_layout(device):
     rng = np.random.default_rng(9)
     n, e, r = 700, 9000, 13
     g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device, hub=True)
-    tcp, ctype, ssrc, sdst, sedge = (t.cpu().numpy() for t in ops._typed_tiles(g))
-    rows = capi.GA_TYPED_TILE_ROWS
+    *arrays, rows = ops._typed_tiles(g)
+    tcp, ctype, ssrc, sdst, sedge = (t.cpu().numpy() for t in arrays)
+    assert rows in (128, 144) and rows == capi.load().ga_typed_tile_rows(n)
     tiles = -(-n // rows)
     assert tcp.shape == (tiles + 1,) and tcp[0] == 0 and np.all(np.diff(tcp) >= 0)
     total = int(tcp[-1])
@@ -113,7 +114,7 @@ def test_typed_tiles_layout(device):
     # every group wastes less than one chunk
     groups = len(np.unique(key))
     assert total <= -(-e // 16) + groups
-    assert total <= capi.load().ga_typed_tiles_chunk_capacity(n, e, r)
+    assert total <= capi.load().ga_typed_tiles_chunk_capacity(n, e, r, rows)
 
 
 @pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
