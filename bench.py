@@ -185,7 +185,7 @@ def main():
         def network():
             x = x0
             for w, a in params:
-                x = F.elu(layers.gat_layer(g, x, w, a, H, slope, fused=True))
+                x = layers.gat_layer(g, x, w, a, H, slope, fused=True, activation="elu")
             return x
 
         ms_step, out = wall_time(network, args.steps, args.warmup)

@@ -74,6 +74,7 @@ struct GatPolicy {
     bool ids_vec;   // row_of_slot and nbr are 16-byte aligned
     int head_lanes; // kGatFromZ: lanes that share a head (dph / VEC)
     int stride_shift;   // SPREAD: log2 of the lanes per group, set by the launcher
+    int act;            // GA_ACT_*: applied to the finished row before it is stored
   };
   static __device__ __forceinline__ void init(float (&st)[VEC + 2]) {
 #pragma unroll
@@ -101,7 +102,19 @@ struct GatPolicy {
   }
   static __device__ __forceinline__ void emit(const Args &A, out_t *out, int64_t row, int feat,
                                               int f0, const float (&st)[kState]) {
-    emit_row<GatPolicy>(out, row, feat, f0, st, A.stride_shift);
+    if (A.act == GA_ACT_NONE) {
+      emit_row<GatPolicy>(out, row, feat, f0, st, A.stride_shift);
+      return;
+    }
+    // the activation of the layer (relu, or elu with alpha = 1) on the fp32 row, before
+    // it is rounded and stored: the row is not written and read again for it
+    typedef RowIO<out_t, VEC, SPREAD> IO;
+    float o[VEC];
+    finish(st, o);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v)
+      o[v] = o[v] > 0.0f ? o[v] : (A.act == GA_ACT_ELU ? __expf(o[v]) - 1.0f : (o[v] != o[v] ? o[v] : 0.0f));
+    IO::store(out + row * feat + f0, o, IO::lane(A.stride_shift, feat - f0));
   }
   static __device__ __forceinline__ void emit_empty(const Args &A, out_t *out, int64_t row,
                                                     int feat, int f0) {
@@ -208,14 +221,14 @@ int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const int32_t *nbr, const float *el, const float *er,
                const void *z, void *out, int64_t n_rows, int64_t n_edges,
                int heads, int dim, float slope, float *ws, hipStream_t stream,
-               size_t ws_bytes = SIZE_MAX) {
+               size_t ws_bytes = SIZE_MAX, int act = GA_ACT_NONE) {
   typedef GatPolicy<T, VEC, MODE, SPREAD> P;
   const bool ids_vec = aligned(row_of_slot, 16) && (!nbr || aligned(nbr, 16));
   const int head_lanes = dim / VEC;
   if (MODE == kGatFromZ &&
       (dim % VEC != 0 || head_lanes > 16 || (head_lanes & (head_lanes - 1)) != 0))
     return GA_EUNSUPPORTED;
-  typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec, head_lanes, 0};
+  typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec, head_lanes, 0, act};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges,
                         heads * dim, ws, stream, ws_bytes);
 }
@@ -226,26 +239,26 @@ int gat_aggregate_dispatch(const int32_t *pointer, const int32_t *row_of_slot,
                            const int32_t *nbr, const float *el, const float *er,
                            const void *z, void *out, int64_t n_rows, int64_t n_edges,
                            int heads, int dim, float slope, int dtype, float *ws,
-                           size_t ws_bytes, hipStream_t s) {
+                           size_t ws_bytes, hipStream_t s, int act = GA_ACT_NONE) {
   const bool vec_ok = aligned(out, 16) && (!z || aligned(z, 16));
   if (dtype == GA_F32) {
     if (vec_ok && dim % 4 == 0)
       return launch_gat<float, 4>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
-                                  heads, dim, slope, ws, s, ws_bytes);
+                                  heads, dim, slope, ws, s, ws_bytes, act);
     if (heads == 1 && dim >= 3 && dim <= 256)   // rows that 16-byte accesses do not tile
       return launch_gat<float, 4, kGatNode, true>(pointer, row_of_slot, nbr, el, er, z, out,
-                                                  n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes);
+                                                  n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes, act);
     return launch_gat<float, 1>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
-                                heads, dim, slope, ws, s, ws_bytes);
+                                heads, dim, slope, ws, s, ws_bytes, act);
   }
   if (vec_ok && dim % 8 == 0)
     return launch_gat<bf16_t, 8>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
-                                 heads, dim, slope, ws, s, ws_bytes);
+                                 heads, dim, slope, ws, s, ws_bytes, act);
   if (heads == 1 && dim >= 3 && dim <= 256)
     return launch_gat<bf16_t, 4, kGatNode, true>(pointer, row_of_slot, nbr, el, er, z, out,
-                                                 n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes);
+                                                 n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes, act);
   return launch_gat<bf16_t, 1>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
-                               heads, dim, slope, ws, s, ws_bytes);
+                               heads, dim, slope, ws, s, ws_bytes, act);
 }
 
 // Argument checks shared by ga_gat_aggregate and ga_gat_aggregate_static
@@ -317,6 +330,16 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
                      int64_t heads, int64_t dim, float slope, int dtype,
                      void *workspace, size_t workspace_bytes,
                      ga_stream_t stream) {
+  return ga_gat_aggregate_act(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges, heads,
+                              dim, slope, GA_ACT_NONE, dtype, workspace, workspace_bytes, stream);
+}
+
+int ga_gat_aggregate_act(const int32_t *pointer, const int32_t *row_of_slot,
+                         const int32_t *nbr, const float *el, const float *er,
+                         const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                         int64_t heads, int64_t dim, float slope, int activation, int dtype,
+                         void *workspace, size_t workspace_bytes, ga_stream_t stream) {
+  if (activation < GA_ACT_NONE || activation > GA_ACT_ELU) return GA_EINVAL;
   bool nothing = false;
   const int rc = ga::gat_aggregate_check(pointer, row_of_slot, nbr, el, er, z, out, n_rows,
                                          n_edges, heads, dim, dtype, &nothing);
@@ -327,7 +350,7 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
     return GA_EWORKSPACE;
   return ga::gat_aggregate_dispatch(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
                                     (int)heads, (int)dim, slope, dtype, (float *)workspace,
-                                    workspace_bytes, (hipStream_t)stream);
+                                    workspace_bytes, (hipStream_t)stream, activation);
 }
 
 int ga_gat_aggregate_static(const int32_t *pointer, const int32_t *row_of_slot,
@@ -402,6 +425,18 @@ int ga_gat_aggregate_from_z(const int32_t *pointer, const int32_t *row_of_slot,
                             const void *z, void *out, int64_t n_rows, int64_t n_edges,
                             int64_t heads, int64_t dim, float slope, int dtype,
                             void *workspace, size_t workspace_bytes, ga_stream_t stream) {
+  return ga_gat_aggregate_from_z_act(pointer, row_of_slot, nbr, a_l, er, z, out, n_rows, n_edges,
+                                     heads, dim, slope, GA_ACT_NONE, dtype, workspace,
+                                     workspace_bytes, stream);
+}
+
+int ga_gat_aggregate_from_z_act(const int32_t *pointer, const int32_t *row_of_slot,
+                                const int32_t *nbr, const float *a_l, const float *er,
+                                const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                                int64_t heads, int64_t dim, float slope, int activation,
+                                int dtype, void *workspace, size_t workspace_bytes,
+                                ga_stream_t stream) {
+  if (activation < GA_ACT_NONE || activation > GA_ACT_ELU) return GA_EINVAL;
   if (n_rows < 0 || n_edges < 0 || heads <= 0 || dim <= 0) return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || heads * dim > 0x7fffffff)
     return GA_EINVAL;
@@ -426,15 +461,15 @@ int ga_gat_aggregate_from_z(const int32_t *pointer, const int32_t *row_of_slot,
   if (dtype == GA_F32) {
     if (vec_ok && dim % 4 == 0)
       return ga::launch_gat<float, 4, ga::kGatFromZ>(pointer, row_of_slot, nbr, a_l, er, z, out,
-                                                     n_rows, n_edges, h, d, slope, ws, s);
+                                                     n_rows, n_edges, h, d, slope, ws, s, SIZE_MAX, activation);
     return ga::launch_gat<float, 1, ga::kGatFromZ>(pointer, row_of_slot, nbr, a_l, er, z, out,
-                                                   n_rows, n_edges, h, d, slope, ws, s);
+                                                   n_rows, n_edges, h, d, slope, ws, s, SIZE_MAX, activation);
   }
   if (vec_ok && dim % 8 == 0)
     return ga::launch_gat<ga::bf16_t, 8, ga::kGatFromZ>(pointer, row_of_slot, nbr, a_l, er, z,
-                                                        out, n_rows, n_edges, h, d, slope, ws, s);
+                                                        out, n_rows, n_edges, h, d, slope, ws, s, SIZE_MAX, activation);
   return ga::launch_gat<ga::bf16_t, 1, ga::kGatFromZ>(pointer, row_of_slot, nbr, a_l, er, z, out,
-                                                      n_rows, n_edges, h, d, slope, ws, s);
+                                                      n_rows, n_edges, h, d, slope, ws, s, SIZE_MAX, activation);
 }
 
 }  // extern "C"

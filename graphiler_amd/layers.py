@@ -71,22 +71,31 @@ def gat_aggregate_plan(g: DGLGraph, z, el, er, negative_slope: float = 0.01):
 
 
 def gat_layer(g: DGLGraph, h, fc_weight, attn_weight, heads: int = 1,
-              negative_slope: float = 0.01, fused: bool = True):
+              negative_slope: float = 0.01, fused: bool = True, activation=None):
     """One GAT layer forward; ``fused`` runs the chain as a single pass.  When
     the (N, heads) table of source terms is too large to stay cached
     (``SOURCE_TERM_TABLE_LIMIT`` bytes), the pass recomputes them from the
-    gathered rows instead of gathering them as well."""
+    gathered rows instead of gathering them as well.  ``activation`` ("relu" |
+    "elu"; the ``F.elu`` between the layers of examples/GAT/GAT.py) is applied by
+    the fused pass to the rows it stores, by a separate call otherwise."""
     z, el, er = gat_project(h, fc_weight, attn_weight, heads)
     if fused:
         if el.numel() * el.element_size() >= SOURCE_TERM_TABLE_LIMIT:
             try:
                 return ops.gat_aggregate_from_z(attn_weight[0].float().contiguous(), er.float(),
-                                                z, g, negative_slope)
+                                                z, g, negative_slope, activation)
             except capi.GraphilerError as err:      # head width the variant does not take
                 if err.code != capi.GA_EUNSUPPORTED:
                     raise
-        return ops.gat_aggregate(el.float(), er.float(), z, g, negative_slope)
-    return gat_aggregate_plan(g, z, el, er, negative_slope)
+        return ops.gat_aggregate(el.float(), er.float(), z, g, negative_slope, activation)
+    out = gat_aggregate_plan(g, z, el, er, negative_slope)
+    if activation == "elu":
+        return F.elu(out)
+    if activation == "relu":
+        return torch.relu(out)
+    if activation is not None:
+        raise RuntimeError("activation must be None, 'relu' or 'elu'")
+    return out
 
 
 def rgcn_layer(g: DGLGraph, h, weight, norm, fused=True):

@@ -712,10 +712,22 @@ def BroadcastEdgeType(features, graph: DGLGraph) -> torch.Tensor:
 
 
 # ----------------------------------------------------------- fused GAT ----
-def gat_aggregate(el, er, z, graph: DGLGraph, negative_slope: float = 0.01):
+_ACTIVATIONS = {None: capi.GA_ACT_NONE, "relu": capi.GA_ACT_RELU, "elu": capi.GA_ACT_ELU}
+
+
+def _activation(name) -> int:
+    if name not in _ACTIVATIONS:
+        raise RuntimeError("activation must be None, 'relu' or 'elu'")
+    return _ACTIVATIONS[name]
+
+
+def gat_aggregate(el, er, z, graph: DGLGraph, negative_slope: float = 0.01, activation=None):
     """u_add_v -> leaky_relu -> edge softmax -> u_mul_e sum in one pass
     (the four-operator chain of examples/GAT/GAT.py:25-36 at opt level 2).
-    el, er: (N, H) fp32 attention terms of source / destination; z: (N, H*D)."""
+    el, er: (N, H) fp32 attention terms of source / destination; z: (N, H*D).
+    ``activation`` ("relu" | "elu"): the layer's activation, applied to the fp32
+    rows before they are stored instead of by a pass of its own."""
+    act = _activation(activation)
     _check_input(el, "el")
     _check_input(er, "er")
     _check_input(z, "z")
@@ -733,20 +745,22 @@ def gat_aggregate(el, er, z, graph: DGLGraph, negative_slope: float = 0.01):
     lib = capi.load()
     ws_bytes = lib.ga_gat_workspace_bytes(graph.num_edges, feat, heads)
     ws = graph.workspace(ws_bytes)
-    capi.check(lib.ga_gat_aggregate(
+    capi.check(lib.ga_gat_aggregate_act(
         graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
         graph.in_node_indices.data_ptr(), el.data_ptr(), er.data_ptr(),
         z.data_ptr(), out.data_ptr(), graph.num_nodes, graph.num_edges, heads,
-        feat // heads, float(negative_slope), dt, ws.data_ptr(), ws.numel(),
+        feat // heads, float(negative_slope), act, dt, ws.data_ptr(), ws.numel(),
         _stream(out)), "ga_gat_aggregate")
     return out
 
 
-def gat_aggregate_from_z(a_l, er, z, graph: DGLGraph, negative_slope: float = 0.01):
+def gat_aggregate_from_z(a_l, er, z, graph: DGLGraph, negative_slope: float = 0.01,
+                         activation=None):
     """``gat_aggregate`` with the source term recomputed from the gathered row:
     logits leaky_relu(<z[src, h], a_l[h]> + er[dst, h]).  a_l: (H, D) fp32;
     er: (N, H) fp32; z: (N, H*D).  For node counts whose (N, H) table of source
     terms no longer fits the caches this saves one memory sector per edge."""
+    act = _activation(activation)
     _check_input(a_l, "a_l")
     _check_input(er, "er")
     _check_input(z, "z")
@@ -760,11 +774,11 @@ def gat_aggregate_from_z(a_l, er, z, graph: DGLGraph, negative_slope: float = 0.
     out = torch.empty(_out_shape(graph.num_nodes, z), dtype=z.dtype, device=z.device)
     lib = capi.load()
     ws = graph.workspace(lib.ga_gat_workspace_bytes(graph.num_edges, feat, heads))
-    capi.check(lib.ga_gat_aggregate_from_z(
+    capi.check(lib.ga_gat_aggregate_from_z_act(
         graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
         graph.in_node_indices.data_ptr(), a_l.data_ptr(), er.data_ptr(), z.data_ptr(),
         out.data_ptr(), graph.num_nodes, graph.num_edges, heads, feat // heads,
-        float(negative_slope), dt, ws.data_ptr(), ws.numel(), _stream(out)),
+        float(negative_slope), act, dt, ws.data_ptr(), ws.numel(), _stream(out)),
         "ga_gat_aggregate_from_z")
     return out
 

@@ -54,6 +54,8 @@ enum ga_bcast_op {
 };
 /* functor.cuh:125-213: sum starts at 0, max at -inf, min at +inf             */
 enum ga_reduce { GA_SUM = 0, GA_MAX = 1, GA_MIN = 2 };
+/* activation applied to an output row before it is stored (the *_act entry points) */
+enum ga_activation { GA_ACT_NONE = 0, GA_ACT_RELU = 1, GA_ACT_ELU = 2 };
 
 /* Library version (major*10000 + minor*100 + patch). */
 int ga_version(void);
@@ -401,6 +403,23 @@ int ga_gat_aggregate_from_z(const int32_t *pointer, const int32_t *row_of_slot,
                             int64_t heads, int64_t dim, float slope, int dtype,
                             void *workspace, size_t workspace_bytes,
                             ga_stream_t stream);
+
+/* ga_gat_aggregate / ga_gat_aggregate_from_z followed by the layer's activation
+ * (`h = F.elu(h)` between the layers of the reference's GAT network,
+ * examples/GAT/GAT.py; relu for GA_ACT_RELU; elu with alpha = 1) applied to the fp32
+ * row before it is rounded and stored, so the (n, heads * dim) result is not written,
+ * read and written again for it.  activation = GA_ACT_NONE is the plain entry point. */
+int ga_gat_aggregate_act(const int32_t *pointer, const int32_t *row_of_slot,
+                         const int32_t *nbr, const float *el, const float *er,
+                         const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                         int64_t heads, int64_t dim, float slope, int activation, int dtype,
+                         void *workspace, size_t workspace_bytes, ga_stream_t stream);
+int ga_gat_aggregate_from_z_act(const int32_t *pointer, const int32_t *row_of_slot,
+                                const int32_t *nbr, const float *a_l, const float *er,
+                                const void *z, void *out, int64_t n_rows, int64_t n_edges,
+                                int64_t heads, int64_t dim, float slope, int activation,
+                                int dtype, void *workspace, size_t workspace_bytes,
+                                ga_stream_t stream);
 
 /* The softmax-weighted reduction with per-edge operands:
  *   a = softmax_v(logit[e, h] over the in-edges e of v),

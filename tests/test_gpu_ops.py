@@ -636,6 +636,42 @@ def test_gat_aggregate_from_z(graph, device, heads, dim, bf16):
                  TOL_BF16 if bf16 else TOL_F32, f"gat from z on {name}")
 
 
+@pytest.mark.parametrize("heads,dim", [(1, 64), (4, 16), (3, 5)])
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("activation", ["elu", "relu"])
+def test_gat_aggregate_with_activation(graph, device, heads, dim, bf16, activation):
+    """The layer's activation applied by the fused pass to the rows it stores (the F.elu
+    between the layers of examples/GAT/GAT.py): activation(oracle chain) in float64; relu
+    also bit for bit against torch.relu of the plain result (it commutes with rounding)."""
+    name, g, arr = graph
+    n = arr.num_nodes
+    rng = np.random.default_rng(heads * 17 + dim)
+    z = rng.standard_normal((n, heads * dim), dtype=np.float32)
+    if bf16:
+        z = to_bf16_f32(z)
+    el = rng.standard_normal((n, heads), dtype=np.float32)
+    er = rng.standard_normal((n, heads), dtype=np.float32)
+    ref = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er, z, heads=heads,
+                               slope=0.2).astype(np.float64)
+    ref = np.where(ref > 0, ref, np.expm1(ref) if activation == "elu" else 0.0)
+    args = (_dev(el, device), _dev(er, device), _dev(z, device, bf16), g, 0.2)
+    got = ops.gat_aggregate(*args, activation=activation)
+    assert_close(got.float().cpu().numpy().reshape(ref.shape), ref,
+                 TOL_BF16 if bf16 else TOL_F32, f"gat + {activation} on {name}")
+    if activation == "relu":
+        assert torch.equal(got, torch.relu(ops.gat_aggregate(*args)))
+    if dim in (16, 64):          # head widths the source-term variant takes
+        a_l = (rng.standard_normal((heads, dim)) / np.sqrt(dim)).astype(np.float32)
+        plain = ops.gat_aggregate_from_z(_dev(a_l, device), _dev(er, device), _dev(z, device, bf16), g, 0.2)
+        fused = ops.gat_aggregate_from_z(_dev(a_l, device), _dev(er, device), _dev(z, device, bf16), g, 0.2,
+                                         activation=activation)
+        want = torch.relu(plain.float()) if activation == "relu" else torch.nn.functional.elu(plain.float())
+        assert_close(fused.float().cpu().numpy(), want.cpu().numpy(), TOL_BF16 if bf16 else TOL_F32,
+                     f"gat from z + {activation} on {name}")
+    with pytest.raises(RuntimeError):
+        ops.gat_aggregate(*args, activation="gelu")
+
+
 def test_gat_aggregate_from_z_unsupported_head_width(device):
     g = prepare_graph(np.array([0, 1]), np.array([1, 0]), 2, device=device)
     with pytest.raises(capi.GraphilerError):          # 24 / 4 = 6 lanes per head
