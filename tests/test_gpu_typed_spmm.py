@@ -34,13 +34,18 @@ def _dev(a, device, bf16=False):
 
 
 def _reference(arr, src, etype, r, x, w, norm):
+    """The operator chain on the oracle, and the magnitude its result is held against:
+    the same chain on absolute values (every product of the typed product and every
+    message of the sum counted with its size)."""
     etp = oracle.type_pointer(etype, r)
-    msg = oracle.segment_mm(etp, oracle.gather_rows(src, x), w)
-    if norm is not None:
-        msg = msg * norm[:, None]
-    msg = msg.astype(np.float32)
     args = (arr.in_pointer, arr.in_node_indices, arr.in_edge_indices)
-    return (oracle.spmm(*args, msg, op="copy_e"), oracle.spmm(*args, np.abs(msg), op="copy_e"))
+    out = []
+    for xx, ww in ((x, w), (np.abs(x), np.abs(w))):
+        msg = oracle.segment_mm(etp, oracle.gather_rows(src, xx), ww)
+        if norm is not None:
+            msg = msg * norm[:, None]
+        out.append(oracle.spmm(*args, msg.astype(np.float32), op="copy_e"))
+    return out[0], out[1]
 
 
 CASES = [  # nodes, edges, relations, K, hub
@@ -179,3 +184,28 @@ def test_typed_spmm_rejects_what_it_does_not_cover(device):
         ops.TypedSpMMEdge(x.cpu(), torch.randn(3, 16, 64), g)
     assert not ops.typed_spmm_supported(x, torch.randn(3, 16, 32, device=device))
     assert ops.typed_spmm_supported(x, torch.randn(3, 16, 64, device=device))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_typed_spmm_random_graphs(device, seed):
+    """Random sizes either side of a tile, relation counts from 1 to 200 (most of them
+    without edges in most tiles), a destination that takes a large share of the edges,
+    both dtypes, with and without the per-edge factor."""
+    rng = np.random.default_rng(500 + seed)
+    n = int(rng.choice([1, 17, 127, 128, 129, 144, 145, 1000, 5000]))
+    e = int(rng.choice([0, 1, 50, 3000, 40000]))
+    r = int(rng.choice([1, 2, 9, 60, 200]))
+    k = int(rng.choice([16, 32, 64]))
+    bf16 = bool(rng.integers(0, 2))
+    scaled = bool(rng.integers(0, 2))
+    g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device, hub=bool(rng.integers(0, 2)))
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    w = (rng.standard_normal((r, k, 64)) / np.sqrt(k)).astype(np.float32)
+    norm = rng.uniform(0.1, 1.5, e).astype(np.float32) if scaled else None
+    if bf16:
+        x, w = to_bf16_f32(x), to_bf16_f32(w)
+    got = ops.TypedSpMMEdge(_dev(x, device, bf16), _dev(w, device, bf16), g,
+                            row_scale=_dev(norm, device) if scaled else None)
+    ref, mag = _reference(arr, src, etype, r, x, w, norm)
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
+                 f"typed random n={n} e={e} r={r} k={k} bf16={bf16}", mag=mag)

@@ -125,3 +125,37 @@ def test_project_attn_wide(device, rows, K, M, heads):
     # el / er come from the fp32 accumulators, not from the rounded z
     assert_close(el.cpu().numpy(), (zh * a[0]).sum(-1), TOL_F32, "wide project el", mag=mag_l)
     assert_close(er.cpu().numpy(), (zh * a[1]).sum(-1), TOL_F32, "wide project er", mag=mag_r)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_wide_products_random_shapes(device, seed):
+    """Random row counts per type (empty types, a single row, types that end inside a
+    step), type counts either side of the kernel's limit of 64, K from 4 to 256, one to
+    four weights of 128 to 512 columns: whatever kernel a shape lands on, the result is
+    the oracle's and the stacked call gives the bits of separate calls."""
+    rng = np.random.default_rng(1000 + seed)
+    n_types = int(rng.choice([1, 2, 5, 63, 64, 65, 130]))
+    counts = rng.choice([0, 1, 7, 31, 128, 129, 300, 1000], size=n_types,
+                        p=[.2, .1, .1, .1, .1, .1, .2, .1])
+    if counts.sum() == 0:
+        counts[0] = 5
+    tp = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(tp[-1])
+    K = int(rng.choice([4, 8, 20, 32, 36, 64, 100, 128, 192, 256]))
+    M = int(rng.choice([128, 256, 384, 512]))
+    n_w = int(rng.integers(1, 5))
+    X = to_bf16_f32(rng.standard_normal((rows, K), dtype=np.float32))
+    Ws = [to_bf16_f32((rng.standard_normal((n_types, K, M)) / np.sqrt(K)).astype(np.float32))
+          for _ in range(n_w)]
+    dX, dtp = _dev(X, device, True), _dev(tp, device)
+    dWs = [_dev(w, device, True) for w in Ws]
+    outs = _stacked(dtp, dX, dWs, M, capi.GA_BF16)
+    lib = capi.load()
+    for w, dw, y in zip(Ws, dWs, outs):
+        assert_close(y.float().cpu().numpy(), oracle.segment_mm(tp, X, w), TOL_BF16,
+                     f"random wide T={n_types} rows={rows} K={K} M={M} n={n_w}")
+        one = torch.empty_like(y)
+        assert lib.ga_segment_mm(dtp.data_ptr(), n_types, dX.data_ptr(), dw.data_ptr(),
+                                 one.data_ptr(), rows, 1, K, M, capi.GA_BF16,
+                                 torch.cuda.current_stream().cuda_stream) == 0
+        assert torch.equal(one.view(torch.int16), y.view(torch.int16))
