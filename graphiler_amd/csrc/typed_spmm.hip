@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kBlock) void typed_fill_kernel(
     int32_t *__restrict__ slot_src, unsigned char *__restrict__ slot_dst,
     int32_t *__restrict__ slot_edge) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (p >= chunk_capacity * kChunk) return;
+  if (p >= chunk_capacity * kChunk) return;      // whole chunks: 16 neighbouring threads leave together
   const int64_t c = p / kChunk;
   int src = -1, edge = -1, dst = 0xff, type = 0;     // pad: no row of a tile
   if (c < chunk_base[n_groups]) {
@@ -130,7 +130,12 @@ __global__ __launch_bounds__(kBlock) void typed_fill_kernel(
   slot_src[p] = src;
   slot_edge[p] = edge;
   slot_dst[p] = (unsigned char)dst;
-  if ((p & (kChunk - 1)) == 0) chunk_type[c] = type;
+  // the 16-row blocks of the tile that the chunk has rows in, beside its relation: the 16
+  // threads of a chunk are neighbours in a wavefront
+  unsigned blocks = src >= 0 ? 1u << (dst >> 4) : 0u;
+#pragma unroll
+  for (int off = 1; off < kChunk; off <<= 1) blocks |= __shfl_xor(blocks, off);
+  if ((p & (kChunk - 1)) == 0) chunk_type[c] = type | (int)(blocks << 16);
 }
 
 inline size_t round_up(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -259,7 +264,7 @@ struct ChunkIds {
   int src;                // source node of row n (-1: pad)
   uint32_t dst4;          // destinations inside the tile of rows 4 q .. 4 q + 3, one byte each
   int edge;               // edge id of row 4 q + (n & 3) (-1: pad)
-  int type;               // relation of the chunk
+  int type;               // relation of the chunk | its block mask << 16
 };
 
 template <typename T, int KS>
@@ -267,6 +272,7 @@ struct ChunkData {
   TypedFrag<T, KS> f;
   float sc;               // scale of row 4 q + (n & 3)
   uint32_t dst4;
+  unsigned hit;           // blocks of the tile the chunk has rows in (the same in every lane)
 };
 
 // lane L of my row of 16 lanes
@@ -369,8 +375,10 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
   };
   auto load_data = [&](const ChunkIds &I, ChunkData<T, KS> &D) __attribute__((always_inline)) {
     TypedFrag<T, KS>::load_x(D.f, (const T *)A.x, (uint32_t)(I.src < 0 ? 0 : I.src), q);
-    const int type = __builtin_amdgcn_readfirstlane(I.type);
-    TypedFrag<T, KS>::load_w(D.f, (const T *)A.W + (int64_t)type * (16 * KS * kTypedM), w_lane);
+    const int word = __builtin_amdgcn_readfirstlane(I.type);     // relation | blocks << 16
+    TypedFrag<T, KS>::load_w(D.f, (const T *)A.W + (int64_t)(word & 0xffff) * (16 * KS * kTypedM),
+                             w_lane);
+    D.hit = (unsigned)word >> 16;
     D.sc = SCALED ? load_at<float>(A.row_scale, (uint32_t)(I.edge < 0 ? 0 : I.edge) * 4u) : 1.0f;
     D.dst4 = I.dst4;
   };
@@ -415,11 +423,7 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
     int u[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) u[j] = (int)((d.dst4 >> (8 * j)) & 0xffu) - n;
-    // blocks of the tile the chunk has rows in (a pad row says block 15)
-    unsigned hit = (1u << (d.dst4 >> 4 & 15u)) | (1u << (d.dst4 >> 12 & 15u)) |
-                   (1u << (d.dst4 >> 20 & 15u)) | (1u << (d.dst4 >> 28 & 15u));
-    hit = __builtin_amdgcn_readlane(hit, 0) | __builtin_amdgcn_readlane(hit, 16) |
-          __builtin_amdgcn_readlane(hit, 32) | __builtin_amdgcn_readlane(hit, 48);
+    const unsigned hit = d.hit;
     // tile[b] += S_b @ messages: S_b[i][r] = 1 where row r of the chunk goes to row
     // 16 b + i of the tile; lane (n, q) holds S_b[n][4 q .. 4 q + 3]
 #pragma unroll
@@ -630,6 +634,7 @@ int ga_typed_tiles_build(const int32_t *row_of_slot, const int32_t *nbr, const i
   if (n_rows < 0 || n_edges < 0 || n_types <= 0) return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || n_types > 0x7fffffff) return GA_EINVAL;
   if (!tile_rows_ok(tile_rows)) return GA_EINVAL;
+  if (n_types > 0xffff) return GA_EUNSUPPORTED;      // the relation shares a word with the block mask
   const int64_t n_tiles = tiles_of(n_rows, tile_rows), n_groups = n_tiles * n_types;
   if (n_groups > 0x7ffffffe) return GA_EUNSUPPORTED;
   const int64_t cap = ga_typed_tiles_chunk_capacity(n_rows, n_edges, n_types, tile_rows);

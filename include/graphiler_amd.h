@@ -200,7 +200,8 @@ int ga_sddmm_u_op_v_adj(const int32_t *pointer, const int32_t *row_of_slot,
  * chunks of 16 slots.  tile_rows is 128 or 144: ga_typed_tile_rows(n_rows) names the one
  * whose tiles fill whole rounds of this device's CUs best; the same value goes to every
  * call for the graph.  Outputs: tile_chunk_pointer (tiles + 1, tiles =
- * ceil(n_rows / tile_rows)), chunk_type (capacity), slot_src and slot_edge
+ * ceil(n_rows / tile_rows)), chunk_type (capacity: relation | mask of the chunk's 16-row
+ * blocks << 16; at most 65535 relations), slot_src and slot_edge
  * (16 * capacity, -1 in pad slots), slot_dst (16 * capacity bytes: destination - tile
  * start, 255 in pad slots; 4-byte aligned), capacity =
  * ga_typed_tiles_chunk_capacity(...).  Everything runs on `stream`; nothing is read

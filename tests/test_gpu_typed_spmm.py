@@ -105,10 +105,13 @@ def test_typed_tiles_layout(device):
     chunk_of_slot = np.arange(16 * total) // 16
     tile_of_chunk = np.searchsorted(tcp, np.arange(total), side="right") - 1
     assert np.array_equal(dst[ed], tile_of_chunk[chunk_of_slot[live]] * rows + sdst[used][live])
-    assert np.array_equal(etype[ed], ctype[:total][chunk_of_slot[live]])
+    assert np.array_equal(etype[ed], (ctype[:total] & 0xffff)[chunk_of_slot[live]])
+    blocks = np.zeros(total, dtype=np.int64)          # 16-row blocks a chunk has rows in
+    np.bitwise_or.at(blocks, chunk_of_slot[live], 1 << (sdst[used][live].astype(np.int64) >> 4))
+    assert np.array_equal(ctype[:total].astype(np.int64) >> 16, blocks)
     # order: relation ascending inside a tile; a group's slots in adjacency order
     for t in range(tiles):
-        ct = ctype[tcp[t]:tcp[t + 1]]
+        ct = ctype[tcp[t]:tcp[t + 1]] & 0xffff
         assert np.all(np.diff(ct) >= 0)
     slot_of_edge = np.empty(e, dtype=np.int64)
     slot_of_edge[arr.in_edge_indices] = np.arange(e)
