@@ -429,6 +429,35 @@ def test_segment_softmax_rows_over_many_chunks(device, heads):
     assert np.abs(sums[np.diff(arr.in_pointer) > 0] - 1.0).max() < 2e-5
 
 
+def test_segment_softmax_in_place(device):
+    """y == x is allowed at the C boundary (rows over many chunks and short ones, heads
+    on both kernel families) and gives the bits of the out-of-place call."""
+    lib = capi.load()
+    src, dst, n = _hub_graph(5)
+    g = prepare_graph(src, dst, n, device=device)
+    rng = np.random.default_rng(5)
+    for heads in (1, 4, 3):
+        x = _dev((rng.standard_normal((dst.shape[0], heads)) * 4.0).astype(np.float32), device)
+        want = ops.SegmentSoftmax(x, 1, None, g)
+        y = x.clone()
+        ws = g.workspace(lib.ga_softmax_workspace_bytes(g.num_edges, heads))
+        rc = lib.ga_segment_softmax(
+            g.in_pointer.data_ptr(), g.in_row_of_slot.data_ptr(),
+            None if g.in_eid_is_identity else g.in_edge_indices.data_ptr(),
+            y.data_ptr(), y.data_ptr(), g.num_nodes, g.num_edges, heads,
+            ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+        assert torch.equal(y, want), f"in-place softmax differs at H={heads}"
+        # an output that starts inside the input is refused before anything runs
+        both = torch.empty(x.numel() + heads, device=device)
+        rc = lib.ga_segment_softmax(
+            g.in_pointer.data_ptr(), g.in_row_of_slot.data_ptr(),
+            None if g.in_eid_is_identity else g.in_edge_indices.data_ptr(),
+            both.data_ptr(), both.data_ptr() + 4 * heads, g.num_nodes, g.num_edges, heads,
+            ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+        assert rc == capi.GA_EINVAL
+
+
 def _mask_some_logits(rng, ptr, eid, x):
     """-inf on about a third of the logits, keeping one finite logit per row and head."""
     x = x.copy()

@@ -121,6 +121,22 @@ def test_gat_aggregate_al_small_and_large_tables(setup, device):
         assert err <= TOL_F32, f"gat_aggregate_al differs by {err:.2e} at {n_nodes} nodes"
 
 
+def test_gat_aggregate_takes_bf16_attention_terms(setup, device):
+    """A bf16 plan whose projection was not rewritten hands el / er over in bf16: the
+    operator takes them (read as fp32) and gives what it gives for the same values in
+    fp32."""
+    sg, arr, rng = setup
+    heads, d = 2, 32
+    z = torch.randn(arr.num_nodes, heads, d, device=device).bfloat16()
+    el = torch.randn(arr.num_nodes, heads, 1, device=device).bfloat16()
+    er = torch.randn(arr.num_nodes, heads, 1, device=device).bfloat16()
+    got = torch.ops.my_ops.gat_aggregate(el, er, z, 0.2, sg)
+    want = torch.ops.my_ops.gat_aggregate(el.float(), er.float(), z, 0.2, sg)
+    assert got.dtype == torch.bfloat16 and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    with pytest.raises(RuntimeError):
+        torch.ops.my_ops.gat_aggregate(el.int(), er, z, 0.2, sg)
+
+
 def test_error_convention(setup, device):
     sg, arr, rng = setup
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):

@@ -50,6 +50,26 @@ def test_argument_rejection_without_gpu():
     assert lib.ga_spmm_workspace_bytes(1000, 64) >= 2 * 64 * 4
 
 
+def test_segment_softmax_rejects_partially_overlapping_buffers():
+    """y may be x (in place) or disjoint from it; anything in between would make a
+    later pass read results as logits.  The check runs before any launch and touches
+    no memory, so made-up addresses do for it (the in-place and disjoint calls stop
+    later, at the missing workspace)."""
+    lib = capi.load()
+    edges, heads = 1000, 4
+    nbytes = edges * heads * 4
+    ptr = row = 0x10000                    # non-null stand-ins, never dereferenced
+    x = 0x4000000
+
+    def call(y):
+        return lib.ga_segment_softmax(ptr, row, None, x, y, 10, edges, heads, None, 0, None)
+
+    for y in (x + 4, x - 4, x + nbytes - 4, x - nbytes + 4, x + nbytes // 2):
+        assert call(y) == capi.GA_EINVAL, hex(y)
+    assert lib.ga_softmax_workspace_bytes(edges, heads) > 0
+    for y in (x, x + nbytes, x - nbytes):
+        assert call(y) == capi.GA_EWORKSPACE, hex(y)
+
 @pytest.mark.parametrize("kind", ["uniform", "skewed", "empty"])
 def test_build_graph_arrays_matches_oracle_bit_exact(kind):
     rng = np.random.default_rng(3)

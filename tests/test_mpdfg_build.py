@@ -154,3 +154,58 @@ def test_build_errors():
         mpdfg_builder(U.gcn_message, bad_softmax)
     with pytest.raises(BuildError, match="annotated"):
         mpdfg_builder(untyped_message, U.gcn_reduce)
+
+
+# --- guards of single rewrites, on hand-written plans -------------------------------
+_DOT_PLAN = """
+graph(%g : __torch__.torch.classes.my_classes.DGLGraph, %x : Tensor, %w : WTYPE,
+      %q : Tensor, %s : Tensor):
+  %zero : int = prim::Constant[value=0]()
+  %one : int = prim::Constant[value=1]()
+  %true : bool = prim::Constant[value=1]()
+  %none : NoneType = prim::Constant()
+  %dims : int[] = prim::ListConstruct(%one)
+  %y : Tensor = my_ops::SegmentMMEdgeGather(%x, %w, %zero, SCALE, %g)
+  %b : Tensor = my_ops::BroadcastDstNode(%q, %g)
+  %m : Tensor = aten::mul(%y, %b)
+  %r : Tensor = aten::sum(%m, %dims, %true, %none)
+  return (%r)
+"""
+
+
+def _late_fused_kinds(ir):
+    from graphiler_amd import torch_boundary
+    from graphiler_amd.mpdfg import passes
+    from graphiler_amd.mpdfg.builder import MPDFG
+    torch_boundary.load()
+    plan = MPDFG(torch._C.parse_ir(ir), {})
+    rw = passes._Rewriter(plan)
+    for _ in range(4):
+        if not rw.late_fusion():
+            break
+    plan.graph.lint()
+    # the operator that produces the plan's result, and everything it reads
+    live, todo = [], [plan.graph.return_node()]
+    while todo:
+        for v in todo.pop().inputs():
+            if v.node().kind().startswith("my_ops::"):
+                live.append(v.node().kind())
+            todo.append(v.node())
+    return live
+
+
+def test_typed_product_and_dot_fuse_only_without_row_factor_and_heads():
+    """sum(gathered typed product * broadcast rows) becomes SegmentMMEdgeDot only when
+    the product has no per-row factor (the dot has no operand for one) and its weights
+    are not known to be (T, H, K, M) (the sum over dim 1 would then run across heads)."""
+    plain = _DOT_PLAN.replace("WTYPE", "Tensor").replace("SCALE", "%none")
+    assert _late_fused_kinds(plain) == ["my_ops::SegmentMMEdgeDot"]
+    three_d = _DOT_PLAN.replace("WTYPE", "Float(4, 16, 8)").replace("SCALE", "%none")
+    assert _late_fused_kinds(three_d) == ["my_ops::SegmentMMEdgeDot"]
+
+    scaled = _DOT_PLAN.replace("WTYPE", "Tensor").replace("SCALE", "%s")
+    assert sorted(_late_fused_kinds(scaled)) == ["my_ops::BroadcastDstNode",
+                                                 "my_ops::SegmentMMEdgeGather"]
+    heads = _DOT_PLAN.replace("WTYPE", "Float(4, 2, 16, 8)").replace("SCALE", "%none")
+    assert sorted(_late_fused_kinds(heads)) == ["my_ops::BroadcastDstNode",
+                                                "my_ops::SegmentMMEdgeGather"]
