@@ -370,18 +370,16 @@ def main():
                 v["ops"][f"rgcn_layer_{K}_{M}"] = op_record(
                     f"c3.rgcn_layer_{K}_{M}_{tag}", lambda: layers.rgcn_layer(g, xin, w, norm, fused=True),
                     lbytes, 2.0 * E * K * M, tag, reps=50)
-                if (K, M) == (16, 64):
-                    # the same layer by its two implementations: the operator pair over an
-                    # (E, M) message tensor, and the single pass over destination tiles
-                    v["ops"]["rgcn_layer_16_64_two_pass"] = op_record(
-                        f"c3.rgcn_layer_16_64_two_pass_{tag}",
-                        lambda: ops.SpMMEdge(ops.SegmentMMEdgeGather(xin, w, 0, g, row_scale=norm),
-                                             [1], False, None, g),
-                        lbytes + 2 * E * M * b, 2.0 * E * K * M, tag, reps=50)
-                    v["ops"]["rgcn_layer_16_64_tiles"] = op_record(
-                        f"c3.rgcn_layer_16_64_tiles_{tag}",
-                        lambda: layers.rgcn_layer(g, xin, w, norm, fused="tiles"),
-                        lbytes, 2.0 * E * K * M, tag, reps=50)
+                # the same layer by its two implementations: the operator pair over an
+                # (E, M) message tensor, and the single pass over destination tiles
+                v["ops"][f"rgcn_layer_{K}_{M}_two_pass"] = op_record(
+                    f"c3.rgcn_layer_{K}_{M}_two_pass_{tag}",
+                    lambda: layers.rgcn_layer(g, xin, w, norm, fused="pair"),
+                    lbytes + 2 * E * M * b, 2.0 * E * K * M, tag, reps=50)
+                v["ops"][f"rgcn_layer_{K}_{M}_tiles"] = op_record(
+                    f"c3.rgcn_layer_{K}_{M}_tiles_{tag}",
+                    lambda: layers.rgcn_layer(g, xin, w, norm, fused="tiles"),
+                    lbytes, 2.0 * E * K * M, tag, reps=50)
                 if args.no_ops:
                     continue
                 v["ops"][f"segment_mm_gather_{K}_{M}"] = op_record(

@@ -537,7 +537,8 @@ torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
 
 // SpMMEdge(SegmentMMEdgeGather(features, weights, 0, row_scale)): an RGCN layer's message
 // and reduce steps (examples/RGCN/RGCN.py:25-33).  One pass without the per-edge
-// messages where that kernel is the faster one (16 -> 64), the two operators elsewhere.
+// messages where that kernel is the faster one (the small products: K * M up to 2048,
+// e.g. 16 -> 64 and 64 -> 8), the two operators elsewhere.
 torch::Tensor TypedSpMMEdge(torch::Tensor features, torch::Tensor weights,
                             at::optional<torch::Tensor> row_scale, const GraphPtr &graph) {
   const MmShape s = edge_mm_shape(features, weights, graph);
@@ -551,7 +552,8 @@ torch::Tensor TypedSpMMEdge(torch::Tensor features, torch::Tensor weights,
       plain_scale = true;
     }
   }
-  if (plain_scale && weights.dim() == 3 && features.dim() == 2 && s.K == 16 && s.M == 64) {
+  if (plain_scale && weights.dim() == 3 && features.dim() == 2 && s.K % 16 == 0 &&
+      s.K * s.M <= 2048) {
     const DGLGraph::TypedTiles &t = graph->typed_tiles();
     torch::Tensor out = torch::empty({graph->num_nodes, s.M}, features.options());
     const int rc = ga_typed_spmm(

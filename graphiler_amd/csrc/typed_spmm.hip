@@ -14,11 +14,13 @@
 //     chunks of 16 slots, and per padded slot the source node, the destination inside
 //     the tile and the edge id are written out, per chunk its relation, per tile its
 //     first chunk.  A pad slot has source and edge id -1.
-//   kernel   one workgroup of four wavefronts per tile; a wavefront owns 32 of the 64
-//     output columns and walks every second chunk of the tile (two wavefronts share a
-//     chunk, one per column half); its 128 x 32 fp32 partial sums stay in matrix-core
-//     accumulators (64 registers), and the partial tiles meet in LDS at the end.  Per chunk it gathers the 16 source
-//     rows (one 16- or 8-byte read per lane), multiplies them with its 16 columns of the
+//   kernel   one workgroup of four wavefronts per tile.  With 64 output columns a
+//     wavefront owns 32 of them and walks every second chunk of the tile (two
+//     wavefronts share a chunk, one per column half); with 32, 16 or 8 columns it owns
+//     them all and walks every fourth chunk.  Its 128 x 32 (or narrower) fp32 partial
+//     sums stay in matrix-core accumulators (64 registers), and the partial tiles meet
+//     in LDS at the end.  Per chunk it gathers the 16 source rows (one 16- or 8-byte
+//     read per lane and 16 input features), multiplies them with its columns of the
 //     relation's weights (K / 4 v_mfma_f32_16x16x4_f32, or K / 16
 //     v_mfma_f32_16x16x16_bf16) and scales the 16 x 16 result rows: the messages.  The
 //     sum over destinations is a second matrix product: tile block b += S_b @ messages
@@ -32,9 +34,10 @@
 //     neighbours: they are replaced by zero and remembered as one bit per element and
 //     kind (+inf, -inf, NaN), which the final write adds back in.
 //
-// Chunk ids and source rows are requested four and two chunks ahead of the arithmetic.
+// Chunk ids and source rows are requested two and one of the wavefront's own chunks
+// ahead of the arithmetic.
 // HBM traffic per edge: 9 index bytes (+ padding), the 4-byte scale, the K b-byte
-// source row (from L2 when x fits) and 64 b / degree output bytes.
+// source row (from L2 when x fits) and M b / degree output bytes.
 #include "common.h"
 
 #include <rocprim/device/device_radix_sort.hpp>
@@ -51,8 +54,9 @@ typedef short shortx4 __attribute__((ext_vector_type(4)));
 constexpr int kMaxTileRows = 144;
 inline bool tile_rows_ok(int64_t r) { return r == 128 || r == 144; }
 constexpr int kChunk = 16;                      // slots per chunk: rows of one MFMA
-constexpr int kTypedM = 64;                     // output columns: 4 wavefronts x 16
-constexpr int kTypedBlock = 4 * kWave;
+constexpr int kTypedWaves = 4;
+constexpr int kTypedBlock = kTypedWaves * kWave;
+inline bool typed_cols_ok(int64_t m) { return m == 8 || m == 16 || m == 32 || m == 64; }
 
 // ------------------------------------------------------------------ preparation ----
 // key of a slot: tile * n_types + relation
@@ -187,17 +191,28 @@ __device__ __forceinline__ V load_at(const void *base, uint32_t byte_offset) {
   return *reinterpret_cast<const V *>(reinterpret_cast<const char *>(base) + byte_offset);
 }
 
-// A wavefront owns kCB of the four 16-column blocks of the tile and walks every kCB-th
-// chunk: 4 / kCB wavefronts share a chunk (one per column group), kCB take turns on the
-// chunks.  Two blocks = a 128 x 32 tile per wavefront (64 accumulator registers): three
-// wavefronts fit a SIMD and the whole grid is resident at once.
-constexpr int kCB = 2;
-constexpr int kColGroups = 4 / kCB;
-template <typename T, int KS>
+// How the MC output columns are shared out.  A wavefront owns kCB 16-column blocks of
+// the tile (at most two: a 128 x 32 tile per wavefront is 64 accumulator registers,
+// three wavefronts fit a SIMD and the whole grid is resident at once); the blocks of a
+// tile make kColGroups groups of kCB, one wavefront per group works on a chunk, and the
+// kTurns wavefronts of a group take turns on the chunks of the tile.  Eight columns run
+// as a block of 16 whose upper half repeats the lower one and is never stored.
+template <int MC>
+struct Cols {
+  static constexpr int kBlocks = MC >= 16 ? MC / 16 : 1;
+  static constexpr int kCB = kBlocks >= 2 ? 2 : 1;
+  static constexpr int kColGroups = kBlocks / kCB;
+  static constexpr int kTurns = kTypedWaves / kColGroups;
+  static constexpr int kMergeStride = MC + 4;   // row stride of the LDS tile the waves meet in
+  // column of the weights behind lane n of block 0
+  static __device__ __forceinline__ uint32_t lane_col(int n) { return MC >= 16 ? n : n % MC; }
+};
+template <typename T, int KS, int MC>
 struct TypedFrag;
 
-template <int KS>
-struct TypedFrag<float, KS> {
+template <int KS, int MC>
+struct TypedFrag<float, KS, MC> {
+  static constexpr int kCB = Cols<MC>::kCB;
   float4 x[KS];           // row n of the chunk: k = 16 j + 4 q .. + 3
   float w[kCB][KS][4];    // my column block c: W[16 j + 4 q + s][16 (cb0 + c) + n]
   static __device__ __forceinline__ void load_x(TypedFrag &f, const float *x, uint32_t row, int q) {
@@ -205,7 +220,9 @@ struct TypedFrag<float, KS> {
     for (int j = 0; j < KS; ++j)
       f.x[j] = load_at<float4>(x, (row * (16u * KS) + 16u * j + 4u * q) * 4u);
   }
-  // wt: the relation's weights (uniform); lane_off: element (4 q, n) of them
+  // wt: the relation's weights (uniform); lane_off: element (4 q, n) of them.  One
+  // element per load: reading them four at a time from a copy of the weights stored
+  // column by column measured slower (16 cache lines per load instead of 4).
   static __device__ __forceinline__ void load_w(TypedFrag &f, const float *wt, uint32_t lane_off) {
 #pragma unroll
     for (int cb = 0; cb < kCB; ++cb)
@@ -213,7 +230,7 @@ struct TypedFrag<float, KS> {
       for (int j = 0; j < KS; ++j)
 #pragma unroll
         for (int s = 0; s < 4; ++s)
-          f.w[cb][j][s] = load_at<float>(wt, (lane_off + (16u * j + s) * kTypedM + 16u * cb) * 4u);
+          f.w[cb][j][s] = load_at<float>(wt, (lane_off + (16u * j + s) * MC + 16u * cb) * 4u);
   }
   static __device__ __forceinline__ floatx4 mma(const TypedFrag &f, int cb) {
     floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -228,8 +245,9 @@ struct TypedFrag<float, KS> {
   }
 };
 
-template <int KS>
-struct TypedFrag<bf16_t, KS> {
+template <int KS, int MC>
+struct TypedFrag<bf16_t, KS, MC> {
+  static constexpr int kCB = Cols<MC>::kCB;
   uint2 x[KS];            // four bf16: k = 16 j + 4 q .. + 3
   uint2 w[kCB][KS];       // my column block c: W[16 j + 4 q .. + 3][16 (cb0 + c) + n]
   static __device__ __forceinline__ void load_x(TypedFrag &f, const bf16_t *x, uint32_t row, int q) {
@@ -245,7 +263,7 @@ struct TypedFrag<bf16_t, KS> {
         uint32_t h[4];
 #pragma unroll
         for (int s = 0; s < 4; ++s)
-          h[s] = load_at<bf16_t>(wt, (lane_off + (16u * j + s) * kTypedM + 16u * cb) * 2u);
+          h[s] = load_at<bf16_t>(wt, (lane_off + (16u * j + s) * MC + 16u * cb) * 2u);
         f.w[cb][j] = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
       }
   }
@@ -267,9 +285,9 @@ struct ChunkIds {
   int type;               // relation of the chunk | its block mask << 16
 };
 
-template <typename T, int KS>
+template <typename T, int KS, int MC>
 struct ChunkData {
-  TypedFrag<T, KS> f;
+  TypedFrag<T, KS, MC> f;
   float sc;               // scale of row 4 q + (n & 3)
   uint32_t dst4;
   unsigned hit;           // blocks of the tile the chunk has rows in (the same in every lane)
@@ -336,10 +354,9 @@ __device__ __forceinline__ void store_row4(bf16_t *p, const float4 &v) {
   *reinterpret_cast<uint2 *>(p) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
 }
 
-constexpr int kMergeStride = kTypedM + 4;     // row stride of the LDS tile the waves meet in
-
 // Elements of a tile that received a message that is not finite, by kind: bit
 // 4 b + i of word cb is element (b, cb, i) of the lane (up to 9 blocks: 36 bits).
+template <int kCB>
 struct Poison {
   uint64_t pinf[kCB], ninf[kCB], nan[kCB];
 };
@@ -351,15 +368,19 @@ struct TypedArgs {
   const float *row_scale;
 };
 
-// The chunks first, first + kCB, ... < c1 of a tile into the lane's share of the
+// The chunks first, first + kTurns, ... < c1 of a tile into the lane's share of the
 // wavefront's 128 x (16 kCB) tile: tile[b][c][i] = row 16 b + 4 q + i, column 16 c + n of
 // the wavefront's columns (w_lane already points at them).  CHECKED: messages that
 // are not finite are replaced by zero and recorded in `poison`.
-template <typename T, int KS, bool SCALED, bool CHECKED, int NB>
+template <typename T, int KS, int MC, bool SCALED, bool CHECKED, int NB>
 __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c1, int n, int q,
-                                            floatx4 (&tile)[NB][kCB], Poison &poison) {
+                                            floatx4 (&tile)[NB][Cols<MC>::kCB],
+                                            Poison<Cols<MC>::kCB> &poison) {
   constexpr int kTerms = Terms<T>::kTerms;
-  const uint32_t w_lane = (4u * q) * kTypedM + n;
+  constexpr int kCB = Cols<MC>::kCB, kTurns = Cols<MC>::kTurns;
+  using Frag = TypedFrag<T, KS, MC>;
+  using Data = ChunkData<T, KS, MC>;
+  const uint32_t w_lane = (4u * q) * MC + Cols<MC>::lane_col(n);
   // Loads are issued without branches around them (a chunk index past the end reads the
   // last chunk again, a pad slot reads row 0 of x and edge 0 of the scale; no row of a
   // tile selects what they produce): the waits for the loads of the chunk before then
@@ -373,16 +394,15 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
     // type of the chunk at hand would also wait for the one requested just now.
     I.type = __hip_atomic_load(A.chunk_type + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
-  auto load_data = [&](const ChunkIds &I, ChunkData<T, KS> &D) __attribute__((always_inline)) {
-    TypedFrag<T, KS>::load_x(D.f, (const T *)A.x, (uint32_t)(I.src < 0 ? 0 : I.src), q);
+  auto load_data = [&](const ChunkIds &I, Data &D) __attribute__((always_inline)) {
+    Frag::load_x(D.f, (const T *)A.x, (uint32_t)(I.src < 0 ? 0 : I.src), q);
     const int word = __builtin_amdgcn_readfirstlane(I.type);     // relation | blocks << 16
-    TypedFrag<T, KS>::load_w(D.f, (const T *)A.W + (int64_t)(word & 0xffff) * (16 * KS * kTypedM),
-                             w_lane);
+    Frag::load_w(D.f, (const T *)A.W + (int64_t)(word & 0xffff) * (16 * KS * MC), w_lane);
     D.hit = (unsigned)word >> 16;
     D.sc = SCALED ? load_at<float>(A.row_scale, (uint32_t)(I.edge < 0 ? 0 : I.edge) * 4u) : 1.0f;
     D.dst4 = I.dst4;
   };
-  auto compute = [&](const ChunkData<T, KS> &d) __attribute__((always_inline)) {
+  auto compute = [&](const Data &d) __attribute__((always_inline)) {
     // ---- messages of the chunk: rows 4 q + i, columns 16 cb + n ------------------------
     float sc[4] = {1.0f, 1.0f, 1.0f, 1.0f};
     if (SCALED) {
@@ -392,7 +412,7 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
     uint2 t[kCB][kTerms];
 #pragma unroll
     for (int cb = 0; cb < kCB; ++cb) {
-      const floatx4 acc = TypedFrag<T, KS>::mma(d.f, cb);
+      const floatx4 acc = Frag::mma(d.f, cb);
       float m[4] = {acc[0] * sc[0], acc[1] * sc[1], acc[2] * sc[2], acc[3] * sc[3]};
       if (CHECKED) {
         bool fin = true;
@@ -443,31 +463,41 @@ __device__ __forceinline__ void walk_chunks(const TypedArgs &A, int first, int c
   };
 
   if (first >= c1) return;
-  // Two sets of registers take turns (the loop is unrolled twice, so no copies): the ids
-  // of one of my chunks are requested two, its rows and weights one of my chunks ahead of
-  // the arithmetic (a third set did not pay for its registers).  Ids are requested before
-  // the rows of the same step: the wait for them at the next step then leaves that step's
-  // rows and weights in flight (loads return in order).
-  ChunkIds ia, ib;
-  ChunkData<T, KS> d0, d1;
-  load_ids(first, ia);
-  load_ids(first + kCB, ib);
-  load_data(ia, d0);
-  for (int c = first; c < c1; c += 2 * kCB) {
-    load_ids(c + 2 * kCB, ia);
-    load_data(ib, d1);
-    compute(d0);
-    load_ids(c + 3 * kCB, ib);
-    load_data(ia, d0);
-    if (c + kCB < c1) compute(d1);
+  // kDepth sets of registers take turns (the loop is unrolled kDepth times, so no
+  // copies): the ids of one of my chunks are requested kDepth, its rows and weights
+  // kDepth - 1 of my chunks ahead of the arithmetic.  Ids are requested before the rows
+  // of the same step: the wait for them at the next step then leaves that step's rows
+  // and weights in flight (loads return in order).  Three and four sets measured slower
+  // at every shape (fewer wavefronts fit, and the kernel is not waiting for memory).
+  constexpr int kDepth = 2;
+  ChunkIds ids[kDepth];
+  Data data[kDepth];
+#pragma unroll
+  for (int s = 0; s < kDepth; ++s) load_ids(first + s * kTurns, ids[s]);
+#pragma unroll
+  for (int s = 0; s + 1 < kDepth; ++s) load_data(ids[s], data[s]);
+  for (int c = first; c < c1; c += kDepth * kTurns) {
+#pragma unroll
+    for (int s = 0; s < kDepth; ++s) {
+      constexpr int kLast = kDepth - 1;
+      load_ids(c + (s + kDepth) * kTurns, ids[s]);
+      load_data(ids[(s + kLast) % kDepth], data[(s + kLast) % kDepth]);
+      if (s == 0 || c + s * kTurns < c1) compute(data[s]);
+    }
   }
 }
 
-template <typename T, int KS, bool SCALED, int NB>
-__global__ __launch_bounds__(kTypedBlock, KS == 1 ? 3 : 1) void typed_tiles_kernel(
+// Wavefronts per SIMD the kernel is compiled for: three where the registers allow it
+// without spilling (one k step of 16), no promise otherwise.
+constexpr int typed_waves_per_simd(int KS, int MC) { return KS == 1 ? 3 : 1; }
+
+template <typename T, int KS, int MC, bool SCALED, int NB>
+__global__ __launch_bounds__(kTypedBlock, typed_waves_per_simd(KS, MC)) void typed_tiles_kernel(
     const int32_t *__restrict__ tile_chunk_pointer, TypedArgs A, T *__restrict__ out,
     int64_t n_rows) {
   constexpr int kTileRows = 16 * NB;
+  constexpr int kCB = Cols<MC>::kCB, kColGroups = Cols<MC>::kColGroups, kTurns = Cols<MC>::kTurns;
+  constexpr int kMergeStride = Cols<MC>::kMergeStride;
   static_assert(4 * NB <= 64 && kTileRows <= kMaxTileRows, "one bit per tile element of a lane");
   __shared__ __attribute__((aligned(16))) float merged[kTileRows * kMergeStride];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -478,7 +508,7 @@ __global__ __launch_bounds__(kTypedBlock, KS == 1 ? 3 : 1) void typed_tiles_kern
   const int colgroup = wave % kColGroups, turn = wave / kColGroups;
   A.W = static_cast<const T *>(A.W) + 16 * kCB * colgroup;
   floatx4 tile[NB][kCB];
-  Poison poison;
+  Poison<kCB> poison;
 #pragma unroll
   for (int cb = 0; cb < kCB; ++cb) poison.pinf[cb] = poison.ninf[cb] = poison.nan[cb] = 0ull;
   auto clear = [&]() __attribute__((always_inline)) {
@@ -488,7 +518,7 @@ __global__ __launch_bounds__(kTypedBlock, KS == 1 ? 3 : 1) void typed_tiles_kern
       for (int cb = 0; cb < kCB; ++cb) tile[b][cb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
   };
   clear();
-  walk_chunks<T, KS, SCALED, false, NB>(A, c0 + turn, c1, n, q, tile, poison);
+  walk_chunks<T, KS, MC, SCALED, false, NB>(A, c0 + turn, c1, n, q, tile, poison);
   // A message that is not finite turns the zeros of the selection matrix into NaN for
   // the rows around it.  Such a message leaves something that is not finite in the tile:
   // then the wavefront walks its chunks again, keeping those messages out of the matrix
@@ -502,7 +532,7 @@ __global__ __launch_bounds__(kTypedBlock, KS == 1 ? 3 : 1) void typed_tiles_kern
       for (int i = 0; i < 4; ++i) fin = fin && is_finite(tile[b][cb][i]);
   if (__builtin_amdgcn_ballot_w64(!fin) != 0) {
     clear();
-    walk_chunks<T, KS, SCALED, true, NB>(A, c0 + turn, c1, n, q, tile, poison);
+    walk_chunks<T, KS, MC, SCALED, true, NB>(A, c0 + turn, c1, n, q, tile, poison);
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -517,8 +547,8 @@ __global__ __launch_bounds__(kTypedBlock, KS == 1 ? 3 : 1) void typed_tiles_kern
   }
   // ---- the partial tiles meet in LDS: the column groups side by side, the wavefronts of
   // a group one after the other in a fixed order ------------------------------------------
-  for (int w = 0; w < kCB; ++w) {
-    if (turn == w) {
+  for (int w = 0; w < kTurns; ++w) {
+    if (turn == w && (MC >= 16 || n < MC)) {
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
 #pragma unroll
@@ -536,32 +566,43 @@ __global__ __launch_bounds__(kTypedBlock, KS == 1 ? 3 : 1) void typed_tiles_kern
   }
   // ---- and go to memory: a thread moves four columns of a row at a time -----------------
   const int64_t row0 = (int64_t)blockIdx.x * kTileRows;
-  for (int i = threadIdx.x; i < kTileRows * (kTypedM / 4); i += kTypedBlock) {
-    const int r = i / (kTypedM / 4), c4 = i % (kTypedM / 4);
+  for (int i = threadIdx.x; i < kTileRows * (MC / 4); i += kTypedBlock) {
+    const int r = i / (MC / 4), c4 = i % (MC / 4);
     if (row0 + r < n_rows)
-      store_row4(out + (row0 + r) * kTypedM + 4 * c4,
+      store_row4(out + (row0 + r) * MC + 4 * c4,
                  *reinterpret_cast<const float4 *>(merged + r * kMergeStride + 4 * c4));
   }
 }
 
-template <typename T, int KS, int NB>
+template <typename T, int KS, int MC, int NB>
 int launch_typed_nb(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows,
                     hipStream_t s) {
   const dim3 grid((unsigned)tiles_of(n_rows, 16 * NB));
   if (A.row_scale)
-    hipLaunchKernelGGL((typed_tiles_kernel<T, KS, true, NB>), grid, dim3(kTypedBlock), 0, s, tcp, A,
-                       (T *)out, n_rows);
+    hipLaunchKernelGGL((typed_tiles_kernel<T, KS, MC, true, NB>), grid, dim3(kTypedBlock), 0, s,
+                       tcp, A, (T *)out, n_rows);
   else
-    hipLaunchKernelGGL((typed_tiles_kernel<T, KS, false, NB>), grid, dim3(kTypedBlock), 0, s, tcp, A,
-                       (T *)out, n_rows);
+    hipLaunchKernelGGL((typed_tiles_kernel<T, KS, MC, false, NB>), grid, dim3(kTypedBlock), 0, s,
+                       tcp, A, (T *)out, n_rows);
   return launch_status();
+}
+
+template <typename T, int KS, int MC>
+int launch_typed_mc(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows,
+                    int64_t tile_rows, hipStream_t s) {
+  if (tile_rows == 144) return launch_typed_nb<T, KS, MC, 9>(tcp, A, out, n_rows, s);
+  return launch_typed_nb<T, KS, MC, 8>(tcp, A, out, n_rows, s);
 }
 
 template <typename T, int KS>
 int launch_typed(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows,
-                 int64_t tile_rows, hipStream_t s) {
-  if (tile_rows == 144) return launch_typed_nb<T, KS, 9>(tcp, A, out, n_rows, s);
-  return launch_typed_nb<T, KS, 8>(tcp, A, out, n_rows, s);
+                 int64_t tile_rows, int64_t M, hipStream_t s) {
+  switch (M) {
+    case 8: return launch_typed_mc<T, KS, 8>(tcp, A, out, n_rows, tile_rows, s);
+    case 16: return launch_typed_mc<T, KS, 16>(tcp, A, out, n_rows, tile_rows, s);
+    case 32: return launch_typed_mc<T, KS, 32>(tcp, A, out, n_rows, tile_rows, s);
+    default: return launch_typed_mc<T, KS, 64>(tcp, A, out, n_rows, tile_rows, s);
+  }
 }
 
 // Workgroups of the kernel that a CU holds at once (three wavefronts per SIMD by its
@@ -695,7 +736,7 @@ int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
   if (!tile_rows_ok(tile_rows)) return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff) return GA_EINVAL;
   if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
-  if (M != kTypedM || K % 16 != 0 || K > 64) return GA_EUNSUPPORTED;
+  if (!typed_cols_ok(M) || K % 16 != 0 || K > 64 || n_types > 0xffff) return GA_EUNSUPPORTED;
   const size_t esz = dtype == GA_F32 ? 4 : 2;
   // the kernel addresses x, one relation of W and row_scale with 32-bit byte offsets,
   // the slot arrays with 32-bit indices
@@ -713,7 +754,8 @@ int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
   hipStream_t s = (hipStream_t)stream;
   const TypedArgs A{chunk_type, slot_src, slot_edge, (const uint32_t *)slot_dst, x, W, row_scale};
   const int ks = (int)(K / 16);
-#define GA_TYPED(T, KS) return launch_typed<T, KS>(tile_chunk_pointer, A, out, n_rows, tile_rows, s)
+#define GA_TYPED(T, KS) \
+  return launch_typed<T, KS>(tile_chunk_pointer, A, out, n_rows, tile_rows, M, s)
   if (dtype == GA_F32) {
     switch (ks) {
       case 1: GA_TYPED(float, 1);

@@ -104,14 +104,16 @@ def rgcn_layer(g: DGLGraph, h, weight, norm, fused=True):
 
     ``fused=True``: the typed product reads the source rows through the COO column
     and applies the norm to the rows it produces, then the neighbour sum (two
-    passes over an (E, M) message tensor); for 16 -> 64 layers, where it is the
-    faster one, the single pass of ``fused="tiles"``.
+    passes over an (E, M) message tensor); for the small products where it is the
+    faster one (ops.typed_spmm_preferred: 16 -> 64, 64 -> 8, ...), the single pass
+    of ``fused="tiles"``.
+    ``fused="pair"``: always the two passes.
     ``fused="tiles"``: ops.TypedSpMMEdge, one pass without the message tensor
-    (M = 64, K in 16, 32, 48, 64).
+    (K in 16, 32, 48, 64; M in 8, 16, 32, 64).
     ``fused=False``: the reference's plan BroadcastSrcNode -> SegmentMMEdge ->
     mul(norm) -> SpMMEdge."""
-    if fused == "tiles" or (fused is True and weight.dim() == 3 and h.dim() == 2
-                            and tuple(weight.shape[1:]) == (16, 64)):
+    if fused == "tiles" or (fused is True and h.dim() == 2
+                            and ops.typed_spmm_preferred(h, weight)):
         return ops.TypedSpMMEdge(h, weight, g, row_scale=norm.float().contiguous())
     if fused:
         msg = ops.SegmentMMEdgeGather(h, weight, 0, g, row_scale=norm.float().contiguous())

@@ -586,10 +586,18 @@ def _typed_tiles(graph: DGLGraph):
 
 
 def typed_spmm_supported(features, weights) -> bool:
-    """Shapes TypedSpMMEdge takes: 64 output features, 16 / 32 / 48 / 64 input features."""
-    return weights.dim() == 3 and int(weights.shape[2]) == 64 \
+    """Shapes TypedSpMMEdge takes: 16 / 32 / 48 / 64 input features, 8 / 16 / 32 / 64
+    output features."""
+    return weights.dim() == 3 and int(weights.shape[2]) in (8, 16, 32, 64) \
         and int(weights.shape[1]) in (16, 32, 48, 64) \
         and get_feat_dim(features) == int(weights.shape[1])
+
+
+def typed_spmm_preferred(features, weights) -> bool:
+    """Shapes at which the one-pass kernel beats SegmentMMEdgeGather + SpMMEdge: the
+    small products (K * M up to 2048; at 64 x 64 the pair is the faster one)."""
+    return typed_spmm_supported(features, weights) \
+        and int(weights.shape[1]) * int(weights.shape[2]) <= 2048
 
 
 def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None) -> torch.Tensor:
@@ -597,7 +605,8 @@ def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None) -> torch.T
     in one pass (examples/RGCN/RGCN.py:25-33; broadcast.cu:58-63, segment_mm.cu:29-33,
     spmm.cu:359-373): out[v] = sum over the in-edges e of v of
     row_scale[e] * features[src(e)] @ weights[type(e)].  No per-edge tensor is written.
-    features (N, K), weights (R, K, 64) with K in 16, 32, 48, 64; ``row_scale`` (E,) or
+    features (N, K), weights (R, K, M) with K in 16, 32, 48, 64 and M in 8, 16, 32, 64;
+    ``row_scale`` (E,) or
     (E, 1) fp32.  The additions of a row happen in the order of the prepared layout
     (by relation, then adjacency order), the same in every call."""
     _check_input(features, "features")

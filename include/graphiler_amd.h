@@ -208,9 +208,10 @@ int ga_sddmm_u_op_v_adj(const int32_t *pointer, const int32_t *row_of_slot,
  * back.
  *
  * ga_typed_spmm: x (n_src, K), W (n_types, K, M), out (n_rows, M) of `dtype`;
- * row_scale (n_edges,) fp32 in edge-id order or null.  M must be 64, K one of 16, 32,
- * 48, 64, and x and row_scale smaller than 4 GiB (GA_EUNSUPPORTED otherwise: use
- * ga_segment_mm_gather + ga_spmm_csr).  The sum over the in-edges runs on the matrix
+ * row_scale (n_edges,) fp32 in edge-id order or null.  M must be 8, 16, 32 or 64, K one
+ * of 16, 32, 48, 64, and x and row_scale smaller than 4 GiB (GA_EUNSUPPORTED otherwise:
+ * use ga_segment_mm_gather + ga_spmm_csr, which are also the faster pair from about
+ * K * M = 4096 on).  The sum over the in-edges runs on the matrix
  * cores with fp32 accumulation: bf16 messages enter as the two-operator chain rounds
  * them, fp32 messages as three bf16 terms that carry 24 bits.  The order of the
  * additions is fixed by the prepared layout, so repeated calls give identical bits;

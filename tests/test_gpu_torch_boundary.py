@@ -166,7 +166,7 @@ def test_typed_sum_and_stacked_products_through_torchscript(device):
     sg = torch_boundary.script_graph(g)
     ops = torch.ops.my_ops
     norm = _t(rng.uniform(0.1, 1.0, (e, 1)).astype(np.float32), device)
-    for k, m in ((16, 64), (32, 64), (16, 24)):
+    for k, m in ((16, 64), (32, 64), (64, 8), (64, 64), (16, 24)):      # one pass, one pass, one pass, pair, pair
         x = _t(rng.standard_normal((n, k), dtype=np.float32), device)
         w = _t((rng.standard_normal((r, k, m)) / np.sqrt(k)).astype(np.float32), device)
         want = pyops.SpMMEdge(pyops.SegmentMMEdgeGather(x, w, 0, g, row_scale=norm), [1], False, None, g)

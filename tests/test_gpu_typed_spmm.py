@@ -48,34 +48,42 @@ def _reference(arr, src, etype, r, x, w, norm):
     return out[0], out[1]
 
 
-CASES = [  # nodes, edges, relations, K, hub
-    (300, 4000, 7, 16, False),
-    (1000, 20000, 60, 16, True),
-    (130, 900, 3, 32, False),
-    (257, 5000, 11, 48, True),
-    (128, 3000, 5, 64, False),
-    (5, 40, 2, 16, False),
-    (700, 0, 4, 16, False),
+CASES = [  # nodes, edges, relations, K, M, hub
+    (300, 4000, 7, 16, 64, False),
+    (1000, 20000, 60, 16, 64, True),
+    (130, 900, 3, 32, 64, False),
+    (257, 5000, 11, 48, 64, True),
+    (128, 3000, 5, 64, 64, False),
+    (5, 40, 2, 16, 64, False),
+    (700, 0, 4, 16, 64, False),
+    # narrower outputs: one wavefront per chunk, four taking turns on a tile's chunks
+    (1000, 20000, 60, 64, 8, True),
+    (300, 4000, 7, 16, 8, False),
+    (257, 5000, 11, 48, 16, True),
+    (130, 900, 3, 32, 32, False),
+    (1000, 20000, 60, 64, 32, True),
+    (5, 40, 2, 64, 16, False),
+    (700, 0, 4, 64, 8, False),
 ]
 
 
-@pytest.mark.parametrize("n,e,r,k,hub", CASES)
+@pytest.mark.parametrize("n,e,r,k,m,hub", CASES)
 @pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
 @pytest.mark.parametrize("scaled", [True, False], ids=["norm", "plain"])
-def test_typed_spmm_matches_operator_chain(device, n, e, r, k, hub, bf16, scaled):
-    rng = np.random.default_rng(n + e + k)
+def test_typed_spmm_matches_operator_chain(device, n, e, r, k, m, hub, bf16, scaled):
+    rng = np.random.default_rng(n + e + k + m)
     g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device, hub)
     x = rng.standard_normal((n, k), dtype=np.float32)
-    w = (rng.standard_normal((r, k, 64)) / np.sqrt(k)).astype(np.float32)
+    w = (rng.standard_normal((r, k, m)) / np.sqrt(k)).astype(np.float32)
     norm = rng.uniform(0.1, 1.5, e).astype(np.float32) if scaled else None
     if bf16:
         x, w = to_bf16_f32(x), to_bf16_f32(w)
     got = ops.TypedSpMMEdge(_dev(x, device, bf16), _dev(w, device, bf16), g,
                             row_scale=_dev(norm, device) if scaled else None)
-    assert got.shape == (n, 64) and got.dtype == (torch.bfloat16 if bf16 else torch.float32)
+    assert got.shape == (n, m) and got.dtype == (torch.bfloat16 if bf16 else torch.float32)
     ref, mag = _reference(arr, src, etype, r, x, w, norm)
     assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
-                 f"typed spmm n={n} e={e} r={r} k={k}", mag=mag)
+                 f"typed spmm n={n} e={e} r={r} k={k} m={m}", mag=mag)
     again = ops.TypedSpMMEdge(_dev(x, device, bf16), _dev(w, device, bf16), g,
                               row_scale=_dev(norm, device) if scaled else None)
     assert torch.equal(got.view(torch.int16 if bf16 else torch.int32),
@@ -125,8 +133,9 @@ def test_typed_tiles_layout(device):
     assert total <= capi.load().ga_typed_tiles_chunk_capacity(n, e, r, rows)
 
 
+@pytest.mark.parametrize("m", [64, 8, 32])
 @pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
-def test_typed_spmm_messages_that_are_not_finite(device, bf16):
+def test_typed_spmm_messages_that_are_not_finite(device, bf16, m):
     """inf and NaN source features: the rows that receive such a message become what
     the chain makes them (inf, -inf or NaN), every other row stays finite and exact to
     tolerance -- the selection matrices of the kernel must not spread them."""
@@ -134,7 +143,7 @@ def test_typed_spmm_messages_that_are_not_finite(device, bf16):
     n, e, r, k = 400, 6000, 6, 16
     g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device)
     x = rng.standard_normal((n, k), dtype=np.float32)
-    w = np.abs(rng.standard_normal((r, k, 64)) / np.sqrt(k)).astype(np.float32) + 0.01
+    w = np.abs(rng.standard_normal((r, k, m)) / np.sqrt(k)).astype(np.float32) + 0.01
     if bf16:
         x, w = to_bf16_f32(x), to_bf16_f32(w)
     x[0, :] = np.inf            # +inf messages (weights are positive); row 0 is also what pad slots read
@@ -167,16 +176,31 @@ def test_rgcn_layer_paths_agree(device):
     a = layers.rgcn_layer(g, x, w, norm, fused="tiles")
     b = layers.rgcn_layer(g, x, w, norm, fused=False)
     c = layers.rgcn_layer(g, x, w, norm, fused=True)
+    d = layers.rgcn_layer(g, x, w, norm, fused="pair")
     assert_close(a.cpu().numpy(), b.cpu().numpy(), 2 * TOL_F32, "tiles against unfused")
     assert_close(c.cpu().numpy(), b.cpu().numpy(), 2 * TOL_F32, "default against unfused")
+    assert_close(d.cpu().numpy(), b.cpu().numpy(), 2 * TOL_F32, "pair against unfused")
+    assert torch.equal(a, c), "16 -> 64 takes the single pass by default"
+    # a second layer as in the two-layer network (64 -> 8: single pass) and a wide one (pair)
+    for k, m, one_pass in ((64, 8, True), (64, 64, False)):
+        x2 = _dev(rng.standard_normal((n, k), dtype=np.float32), device)
+        w2 = _dev((rng.standard_normal((r, k, m)) / 8).astype(np.float32), device)
+        assert ops.typed_spmm_preferred(x2, w2) == one_pass
+        got = layers.rgcn_layer(g, x2, w2, norm, fused=True)
+        want = layers.rgcn_layer(g, x2, w2, norm, fused="tiles" if one_pass else "pair")
+        assert torch.equal(got, want)
+        assert_close(got.cpu().numpy(), layers.rgcn_layer(g, x2, w2, norm, fused=False).cpu().numpy(),
+                     2 * TOL_F32, f"{k} -> {m} against unfused")
 
 
 def test_typed_spmm_rejects_what_it_does_not_cover(device):
     rng = np.random.default_rng(6)
     g, arr, src, dst, etype = _typed_graph(rng, 100, 500, 3, device)
     x = torch.randn(100, 16, device=device)
-    with pytest.raises(capi.GraphilerError):          # M != 64
-        ops.TypedSpMMEdge(x, torch.randn(3, 16, 32, device=device), g)
+    with pytest.raises(capi.GraphilerError):          # M not one of 8, 16, 32, 64
+        ops.TypedSpMMEdge(x, torch.randn(3, 16, 24, device=device), g)
+    with pytest.raises(capi.GraphilerError):
+        ops.TypedSpMMEdge(x, torch.randn(3, 16, 128, device=device), g)
     with pytest.raises(capi.GraphilerError):          # K not a multiple of 16
         ops.TypedSpMMEdge(torch.randn(100, 8, device=device), torch.randn(3, 8, 64, device=device), g)
     with pytest.raises(RuntimeError):                 # one weight per relation
@@ -185,11 +209,12 @@ def test_typed_spmm_rejects_what_it_does_not_cover(device):
         ops.TypedSpMMEdge(x, torch.randn(3, 16, 64, device=device).bfloat16(), g)
     with pytest.raises(RuntimeError):
         ops.TypedSpMMEdge(x.cpu(), torch.randn(3, 16, 64), g)
-    assert not ops.typed_spmm_supported(x, torch.randn(3, 16, 32, device=device))
+    assert not ops.typed_spmm_supported(x, torch.randn(3, 16, 24, device=device))
     assert ops.typed_spmm_supported(x, torch.randn(3, 16, 64, device=device))
+    assert ops.typed_spmm_supported(x, torch.randn(3, 16, 8, device=device))
 
 
-@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("seed", range(16))
 def test_typed_spmm_random_graphs(device, seed):
     """Random sizes either side of a tile, relation counts from 1 to 200 (most of them
     without edges in most tiles), a destination that takes a large share of the edges,
@@ -199,11 +224,12 @@ def test_typed_spmm_random_graphs(device, seed):
     e = int(rng.choice([0, 1, 50, 3000, 40000]))
     r = int(rng.choice([1, 2, 9, 60, 200]))
     k = int(rng.choice([16, 32, 64]))
+    m = int(rng.choice([8, 16, 32, 64]))
     bf16 = bool(rng.integers(0, 2))
     scaled = bool(rng.integers(0, 2))
     g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device, hub=bool(rng.integers(0, 2)))
     x = rng.standard_normal((n, k), dtype=np.float32)
-    w = (rng.standard_normal((r, k, 64)) / np.sqrt(k)).astype(np.float32)
+    w = (rng.standard_normal((r, k, m)) / np.sqrt(k)).astype(np.float32)
     norm = rng.uniform(0.1, 1.5, e).astype(np.float32) if scaled else None
     if bf16:
         x, w = to_bf16_f32(x), to_bf16_f32(w)
@@ -211,4 +237,4 @@ def test_typed_spmm_random_graphs(device, seed):
                             row_scale=_dev(norm, device) if scaled else None)
     ref, mag = _reference(arr, src, etype, r, x, w, norm)
     assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
-                 f"typed random n={n} e={e} r={r} k={k} bf16={bf16}", mag=mag)
+                 f"typed random n={n} e={e} r={r} k={k} m={m} bf16={bf16}", mag=mag)
