@@ -985,7 +985,7 @@ namespace {
 // wide_mm.hip reads X once for all of `n_w` weight tensors.  GA_EUNSUPPORTED: not its shape.
 int wide_typed(const int32_t *type_pointer, int64_t n_types, const void *X,
                const void *const *W, void *const *Y, int n_w, int64_t rows, int64_t K,
-               int64_t M, hipStream_t s) {
+               int64_t M, const float *row_scale, hipStream_t s) {
   if (M % kWideGroupCols != 0 || n_types > 64) return GA_EUNSUPPORTED;
   const int per_w = (int)(M / kWideGroupCols);
   if (!wide_mm_fits((int)K, n_w * per_w)) return GA_EUNSUPPORTED;
@@ -996,6 +996,7 @@ int wide_typed(const int32_t *type_pointer, int64_t n_types, const void *X,
   p.X = (const bf16_t *)X;
   p.K = (int)K;
   p.n_groups = n_w * per_w;
+  p.row_scale = row_scale;
   for (int w = 0; w < n_w; ++w)
     for (int c = 0; c < per_w; ++c) {
       const int g = w * per_w + c;
@@ -1013,8 +1014,8 @@ int segment_mm_any(const int32_t *type_pointer, int64_t n_types, const void *X,
                    int64_t M, int dtype, const MmExt &ext, hipStream_t s) {
   const bool fused = ext.x_index || ext.Q;
   int rc = GA_EUNSUPPORTED;
-  if (dtype == GA_BF16 && heads == 1 && !fused && !ext.row_scale && Y) {
-    rc = wide_typed(type_pointer, n_types, X, &W, &Y, 1, rows, K, M, s);
+  if (dtype == GA_BF16 && heads == 1 && !fused && Y) {
+    rc = wide_typed(type_pointer, n_types, X, &W, &Y, 1, rows, K, M, ext.row_scale, s);
     if (rc != GA_EUNSUPPORTED) return rc;
   }
   if (aligned(X, 16) && (!Y || aligned(Y, 16)) && (!ext.Q || aligned(ext.Q, 16))) {
@@ -1028,7 +1029,8 @@ int segment_mm_any(const int32_t *type_pointer, int64_t n_types, const void *X,
       rc = launch_mfma<bf16_t, 16>(type_pointer, (int)n_types, X, W, Y, rows,
                                    (int)heads, (int)K, (int)M, ext, s);
   }
-  if (rc != GA_EUNSUPPORTED || fused) return rc;
+  // (the scalar kernel below takes no index column, dot operand or row factor)
+  if (rc != GA_EUNSUPPORTED || fused || ext.row_scale) return rc;
 
   // shapes the MFMA path does not take (odd K, weights beyond the LDS budget)
   const int64_t total = rows * heads * M;
@@ -1217,7 +1219,7 @@ extern "C" int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_type
   }
   hipStream_t s = (hipStream_t)stream;
   if (dtype == GA_BF16) {
-    const int rc = wide_typed(type_pointer, n_types, X, W, Y, (int)n_weights, rows, K, M, s);
+    const int rc = wide_typed(type_pointer, n_types, X, W, Y, (int)n_weights, rows, K, M, nullptr, s);
     if (rc != GA_EUNSUPPORTED) return rc;
   }
   // any other shape: one product per weight tensor

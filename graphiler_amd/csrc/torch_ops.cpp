@@ -431,6 +431,42 @@ torch::Tensor SegmentMMNode(torch::Tensor features, torch::Tensor weights,
   return segment_mm(features, weights, graph->ntype_pointer, graph->num_ntypes,
                     graph->num_nodes);
 }
+// SegmentMMNode(features, weights) * row_scale with an (N, 1) factor applied to the fp32
+// sums before they are rounded: the `trans_out * alpha.unsqueeze(1)` of
+// examples/HGT/HGT.py:58-60 without a pass over the result.  Any other factor (another
+// shape, a dtype that would promote the product) multiplies the result afterwards.
+torch::Tensor SegmentMMNodeScaled(torch::Tensor features, torch::Tensor weights,
+                                  torch::Tensor row_scale, const GraphPtr &graph) {
+  const bool fits = row_scale.is_cuda() && row_scale.dim() == 2 && row_scale.size(1) == 1 &&
+                    row_scale.size(0) == graph->num_nodes && row_scale.is_floating_point() &&
+                    features.is_floating_point() && features.dim() == 2 &&
+                    features.size(0) == graph->num_nodes && (weights.dim() == 3 || weights.dim() == 4) &&
+                    at::promote_types(features.scalar_type(), row_scale.scalar_type()) ==
+                        features.scalar_type();
+  if (fits) {
+    check_input(features, "features");
+    check_input(weights, "weights");
+    const int dt = feat_dtype(features, "features");
+    TORCH_CHECK(weights.scalar_type() == features.scalar_type(),
+                "features and weights must share a dtype");
+    TORCH_CHECK(graph->ntype_pointer.has_value(), "the graph has no type pointer for this operator");
+    const int64_t heads = weights.dim() == 4 ? weights.size(1) : 1;
+    const int64_t K = weights.size(weights.dim() - 2), M = weights.size(weights.dim() - 1);
+    TORCH_CHECK(weights.size(0) == graph->num_ntypes, "weights must have one matrix per type");
+    TORCH_CHECK(feat_dim(features) == heads * K, "features must be (rows, heads*K)");
+    torch::Tensor rs = row_scale.to(at::kFloat).contiguous();
+    torch::Tensor out = torch::empty({graph->num_nodes, heads * M}, features.options());
+    const int rc = ga_segment_mm_gather(
+        graph->ntype_pointer.value().data_ptr<int>(), graph->num_ntypes, features.data_ptr(),
+        nullptr, weights.data_ptr(), out.data_ptr(), nullptr, nullptr, nullptr, nullptr,
+        rs.data_ptr<float>(), graph->num_nodes, heads, K, M, dt, current_stream(out));
+    if (rc != GA_EUNSUPPORTED) {
+      check_ga(rc, "ga_segment_mm_gather");
+      return out;
+    }
+  }
+  return SegmentMMNode(features, weights, graph) * row_scale;
+}
 // segment_mm.cu:29-33
 torch::Tensor SegmentMMEdge(torch::Tensor features, torch::Tensor weights,
                             const GraphPtr &graph) {
@@ -907,6 +943,9 @@ static auto registry =
             &TypedSpMMEdge)
         .op("my_ops::SegmentMMNodeStacked(Tensor x, Tensor[] ws, " GRAPH_T " g) -> Tensor[] zs",
             &SegmentMMNodeStacked)
+        .op("my_ops::SegmentMMNodeScaled(Tensor x, Tensor w, Tensor row_scale, " GRAPH_T
+            " g) -> Tensor z",
+            &SegmentMMNodeScaled)
         .op("my_ops::SegmentMMEdgeDot(Tensor x, Tensor w, int endpoint, Tensor q, "
             "int q_endpoint, Tensor? scale, " GRAPH_T " g) -> Tensor z",
             &SegmentMMEdgeDot)

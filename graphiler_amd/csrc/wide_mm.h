@@ -27,6 +27,7 @@ struct WideMm {
   // on the fp32 accumulators; a_l / a_r / el / er point at the group's first column / head
   const float *a_l[kWideMaxGroups], *a_r[kWideMaxGroups];
   float *el[kWideMaxGroups], *er[kWideMaxGroups];
+  const float *row_scale;     // Y[r, :] of every group times row_scale[r]; null: 1 (not with a_l / a_r)
   int64_t ldd;                // heads per row of el / er
   int dph;                    // columns per head: 32, 64 or 128
   bool w_wide;                // set by wide_mm_launch: rows of every W are 16-byte aligned

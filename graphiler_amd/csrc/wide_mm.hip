@@ -174,6 +174,15 @@ __global__ __launch_bounds__(kWideBlock) void wide_mm_kernel(WideMm p, int chunk
       for (int f = 0; f < NF; ++f) xa[t][f] = xn[t][f];
     if (rel + kStepRows < nrows) load_rows(rel + kStepRows, xn);
     const bool full = rel + kWaveRows <= nrows;
+    // factors of my rows rel + 16 t + 4 q + i (requested now, used after the products)
+    float rs[TW][4];
+#pragma unroll
+    for (int t = 0; t < TW; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = rel + 16 * t + 4 * q + i;
+        rs[t][i] = !ATTN && p.row_scale ? p.row_scale[row0 + (r < nrows ? r : nrows - 1)] : 1.0f;
+      }
 #pragma unroll 1
     for (int g = 0; g < NG; ++g) {
       // The weight fragments do not change from step to step, and the compiler would
@@ -199,6 +208,14 @@ __global__ __launch_bounds__(kWideBlock) void wide_mm_kernel(WideMm p, int chunk
         }
       }
       // lane (n, q) holds rows rel + 16 t + 4 q + i, columns 8 n .. 8 n + 7 of the group
+      if (!ATTN && p.row_scale) {
+#pragma unroll
+        for (int t = 0; t < TW; ++t)
+#pragma unroll
+          for (int cb = 0; cb < 8; ++cb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[t][cb][i] *= rs[t][i];
+      }
       char *ybase = reinterpret_cast<char *>(p.Y[g] + (int64_t)row0 * p.ldy[g]);
       const uint32_t yrow = (uint32_t)p.ldy[g] * 2u;
       const uint32_t yoff = (uint32_t)(rel + 4 * q) * yrow + (uint32_t)n * 16u;
@@ -344,6 +361,7 @@ int wide_mm_launch(const WideMm &p, hipStream_t s) {
   if (!wide_mm_fits(p.K, p.n_groups)) return GA_EUNSUPPORTED;
   if (p.rows <= 0) return GA_OK;
   if (p.rows > 0x7fffffff || !aligned(p.X, p.K % 8 == 0 ? 16 : 8)) return GA_EUNSUPPORTED;
+  if (p.row_scale && (!aligned(p.row_scale, 4) || p.a_l[0])) return GA_EUNSUPPORTED;
   const bool attn = p.a_l[0] != nullptr;
   if (attn && p.dph != 32 && p.dph != 64 && p.dph != 128) return GA_EUNSUPPORTED;
   for (int g = 0; g < p.n_groups; ++g) {

@@ -165,6 +165,8 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
         a = ops.SegmentSoftmax(attn.contiguous(), 1, None, g)      # (E, heads) fp32
         m = (v_e.view(e, heads, d).float() * a.unsqueeze(-1)).to(h.dtype).view(e, hidden)
         t = ops.SpMMEdge(m, [1], False, None, g)
-    alpha = torch.sigmoid(ops.BroadcastNodeType(skip.float().unsqueeze(1), g))
+    alpha = ops.BroadcastNodeType(torch.sigmoid(skip.float()).unsqueeze(1), g)
+    if fused:       # the gate goes into the product's epilogue
+        return ops.SegmentMMNode(t, a_weight, g, row_scale=alpha)
     out = ops.SegmentMMNode(t, a_weight, g)
     return (out.float() * alpha).to(h.dtype)

@@ -504,6 +504,9 @@ class _Rewriter:
         for n in list(self.G.nodes()):
             if n.kind() == "my_ops::SpMMEdge":
                 changed |= self._fuse_typed_spmm(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "aten::mul":
+                changed |= self._fuse_node_scale(n)
         changed |= self._fuse_stacked_mm()
         return changed
 
@@ -653,6 +656,23 @@ class _Rewriter:
         n.destroy()
         mm.destroy()
         return True
+
+    def _fuse_node_scale(self, n) -> bool:
+        """SegmentMMNode(x, w) * BroadcastNodeType(s) -> SegmentMMNodeScaled(x, w,
+        BroadcastNodeType(s)): the per-node factor is applied to the product's fp32 sums
+        (HGT's gate on the output projection).  The operator itself falls back to the
+        two steps when the factor is not (N, 1) or would promote the result."""
+        for a, b in ((n.inputsAt(0), n.inputsAt(1)), (n.inputsAt(1), n.inputsAt(0))):
+            mm, bc = a.node(), b.node()
+            if mm.kind() == "my_ops::SegmentMMNode" and self.single_use(a) and \
+                    bc.kind() == "my_ops::BroadcastNodeType":
+                out = self.make("my_ops::SegmentMMNodeScaled",
+                                [mm.inputsAt(0), mm.inputsAt(1), b, self.dglgraph], n, NODE)
+                n.output().replaceAllUsesWith(out)
+                n.destroy()
+                mm.destroy()
+                return True
+        return False
 
     def _fuse_stacked_mm(self) -> bool:
         """Two to four SegmentMMNode(x, w_i) of one x -> SegmentMMNodeStacked(x, [w_i]):

@@ -425,7 +425,7 @@ def SegmentSoftmax(features, dim: int, dtype, graph: DGLGraph) -> torch.Tensor:
 
 
 # ----------------------------------------------------------- segment_mm ----
-def _segment_mm(features, weights, type_pointer, num_types, rows_expected):
+def _segment_mm(features, weights, type_pointer, num_types, rows_expected, row_scale=None):
     _check_input(features, "features")
     _check_input(weights, "weights")
     dt = _feat_dtype(features, "features")
@@ -447,17 +447,32 @@ def _segment_mm(features, weights, type_pointer, num_types, rows_expected):
         raise RuntimeError("features must be (rows, heads*K)")
     out = torch.empty((rows, heads * M), dtype=features.dtype,
                       device=features.device)
+    if row_scale is not None:
+        _check_input(row_scale, "row_scale")
+        if row_scale.dtype != torch.float32 or row_scale.numel() != rows:
+            raise RuntimeError("row_scale must be one float32 per row")
+        rc = capi.load().ga_segment_mm_gather(
+            type_pointer.data_ptr(), num_types, features.data_ptr(), None,
+            weights.data_ptr(), out.data_ptr(), None, None, None, None,
+            row_scale.data_ptr(), rows, heads, K, M, dt, _stream(out))
+        if rc != capi.GA_EUNSUPPORTED:
+            capi.check(rc, "ga_segment_mm_gather")
+            return out
     capi.check(capi.load().ga_segment_mm(
         type_pointer.data_ptr(), num_types, features.data_ptr(),
         weights.data_ptr(), out.data_ptr(), rows, heads, K, M, dt,
         _stream(out)), "ga_segment_mm")
+    if row_scale is not None:       # a shape outside the kernels that take the factor
+        out = (out.float() * row_scale.reshape(-1, 1)).to(out.dtype)
     return out
 
 
-def SegmentMMNode(features, weights, graph: DGLGraph) -> torch.Tensor:
-    """segment_mm.cu:23-27: per-node-type linear, nodes sorted by type."""
+def SegmentMMNode(features, weights, graph: DGLGraph, row_scale=None) -> torch.Tensor:
+    """segment_mm.cu:23-27: per-node-type linear, nodes sorted by type.  ``row_scale``
+    (N,) or (N, 1) fp32 multiplies row r of the result, applied to the fp32 sums before
+    they are rounded (the ``trans_out * alpha.unsqueeze(1)`` of examples/HGT/HGT.py:58-60)."""
     return _segment_mm(features, weights, graph.ntype_pointer,
-                       graph.num_ntypes, graph.num_nodes)
+                       graph.num_ntypes, graph.num_nodes, row_scale)
 
 
 def SegmentMMNodeStacked(features, weights: Sequence[torch.Tensor], graph: DGLGraph):

@@ -313,7 +313,10 @@ int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_types, const vo
  * two results:
  *   Y   (rows, heads*M) `dtype`, with Q / q_index / dot NULL; row_scale, when
  *       not NULL, is (rows,) fp32 and multiplies row r of Y (the per-edge norm
- *       of examples/RGCN/RGCN.py:29, read in edge order with the rows);
+ *       of examples/RGCN/RGCN.py:29, read in edge order with the rows; with x_index
+ *       NULL and the node type pointer it is the gate of examples/HGT/HGT.py:58-60
+ *       on the output projection).  The factor multiplies the fp32 sums before they
+ *       are rounded;
  *   dot (rows, heads) fp32 with Y NULL: dot[r, h] = <Y[r, h, :], Q[q_index[r], h, :]>
  *       (q_index NULL: Q[r]); Q (*, heads*M) `dtype`.  The product rows stay in
  *       registers (HGT's sum(k * q, dim=1), HGT.py:44-45).  scale, when not
@@ -325,7 +328,10 @@ int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_types, const vo
  * heads*M > 128, K % 4 (fp32) or K % 8 (bf16) != 0; for dot also a head width M
  * that is not c, 2c, 4c, 8c or 16c with c = ceil(heads*M / 16) rounded up to a
  * power of two (at least 2 for bf16)); the caller then gathers with
- * ga_gather_rows.
+ * ga_gather_rows.  Without index columns and dot operand, bf16 shapes of the wide
+ * kernel (see ga_segment_mm_stacked) are taken as well; a call with row_scale whose
+ * shape no matrix-core kernel takes also returns GA_EUNSUPPORTED (ga_segment_mm, then
+ * the factor).
  */
 int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types, const void *X,
                          const int64_t *x_index, const void *W, void *Y,

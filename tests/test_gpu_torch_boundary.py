@@ -181,6 +181,18 @@ def test_typed_sum_and_stacked_products_through_torchscript(device):
     assert len(outs) == 3
     for w, y in zip(ws, outs):
         assert torch.equal(y.view(torch.int16), ops.SegmentMMNode(h, w, sg).view(torch.int16))
+    # the product with a per-node factor: in the kernel when the factor is (N, 1) and does
+    # not promote the result, as two steps otherwise -- the same values either way
+    for w, dt in ((ws[0], torch.bfloat16), (ws[0].float(), torch.float32)):
+        hh = h.to(dt)
+        plain = ops.SegmentMMNode(hh, w, sg)
+        for fac in (torch.rand(n, 1, device=device).to(dt), torch.rand(n, 1, device=device),
+                    torch.rand(n, device=device).to(dt)[:, None].expand(n, 128)):
+            got = ops.SegmentMMNodeScaled(hh, w, fac, sg)
+            want = plain * fac
+            assert got.dtype == want.dtype and got.shape == want.shape
+            assert_close(got.float().cpu().numpy(), want.float().cpu().numpy(),
+                         2e-2 if dt == torch.bfloat16 else 2 * TOL_F32, f"SegmentMMNodeScaled {dt}")
     mixed = [ws[0], ws[1][:, :, :64].contiguous()]          # different shapes: one product each
     outs = ops.SegmentMMNodeStacked(h, mixed, sg)
     assert outs[1].shape == (n, 64)

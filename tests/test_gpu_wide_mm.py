@@ -103,6 +103,37 @@ def test_stacked_operator_and_hgt_projections(device):
         ops.SegmentMMNodeStacked(h, [], g)
 
 
+@pytest.mark.parametrize("K,M,bf16", [(128, 128, True), (256, 256, True), (100, 128, True),
+                                      (64, 384, True), (102, 128, True), (128, 64, True),
+                                      (20, 24, False), (128, 128, False)])
+def test_node_product_with_row_factor(device, K, M, bf16):
+    """ops.SegmentMMNode(..., row_scale): the factor multiplies the fp32 sums (wide kernel,
+    tile kernels, and shapes where it is applied afterwards)."""
+    from graphiler_amd import prepare_graph
+    rng = np.random.default_rng(K + M)
+    tn = len(COUNTS)
+    ntype = np.repeat(np.arange(tn), COUNTS)
+    n = ntype.shape[0]
+    src, dst = rng.integers(0, n, 2000), rng.integers(0, n, 2000)
+    g = prepare_graph(src, dst, n, device=device, ntype_of=ntype, num_ntypes=tn)
+    tp = np.concatenate([[0], np.cumsum(COUNTS)]).astype(np.int32)
+    x = rng.standard_normal((n, K), dtype=np.float32)
+    w = (rng.standard_normal((tn, K, M)) / np.sqrt(K)).astype(np.float32)
+    if bf16:
+        x, w = to_bf16_f32(x), to_bf16_f32(w)
+    scale = rng.uniform(0.1, 2.0, n).astype(np.float32)
+    got = ops.SegmentMMNode(_dev(x, device, bf16), _dev(w, device, bf16), g,
+                            row_scale=_dev(scale, device).reshape(-1, 1))
+    assert got.dtype == (torch.bfloat16 if bf16 else torch.float32) and got.shape == (n, M)
+    ref = oracle.segment_mm(tp, x, w) * scale[:, None]
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
+                 f"scaled node product K={K} M={M}",
+                 mag=oracle.segment_mm(tp, np.abs(x), np.abs(w)) * scale[:, None])
+    with pytest.raises(RuntimeError):
+        ops.SegmentMMNode(_dev(x, device, bf16), _dev(w, device, bf16), g,
+                          row_scale=_dev(scale[:-1], device))
+
+
 @pytest.mark.parametrize("rows,K,M,heads", [
     (1500, 256, 256, 4), (1500, 256, 256, 2), (1500, 256, 256, 8),   # heads of 64, 128, 32 columns
     (777, 128, 128, 1), (777, 128, 128, 4), (333, 64, 384, 3), (255, 32, 512, 8),

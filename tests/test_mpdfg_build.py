@@ -73,7 +73,9 @@ def test_level2_fuses_into_graph_operators():
     _, k = _kinds("hgt", 2)
     ours = [x for x in k if x.startswith("my_ops::")]
     # K, V, Q read the node rows once; the output projection stays on its own
-    assert ours.count("my_ops::SegmentMMNodeStacked") == 1 and ours.count("my_ops::SegmentMMNode") == 1
+    # K, V, Q in one pass over h; the output projection takes the gate as its row factor
+    assert ours.count("my_ops::SegmentMMNodeStacked") == 1 and ours.count("my_ops::SegmentMMNode") == 0
+    assert ours.count("my_ops::SegmentMMNodeScaled") == 1 and "aten::mul" not in ours
     assert "my_ops::SegmentMMEdgeDot" in ours            # sum(bmm(k, W_att) * q) in one pass
     assert "my_ops::SegmentMMEdgeGather" in ours and "my_ops::edge_softmax_sum" in ours
     assert "my_ops::SegmentSoftmax" not in ours and "my_ops::gspmm_e_mul_e_sum" not in ours
