@@ -426,12 +426,33 @@ def main():
                            "x 16, hidden 128, bf16 with fp32 accumulation; power-law out-degree, seed 3",
                "num_nodes": N, "num_edges": E, "dtype": "bf16",
                "ms_per_step": round(ms_step, 4), "edges_per_s": round(E / (ms_step * 1e-3), 1)}
-        # bytes of the fused layer: h in, K/V/Q/t/out node rows, three gathered rows per edge,
-        # the transformed values written and read once, scores written and read once
-        layer_bytes = N * hid * b * 9 + E * (3 * hid * b + 2 * hid * b + 24 + 4 * 4 * H)
-        opsr = {"hgt_layer": op_record("c4.hgt_layer", layer, layer_bytes,
-                                       2.0 * N * hid * hid * 4 + 4.0 * E * H * D * D, "bf16")}
+        # bytes of the layer with its relation products per edge: h in, K/V/Q/t/out node rows,
+        # three gathered rows per edge, the transformed values written and read once, scores
+        # written and read once
+        edges_bytes = N * hid * b * 9 + E * (3 * hid * b + 2 * hid * b + 24 + 4 * 4 * H)
+        edges_flops = 2.0 * N * hid * hid * 4 + 4.0 * E * H * D * D
+        # ... per (destination, relation) pair, the form the layer takes on this graph: node
+        # rows as before, per edge the gathered k / v rows, the pair's transformed q row, five
+        # index reads and the scores (written, normalised in place, read); per pair the q row
+        # read, its transform written, the weighted sum and its transform written and read
+        P = g.relation_pairs().num_pairs
+        pairs_bytes = N * hid * b * 9 + P * hid * b * 6 + E * (3 * hid * b + 20 + 4 * 4 * H)
+        pairs_flops = 2.0 * N * hid * hid * 4 + 4.0 * P * H * D * D + 4.0 * E * hid
+        by_pairs = E >= layers.PAIRS_MIN_EDGES_PER_PAIR * P
+        rec["num_pairs"] = P
+        rec["relation_products"] = "per (destination, relation) pair" if by_pairs else "per edge"
+        opsr = {"hgt_layer": op_record("c4.hgt_layer", layer, pairs_bytes if by_pairs else edges_bytes,
+                                       pairs_flops if by_pairs else edges_flops, "bf16")}
         if not args.no_ops:
+            opsr["hgt_layer_per_edge"] = op_record(
+                "c4.hgt_layer_per_edge",
+                lambda: layers.hgt_layer(g, X, wk, wq, wv, wa, ra, rm, rp, skip, H, fused="edges"),
+                edges_bytes, edges_flops, "bf16")
+            kk, vv, qq = ops.SegmentMMNodeStacked(X, [wk, wv, wq], g)
+            opsr["relation_pair_attention"] = op_record(
+                "c4.relation_pair_attention",
+                lambda: ops.relation_pair_attention(kk, qq, vv, ra, rm, rp.float() / D ** 0.5, g),
+                pairs_bytes - N * hid * b * 6, pairs_flops - 2.0 * N * hid * hid * 4, "bf16")
             opsr["segment_mm_node_128_128"] = op_record(
                 "c4.segment_mm_node", lambda: ops.SegmentMMNode(X, wk, g),
                 N * 2 * hid * b + Tn * hid * hid * b, 2.0 * N * hid * hid, "bf16", reps=50)
@@ -462,8 +483,9 @@ def main():
                 "c4.edge_softmax_sum", lambda: ops.edge_softmax_sum(lg, ve, g),
                 4 * (N + 1) + E * (4 + 4 + 4 * H + hid * b) + N * hid * b, reps=50)
         rec["ops"] = opsr
-        rec["roofline"] = dict(opsr["hgt_layer"], kernel="hgt_layer (3 node projections, dot-product "
-                               "scores, gathered values, softmax-weighted sum, output projection)")
+        rec["roofline"] = dict(opsr["hgt_layer"], kernel="hgt_layer (3 node projections, relation "
+                               "products " + rec["relation_products"] + ", dot-product scores, edge "
+                               "softmax, weighted sum of gathered values, output projection)")
         return rec
 
     runners = {"c2": run_c2, "c3": run_c3, "c4": run_c4, "c5": run_c5}

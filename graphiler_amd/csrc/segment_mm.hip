@@ -904,7 +904,7 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
   g.perm_shift = -1;
   // rows per workgroup: a multiple of the 64-row step, large enough to
   // amortise the weight staging, small enough to keep every CU busy
-  int64_t steps = rows / (kTileBlock * 2048);
+  int64_t steps = rows / (kTileBlock * 1024);
   if (steps < 1) steps = 1;
   if (steps > 16) steps = 16;
   g.chunk_rows = (int)steps * kTileBlock;

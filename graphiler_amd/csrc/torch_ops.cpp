@@ -588,7 +588,8 @@ torch::Tensor TypedSpMMEdge(torch::Tensor features, torch::Tensor weights,
       plain_scale = true;
     }
   }
-  if (plain_scale && weights.dim() == 3 && features.dim() == 2 && s.K % 16 == 0 &&
+  const bool cols_ok = s.M == 8 || s.M == 16 || s.M == 32 || s.M == 64;
+  if (plain_scale && weights.dim() == 3 && features.dim() == 2 && s.K % 16 == 0 && cols_ok &&
       s.K * s.M <= 2048) {
     const DGLGraph::TypedTiles &t = graph->typed_tiles();
     torch::Tensor out = torch::empty({graph->num_nodes, s.M}, features.options());

@@ -195,6 +195,18 @@ class DGLGraph:
     def out_eid_is_identity(self) -> bool:
         return self._identity("out_ident", self.out_edge_indices)
 
+    def relation_pairs(self) -> Optional["RelationPairs"]:
+        """The (destination, relation) pairs of the in-adjacency, built once on the
+        device: a layer whose per-edge work is linear in a per-relation matrix (HGT's
+        ``bmm(k, relation_att)`` and ``bmm(v, relation_msg)``, examples/HGT/HGT.py:35-44)
+        can apply that matrix once per pair instead of once per edge.  None when the
+        graph has no edge types or the slots of a destination are not grouped by
+        relation (they are when edge ids are sorted by type, as
+        include/dglgraph.h:24-27 requires for the type pointer)."""
+        if "pairs" not in self._cache:
+            self._cache["pairs"] = _build_relation_pairs(self)
+        return self._cache["pairs"]
+
     def workspace(self, nbytes: int) -> torch.Tensor:
         """Scratch buffer shared by the operators called on this graph (grows on
         demand).  Calls that use it must be ordered on one stream: two streams
@@ -209,6 +221,59 @@ class DGLGraph:
                              device=self.device)
             self._cache["ws"] = ws
         return ws
+
+
+@dataclass
+class RelationPairs:
+    """Slots of the in-adjacency grouped into runs of one (destination, relation).
+    Pairs are numbered in slot order (by destination, then relation); ``by_type``
+    lists them by relation (stable), which is the row order the typed products need."""
+    num_pairs: int
+    pair_pointer: torch.Tensor      # (P + 1) int32: first slot of every pair
+    pair_of_slot: torch.Tensor      # (E) int32
+    pair_dst: torch.Tensor          # (P) int32, ascending
+    dst_pointer: torch.Tensor       # (N + 1) int32: first pair of every destination
+    type_pointer: torch.Tensor      # (T + 1) int32 over by_type
+    by_type: torch.Tensor           # (P) int64: pair ids ordered by relation
+    rank: torch.Tensor              # (P) int32: position of a pair in by_type
+    rank_of_slot: torch.Tensor      # (E) int32: rank[pair_of_slot]
+    dst_by_type: torch.Tensor       # (P) int64: pair_dst[by_type]
+
+
+def _build_relation_pairs(g: "DGLGraph") -> Optional[RelationPairs]:
+    if g.etype_pointer is None or g.num_edges == 0:
+        return None
+    dev, n_edges, n_types = g.device, g.num_edges, g.num_etypes
+    rows = g.in_row_of_slot.long()
+    eid = g.in_edge_indices.long()
+    etype = torch.bucketize(eid, g.etype_pointer[1:].long(), right=True)
+    key = rows * n_types + etype
+    if n_edges > 1 and not bool((key[1:] >= key[:-1]).all()):
+        return None
+    first = torch.ones(n_edges, dtype=torch.bool, device=dev)
+    first[1:] = key[1:] != key[:-1]
+    pair_of_slot = torch.cumsum(first, 0) - 1
+    starts = torch.nonzero(first).reshape(-1)
+    n_pairs = int(starts.numel())
+    pair_key = key[starts]
+    pair_dst = torch.div(pair_key, n_types, rounding_mode="floor")
+    pair_type = pair_key - pair_dst * n_types
+    by_type = torch.argsort(pair_type, stable=True)
+    rank = torch.empty_like(by_type)
+    rank[by_type] = torch.arange(n_pairs, device=dev)
+    return RelationPairs(
+        num_pairs=n_pairs,
+        pair_pointer=torch.cat([starts, starts.new_tensor([n_edges])]).int().contiguous(),
+        pair_of_slot=pair_of_slot.int().contiguous(),
+        pair_dst=pair_dst.int().contiguous(),
+        dst_pointer=torch.searchsorted(pair_dst.contiguous(),
+                                       torch.arange(g.num_nodes + 1, device=dev)).int().contiguous(),
+        type_pointer=torch.searchsorted(pair_type[by_type].contiguous(),
+                                        torch.arange(n_types + 1, device=dev)).int().contiguous(),
+        by_type=by_type.contiguous(),
+        rank=rank.int().contiguous(),
+        rank_of_slot=rank[pair_of_slot].int().contiguous(),
+        dst_by_type=pair_dst[by_type].contiguous())
 
 
 def group_on_device(key: torch.Tensor, other: Optional[torch.Tensor], n_keys: int):

@@ -124,9 +124,15 @@ def rgcn_layer(g: DGLGraph, h, weight, norm, fused=True):
     return ops.SpMMEdge(msg, [1], False, None, g)
 
 
+# Edges per (destination, relation) pair from which an HGT layer applies its relation
+# matrices per pair: the pair form replaces two typed products over E rows by two over
+# P rows plus two passes over the pairs.
+PAIRS_MIN_EDGES_PER_PAIR = 2.0
+
+
 def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
               relation_att, relation_msg, relation_pri, skip, heads: int = 1,
-              fused: bool = True):
+              fused=True):
     """examples/HGT/HGT.py:28-60 as the operator sequence of its optimised plan,
     generalised from one head to ``heads`` heads of width D = hidden / heads:
 
@@ -141,22 +147,39 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
     k/q/v/a_weight: (T_n, hidden, hidden); relation_att / relation_msg:
     (T_e, heads, D, D); relation_pri: (T_e, heads); skip: (T_n,).
 
-    ``fused`` replaces the per-edge copies and products by
+    ``fused="edges"`` replaces the per-edge copies and products by
       attn = SegmentMMEdgeDot(K, relation_att, src, Q, dst) * pri / sqrt(D)
       t    = edge_softmax_sum(attn, SegmentMMEdgeGather(V, relation_msg, src))
     so the only per-edge tensors are the scores and the transformed values.
+    ``fused="pairs"`` applies the relation matrices once per (destination, relation)
+    pair instead (ops.relation_pair_attention): no per-edge tensor but the scores.
+    ``fused=True`` takes the pairs when the graph has at least ``PAIRS_MIN_EDGES_PER_PAIR``
+    edges per pair (config 4: 7.4) and the per-edge form otherwise.
     """
     n, hidden = h.shape
     d = hidden // heads
     e = g.num_edges
     # the three projections of h in one pass over its rows
     k, v, q = ops.SegmentMMNodeStacked(h, [k_weight, v_weight, q_weight], g)
-    if fused:
+    t = None
+    if fused == "pairs" or fused is True:
+        pairs = g.relation_pairs()
+        if fused == "pairs" and pairs is None:
+            raise RuntimeError("the in-adjacency of this graph is not grouped by relation")
+        if pairs is not None and (fused == "pairs"
+                                  or e >= PAIRS_MIN_EDGES_PER_PAIR * pairs.num_pairs):
+            try:
+                t = ops.relation_pair_attention(k, q, v, relation_att, relation_msg,
+                                                relation_pri.float() / (d ** 0.5), g)
+            except capi.GraphilerError as err:      # head width outside the typed product
+                if err.code != capi.GA_EUNSUPPORTED or fused == "pairs":
+                    raise
+    if t is None and fused:
         attn = ops.SegmentMMEdgeDot(k, relation_att, 0, q, 1, g,
                                     scale=relation_pri.float() / (d ** 0.5))
         v_e = ops.SegmentMMEdgeGather(v, relation_msg, 0, g)
         t = ops.edge_softmax_sum(attn, v_e, g)
-    else:
+    elif t is None:
         pri = ops.BroadcastEdgeType(relation_pri.float(), g) / (d ** 0.5)
         k_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(k, g), relation_att, g)
         v_e = ops.SegmentMMEdge(ops.BroadcastSrcNode(v, g), relation_msg, g)

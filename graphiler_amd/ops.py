@@ -835,6 +835,84 @@ def edge_softmax_sum(logits, messages, graph: DGLGraph) -> torch.Tensor:
     return out
 
 
+def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
+                            graph: DGLGraph) -> torch.Tensor:
+    """The message and reduce stages of an HGT layer (examples/HGT/HGT.py:35-53) with
+    the per-relation matrices applied once per (destination, relation) pair instead
+    of once per edge -- both stages are linear in them:
+
+      score[e, h] = <k[src] @ A[t], q[dst]> * s[t, h] = <k[src], q[dst] @ (s A[t])^T>
+      out[v]      = sum_e a[e] * (v[src] @ M[t])      = sum_{pairs (v, t)} (sum_{e in pair} a[e] * v[src]) @ M[t]
+
+    with a = softmax of the scores over the in-edges of v.  k, q, v (N, H*D);
+    relation_att, relation_msg (T, H, D, D); relation_scale (T, H) fp32 (the prior
+    over sqrt(D)) or None.  The typed products run over P pairs, the scores are a
+    plain dot product per edge and the weighted sum gathers rows of v: no (E, H*D)
+    tensor is written.  Returns (N, H*D).  Raises GraphilerError(GA_EUNSUPPORTED) for
+    shapes the typed-product kernel does not take and RuntimeError when the graph has
+    no pair layout (DGLGraph.relation_pairs)."""
+    for name, x in (("k", k), ("q", q), ("v", v), ("relation_att", relation_att),
+                    ("relation_msg", relation_msg)):
+        _check_input(x, name)
+    dt = _feat_dtype(k, "k")
+    if relation_att.dim() != 4 or relation_att.shape != relation_msg.shape \
+            or int(relation_att.shape[0]) != graph.num_etypes \
+            or relation_att.shape[2] != relation_att.shape[3]:
+        raise RuntimeError("relation matrices must be (edge types, heads, D, D)")
+    heads, d = int(relation_att.shape[1]), int(relation_att.shape[2])
+    n, e, hid, n_types = graph.num_nodes, graph.num_edges, heads * d, graph.num_etypes
+    for x in (k, q, v):
+        if x.dtype != k.dtype or tuple(x.shape) != (n, hid):
+            raise RuntimeError("k, q and v must be (nodes, heads*D) of one dtype")
+    if relation_att.dtype != k.dtype or relation_msg.dtype != k.dtype:
+        raise RuntimeError("relation matrices must have the features' dtype")
+    pairs = graph.relation_pairs()
+    if pairs is None:
+        raise RuntimeError("the in-adjacency of this graph is not grouped by relation")
+    att_t = relation_att.transpose(-1, -2)
+    if relation_scale is not None:
+        if tuple(relation_scale.shape) != (n_types, heads):
+            raise RuntimeError("relation_scale must be (edge types, heads)")
+        # an fp32 product, rounded once to the features' dtype
+        att_t = att_t * relation_scale.float()[:, :, None, None]
+    if att_t.dtype != k.dtype:
+        att_t = att_t.to(k.dtype, memory_format=torch.contiguous_format)
+    att_t = att_t.contiguous()       # (a no-op after the conversion)
+    lib, stream, dev, P = capi.load(), _stream(k), k.device, pairs.num_pairs
+
+    def typed_rows(x, index, w):        # row r = x[index[r]] @ w[relation of pair by_type[r]]
+        y = torch.empty((P, hid), dtype=x.dtype, device=dev)
+        capi.check(lib.ga_segment_mm_gather(
+            pairs.type_pointer.data_ptr(), n_types, x.data_ptr(), index.data_ptr(),
+            w.data_ptr(), y.data_ptr(), None, None, None, None, None, P, heads, d, d, dt,
+            stream), "ga_segment_mm_gather")
+        return y
+
+    q_pair = typed_rows(q, pairs.dst_by_type, att_t)
+    score = torch.empty((e, heads), dtype=torch.float32, device=dev)      # slot order
+    capi.check(lib.ga_sddmm_u_dot_v(
+        graph.in_node_indices.data_ptr(), pairs.rank_of_slot.data_ptr(), 32, k.data_ptr(),
+        q_pair.data_ptr(), score.data_ptr(), e, heads, d, dt, stream), "ga_sddmm_u_dot_v")
+    ws = graph.workspace(max(lib.ga_softmax_workspace_bytes(e, heads),
+                             lib.ga_spmm_workspace_bytes(e, hid)))
+    capi.check(lib.ga_segment_softmax(
+        graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(), None, score.data_ptr(),
+        score.data_ptr(), n, e, heads, ws.data_ptr(), ws.numel(), stream), "ga_segment_softmax")
+    v_pair = torch.empty((P, hid), dtype=v.dtype, device=dev)            # pair order
+    capi.check(lib.ga_spmm_csr(
+        pairs.pair_pointer.data_ptr(), pairs.pair_of_slot.data_ptr(),
+        graph.in_node_indices.data_ptr(), None, v.data_ptr(), score.data_ptr(),
+        v_pair.data_ptr(), P, e, hid, heads, capi.GA_U_MUL_E, capi.GA_SUM, dt, ws.data_ptr(),
+        ws.numel(), stream), "ga_spmm_csr")
+    m_pair = typed_rows(v_pair, pairs.by_type, relation_msg)             # by_type order
+    out = torch.empty((n, hid), dtype=v.dtype, device=dev)
+    capi.check(lib.ga_spmm_csr(
+        pairs.dst_pointer.data_ptr(), pairs.pair_dst.data_ptr(), pairs.rank.data_ptr(),
+        pairs.rank.data_ptr(), m_pair.data_ptr(), None, out.data_ptr(), n, P, hid, 1,
+        capi.GA_COPY_E, capi.GA_SUM, dt, ws.data_ptr(), ws.numel(), stream), "ga_spmm_csr")
+    return out
+
+
 # ------------------------------------------------------ dense projection ----
 # fp32 projections with at most this many output columns and at least this many rows
 # run on the library's own kernel (one pass over the rows, 1.2-2.1x the rate of the

@@ -5,8 +5,8 @@ import pytest
 import torch
 
 import oracle
-from graphiler_amd import datasets, layers, prepare_graph
-from graphiler_amd.graph import build_graph_arrays
+from graphiler_amd import capi, datasets, layers, prepare_graph
+from graphiler_amd.graph import build_graph_arrays, sort_edges_by_type
 from helpers import TOL_BF16, TOL_F32, assert_close, to_bf16_f32
 
 pytestmark = pytest.mark.gpu
@@ -121,7 +121,7 @@ def test_rgcn_two_layers(device, bf16, fused):
     assert_close(h2.float().cpu().numpy(), ref_layer(r1, w2), 2 * tol, "RGCN layer 2")
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", [True, "pairs", "edges", False])
 @pytest.mark.parametrize("bf16", [False, True])
 def test_hgt_layer(device, bf16, fused):
     wl = datasets.hgt_hetero(counts=(800, 600, 400, 200), edges_per_type=4000)
@@ -161,3 +161,39 @@ def test_hgt_layer(device, bf16, fused):
     out = oracle.segment_mm(ntp, t, wa) * (1.0 / (1.0 + np.exp(-skip[wl.ntype])))[:, None]
     assert_close(got.float().cpu().numpy(), out, TOL_BF16 if bf16 else TOL_F32,
                  f"HGT layer bf16={bf16}")
+
+
+@pytest.mark.parametrize("heads,d", [(8, 16), (2, 32), (1, 16), (4, 8)])
+def test_hgt_pair_form_equals_edge_form(device, heads, d):
+    """The relation matrices applied per (destination, relation) pair against per edge:
+    few edges per pair, destinations without in-edges, a relation without edges, a
+    destination with a large share of the edges; fp32, so the two forms differ by
+    rounding order only.  Head widths the typed product does not take fall back."""
+    rng = np.random.default_rng(heads * 100 + d)
+    n, e, tn, te = 900, 7000, 3, 6
+    hid = heads * d
+    src = rng.integers(0, n, e)
+    dst = rng.integers(0, n // 2, e)                 # upper half: no in-edges
+    dst[: e // 4] = 7                                 # one destination with a quarter of the edges
+    et = rng.choice([0, 1, 2, 4, 5], size=e)          # relation 3 has no edges
+    src, dst, et, _ = sort_edges_by_type(src, dst, et)
+    nt = np.sort(rng.integers(0, tn, n))
+    g = prepare_graph(src, dst, n, device=device, ntype_of=nt, num_ntypes=tn, etype_of=et,
+                      num_etypes=te)
+    pairs = g.relation_pairs()
+    key = np.unique(dst.astype(np.int64) * te + et)
+    assert pairs is not None and pairs.num_pairs == len(key)
+    assert np.array_equal(pairs.pair_dst.cpu().numpy(), key // te)
+    counts = np.diff(pairs.pair_pointer.cpu().numpy())
+    assert counts.sum() == e and counts.min() >= 1
+    h = _t(rng.standard_normal((n, hid), dtype=np.float32), device)
+    wk, wq, wv, wa = (_t(datasets.glorot(rng, (tn, hid, hid)), device) for _ in range(4))
+    ratt, rmsg = (_t(datasets.glorot(rng, (te, heads, d, d)), device) for _ in range(2))
+    rpri = _t(rng.uniform(0.5, 1.5, (te, heads)).astype(np.float32), device)
+    skip = _t(rng.standard_normal(tn).astype(np.float32), device)
+    args = (g, h, wk, wq, wv, wa, ratt, rmsg, rpri, skip, heads)
+    want = layers.hgt_layer(*args, fused=False)
+    got = layers.hgt_layer(*args, fused="pairs")
+    assert_close(got.cpu().numpy(), want.cpu().numpy(), 2 * TOL_F32, f"HGT pairs {heads}x{d}")
+    auto = layers.hgt_layer(*args, fused=True)
+    assert_close(auto.cpu().numpy(), want.cpu().numpy(), 2 * TOL_F32, f"HGT auto {heads}x{d}")
