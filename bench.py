@@ -432,11 +432,12 @@ def main():
         edges_bytes = N * hid * b * 9 + E * (3 * hid * b + 2 * hid * b + 24 + 4 * 4 * H)
         edges_flops = 2.0 * N * hid * hid * 4 + 4.0 * E * H * D * D
         # ... per (destination, relation) pair, the form the layer takes on this graph: node
-        # rows as before, per edge the gathered k / v rows, the pair's transformed q row, five
-        # index reads and the scores (written, normalised in place, read); per pair the q row
-        # read, its transform written, the weighted sum and its transform written and read
+        # rows as before, per edge the gathered k / v rows, the pair's transformed q row and
+        # three index reads (scores stay in registers); per pair the q row read, its transform
+        # written, the weighted sum and its transform written and read, the log-sum-exp
+        # written, normalised in place and read
         P = g.relation_pairs().num_pairs
-        pairs_bytes = N * hid * b * 9 + P * hid * b * 6 + E * (3 * hid * b + 20 + 4 * 4 * H)
+        pairs_bytes = N * hid * b * 9 + P * (hid * b * 6 + 4 * 4 * H) + E * (3 * hid * b + 12)
         pairs_flops = 2.0 * N * hid * hid * 4 + 4.0 * P * H * D * D + 4.0 * E * hid
         by_pairs = E >= layers.PAIRS_MIN_EDGES_PER_PAIR * P
         rec["num_pairs"] = P

@@ -216,6 +216,133 @@ struct GatPolicy {
   }
 };
 
+// Dot-product attention over an adjacency: slot i of row r weighs the value row
+// v[nbr[i]] with softmax_r(<k[nbr[i]], q[qrow[i]]>), per head; beside the weighted sum
+// the row's log-sum-exp is written, so that rows which are pieces of one softmax (the
+// (destination, relation) pairs of an HGT layer) can be combined afterwards.  State,
+// merge and finish are the fused GAT aggregation's; only the logits differ: a second
+// gathered row (k) and the slot's query row, which consecutive slots of a pair share.
+template <typename T, int VEC>
+struct DotAttnPolicy : GatPolicy<T, VEC, kGatEdge, false> {
+  typedef GatPolicy<T, VEC, kGatEdge, false> Base;
+  struct Args {
+    const int32_t *nbr;    // key / value row of a slot
+    const int32_t *qrow;   // query row of a slot
+    const T *k, *q, *v;    // rows of heads * dph features
+    float *lse;            // (n_rows, heads) or null
+    int heads;
+    int dph;
+    int head_lanes;        // lanes that share a head (dph / VEC)
+    bool ids_vec;          // row_of_slot, nbr and qrow are 16-byte aligned
+  };
+  static __device__ __forceinline__ void emit(const Args &A, T *out, int64_t row, int feat, int f0,
+                                              const float (&st)[VEC + 2]) {
+    emit_row<DotAttnPolicy>(out, row, feat, f0, st);
+    if (A.lse && f0 % A.dph == 0)
+      A.lse[row * A.heads + f0 / A.dph] = st[VEC] + logf(st[VEC + 1]);
+  }
+  static __device__ __forceinline__ void emit_empty(const Args &A, T *out, int64_t row, int feat,
+                                                    int f0) {
+    emit_empty_row<DotAttnPolicy>(out, row, feat, f0);
+    if (A.lse && f0 % A.dph == 0) A.lse[row * A.heads + f0 / A.dph] = -INFINITY;
+  }
+
+  template <class Close>
+  static __device__ __forceinline__ void walk(const Args &A,
+                                              const int32_t *__restrict__ row_of_slot,
+                                              int64_t a, int64_t b, int f0, int feat,
+                                              float (&st)[VEC + 2], int &cur,
+                                              Close &&close_segment) {
+    typedef RowIO<T, VEC, false> IO;
+    const typename IO::lane_t ln = IO::lane(0, feat - f0);
+    for (int64_t j = a; j < b; j += kUnroll) {
+      int r[kUnroll], g[kUnroll], qr[kUnroll];
+      float s[kUnroll];
+      typename IO::raw_t x[kUnroll], kx[kUnroll], qx[kUnroll];
+      load_ids8(row_of_slot, j, b, A.ids_vec, r);
+      load_ids8(A.nbr, j, b, A.ids_vec, g);
+      load_ids8(A.qrow, j, b, A.ids_vec, qr);
+#pragma unroll
+      for (int t = 0; t < kUnroll; ++t) {
+        kx[t] = IO::load(A.k + (int64_t)g[t] * feat + f0, ln);
+        qx[t] = IO::load(A.q + (int64_t)qr[t] * feat + f0, ln);
+        x[t] = IO::load(A.v + (int64_t)g[t] * feat + f0, ln);
+      }
+      // every live lane of a head runs this together (heads tile the row)
+#pragma unroll
+      for (int t = 0; t < kUnroll; ++t) {
+        float kf[VEC], qf[VEC];
+        IO::widen(kx[t], kf);
+        IO::widen(qx[t], qf);
+        float d = 0.0f;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) d = fmaf(kf[v], qf[v], d);
+        s[t] = lanes_sum(d, A.head_lanes);
+      }
+      const bool one_row = j + kUnroll <= b && r[0] == cur && r[kUnroll - 1] == cur;
+      if (one_row) {
+        // whole batch inside the open row (rows are sorted): one rescale
+        float bm = s[0];
+#pragma unroll
+        for (int t = 1; t < kUnroll; ++t) bm = fmaxf(bm, s[t]);
+        const float nm = fmaxf(st[VEC], bm);
+        const float ref = finite_or_zero(nm);
+        const float sc = __expf(st[VEC] - ref);
+        st[VEC + 1] *= sc;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) st[v] *= sc;
+        st[VEC] = nm;
+#pragma unroll
+        for (int t = 0; t < kUnroll; ++t) {
+          const float p = __expf(s[t] - ref);
+          st[VEC + 1] += p;
+          float xf[VEC];
+          IO::widen(x[t], xf);
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) st[v] = fmaf(p, xf[v], st[v]);
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < kUnroll; ++t) {
+          if (j + t < b) {
+            if (r[t] != cur) {
+              close_segment();
+              cur = r[t];
+              Base::init(st);
+            }
+            const float nm = fmaxf(st[VEC], s[t]);
+            const float ref = finite_or_zero(nm);
+            const float sc = __expf(st[VEC] - ref);
+            const float p = __expf(s[t] - ref);
+            st[VEC + 1] = st[VEC + 1] * sc + p;
+            float xf[VEC];
+            IO::widen(x[t], xf);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) st[v] = fmaf(p, xf[v], st[v] * sc);
+            st[VEC] = nm;
+          }
+        }
+      }
+    }
+  }
+};
+
+template <typename T, int VEC>
+int launch_dot_attn(const int32_t *pointer, const int32_t *row_of_slot, const int32_t *nbr,
+                    const int32_t *qrow, const void *k, const void *q, const void *v, void *out,
+                    float *lse, int64_t n_rows, int64_t n_edges, int heads, int dim, float *ws,
+                    size_t ws_bytes, hipStream_t stream) {
+  typedef DotAttnPolicy<T, VEC> P;
+  const int head_lanes = dim / VEC;
+  if (dim % VEC != 0 || head_lanes > 16 || (head_lanes & (head_lanes - 1)) != 0)
+    return GA_EUNSUPPORTED;
+  const bool ids_vec = aligned(row_of_slot, 16) && aligned(nbr, 16) && aligned(qrow, 16);
+  typename P::Args args{nbr, qrow, (const T *)k, (const T *)q, (const T *)v, lse,
+                        heads, dim, head_lanes, ids_vec};
+  return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, heads * dim, ws,
+                        stream, ws_bytes);
+}
+
 template <typename T, int VEC, int MODE = kGatNode, bool SPREAD = false>
 int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const int32_t *nbr, const float *el, const float *er,
@@ -418,6 +545,40 @@ int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,
                                                              m, out, n_rows, n_edges, 1, d, 0.0f, ws, s);
   return ga::launch_gat<ga::bf16_t, 1, ga::kGatEdge>(pointer, row_of_slot, eid, logit, nullptr, m,
                                              out, n_rows, n_edges, h, d, 0.0f, ws, s);
+}
+
+int ga_dot_attention_sum(const int32_t *pointer, const int32_t *row_of_slot,
+                         const int32_t *nbr, const int32_t *qrow, const void *k, const void *q,
+                         const void *v, void *out, float *lse, int64_t n_rows, int64_t n_edges,
+                         int64_t heads, int64_t dim, int dtype, void *workspace,
+                         size_t workspace_bytes, ga_stream_t stream) {
+  if (n_rows < 0 || n_edges < 0 || heads <= 0 || dim <= 0) return GA_EINVAL;
+  if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || heads * dim > 0x7fffffff)
+    return GA_EINVAL;
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  if (n_rows == 0) return GA_OK;
+  if (!pointer || !out) return GA_EINVAL;
+  const int64_t feat = heads * dim;
+  if (n_edges > 0) {
+    if (!row_of_slot || !nbr || !qrow || !k || !q || !v) return GA_EINVAL;
+    if (!workspace || !ga::aligned(workspace, 16) ||
+        ga_gat_workspace_bytes(n_edges, feat, heads) > workspace_bytes)
+      return GA_EWORKSPACE;
+  }
+  if (lse && !ga::aligned(lse, 4)) return GA_EALIGN;
+  // rows are read and written in 16-byte pieces that do not straddle a head
+  const int vec = dtype == GA_F32 ? 4 : 8;
+  if (!ga::aligned(out, 16) || (k && !ga::aligned(k, 16)) || (q && !ga::aligned(q, 16)) ||
+      (v && !ga::aligned(v, 16)) || dim % vec != 0)
+    return GA_EUNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == GA_F32)
+    return ga::launch_dot_attn<float, 4>(pointer, row_of_slot, nbr, qrow, k, q, v, out, lse, n_rows,
+                                         n_edges, (int)heads, (int)dim, (float *)workspace,
+                                         workspace_bytes, s);
+  return ga::launch_dot_attn<ga::bf16_t, 8>(pointer, row_of_slot, nbr, qrow, k, q, v, out, lse,
+                                            n_rows, n_edges, (int)heads, (int)dim,
+                                            (float *)workspace, workspace_bytes, s);
 }
 
 int ga_gat_aggregate_from_z(const int32_t *pointer, const int32_t *row_of_slot,

@@ -835,6 +835,33 @@ def edge_softmax_sum(logits, messages, graph: DGLGraph) -> torch.Tensor:
     return out
 
 
+def dot_attention_sum(k, q, v, graph: DGLGraph, return_lse: bool = False):
+    """out[v] = sum over the in-edges e of v of softmax_v(<k[src], q[v]>)[e] * v[src], per
+    head: ``sum(k * q)`` -> SegmentSoftmax -> mul -> SpMM (examples/HGT/HGT.py:44-53
+    without its relation matrices) in one pass, nothing per edge written.  k, q, v
+    (N, H, D) or (N, D) (one head).  ``return_lse``: also the (N, H) fp32 log of every
+    destination's sum of exponentials (-inf without in-edges)."""
+    for name, x in (("k", k), ("q", q), ("v", v)):
+        _check_input(x, name)
+    dt = _feat_dtype(k, "k")
+    if q.dtype != k.dtype or v.dtype != k.dtype or q.shape != k.shape or v.shape != k.shape \
+            or k.dim() not in (2, 3) or int(k.shape[0]) != graph.num_nodes:
+        raise RuntimeError("k, q and v must be (nodes, heads, D) or (nodes, D) of one dtype")
+    heads = 1 if k.dim() == 2 else int(k.shape[1])
+    d = int(k.shape[-1])
+    out = torch.empty_like(v)
+    lse = torch.empty((graph.num_nodes, heads), dtype=torch.float32, device=k.device) \
+        if return_lse else None
+    lib = capi.load()
+    ws = graph.workspace(lib.ga_gat_workspace_bytes(graph.num_edges, heads * d, heads))
+    capi.check(lib.ga_dot_attention_sum(
+        graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
+        graph.in_node_indices.data_ptr(), graph.in_row_of_slot.data_ptr(), k.data_ptr(),
+        q.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(lse), graph.num_nodes, graph.num_edges,
+        heads, d, dt, ws.data_ptr(), ws.numel(), _stream(out)), "ga_dot_attention_sum")
+    return (out, lse) if return_lse else out
+
+
 def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
                             graph: DGLGraph) -> torch.Tensor:
     """The message and reduce stages of an HGT layer (examples/HGT/HGT.py:35-53) with
@@ -889,16 +916,39 @@ def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
         return y
 
     q_pair = typed_rows(q, pairs.dst_by_type, att_t)
+    ws = graph.workspace(max(lib.ga_softmax_workspace_bytes(e, heads),
+                             lib.ga_spmm_workspace_bytes(e, hid),
+                             lib.ga_gat_workspace_bytes(e, hid, heads)))
+    # scores, softmax inside every pair and the pair's weighted sum of value rows in one
+    # pass; the pairs of a destination are then weighed by the softmax of their
+    # log-sum-exps, which makes the weights the softmax over all its in-edges
+    v_pair = torch.empty((P, hid), dtype=v.dtype, device=dev)            # pair order
+    lse = torch.empty((P, heads), dtype=torch.float32, device=dev)
+    rc = lib.ga_dot_attention_sum(
+        pairs.pair_pointer.data_ptr(), pairs.pair_of_slot.data_ptr(),
+        graph.in_node_indices.data_ptr(), pairs.rank_of_slot.data_ptr(), k.data_ptr(),
+        q_pair.data_ptr(), v.data_ptr(), v_pair.data_ptr(), lse.data_ptr(), P, e, heads, d, dt,
+        ws.data_ptr(), ws.numel(), stream)
+    if rc != capi.GA_EUNSUPPORTED:
+        capi.check(rc, "ga_dot_attention_sum")
+        capi.check(lib.ga_segment_softmax(
+            pairs.dst_pointer.data_ptr(), pairs.pair_dst.data_ptr(), None, lse.data_ptr(),
+            lse.data_ptr(), n, P, heads, ws.data_ptr(), ws.numel(), stream), "ga_segment_softmax")
+        m_pair = typed_rows(v_pair, pairs.by_type, relation_msg)         # by_type order
+        out = torch.empty((n, hid), dtype=v.dtype, device=dev)
+        capi.check(lib.ga_spmm_csr(
+            pairs.dst_pointer.data_ptr(), pairs.pair_dst.data_ptr(), pairs.rank.data_ptr(), None,
+            m_pair.data_ptr(), lse.data_ptr(), out.data_ptr(), n, P, hid, heads, capi.GA_U_MUL_E,
+            capi.GA_SUM, dt, ws.data_ptr(), ws.numel(), stream), "ga_spmm_csr")
+        return out
+    # head widths outside that kernel: the three steps as separate operators
     score = torch.empty((e, heads), dtype=torch.float32, device=dev)      # slot order
     capi.check(lib.ga_sddmm_u_dot_v(
         graph.in_node_indices.data_ptr(), pairs.rank_of_slot.data_ptr(), 32, k.data_ptr(),
         q_pair.data_ptr(), score.data_ptr(), e, heads, d, dt, stream), "ga_sddmm_u_dot_v")
-    ws = graph.workspace(max(lib.ga_softmax_workspace_bytes(e, heads),
-                             lib.ga_spmm_workspace_bytes(e, hid)))
     capi.check(lib.ga_segment_softmax(
         graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(), None, score.data_ptr(),
         score.data_ptr(), n, e, heads, ws.data_ptr(), ws.numel(), stream), "ga_segment_softmax")
-    v_pair = torch.empty((P, hid), dtype=v.dtype, device=dev)            # pair order
     capi.check(lib.ga_spmm_csr(
         pairs.pair_pointer.data_ptr(), pairs.pair_of_slot.data_ptr(),
         graph.in_node_indices.data_ptr(), None, v.data_ptr(), score.data_ptr(),

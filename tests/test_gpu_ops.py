@@ -358,6 +358,89 @@ def _hub_graph(seed):
     return src, dst, n
 
 
+def _dot_attention_reference(arr, k, q, v, heads):
+    """sum(k * q) -> segment softmax -> weighted sum on the oracle, and the rows' log-sum-exp."""
+    n, e = arr.num_nodes, arr.COO_src.shape[0]
+    score = oracle.sddmm_u_dot_v(arr.COO_src, arr.COO_dst, k, q).astype(np.float32)
+    att = oracle.segment_softmax(arr.in_pointer, arr.in_edge_indices, score)
+    out = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      v.reshape(n, -1), att, op="u_mul_e", heads=heads)
+    mag = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
+                      np.abs(v).reshape(n, -1), att, op="u_mul_e", heads=heads)
+    lse = np.full((n, heads), -np.inf)
+    big = np.full((n, heads), -np.inf)
+    np.maximum.at(big, arr.COO_dst, score.astype(np.float64))
+    tot = np.zeros((n, heads))
+    np.add.at(tot, arr.COO_dst, np.exp(score.astype(np.float64) - big[arr.COO_dst]))
+    has = np.diff(arr.in_pointer) > 0
+    lse[has] = big[has] + np.log(tot[has])
+    return out, mag, lse
+
+
+@pytest.mark.parametrize("heads,dim", [(8, 16), (1, 64), (4, 8), (2, 32), (1, 128), (16, 8)])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_dot_attention_sum(graph, device, heads, dim, bf16):
+    """ga_dot_attention_sum over the graph's in-adjacency (queries on the destinations)."""
+    name, g, arr = graph
+    rng = np.random.default_rng(heads * 1000 + dim)
+    n = arr.num_nodes
+    k, q, v = (rng.standard_normal((n, heads, dim), dtype=np.float32) for _ in range(3))
+    k *= 0.5
+    if bf16:
+        k, q, v = to_bf16_f32(k), to_bf16_f32(q), to_bf16_f32(v)
+    if dim // (8 if bf16 else 4) > 16:          # a head wider than 16 lanes of 16 bytes
+        if arr.COO_src.shape[0]:
+            with pytest.raises(capi.GraphilerError) as err:
+                ops.dot_attention_sum(_dev(k, device, bf16), _dev(q, device, bf16),
+                                      _dev(v, device, bf16), g)
+            assert err.value.code == capi.GA_EUNSUPPORTED
+        return
+    out, lse = ops.dot_attention_sum(_dev(k, device, bf16), _dev(q, device, bf16),
+                                     _dev(v, device, bf16), g, return_lse=True)
+    assert out.shape == (n, heads, dim) and lse.shape == (n, heads)
+    ref, mag, ref_lse = _dot_attention_reference(arr, k, q, v, heads)
+    assert_close(out.float().cpu().numpy().reshape(n, -1), ref, TOL_BF16 if bf16 else TOL_F32,
+                 f"dot attention {name} {heads}x{dim}", mag=mag)
+    got_lse = lse.cpu().numpy()
+    has = np.diff(arr.in_pointer) > 0
+    assert np.all(np.isneginf(got_lse[~has])) and np.all(np.isfinite(got_lse[has]))
+    if has.any():
+        assert np.abs(got_lse[has] - ref_lse[has]).max() <= 2e-5 * max(1.0, np.abs(ref_lse[has]).max())
+    only = ops.dot_attention_sum(_dev(k, device, bf16), _dev(q, device, bf16), _dev(v, device, bf16), g)
+    assert torch.equal(only.view(torch.int16 if bf16 else torch.int32),
+                       out.view(torch.int16 if bf16 else torch.int32))
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_dot_attention_sum_long_rows_and_rejects(device, bf16):
+    """Rows of 150,000 / 5,000 / 2,500 slots (partial states chained across workgroups),
+    and the shapes the kernel does not take."""
+    src, dst, n = _hub_graph(11)
+    g = prepare_graph(src, dst, n, device=device)
+    arr = build_graph_arrays(src, dst, n)
+    rng = np.random.default_rng(12)
+    heads, dim = 4, 16
+    k, q, v = (rng.standard_normal((n, heads, dim), dtype=np.float32) for _ in range(3))
+    k *= 0.25
+    if bf16:
+        k, q, v = to_bf16_f32(k), to_bf16_f32(q), to_bf16_f32(v)
+    out, lse = ops.dot_attention_sum(_dev(k, device, bf16), _dev(q, device, bf16),
+                                     _dev(v, device, bf16), g, return_lse=True)
+    ref, mag, ref_lse = _dot_attention_reference(arr, k, q, v, heads)
+    assert_close(out.float().cpu().numpy().reshape(n, -1), ref, TOL_BF16 if bf16 else TOL_F32,
+                 "dot attention, long rows", mag=mag)
+    has = np.diff(arr.in_pointer) > 0
+    assert np.abs(lse.cpu().numpy()[has] - ref_lse[has]).max() <= 2e-5 * np.abs(ref_lse[has]).max()
+    bad = torch.randn(n, 2, 6, device=device)                    # heads of 6: not 4 (8) values wide
+    if bf16:
+        bad = bad.bfloat16()
+    with pytest.raises(capi.GraphilerError) as err:
+        ops.dot_attention_sum(bad, bad, bad, g)
+    assert err.value.code == capi.GA_EUNSUPPORTED
+    with pytest.raises(RuntimeError):
+        ops.dot_attention_sum(_dev(k, device, bf16), _dev(q, device, bf16)[:, :2], _dev(v, device, bf16), g)
+
+
 @pytest.mark.parametrize("feat,heads,bf16", [(64, 1, False), (256, 4, True), (17, 1, False),
                                              (1, 1, False), (128, 8, False)])
 def test_row_reductions_over_many_workgroups(device, feat, heads, bf16):
