@@ -884,6 +884,19 @@ inline int pow2_ceil_int(int v) {
   return p;
 }
 
+int mm_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      cus = v;
+    else
+      cus = 256;
+  }
+  return cus;
+}
+
 // One launch for `hb` folded heads starting at head h0.
 template <typename T, int KBLK>
 int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
@@ -904,7 +917,11 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
   g.perm_shift = -1;
   // rows per workgroup: a multiple of the 64-row step, large enough to
   // amortise the weight staging, small enough to keep every CU busy
-  int64_t steps = rows / (kTileBlock * 1024);
+  // (the device holds three of these workgroups per CU at once: up to 16 steps, the
+  // fewest with which the grid still fits one such round -- at 269 k rows 6 steps take
+  // 30 us, 4 steps 38 and 12 steps 40)
+  const int64_t slots = 3 * (int64_t)mm_cu_count() - n_types;
+  int64_t steps = (rows + kTileBlock * (slots > 1 ? slots : 1) - 1) / (kTileBlock * (slots > 1 ? slots : 1));
   if (steps < 1) steps = 1;
   if (steps > 16) steps = 16;
   g.chunk_rows = (int)steps * kTileBlock;
