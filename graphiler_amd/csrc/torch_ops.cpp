@@ -190,6 +190,67 @@ struct DGLGraph : torch::CustomClassHolder {
     }
     return tiles_;
   }
+  // The (destination, relation) pairs of the in-adjacency: runs of slots with one
+  // destination and one relation (the slots of a destination are grouped by relation
+  // when edge ids are sorted by type).  Pairs are numbered in slot order; `by_type`
+  // lists them by relation, the row order of the typed products.  Built on first use
+  // with library sorts and scans; `valid` is false when the slots are not so grouped.
+  struct RelationPairs {
+    int64_t num_pairs = 0;
+    torch::Tensor pair_pointer, pair_of_slot, pair_dst, dst_pointer, type_pointer;   // int32
+    torch::Tensor by_type, dst_by_type;                                              // int64
+    torch::Tensor rank, rank_of_slot;                                                // int32
+    bool valid = false;
+    bool ready = false;
+  };
+  const RelationPairs &relation_pairs() {
+    const Side &in = side(false);
+    std::lock_guard<std::mutex> lock(mu_);
+    if (!pairs_.ready) {
+      pairs_.ready = true;
+      if (etype_pointer.has_value() && num_edges > 0) {
+        const auto i64 = in_pointer.options().dtype(at::kLong);
+        torch::Tensor rows = in.rows.to(at::kLong), eid = in_edge_indices.to(at::kLong);
+        torch::Tensor bounds = etype_pointer.value().slice(0, 1).to(at::kLong).contiguous();
+        torch::Tensor etype = torch::bucketize(eid, bounds, /*out_int32=*/false, /*right=*/true);
+        torch::Tensor key = rows * num_etypes + etype;
+        const bool grouped =
+            num_edges < 2 || key.slice(0, 1).ge(key.slice(0, 0, num_edges - 1)).all().item<bool>();
+        if (grouped) {
+          torch::Tensor first = torch::ones({num_edges}, i64.dtype(at::kBool));
+          if (num_edges > 1)
+            first.slice(0, 1).copy_(key.slice(0, 1).ne(key.slice(0, 0, num_edges - 1)));
+          torch::Tensor pair_of_slot = torch::cumsum(first, 0) - 1;
+          torch::Tensor starts = torch::nonzero(first).reshape({-1});
+          const int64_t P = starts.size(0);
+          torch::Tensor pair_key = key.index_select(0, starts);
+          torch::Tensor pair_dst = torch::floor_divide(pair_key, num_etypes);
+          torch::Tensor pair_type = pair_key - pair_dst * num_etypes;
+          torch::Tensor by_type = torch::argsort(pair_type, /*stable=*/true, 0, false);
+          torch::Tensor rank = torch::empty_like(by_type);
+          rank.index_copy_(0, by_type, torch::arange(P, i64));
+          pairs_.num_pairs = P;
+          pairs_.pair_pointer =
+              torch::cat({starts, torch::full({1}, num_edges, i64)}).to(at::kInt).contiguous();
+          pairs_.pair_of_slot = pair_of_slot.to(at::kInt).contiguous();
+          pairs_.pair_dst = pair_dst.to(at::kInt).contiguous();
+          pairs_.dst_pointer = torch::searchsorted(pair_dst.contiguous(),
+                                                   torch::arange(num_nodes + 1, i64))
+                                   .to(at::kInt).contiguous();
+          pairs_.type_pointer =
+              torch::searchsorted(pair_type.index_select(0, by_type).contiguous(),
+                                  torch::arange(num_etypes + 1, i64))
+                  .to(at::kInt).contiguous();
+          pairs_.by_type = by_type.contiguous();
+          pairs_.dst_by_type = pair_dst.index_select(0, by_type).contiguous();
+          pairs_.rank = rank.to(at::kInt).contiguous();
+          pairs_.rank_of_slot = rank.index_select(0, pair_of_slot).to(at::kInt).contiguous();
+          pairs_.valid = true;
+        }
+      }
+    }
+    return pairs_;
+  }
   // Scratch shared by the operators called on this graph: calls that use it must be
   // ordered on one stream (two streams working on one graph object race on it).  It
   // grows on demand; a buffer that was handed out is never freed while the graph
@@ -208,6 +269,7 @@ struct DGLGraph : torch::CustomClassHolder {
   std::mutex mu_;
   Side in_side_, out_side_;
   TypedTiles tiles_;
+  RelationPairs pairs_;
   torch::Tensor ws_;
   std::vector<torch::Tensor> retired_ws_;
 };
@@ -783,6 +845,94 @@ torch::Tensor edge_softmax_sum(torch::Tensor logits, torch::Tensor messages,
   return out;
 }
 
+// edge_softmax_sum(SegmentMMEdgeDot(k, att, 0, q, 1, scale) / divisor,
+//                  SegmentMMEdgeGather(v, msg, 0)): the message and reduce stages of an HGT
+// layer (examples/HGT/HGT.py:35-53).  Both relation products are linear in a matrix per
+// relation, so with at least two edges per (destination, relation) pair they are applied
+// per pair instead of per edge:
+//   score = <k[src], q[dst] (s A)^T>,  out[v] = sum_pairs (sum_{e in pair} a_e v[src]) M
+// with one pass over the slots for scores, softmax inside the pair and weighted sum
+// (ga_dot_attention_sum), the pairs of a destination weighed by the softmax of their
+// log-sum-exps.  Graphs without such pairs and shapes outside those kernels run the
+// three per-edge operators.
+torch::Tensor relation_pair_attention(torch::Tensor k, torch::Tensor q, torch::Tensor v,
+                                      torch::Tensor relation_att, torch::Tensor relation_msg,
+                                      at::optional<torch::Tensor> scale, double divisor,
+                                      const GraphPtr &graph) {
+  auto per_edge = [&]() {
+    torch::Tensor score = SegmentMMEdgeDot(k, relation_att, 0, q, 1, scale, graph);
+    if (divisor != 1.0) score = score / divisor;
+    return edge_softmax_sum(score, SegmentMMEdgeGather(v, relation_msg, 0, at::nullopt, graph),
+                            graph);
+  };
+  // (T, D, D) matrices are one head
+  const int64_t wd = relation_att.dim();
+  const bool shapes = (wd == 3 || wd == 4) && relation_att.sizes() == relation_msg.sizes() &&
+                      relation_att.size(wd - 2) == relation_att.size(wd - 1) && k.dim() == 2 &&
+                      k.sizes() == q.sizes() && k.sizes() == v.sizes() && k.is_cuda() &&
+                      q.is_cuda() && v.is_cuda() && relation_att.is_cuda() &&
+                      relation_msg.is_cuda() && k.is_contiguous() && q.is_contiguous() &&
+                      v.is_contiguous() && relation_msg.is_contiguous() &&
+                      (k.scalar_type() == at::kFloat || k.scalar_type() == at::kBFloat16) &&
+                      q.scalar_type() == k.scalar_type() && v.scalar_type() == k.scalar_type() &&
+                      relation_att.scalar_type() == k.scalar_type() &&
+                      relation_msg.scalar_type() == k.scalar_type() &&
+                      relation_att.size(0) == graph->num_etypes &&
+                      k.size(0) == graph->num_nodes &&
+                      k.size(1) == (wd == 4 ? relation_att.size(1) : 1) * relation_att.size(wd - 1) &&
+                      graph->etype_pointer.has_value();
+  if (!shapes) return per_edge();
+  const int64_t heads = wd == 4 ? relation_att.size(1) : 1, d = relation_att.size(wd - 1);
+  const int64_t hid = heads * d;
+  if (scale.has_value() && scale.value().numel() != graph->num_etypes * heads) return per_edge();
+  const DGLGraph::RelationPairs &pairs = graph->relation_pairs();
+  const int64_t n = graph->num_nodes, e = graph->num_edges, P = pairs.num_pairs;
+  if (!pairs.valid || e < 2 * P) return per_edge();
+  const int dt = feat_dtype(k, "k");
+  torch::Tensor att_t = relation_att.reshape({graph->num_etypes, heads, d, d}).transpose(-1, -2);
+  if (scale.has_value())
+    att_t = att_t * scale.value().to(at::kFloat).reshape({graph->num_etypes, heads, 1, 1});
+  if (divisor != 1.0) att_t = att_t.to(at::kFloat) / divisor;
+  att_t = att_t.to(k.scalar_type()).contiguous();
+  const auto stream = current_stream(k);
+  auto typed_rows = [&](const torch::Tensor &x, const torch::Tensor &index,
+                        const torch::Tensor &w, torch::Tensor &y) {
+    return ga_segment_mm_gather(pairs.type_pointer.data_ptr<int>(), graph->num_etypes,
+                                x.data_ptr(), index.data_ptr<int64_t>(), w.data_ptr(),
+                                y.data_ptr(), nullptr, nullptr, nullptr, nullptr, nullptr, P, heads,
+                                d, d, dt, stream);
+  };
+  torch::Tensor q_pair = torch::empty({P, hid}, k.options());
+  int rc = typed_rows(q, pairs.dst_by_type, att_t, q_pair);
+  if (rc == GA_EUNSUPPORTED) return per_edge();
+  check_ga(rc, "ga_segment_mm_gather");
+  torch::Tensor ws = graph->workspace(std::max(
+      {ga_gat_workspace_bytes(e, hid, heads), ga_softmax_workspace_bytes(P, heads),
+       ga_spmm_workspace_bytes(P, hid)}));
+  torch::Tensor v_pair = torch::empty({P, hid}, k.options());
+  torch::Tensor lse = torch::empty({P, heads}, k.options().dtype(at::kFloat));
+  rc = ga_dot_attention_sum(pairs.pair_pointer.data_ptr<int>(), pairs.pair_of_slot.data_ptr<int>(),
+                            graph->in_node_indices.data_ptr<int>(),
+                            pairs.rank_of_slot.data_ptr<int>(), k.data_ptr(), q_pair.data_ptr(),
+                            v.data_ptr(), v_pair.data_ptr(), lse.data_ptr<float>(), P, e, heads, d,
+                            dt, ws.data_ptr(), (size_t)ws.numel(), stream);
+  if (rc == GA_EUNSUPPORTED) return per_edge();
+  check_ga(rc, "ga_dot_attention_sum");
+  check_ga(ga_segment_softmax(pairs.dst_pointer.data_ptr<int>(), pairs.pair_dst.data_ptr<int>(),
+                              nullptr, lse.data_ptr<float>(), lse.data_ptr<float>(), n, P, heads,
+                              ws.data_ptr(), (size_t)ws.numel(), stream),
+           "ga_segment_softmax");
+  torch::Tensor m_pair = torch::empty({P, hid}, k.options());
+  check_ga(typed_rows(v_pair, pairs.by_type, relation_msg, m_pair), "ga_segment_mm_gather");
+  torch::Tensor out = torch::empty({n, hid}, k.options());
+  check_ga(ga_spmm_csr(pairs.dst_pointer.data_ptr<int>(), pairs.pair_dst.data_ptr<int>(),
+                       pairs.rank.data_ptr<int>(), nullptr, m_pair.data_ptr(),
+                       lse.data_ptr<float>(), out.data_ptr(), n, P, hid, heads, GA_U_MUL_E, GA_SUM,
+                       dt, ws.data_ptr(), (size_t)ws.numel(), stream),
+           "ga_spmm_csr");
+  return out;
+}
+
 // z = x @ w with the GAT attention terms from the same kernel (GAT.py:25-29);
 // fp32 or bf16 storage, el / er always fp32.  Returns the C-ABI code so that a
 // caller can fall back on GA_EUNSUPPORTED.
@@ -950,6 +1100,9 @@ static auto registry =
         .op("my_ops::SegmentMMEdgeDot(Tensor x, Tensor w, int endpoint, Tensor q, "
             "int q_endpoint, Tensor? scale, " GRAPH_T " g) -> Tensor z",
             &SegmentMMEdgeDot)
+        .op("my_ops::relation_pair_attention(Tensor k, Tensor q, Tensor v, Tensor att, Tensor msg, "
+            "Tensor? scale, float divisor, " GRAPH_T " g) -> Tensor t",
+            &relation_pair_attention)
         .op("my_ops::gat_aggregate(Tensor el, Tensor er, Tensor z, float slope, " GRAPH_T
             " g) -> Tensor y",
             &gat_aggregate)

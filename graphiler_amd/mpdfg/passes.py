@@ -507,6 +507,9 @@ class _Rewriter:
         for n in list(self.G.nodes()):
             if n.kind() == "aten::mul":
                 changed |= self._fuse_node_scale(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::edge_softmax_sum":
+                changed |= self._fuse_pair_attention(n)
         changed |= self._fuse_stacked_mm()
         return changed
 
@@ -655,6 +658,44 @@ class _Rewriter:
         n.output().replaceAllUsesWith(out)
         n.destroy()
         mm.destroy()
+        return True
+
+    def _fuse_pair_attention(self, n) -> bool:
+        """edge_softmax_sum(SegmentMMEdgeDot(k, A, src, q, dst, s) [/ c],
+        SegmentMMEdgeGather(v, M, src)) -> relation_pair_attention(k, q, v, A, M, s, c):
+        HGT's message and reduce stages as one operator, which applies the relation
+        matrices per (destination, relation) pair where the graph has such pairs and
+        runs these three operators otherwise."""
+        score, msg = n.inputsAt(0).node(), n.inputsAt(1).node()
+        if msg.kind() != "my_ops::SegmentMMEdgeGather" or not self.single_use(n.inputsAt(1)) \
+                or self.const_of(msg.inputsAt(2)) != 0 \
+                or msg.inputsAt(3).node().kind() != "prim::Constant" \
+                or not isinstance(msg.inputsAt(3).type(), torch._C.NoneType):
+            return False
+        divisor, div = None, None
+        if score.kind() == "aten::div" and self.single_use(n.inputsAt(0)) \
+                and score.inputsSize() == 2 \
+                and isinstance(score.inputsAt(1).type(), torch._C.FloatType):
+            div, divisor = score, score.inputsAt(1)
+            score = score.inputsAt(0).node()
+            if not self.single_use(div.inputsAt(0)):
+                return False
+        elif not self.single_use(n.inputsAt(0)):
+            return False
+        if score.kind() != "my_ops::SegmentMMEdgeDot" or self.const_of(score.inputsAt(2)) != 0 \
+                or self.const_of(score.inputsAt(4)) != 1:
+            return False
+        if divisor is None:
+            divisor = self.const(1.0, n)
+        out = self.make("my_ops::relation_pair_attention",
+                        [score.inputsAt(0), score.inputsAt(3), msg.inputsAt(0), score.inputsAt(1),
+                         msg.inputsAt(1), score.inputsAt(5), divisor, self.dglgraph], n, NODE)
+        n.output().replaceAllUsesWith(out)
+        n.destroy()
+        if div is not None:
+            div.destroy()
+        score.destroy()
+        msg.destroy()
         return True
 
     def _fuse_node_scale(self, n) -> bool:

@@ -137,6 +137,50 @@ def test_gat_aggregate_takes_bf16_attention_terms(setup, device):
         torch.ops.my_ops.gat_aggregate(el.int(), er, z, 0.2, sg)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_relation_pair_attention_op(device, bf16):
+    """my_ops::relation_pair_attention = edge_softmax_sum(SegmentMMEdgeDot(...) / c,
+    SegmentMMEdgeGather(...)): on a graph with many edges per (destination, relation)
+    pair it takes the per-pair form, on one with a pair per edge the per-edge operators;
+    (T, H, D, D) and (T, D, D) relation matrices."""
+    torch_boundary.load()
+    from graphiler_amd import ops as pyops
+    from graphiler_amd.graph import sort_edges_by_type
+    ops = torch.ops.my_ops
+    rng = np.random.default_rng(77)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    tol = 2e-2 if bf16 else 2 * TOL_F32
+    for n, e, te, dst_range in ((600, 9000, 3, 150), (3000, 2500, 5, 3000)):
+        src = rng.integers(0, n, e)
+        dst = rng.integers(0, dst_range, e)
+        et = rng.integers(0, te, e)
+        src, dst, et, _ = sort_edges_by_type(src, dst, et)
+        g = prepare_graph(src, dst, n, device=device, etype_of=et, num_etypes=te)
+        pairs = len(np.unique(dst.astype(np.int64) * te + et))
+        assert (e >= 2 * pairs) == (dst_range == 150)
+        sg = torch_boundary.script_graph(g)
+        for heads, d in ((4, 16), (1, 32)):
+            hid = heads * d
+            k, q, v = (torch.randn(n, hid, device=device).to(dt) for _ in range(3))
+            shape = (te, heads, d, d) if heads > 1 else (te, d, d)
+            att, msg = ((torch.randn(*shape, device=device) / d ** 0.5).to(dt) for _ in range(2))
+            pri = (torch.rand(te, heads, device=device) + 0.5).to(dt)
+            for scale, divisor in ((pri, 4.0), (None, 1.0)):
+                got = ops.relation_pair_attention(k, q, v, att, msg, scale, divisor, sg)
+                score = ops.SegmentMMEdgeDot(k, att, 0, q, 1, scale, sg) / divisor
+                want = ops.edge_softmax_sum(score, ops.SegmentMMEdgeGather(v, msg, 0, None, sg), sg)
+                assert got.shape == want.shape and got.dtype == want.dtype
+                assert_close(got.float().cpu().numpy(), want.float().cpu().numpy(), tol,
+                             f"relation_pair_attention {heads}x{d} e={e} scale={scale is not None}")
+                if scale is None and heads > 1 and e >= 2 * pairs:
+                    # the per-pair form was taken: the bits of the Python composition of the
+                    # same entry points, not those of the per-edge operators
+                    same = pyops.relation_pair_attention(k, q, v, att, msg, None, g)
+                    assert torch.equal(got.view(torch.int16 if bf16 else torch.int32),
+                                       same.view(torch.int16 if bf16 else torch.int32))
+                    assert not torch.equal(got, want)
+
+
 def test_error_convention(setup, device):
     sg, arr, rng = setup
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):

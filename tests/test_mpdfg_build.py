@@ -72,12 +72,14 @@ def test_level2_fuses_into_graph_operators():
     assert "aten::bmm" not in k and "aten::mul" not in k
     _, k = _kinds("hgt", 2)
     ours = [x for x in k if x.startswith("my_ops::")]
-    # K, V, Q read the node rows once; the output projection stays on its own
     # K, V, Q in one pass over h; the output projection takes the gate as its row factor
     assert ours.count("my_ops::SegmentMMNodeStacked") == 1 and ours.count("my_ops::SegmentMMNode") == 0
     assert ours.count("my_ops::SegmentMMNodeScaled") == 1 and "aten::mul" not in ours
-    assert "my_ops::SegmentMMEdgeDot" in ours            # sum(bmm(k, W_att) * q) in one pass
-    assert "my_ops::SegmentMMEdgeGather" in ours and "my_ops::edge_softmax_sum" in ours
+    # scores, softmax and weighted sum of transformed values as one operator (it picks the
+    # per-pair or the per-edge form from the graph it is given)
+    assert ours.count("my_ops::relation_pair_attention") == 1 and "aten::div" not in ours
+    assert not any(k in ours for k in ("my_ops::SegmentMMEdgeDot", "my_ops::SegmentMMEdgeGather",
+                                       "my_ops::edge_softmax_sum"))
     assert "my_ops::SegmentSoftmax" not in ours and "my_ops::gspmm_e_mul_e_sum" not in ours
     assert not any(x in ("my_ops::BroadcastSrcNode", "my_ops::BroadcastDstNode",
                          "my_ops::SegmentMMEdge", "my_ops::SpMMEdge") for x in ours)
