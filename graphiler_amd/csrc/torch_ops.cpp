@@ -845,6 +845,31 @@ torch::Tensor edge_softmax_sum(torch::Tensor logits, torch::Tensor messages,
   return out;
 }
 
+// out[v] = sum over the in-edges e of v of softmax_v(<k[src], q[v]>)[e] * v[src], per head
+// (sum(k * q) -> SegmentSoftmax -> mul -> SpMM in one pass): k, q, v (N, H, D) or (N, D).
+torch::Tensor dot_attention_sum(torch::Tensor k, torch::Tensor q, torch::Tensor v,
+                                const GraphPtr &graph) {
+  check_input(k, "k");
+  check_input(q, "q");
+  check_input(v, "v");
+  const int dt = feat_dtype(k, "k");
+  TORCH_CHECK((k.dim() == 2 || k.dim() == 3) && k.sizes() == q.sizes() && k.sizes() == v.sizes() &&
+                  q.scalar_type() == k.scalar_type() && v.scalar_type() == k.scalar_type() &&
+                  k.size(0) == graph->num_nodes,
+              "k, q and v must be (nodes, heads, D) or (nodes, D) of one dtype");
+  const int64_t heads = k.dim() == 3 ? k.size(1) : 1, d = k.size(k.dim() - 1);
+  const auto &side = graph->side(false);
+  torch::Tensor out = torch::empty_like(v);
+  torch::Tensor ws = graph->workspace(ga_gat_workspace_bytes(graph->num_edges, heads * d, heads));
+  check_ga(ga_dot_attention_sum(graph->in_pointer.data_ptr<int>(), side.rows.data_ptr<int>(),
+                                graph->in_node_indices.data_ptr<int>(), side.rows.data_ptr<int>(),
+                                k.data_ptr(), q.data_ptr(), v.data_ptr(), out.data_ptr(), nullptr,
+                                graph->num_nodes, graph->num_edges, heads, d, dt, ws.data_ptr(),
+                                (size_t)ws.numel(), current_stream(out)),
+           "ga_dot_attention_sum");
+  return out;
+}
+
 // edge_softmax_sum(SegmentMMEdgeDot(k, att, 0, q, 1, scale) / divisor,
 //                  SegmentMMEdgeGather(v, msg, 0)): the message and reduce stages of an HGT
 // layer (examples/HGT/HGT.py:35-53).  Both relation products are linear in a matrix per
@@ -1100,6 +1125,8 @@ static auto registry =
         .op("my_ops::SegmentMMEdgeDot(Tensor x, Tensor w, int endpoint, Tensor q, "
             "int q_endpoint, Tensor? scale, " GRAPH_T " g) -> Tensor z",
             &SegmentMMEdgeDot)
+        .op("my_ops::dot_attention_sum(Tensor k, Tensor q, Tensor v, " GRAPH_T " g) -> Tensor y",
+            &dot_attention_sum)
         .op("my_ops::relation_pair_attention(Tensor k, Tensor q, Tensor v, Tensor att, Tensor msg, "
             "Tensor? scale, float divisor, " GRAPH_T " g) -> Tensor t",
             &relation_pair_attention)

@@ -172,6 +172,13 @@ def test_relation_pair_attention_op(device, bf16):
                 assert got.shape == want.shape and got.dtype == want.dtype
                 assert_close(got.float().cpu().numpy(), want.float().cpu().numpy(), tol,
                              f"relation_pair_attention {heads}x{d} e={e} scale={scale is not None}")
+                if scale is None and divisor == 1.0:
+                    k3 = k.view(n, heads, d)
+                    att_only = ops.dot_attention_sum(k3, q.view(n, heads, d), v.view(n, heads, d), sg)
+                    same_op = pyops.dot_attention_sum(k3, q.view(n, heads, d), v.view(n, heads, d), g)
+                    assert att_only.shape == (n, heads, d) and torch.equal(
+                        att_only.view(torch.int16 if bf16 else torch.int32),
+                        same_op.view(torch.int16 if bf16 else torch.int32))
                 if scale is None and heads > 1 and e >= 2 * pairs:
                     # the per-pair form was taken: the bits of the Python composition of the
                     # same entry points, not those of the per-edge operators
