@@ -163,7 +163,7 @@ def test_hgt_layer(device, bf16, fused):
                  f"HGT layer bf16={bf16}")
 
 
-@pytest.mark.parametrize("heads,d", [(8, 16), (2, 32), (1, 16), (4, 8)])
+@pytest.mark.parametrize("heads,d", [(8, 16), (2, 32), (1, 16), (4, 8), (8, 12), (2, 24)])
 def test_hgt_pair_form_equals_edge_form(device, heads, d):
     """The relation matrices applied per (destination, relation) pair against per edge:
     few edges per pair, destinations without in-edges, a relation without edges, a
