@@ -377,7 +377,8 @@ def _dot_attention_reference(arr, k, q, v, heads):
     return out, mag, lse
 
 
-@pytest.mark.parametrize("heads,dim", [(8, 16), (1, 64), (4, 8), (2, 32), (1, 128), (16, 8)])
+@pytest.mark.parametrize("heads,dim", [(8, 16), (1, 64), (4, 8), (2, 32), (1, 128), (16, 8),
+                                       (16, 64), (8, 128)])     # more than one tile of 64 lanes per row
 @pytest.mark.parametrize("bf16", [False, True])
 def test_dot_attention_sum(graph, device, heads, dim, bf16):
     """ga_dot_attention_sum over the graph's in-adjacency (queries on the destinations)."""
