@@ -452,7 +452,8 @@ def main():
             kk, vv, qq = ops.SegmentMMNodeStacked(X, [wk, wv, wq], g)
             opsr["relation_pair_attention"] = op_record(
                 "c4.relation_pair_attention",
-                lambda: ops.relation_pair_attention(kk, qq, vv, ra, rm, rp.float() / D ** 0.5, g),
+                lambda: ops.relation_pair_attention(kk, qq, vv, ra, rm, rp.float(), g,
+                                                    factor=1.0 / D ** 0.5),
                 pairs_bytes - N * hid * b * 6, pairs_flops - 2.0 * N * hid * hid * 4, "bf16")
             opsr["segment_mm_node_128_128"] = op_record(
                 "c4.segment_mm_node", lambda: ops.SegmentMMNode(X, wk, g),

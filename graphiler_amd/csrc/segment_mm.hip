@@ -1202,6 +1202,46 @@ extern "C" int ga_project_attn(const void *X, const void *W, const float *a_l,
   return GA_EUNSUPPORTED;
 }
 
+namespace ga {
+namespace {
+// out[b][j][i] = W[b][i][j] * scale[b] * factor over square blocks of D x D values
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transpose_scale_blocks_kernel(
+    const T *__restrict__ W, const float *__restrict__ scale, float factor, T *__restrict__ out,
+    int D, int64_t total) {
+  const int64_t o = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (o >= total) return;
+  const int i = (int)(o % D), j = (int)(o / D % D);
+  const int64_t b = o / ((int64_t)D * D);
+  const float v = elem_to_f32(W[(b * D + i) * D + j]) * (scale ? scale[b] : 1.0f) * factor;
+  f32_to_elem(v, out[o]);
+}
+}  // namespace
+}  // namespace ga
+
+extern "C" int ga_transpose_scale_blocks(const void *W, const float *scale, float factor,
+                                         void *out, int64_t n_blocks, int64_t D, int dtype,
+                                         ga_stream_t stream) {
+  using namespace ga;
+  if (n_blocks < 0 || D <= 0 || D > 0x7fff) return GA_EINVAL;
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  const int64_t total = n_blocks * D * D;
+  if (total == 0) return GA_OK;
+  if (!W || !out || W == out) return GA_EINVAL;
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!aligned(W, esz) || !aligned(out, esz) || (scale && !aligned(scale, 4))) return GA_EALIGN;
+  const int64_t blocks = (total + kBlock - 1) / kBlock;
+  if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == GA_F32)
+    hipLaunchKernelGGL(transpose_scale_blocks_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0,
+                       s, (const float *)W, scale, factor, (float *)out, (int)D, total);
+  else
+    hipLaunchKernelGGL(transpose_scale_blocks_kernel<bf16_t>, dim3((unsigned)blocks), dim3(kBlock),
+                       0, s, (const bf16_t *)W, scale, factor, (bf16_t *)out, (int)D, total);
+  return launch_status();
+}
+
 extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
                              const void *X, const void *W, void *Y, int64_t rows,
                              int64_t heads, int64_t K, int64_t M, int dtype,

@@ -914,12 +914,17 @@ torch::Tensor relation_pair_attention(torch::Tensor k, torch::Tensor q, torch::T
   const int64_t n = graph->num_nodes, e = graph->num_edges, P = pairs.num_pairs;
   if (!pairs.valid || e < 2 * P) return per_edge();
   const int dt = feat_dtype(k, "k");
-  torch::Tensor att_t = relation_att.reshape({graph->num_etypes, heads, d, d}).transpose(-1, -2);
-  if (scale.has_value())
-    att_t = att_t * scale.value().to(at::kFloat).reshape({graph->num_etypes, heads, 1, 1});
-  if (divisor != 1.0) att_t = att_t.to(at::kFloat) / divisor;
-  att_t = att_t.to(k.scalar_type()).contiguous();
   const auto stream = current_stream(k);
+  if (!relation_att.is_contiguous()) return per_edge();
+  // the matrices as the query side needs them: transposed, times scale / divisor
+  torch::Tensor att_t = torch::empty_like(relation_att);
+  torch::Tensor sc;
+  if (scale.has_value()) sc = scale.value().to(at::kFloat).contiguous();
+  check_ga(ga_transpose_scale_blocks(relation_att.data_ptr(),
+                                     sc.defined() ? sc.data_ptr<float>() : nullptr,
+                                     (float)(1.0 / divisor), att_t.data_ptr(),
+                                     graph->num_etypes * heads, d, dt, stream),
+           "ga_transpose_scale_blocks");
   auto typed_rows = [&](const torch::Tensor &x, const torch::Tensor &index,
                         const torch::Tensor &w, torch::Tensor &y) {
     return ga_segment_mm_gather(pairs.type_pointer.data_ptr<int>(), graph->num_etypes,

@@ -170,7 +170,8 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
                                   or e >= PAIRS_MIN_EDGES_PER_PAIR * pairs.num_pairs):
             try:
                 t = ops.relation_pair_attention(k, q, v, relation_att, relation_msg,
-                                                relation_pri.float() / (d ** 0.5), g)
+                                                relation_pri.float().contiguous(), g,
+                                                factor=1.0 / (d ** 0.5))
             except capi.GraphilerError as err:      # head width outside the typed product
                 if err.code != capi.GA_EUNSUPPORTED or fused == "pairs":
                     raise

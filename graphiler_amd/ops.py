@@ -863,7 +863,7 @@ def dot_attention_sum(k, q, v, graph: DGLGraph, return_lse: bool = False):
 
 
 def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
-                            graph: DGLGraph) -> torch.Tensor:
+                            graph: DGLGraph, factor: float = 1.0) -> torch.Tensor:
     """The message and reduce stages of an HGT layer (examples/HGT/HGT.py:35-53) with
     the per-relation matrices applied once per (destination, relation) pair instead
     of once per edge -- both stages are linear in them:
@@ -872,8 +872,8 @@ def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
       out[v]      = sum_e a[e] * (v[src] @ M[t])      = sum_{pairs (v, t)} (sum_{e in pair} a[e] * v[src]) @ M[t]
 
     with a = softmax of the scores over the in-edges of v.  k, q, v (N, H*D);
-    relation_att, relation_msg (T, H, D, D); relation_scale (T, H) fp32 (the prior
-    over sqrt(D)) or None.  The typed products run over P pairs, the scores are a
+    relation_att, relation_msg (T, H, D, D); relation_scale (T, H) fp32 (the prior)
+    or None, ``factor`` a further constant on the scores (1 / sqrt(D)): s = scale * factor.  The typed products run over P pairs, the scores are a
     plain dot product per edge and the weighted sum gathers rows of v: no (E, H*D)
     tensor is written.  Returns (N, H*D).  Raises GraphilerError(GA_EUNSUPPORTED) for
     shapes the typed-product kernel does not take and RuntimeError when the graph has
@@ -896,16 +896,17 @@ def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
     pairs = graph.relation_pairs()
     if pairs is None:
         raise RuntimeError("the in-adjacency of this graph is not grouped by relation")
-    att_t = relation_att.transpose(-1, -2)
-    if relation_scale is not None:
-        if tuple(relation_scale.shape) != (n_types, heads):
-            raise RuntimeError("relation_scale must be (edge types, heads)")
-        # an fp32 product, rounded once to the features' dtype
-        att_t = att_t * relation_scale.float()[:, :, None, None]
-    if att_t.dtype != k.dtype:
-        att_t = att_t.to(k.dtype, memory_format=torch.contiguous_format)
-    att_t = att_t.contiguous()       # (a no-op after the conversion)
     lib, stream, dev, P = capi.load(), _stream(k), k.device, pairs.num_pairs
+    if relation_scale is not None:
+        _check_input(relation_scale, "relation_scale")
+        if tuple(relation_scale.shape) != (n_types, heads) or relation_scale.dtype != torch.float32:
+            raise RuntimeError("relation_scale must be (edge types, heads) float32")
+    # the matrices as the query side needs them: transposed, times the scale (an fp32
+    # product rounded once to the features' dtype)
+    att_t = torch.empty_like(relation_att)
+    capi.check(lib.ga_transpose_scale_blocks(
+        relation_att.data_ptr(), _ptr(relation_scale), float(factor), att_t.data_ptr(), n_types * heads, d,
+        dt, stream), "ga_transpose_scale_blocks")
 
     def typed_rows(x, index, w):        # row r = x[index[r]] @ w[relation of pair by_type[r]]
         y = torch.empty((P, hid), dtype=x.dtype, device=dev)

@@ -305,6 +305,14 @@ int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_types, const vo
                           const void *const *W, void *const *Y, int64_t n_weights,
                           int64_t rows, int64_t K, int64_t M, int dtype, ga_stream_t stream);
 
+/* out[b, j, i] = W[b, i, j] * scale[b] * factor over n_blocks square D x D blocks (scale
+ * NULL: 1), computed in fp32 and rounded once to `dtype`: the relation matrices of
+ * examples/HGT/HGT.py:39-45 transposed and carrying `relation_pri / sqrt(D)`, as the query
+ * side of the scores needs them when the product is moved from the keys to the queries
+ * (ga_dot_attention_sum).  out must not be W. */
+int ga_transpose_scale_blocks(const void *W, const float *scale, float factor, void *out,
+                              int64_t n_blocks, int64_t D, int dtype, ga_stream_t stream);
+
 /* Per-edge typed linear whose operand lives on the nodes, without the per-edge
  * copy: Y[r] = X[x_index[r]] @ W[type(r)] (x_index NULL: X[r]).  Replaces the
  * pair BroadcastSrcNode / BroadcastDstNode (broadcast.cu:58-66) -> SegmentMMEdge

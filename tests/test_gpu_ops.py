@@ -442,6 +442,34 @@ def test_dot_attention_sum_long_rows_and_rejects(device, bf16):
         ops.dot_attention_sum(_dev(k, device, bf16), _dev(q, device, bf16)[:, :2], _dev(v, device, bf16), g)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_transpose_scale_blocks(device, bf16):
+    """ga_transpose_scale_blocks: every D x D block transposed, times its scale and a
+    constant, in fp32 with one rounding -- bit for bit the same arithmetic in ATen."""
+    lib = capi.load()
+    dt = torch.bfloat16 if bf16 else torch.float32
+    stream = torch.cuda.current_stream().cuda_stream
+    for t, h, d in ((5, 3, 8), (10, 8, 16), (1, 1, 1), (2, 1, 33)):
+        w = torch.randn(t, h, d, d, device=device).to(dt)
+        scale = torch.rand(t, h, device=device) + 0.5
+        for sc, factor in ((scale, 0.25), (None, 1.0), (scale, 1.0 / 3.0)):
+            out = torch.full_like(w, float("nan"))
+            rc = lib.ga_transpose_scale_blocks(w.data_ptr(), None if sc is None else sc.data_ptr(),
+                                               factor, out.data_ptr(), t * h, d,
+                                               capi.GA_BF16 if bf16 else capi.GA_F32, stream)
+            assert rc == 0, rc
+            want = w.float().transpose(-1, -2)
+            if sc is not None:
+                want = want * sc[:, :, None, None]
+            want = (want * torch.tensor(factor, dtype=torch.float32, device=device)).to(dt)
+            assert torch.equal(out.view(torch.int16 if bf16 else torch.int32),
+                               want.contiguous().view(torch.int16 if bf16 else torch.int32))
+    w = torch.randn(2, 4, 4, device=device)
+    assert lib.ga_transpose_scale_blocks(w.data_ptr(), None, 1.0, w.data_ptr(), 2, 4, capi.GA_F32,
+                                         stream) == capi.GA_EINVAL           # in place
+    assert lib.ga_transpose_scale_blocks(None, None, 1.0, None, 0, 4, capi.GA_F32, stream) == 0
+
+
 @pytest.mark.parametrize("feat,heads,bf16", [(64, 1, False), (256, 4, True), (17, 1, False),
                                              (1, 1, False), (128, 8, False)])
 def test_row_reductions_over_many_workgroups(device, feat, heads, bf16):
