@@ -358,7 +358,7 @@ def main():
             x, w1, w2 = (torch.from_numpy(t).to(dev).to(dt) for t in (x_h, w1_h, w2_h))
 
             def network():
-                h1 = torch.relu(layers.rgcn_layer(g, x, w1, norm, fused=True))
+                h1 = layers.rgcn_layer(g, x, w1, norm, fused=True, activation="relu")
                 return layers.rgcn_layer(g, h1, w2, norm, fused=True)
 
             ms_step, _ = wall_time(network, max(args.steps, 100), max(args.warmup, 10))

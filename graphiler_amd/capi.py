@@ -55,6 +55,8 @@ SIGNATURES = {
                                     _vp, _vp, _vp, _sz, _vp]),
     "ga_typed_spmm": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                              _i64, _i64, _i64, _i64, _int, _vp]),
+    "ga_typed_spmm_act": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+                                 _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "ga_sddmm_u_dot_v": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64,
                                 _int, _vp]),
     "ga_softmax_workspace_bytes": (_sz, [_i64, _i64]),

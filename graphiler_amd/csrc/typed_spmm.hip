@@ -347,6 +347,10 @@ __device__ __forceinline__ bool is_finite(float v) {
   return (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u;
 }
 
+__device__ __forceinline__ float activated(float o, int act) {
+  return o > 0.0f ? o : (act == GA_ACT_ELU ? __expf(o) - 1.0f : (o != o ? o : 0.0f));
+}
+
 __device__ __forceinline__ void store_row4(float *p, const float4 &v) {
   *reinterpret_cast<float4 *>(p) = v;
 }
@@ -494,7 +498,7 @@ constexpr int typed_waves_per_simd(int KS, int MC) { return KS == 1 ? 3 : 1; }
 template <typename T, int KS, int MC, bool SCALED, int NB>
 __global__ __launch_bounds__(kTypedBlock, typed_waves_per_simd(KS, MC)) void typed_tiles_kernel(
     const int32_t *__restrict__ tile_chunk_pointer, TypedArgs A, T *__restrict__ out,
-    int64_t n_rows) {
+    int64_t n_rows, int act) {
   constexpr int kTileRows = 16 * NB;
   constexpr int kCB = Cols<MC>::kCB, kColGroups = Cols<MC>::kColGroups, kTurns = Cols<MC>::kTurns;
   constexpr int kMergeStride = Cols<MC>::kMergeStride;
@@ -568,40 +572,47 @@ __global__ __launch_bounds__(kTypedBlock, typed_waves_per_simd(KS, MC)) void typ
   const int64_t row0 = (int64_t)blockIdx.x * kTileRows;
   for (int i = threadIdx.x; i < kTileRows * (MC / 4); i += kTypedBlock) {
     const int r = i / (MC / 4), c4 = i % (MC / 4);
-    if (row0 + r < n_rows)
-      store_row4(out + (row0 + r) * MC + 4 * c4,
-                 *reinterpret_cast<const float4 *>(merged + r * kMergeStride + 4 * c4));
+    if (row0 + r < n_rows) {
+      float4 v = *reinterpret_cast<const float4 *>(merged + r * kMergeStride + 4 * c4);
+      if (act != GA_ACT_NONE) {
+        // the activation between layers (examples/RGCN/RGCN.py:69) on the fp32 sums, before
+        // they are rounded and stored; NaN stays NaN
+        v.x = activated(v.x, act); v.y = activated(v.y, act);
+        v.z = activated(v.z, act); v.w = activated(v.w, act);
+      }
+      store_row4(out + (row0 + r) * MC + 4 * c4, v);
+    }
   }
 }
 
 template <typename T, int KS, int MC, int NB>
-int launch_typed_nb(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows,
+int launch_typed_nb(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows, int act,
                     hipStream_t s) {
   const dim3 grid((unsigned)tiles_of(n_rows, 16 * NB));
   if (A.row_scale)
     hipLaunchKernelGGL((typed_tiles_kernel<T, KS, MC, true, NB>), grid, dim3(kTypedBlock), 0, s,
-                       tcp, A, (T *)out, n_rows);
+                       tcp, A, (T *)out, n_rows, act);
   else
     hipLaunchKernelGGL((typed_tiles_kernel<T, KS, MC, false, NB>), grid, dim3(kTypedBlock), 0, s,
-                       tcp, A, (T *)out, n_rows);
+                       tcp, A, (T *)out, n_rows, act);
   return launch_status();
 }
 
 template <typename T, int KS, int MC>
 int launch_typed_mc(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows,
-                    int64_t tile_rows, hipStream_t s) {
-  if (tile_rows == 144) return launch_typed_nb<T, KS, MC, 9>(tcp, A, out, n_rows, s);
-  return launch_typed_nb<T, KS, MC, 8>(tcp, A, out, n_rows, s);
+                    int64_t tile_rows, int act, hipStream_t s) {
+  if (tile_rows == 144) return launch_typed_nb<T, KS, MC, 9>(tcp, A, out, n_rows, act, s);
+  return launch_typed_nb<T, KS, MC, 8>(tcp, A, out, n_rows, act, s);
 }
 
 template <typename T, int KS>
 int launch_typed(const int32_t *tcp, const TypedArgs &A, void *out, int64_t n_rows,
-                 int64_t tile_rows, int64_t M, hipStream_t s) {
+                 int64_t tile_rows, int64_t M, int act, hipStream_t s) {
   switch (M) {
-    case 8: return launch_typed_mc<T, KS, 8>(tcp, A, out, n_rows, tile_rows, s);
-    case 16: return launch_typed_mc<T, KS, 16>(tcp, A, out, n_rows, tile_rows, s);
-    case 32: return launch_typed_mc<T, KS, 32>(tcp, A, out, n_rows, tile_rows, s);
-    default: return launch_typed_mc<T, KS, 64>(tcp, A, out, n_rows, tile_rows, s);
+    case 8: return launch_typed_mc<T, KS, 8>(tcp, A, out, n_rows, tile_rows, act, s);
+    case 16: return launch_typed_mc<T, KS, 16>(tcp, A, out, n_rows, tile_rows, act, s);
+    case 32: return launch_typed_mc<T, KS, 32>(tcp, A, out, n_rows, tile_rows, act, s);
+    default: return launch_typed_mc<T, KS, 64>(tcp, A, out, n_rows, tile_rows, act, s);
   }
 }
 
@@ -731,7 +742,19 @@ int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
                   const float *row_scale, void *out, int64_t n_rows, int64_t n_src,
                   int64_t n_edges, int64_t n_types, int64_t tile_rows, int64_t K, int64_t M,
                   int dtype, ga_stream_t stream) {
+  return ga_typed_spmm_act(tile_chunk_pointer, chunk_type, slot_src, slot_dst, slot_edge, x, W,
+                           row_scale, out, n_rows, n_src, n_edges, n_types, tile_rows, K, M,
+                           GA_ACT_NONE, dtype, stream);
+}
+
+int ga_typed_spmm_act(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
+                      const int32_t *slot_src, const unsigned char *slot_dst,
+                      const int32_t *slot_edge, const void *x, const void *W,
+                      const float *row_scale, void *out, int64_t n_rows, int64_t n_src,
+                      int64_t n_edges, int64_t n_types, int64_t tile_rows, int64_t K, int64_t M,
+                      int activation, int dtype, ga_stream_t stream) {
   using namespace ga;
+  if (activation < GA_ACT_NONE || activation > GA_ACT_ELU) return GA_EINVAL;
   if (n_rows < 0 || n_src < 0 || n_edges < 0 || n_types <= 0 || K <= 0 || M <= 0) return GA_EINVAL;
   if (!tile_rows_ok(tile_rows)) return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff) return GA_EINVAL;
@@ -755,7 +778,7 @@ int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
   const TypedArgs A{chunk_type, slot_src, slot_edge, (const uint32_t *)slot_dst, x, W, row_scale};
   const int ks = (int)(K / 16);
 #define GA_TYPED(T, KS) \
-  return launch_typed<T, KS>(tile_chunk_pointer, A, out, n_rows, tile_rows, M, s)
+  return launch_typed<T, KS>(tile_chunk_pointer, A, out, n_rows, tile_rows, M, activation, s)
   if (dtype == GA_F32) {
     switch (ks) {
       case 1: GA_TYPED(float, 1);

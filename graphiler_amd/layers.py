@@ -98,7 +98,7 @@ def gat_layer(g: DGLGraph, h, fc_weight, attn_weight, heads: int = 1,
     return out
 
 
-def rgcn_layer(g: DGLGraph, h, weight, norm, fused=True):
+def rgcn_layer(g: DGLGraph, h, weight, norm, fused=True, activation=None):
     """examples/RGCN/RGCN.py:25-33.  weight (R, K, M); norm (E, 1) fp32; edges
     sorted by type.
 
@@ -111,17 +111,27 @@ def rgcn_layer(g: DGLGraph, h, weight, norm, fused=True):
     ``fused="tiles"``: ops.TypedSpMMEdge, one pass without the message tensor
     (K in 16, 32, 48, 64; M in 8, 16, 32, 64).
     ``fused=False``: the reference's plan BroadcastSrcNode -> SegmentMMEdge ->
-    mul(norm) -> SpMMEdge."""
+    mul(norm) -> SpMMEdge.
+    ``activation`` ("relu" | "elu"; the ``relu`` between the layers of
+    examples/RGCN/RGCN.py:69): applied by the single pass to the sums it stores, by a
+    separate call otherwise."""
+    if activation not in (None, "relu", "elu"):
+        raise RuntimeError("activation must be None, 'relu' or 'elu'")
     if fused == "tiles" or (fused is True and h.dim() == 2
                             and ops.typed_spmm_preferred(h, weight)):
-        return ops.TypedSpMMEdge(h, weight, g, row_scale=norm.float().contiguous())
+        return ops.TypedSpMMEdge(h, weight, g, row_scale=norm.float().contiguous(),
+                                 activation=activation)
     if fused:
         msg = ops.SegmentMMEdgeGather(h, weight, 0, g, row_scale=norm.float().contiguous())
-        return ops.SpMMEdge(msg, [1], False, None, g)
-    hs = ops.BroadcastSrcNode(h, g)
-    msg = ops.SegmentMMEdge(hs, weight, g)
-    msg = msg * norm.to(msg.dtype)
-    return ops.SpMMEdge(msg, [1], False, None, g)
+        out = ops.SpMMEdge(msg, [1], False, None, g)
+    else:
+        hs = ops.BroadcastSrcNode(h, g)
+        msg = ops.SegmentMMEdge(hs, weight, g)
+        msg = msg * norm.to(msg.dtype)
+        out = ops.SpMMEdge(msg, [1], False, None, g)
+    if activation == "relu":
+        return torch.relu(out)
+    return F.elu(out) if activation == "elu" else out
 
 
 # Edges per (destination, relation) pair from which an HGT layer applies its relation

@@ -615,7 +615,8 @@ def typed_spmm_preferred(features, weights) -> bool:
         and int(weights.shape[1]) * int(weights.shape[2]) <= 2048
 
 
-def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None) -> torch.Tensor:
+def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None,
+                  activation=None) -> torch.Tensor:
     """``SpMMEdge(SegmentMMEdge(BroadcastSrcNode(features), weights) * row_scale)``
     in one pass (examples/RGCN/RGCN.py:25-33; broadcast.cu:58-63, segment_mm.cu:29-33,
     spmm.cu:359-373): out[v] = sum over the in-edges e of v of
@@ -623,7 +624,8 @@ def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None) -> torch.T
     features (N, K), weights (R, K, M) with K in 16, 32, 48, 64 and M in 8, 16, 32, 64;
     ``row_scale`` (E,) or
     (E, 1) fp32.  The additions of a row happen in the order of the prepared layout
-    (by relation, then adjacency order), the same in every call."""
+    (by relation, then adjacency order), the same in every call.  ``activation``
+    ("relu" | "elu"): applied to the fp32 sums before they are stored."""
     _check_input(features, "features")
     _check_input(weights, "weights")
     dt = _feat_dtype(features, "features")
@@ -643,11 +645,11 @@ def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None) -> torch.T
     K, M = int(weights.shape[1]), int(weights.shape[2])
     tcp, ctype, ssrc, sdst, sedge, tile_rows = _typed_tiles(graph)
     out = torch.empty((graph.num_nodes, M), dtype=features.dtype, device=features.device)
-    capi.check(capi.load().ga_typed_spmm(
+    capi.check(capi.load().ga_typed_spmm_act(
         tcp.data_ptr(), ctype.data_ptr(), ssrc.data_ptr(), sdst.data_ptr(), sedge.data_ptr(),
         features.data_ptr(), weights.data_ptr(), _ptr(row_scale), out.data_ptr(),
         graph.num_nodes, int(features.shape[0]), graph.num_edges, graph.num_etypes, tile_rows,
-        K, M, dt, _stream(out)), "ga_typed_spmm")
+        K, M, _activation(activation), dt, _stream(out)), "ga_typed_spmm_act")
     return out
 
 

@@ -235,6 +235,16 @@ int ga_typed_spmm(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
                   int64_t n_edges, int64_t n_types, int64_t tile_rows, int64_t K, int64_t M,
                   int dtype, ga_stream_t stream);
 
+/* ga_typed_spmm with the activation that follows the layer (relu between the layers of
+ * examples/RGCN/RGCN.py:69; GA_ACT_RELU, GA_ACT_ELU with alpha = 1) applied to the fp32
+ * sums before they are rounded and stored.  GA_ACT_NONE is ga_typed_spmm. */
+int ga_typed_spmm_act(const int32_t *tile_chunk_pointer, const int32_t *chunk_type,
+                      const int32_t *slot_src, const unsigned char *slot_dst,
+                      const int32_t *slot_edge, const void *x, const void *W,
+                      const float *row_scale, void *out, int64_t n_rows, int64_t n_src,
+                      int64_t n_edges, int64_t n_types, int64_t tile_rows, int64_t K, int64_t M,
+                      int activation, int dtype, ga_stream_t stream);
+
 /* The general SDDMM of the reference (SDDMMCooKernel / SDDMMCooTreeReduceKernel,
  * sddmm.cuh:34-120): operands on the source nodes (target 0), on the edges (1) or on
  * the destination nodes (2) in any combination (selector.h:30-60), feature shapes

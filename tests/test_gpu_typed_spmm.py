@@ -193,6 +193,35 @@ def test_rgcn_layer_paths_agree(device):
                      2 * TOL_F32, f"{k} -> {m} against unfused")
 
 
+@pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
+def test_typed_spmm_activation(device, bf16):
+    """The activation applied to the fp32 sums inside the kernel against the same
+    activation on the plain result (relu: exactly; elu: to rounding), for both column
+    layouts, and through rgcn_layer for the one-pass and the two-pass form."""
+    import torch.nn.functional as F
+    rng = np.random.default_rng(15)
+    n, e, r = 700, 9000, 8
+    g, arr, src, dst, etype = _typed_graph(rng, n, e, r, device)
+    norm = _dev(rng.uniform(0.1, 1.5, (e, 1)).astype(np.float32), device)
+    for k, m in ((16, 64), (64, 8)):
+        x = _dev(rng.standard_normal((n, k), dtype=np.float32), device, bf16)
+        w = _dev((rng.standard_normal((r, k, m)) / np.sqrt(k)).astype(np.float32), device, bf16)
+        plain = ops.TypedSpMMEdge(x, w, g, row_scale=norm.reshape(-1))
+        relu = ops.TypedSpMMEdge(x, w, g, row_scale=norm.reshape(-1), activation="relu")
+        assert torch.equal(relu, torch.relu(plain)) and bool((relu == 0).any())
+        elu = ops.TypedSpMMEdge(x, w, g, row_scale=norm.reshape(-1), activation="elu")
+        assert_close(elu.float().cpu().numpy(), F.elu(plain.float()).cpu().numpy(),
+                     TOL_BF16 if bf16 else TOL_F32, f"typed elu {k}->{m}")
+        for fused in ("tiles", "pair", False):
+            got = layers.rgcn_layer(g, x, w, norm, fused=fused, activation="relu")
+            want = torch.relu(layers.rgcn_layer(g, x, w, norm, fused=fused))
+            assert torch.equal(got, want), fused
+    with pytest.raises(RuntimeError):
+        ops.TypedSpMMEdge(x, w, g, activation="tanh")
+    with pytest.raises(RuntimeError):
+        layers.rgcn_layer(g, x, w, norm, activation="tanh")
+
+
 def test_typed_spmm_rejects_what_it_does_not_cover(device):
     rng = np.random.default_rng(6)
     g, arr, src, dst, etype = _typed_graph(rng, 100, 500, 3, device)
