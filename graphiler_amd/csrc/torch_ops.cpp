@@ -110,8 +110,12 @@ struct DGLGraph : torch::CustomClassHolder {
   }
   void SetEtypePointer(at::optional<torch::Tensor> pointer) {
     if (pointer.has_value()) check_index(pointer.value(), at::kInt, "etype_pointer");
+    std::lock_guard<std::mutex> lock(mu_);
     etype_pointer = pointer;
     num_etypes = pointer.has_value() ? pointer.value().size(0) - 1 : 1;
+    // the layouts prepared from the edge types belong to the old pointer
+    tiles_ = TypedTiles();
+    pairs_ = RelationPairs();
   }
   void SetNtypeCOO(torch::Tensor column) {
     check_index(column, at::kLong, "ntype_COO");

@@ -123,9 +123,9 @@ class DGLGraph:
         self.num_edges = int(in_node_indices.size(0))
         self.num_ntypes = 1
         self.num_etypes = 1
+        self._cache = {}
         self.SetNtypePointer(ntype_pointer)
         self.SetEtypePointer(etype_pointer)
-        self._cache = {}
 
     # -- setters (include/dglgraph.h:29-46) ---------------------------------
     def SetNtypePointer(self, pointer):
@@ -139,6 +139,10 @@ class DGLGraph:
             _check_index(pointer, torch.int32, "etype_pointer")
         self.etype_pointer = pointer
         self.num_etypes = int(pointer.size(0)) - 1 if pointer is not None else 1
+        # the layouts prepared from the edge types belong to the old pointer (a layout
+        # already handed to a launch stays alive with that launch's tensors)
+        self._cache.pop("typed_tiles", None)
+        self._cache.pop("pairs", None)
 
     def SetNtypeCOO(self, column):
         _check_index(column, torch.int64, "ntype_COO")

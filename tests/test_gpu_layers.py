@@ -197,3 +197,26 @@ def test_hgt_pair_form_equals_edge_form(device, heads, d):
     assert_close(got.cpu().numpy(), want.cpu().numpy(), 2 * TOL_F32, f"HGT pairs {heads}x{d}")
     auto = layers.hgt_layer(*args, fused=True)
     assert_close(auto.cpu().numpy(), want.cpu().numpy(), 2 * TOL_F32, f"HGT auto {heads}x{d}")
+
+
+def test_type_dependent_layouts_follow_the_edge_type_pointer(device):
+    """Replacing a graph's edge type pointer drops the layouts prepared from the old one
+    (the (destination, relation) pairs and the typed tiles)."""
+    from graphiler_amd import ops
+    rng = np.random.default_rng(3)
+    n, e = 300, 4000
+    src, dst = rng.integers(0, n, e), rng.integers(0, 60, e)
+    et = np.sort(rng.integers(0, 4, e))
+    g = prepare_graph(src, dst, n, device=device, etype_of=et, num_etypes=4)
+    before = g.relation_pairs().num_pairs
+    tiles_before = ops._typed_tiles(g)
+    assert before == len(np.unique(dst * 4 + et))
+    one_type = torch.tensor([0, e], dtype=torch.int32, device=device)
+    g.SetEtypePointer(one_type)
+    assert g.num_etypes == 1 and g.relation_pairs().num_pairs == len(np.unique(dst))
+    assert ops._typed_tiles(g) is not tiles_before
+    x = _t(rng.standard_normal((n, 16), dtype=np.float32), device)
+    w = _t(rng.standard_normal((1, 16, 8), dtype=np.float32), device)
+    got = ops.TypedSpMMEdge(x, w, g)
+    want = ops.SpMMEdge(ops.SegmentMMEdgeGather(x, w, 0, g), [1], False, None, g)
+    assert_close(got.cpu().numpy(), want.cpu().numpy(), 2 * TOL_F32, "typed sum after a new type pointer")
