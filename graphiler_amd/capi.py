@@ -79,7 +79,7 @@ SIGNATURES = {
                                        _i64, _i64, ctypes.c_float, _int, _vp, _sz, _vp]),
     "ga_edge_softmax_sum": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                    _int, _vp, _sz, _vp]),
-    "ga_dot_attention_sum": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+    "ga_dot_attention_sum": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
                                     _i64, _i64, _int, _vp, _sz, _vp]),
     "ga_gat_aggregate_static": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
                                        _i64, _i64, ctypes.c_float, _int, _vp]),

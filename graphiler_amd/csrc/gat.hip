@@ -230,6 +230,7 @@ struct DotAttnPolicy : GatPolicy<T, VEC, kGatEdge, false> {
     const int32_t *qrow;   // query row of a slot
     const T *k, *q, *v;    // rows of heads * dph features
     float *lse;            // (n_rows, heads) or null
+    const int32_t *lse_index;   // row r's log-sum-exp goes to row lse_index[r] of lse; null: r
     int heads;
     int dph;
     int head_lanes;        // lanes that share a head (dph / VEC)
@@ -239,12 +240,14 @@ struct DotAttnPolicy : GatPolicy<T, VEC, kGatEdge, false> {
                                               const float (&st)[VEC + 2]) {
     emit_row<DotAttnPolicy>(out, row, feat, f0, st);
     if (A.lse && f0 % A.dph == 0)
-      A.lse[row * A.heads + f0 / A.dph] = st[VEC] + logf(st[VEC + 1]);
+      A.lse[(A.lse_index ? (int64_t)A.lse_index[row] : row) * A.heads + f0 / A.dph] =
+          st[VEC] + logf(st[VEC + 1]);
   }
   static __device__ __forceinline__ void emit_empty(const Args &A, T *out, int64_t row, int feat,
                                                     int f0) {
     emit_empty_row<DotAttnPolicy>(out, row, feat, f0);
-    if (A.lse && f0 % A.dph == 0) A.lse[row * A.heads + f0 / A.dph] = -INFINITY;
+    if (A.lse && f0 % A.dph == 0)
+      A.lse[(A.lse_index ? (int64_t)A.lse_index[row] : row) * A.heads + f0 / A.dph] = -INFINITY;
   }
 
   template <class Close>
@@ -330,14 +333,14 @@ struct DotAttnPolicy : GatPolicy<T, VEC, kGatEdge, false> {
 template <typename T, int VEC>
 int launch_dot_attn(const int32_t *pointer, const int32_t *row_of_slot, const int32_t *nbr,
                     const int32_t *qrow, const void *k, const void *q, const void *v, void *out,
-                    float *lse, int64_t n_rows, int64_t n_edges, int heads, int dim, float *ws,
-                    size_t ws_bytes, hipStream_t stream) {
+                    float *lse, const int32_t *lse_index, int64_t n_rows, int64_t n_edges, int heads,
+                    int dim, float *ws, size_t ws_bytes, hipStream_t stream) {
   typedef DotAttnPolicy<T, VEC> P;
   const int head_lanes = dim / VEC;
   if (dim % VEC != 0 || head_lanes > 16 || (head_lanes & (head_lanes - 1)) != 0)
     return GA_EUNSUPPORTED;
   const bool ids_vec = aligned(row_of_slot, 16) && aligned(nbr, 16) && aligned(qrow, 16);
-  typename P::Args args{nbr, qrow, (const T *)k, (const T *)q, (const T *)v, lse,
+  typename P::Args args{nbr, qrow, (const T *)k, (const T *)q, (const T *)v, lse, lse_index,
                         heads, dim, head_lanes, ids_vec};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, heads * dim, ws,
                         stream, ws_bytes);
@@ -549,9 +552,9 @@ int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,
 
 int ga_dot_attention_sum(const int32_t *pointer, const int32_t *row_of_slot,
                          const int32_t *nbr, const int32_t *qrow, const void *k, const void *q,
-                         const void *v, void *out, float *lse, int64_t n_rows, int64_t n_edges,
-                         int64_t heads, int64_t dim, int dtype, void *workspace,
-                         size_t workspace_bytes, ga_stream_t stream) {
+                         const void *v, void *out, float *lse, const int32_t *lse_index,
+                         int64_t n_rows, int64_t n_edges, int64_t heads, int64_t dim, int dtype,
+                         void *workspace, size_t workspace_bytes, ga_stream_t stream) {
   if (n_rows < 0 || n_edges < 0 || heads <= 0 || dim <= 0) return GA_EINVAL;
   if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || heads * dim > 0x7fffffff)
     return GA_EINVAL;
@@ -565,7 +568,8 @@ int ga_dot_attention_sum(const int32_t *pointer, const int32_t *row_of_slot,
         ga_gat_workspace_bytes(n_edges, feat, heads) > workspace_bytes)
       return GA_EWORKSPACE;
   }
-  if (lse && !ga::aligned(lse, 4)) return GA_EALIGN;
+  if ((lse && !ga::aligned(lse, 4)) || (lse_index && !ga::aligned(lse_index, 4))) return GA_EALIGN;
+  if (lse_index && !lse) return GA_EINVAL;
   // rows are read and written in 16-byte pieces that do not straddle a head
   const int vec = dtype == GA_F32 ? 4 : 8;
   if (!ga::aligned(out, 16) || (k && !ga::aligned(k, 16)) || (q && !ga::aligned(q, 16)) ||
@@ -573,11 +577,11 @@ int ga_dot_attention_sum(const int32_t *pointer, const int32_t *row_of_slot,
     return GA_EUNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == GA_F32)
-    return ga::launch_dot_attn<float, 4>(pointer, row_of_slot, nbr, qrow, k, q, v, out, lse, n_rows,
-                                         n_edges, (int)heads, (int)dim, (float *)workspace,
-                                         workspace_bytes, s);
+    return ga::launch_dot_attn<float, 4>(pointer, row_of_slot, nbr, qrow, k, q, v, out, lse,
+                                         lse_index, n_rows, n_edges, (int)heads, (int)dim,
+                                         (float *)workspace, workspace_bytes, s);
   return ga::launch_dot_attn<ga::bf16_t, 8>(pointer, row_of_slot, nbr, qrow, k, q, v, out, lse,
-                                            n_rows, n_edges, (int)heads, (int)dim,
+                                            lse_index, n_rows, n_edges, (int)heads, (int)dim,
                                             (float *)workspace, workspace_bytes, s);
 }
 

@@ -868,7 +868,7 @@ torch::Tensor dot_attention_sum(torch::Tensor k, torch::Tensor q, torch::Tensor 
   check_ga(ga_dot_attention_sum(graph->in_pointer.data_ptr<int>(), side.rows.data_ptr<int>(),
                                 graph->in_node_indices.data_ptr<int>(), side.rows.data_ptr<int>(),
                                 k.data_ptr(), q.data_ptr(), v.data_ptr(), out.data_ptr(), nullptr,
-                                graph->num_nodes, graph->num_edges, heads, d, dt, ws.data_ptr(),
+                                nullptr, graph->num_nodes, graph->num_edges, heads, d, dt, ws.data_ptr(),
                                 (size_t)ws.numel(), current_stream(out)),
            "ga_dot_attention_sum");
   return out;
@@ -948,22 +948,20 @@ torch::Tensor relation_pair_attention(torch::Tensor k, torch::Tensor q, torch::T
   rc = ga_dot_attention_sum(pairs.pair_pointer.data_ptr<int>(), pairs.pair_of_slot.data_ptr<int>(),
                             graph->in_node_indices.data_ptr<int>(),
                             pairs.rank_of_slot.data_ptr<int>(), k.data_ptr(), q_pair.data_ptr(),
-                            v.data_ptr(), v_pair.data_ptr(), lse.data_ptr<float>(), P, e, heads, d,
-                            dt, ws.data_ptr(), (size_t)ws.numel(), stream);
+                            v.data_ptr(), v_pair.data_ptr(), lse.data_ptr<float>(),
+                            pairs.rank.data_ptr<int>(), P, e, heads, d, dt, ws.data_ptr(),
+                            (size_t)ws.numel(), stream);
   if (rc == GA_EUNSUPPORTED) return per_edge();
   check_ga(rc, "ga_dot_attention_sum");
-  check_ga(ga_segment_softmax(pairs.dst_pointer.data_ptr<int>(), pairs.pair_dst.data_ptr<int>(),
-                              nullptr, lse.data_ptr<float>(), lse.data_ptr<float>(), n, P, heads,
-                              ws.data_ptr(), (size_t)ws.numel(), stream),
-           "ga_segment_softmax");
+  // (the log-sum-exps were written in by_type order, the row order of m_pair)
   torch::Tensor m_pair = torch::empty({P, hid}, k.options());
   check_ga(typed_rows(v_pair, pairs.by_type, relation_msg, m_pair), "ga_segment_mm_gather");
   torch::Tensor out = torch::empty({n, hid}, k.options());
-  check_ga(ga_spmm_csr(pairs.dst_pointer.data_ptr<int>(), pairs.pair_dst.data_ptr<int>(),
-                       pairs.rank.data_ptr<int>(), nullptr, m_pair.data_ptr(),
-                       lse.data_ptr<float>(), out.data_ptr(), n, P, hid, heads, GA_U_MUL_E, GA_SUM,
-                       dt, ws.data_ptr(), (size_t)ws.numel(), stream),
-           "ga_spmm_csr");
+  check_ga(ga_edge_softmax_sum(pairs.dst_pointer.data_ptr<int>(), pairs.pair_dst.data_ptr<int>(),
+                               pairs.rank.data_ptr<int>(), lse.data_ptr<float>(), m_pair.data_ptr(),
+                               out.data_ptr(), n, P, heads, d, dt, ws.data_ptr(), (size_t)ws.numel(),
+                               stream),
+           "ga_edge_softmax_sum");
   return out;
 }
 

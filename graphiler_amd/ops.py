@@ -859,8 +859,9 @@ def dot_attention_sum(k, q, v, graph: DGLGraph, return_lse: bool = False):
     capi.check(lib.ga_dot_attention_sum(
         graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
         graph.in_node_indices.data_ptr(), graph.in_row_of_slot.data_ptr(), k.data_ptr(),
-        q.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(lse), graph.num_nodes, graph.num_edges,
-        heads, d, dt, ws.data_ptr(), ws.numel(), _stream(out)), "ga_dot_attention_sum")
+        q.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(lse), None, graph.num_nodes,
+        graph.num_edges, heads, d, dt, ws.data_ptr(), ws.numel(), _stream(out)),
+        "ga_dot_attention_sum")
     return (out, lse) if return_lse else out
 
 
@@ -924,25 +925,23 @@ def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
                              lib.ga_gat_workspace_bytes(e, hid, heads)))
     # scores, softmax inside every pair and the pair's weighted sum of value rows in one
     # pass; the pairs of a destination are then weighed by the softmax of their
-    # log-sum-exps, which makes the weights the softmax over all its in-edges
+    # log-sum-exps (the softmax-weighted sum of per-"edge" rows, with the pairs as the
+    # edges), which makes the weights the softmax over all its in-edges
     v_pair = torch.empty((P, hid), dtype=v.dtype, device=dev)            # pair order
-    lse = torch.empty((P, heads), dtype=torch.float32, device=dev)
+    lse = torch.empty((P, heads), dtype=torch.float32, device=dev)       # by_type order, like m_pair
     rc = lib.ga_dot_attention_sum(
         pairs.pair_pointer.data_ptr(), pairs.pair_of_slot.data_ptr(),
         graph.in_node_indices.data_ptr(), pairs.rank_of_slot.data_ptr(), k.data_ptr(),
-        q_pair.data_ptr(), v.data_ptr(), v_pair.data_ptr(), lse.data_ptr(), P, e, heads, d, dt,
-        ws.data_ptr(), ws.numel(), stream)
+        q_pair.data_ptr(), v.data_ptr(), v_pair.data_ptr(), lse.data_ptr(), pairs.rank.data_ptr(),
+        P, e, heads, d, dt, ws.data_ptr(), ws.numel(), stream)
     if rc != capi.GA_EUNSUPPORTED:
         capi.check(rc, "ga_dot_attention_sum")
-        capi.check(lib.ga_segment_softmax(
-            pairs.dst_pointer.data_ptr(), pairs.pair_dst.data_ptr(), None, lse.data_ptr(),
-            lse.data_ptr(), n, P, heads, ws.data_ptr(), ws.numel(), stream), "ga_segment_softmax")
         m_pair = typed_rows(v_pair, pairs.by_type, relation_msg)         # by_type order
         out = torch.empty((n, hid), dtype=v.dtype, device=dev)
-        capi.check(lib.ga_spmm_csr(
-            pairs.dst_pointer.data_ptr(), pairs.pair_dst.data_ptr(), pairs.rank.data_ptr(), None,
-            m_pair.data_ptr(), lse.data_ptr(), out.data_ptr(), n, P, hid, heads, capi.GA_U_MUL_E,
-            capi.GA_SUM, dt, ws.data_ptr(), ws.numel(), stream), "ga_spmm_csr")
+        capi.check(lib.ga_edge_softmax_sum(
+            pairs.dst_pointer.data_ptr(), pairs.pair_dst.data_ptr(), pairs.rank.data_ptr(),
+            lse.data_ptr(), m_pair.data_ptr(), out.data_ptr(), n, P, heads, d, dt, ws.data_ptr(),
+            ws.numel(), stream), "ga_edge_softmax_sum")
         return out
     # head widths outside that kernel: the three steps as separate operators
     score = torch.empty((e, heads), dtype=torch.float32, device=dev)      # slot order

@@ -450,7 +450,9 @@ int ga_gat_aggregate_from_z_act(const int32_t *pointer, const int32_t *row_of_sl
 /* Dot-product attention over an adjacency, in one pass:
  *   s_i[h]       = <k[nbr[i], h, :], q[qrow[i], h, :]>      for the slots i of row r,
  *   out[r, h, :] = sum_i softmax_r(s)[i, h] * v[nbr[i], h, :],
- *   lse[r, h]    = log sum_i exp(s_i[h])                     (lse may be NULL)
+ *   lse[r, h]    = log sum_i exp(s_i[h])                     (lse may be NULL; with lse_index,
+ *                                                              int32 (n_rows), written to row
+ *                                                              lse_index[r] instead of r)
  * i.e. sum(k * q) -> SegmentSoftmax -> mul -> SpMM of examples/HGT/HGT.py:44-53 with the
  * keys and values gathered from node rows and no per-edge tensor.  With the rows being
  * the (destination, relation) pairs of a graph (qrow: the pair's transformed query
@@ -462,9 +464,9 @@ int ga_gat_aggregate_from_z_act(const int32_t *pointer, const int32_t *row_of_sl
  * ga_gat_workspace_bytes(n_edges, heads*dim, heads) bytes, 16-byte aligned. */
 int ga_dot_attention_sum(const int32_t *pointer, const int32_t *row_of_slot,
                          const int32_t *nbr, const int32_t *qrow, const void *k, const void *q,
-                         const void *v, void *out, float *lse, int64_t n_rows, int64_t n_edges,
-                         int64_t heads, int64_t dim, int dtype, void *workspace,
-                         size_t workspace_bytes, ga_stream_t stream);
+                         const void *v, void *out, float *lse, const int32_t *lse_index,
+                         int64_t n_rows, int64_t n_edges, int64_t heads, int64_t dim, int dtype,
+                         void *workspace, size_t workspace_bytes, ga_stream_t stream);
 
 /* The softmax-weighted reduction with per-edge operands:
  *   a = softmax_v(logit[e, h] over the in-edges e of v),
