@@ -360,6 +360,165 @@ torch::Tensor gspmm(torch::Tensor ufeature, at::optional<torch::Tensor> efeature
   return spmm(graph, o, r, ufeature, efeature, false);
 }
 
+// ---- operands whose feature shapes broadcast -----------------------------------
+// UseBcast / CalcBcastOff (bcast.cc:6-71): dimension 0 (nodes or edges) never takes
+// part; the others are aligned at the right.  For every element of the flattened
+// per-row output, the element of the left and of the right operand that feeds it;
+// for the dot product the last dimension is the reduction length and offsets count
+// vectors of that length.
+struct BcastTables {
+  bool use = false;
+  int64_t lhs_len = 1, rhs_len = 1, out_len = 1, reduce_size = 1;
+  std::vector<int64_t> lhs_off{0}, rhs_off{0}, feat_shape;
+};
+BcastTables bcast_tables(int op, at::IntArrayRef ls, at::IntArrayRef rs) {
+  BcastTables b;
+  const int64_t l_nd = ls.size(), r_nd = rs.size();
+  for (int64_t i = 1; i < l_nd; ++i) b.lhs_len *= ls[i];
+  for (int64_t i = 1; i < r_nd; ++i) b.rhs_len *= rs[i];
+  const bool copy = op == GA_BCAST_COPY_LHS || op == GA_BCAST_COPY_RHS;
+  if (!copy) {
+    b.use = l_nd != r_nd;
+    for (int64_t i = 1; !b.use && i < l_nd; ++i) b.use = ls[i] != rs[i];
+  }
+  const bool dot = op == GA_BCAST_DOT;
+  if (dot) {
+    TORCH_CHECK(l_nd >= 2 && ls[l_nd - 1] > 0, "dot needs a last dimension to sum over");
+    b.reduce_size = ls[l_nd - 1];
+  }
+  if (!b.use) {
+    const at::IntArrayRef &from = op == GA_BCAST_COPY_RHS ? rs : ls;
+    b.out_len = (op == GA_BCAST_COPY_RHS ? b.rhs_len : b.lhs_len) / b.reduce_size;
+    b.feat_shape.assign(from.begin() + 1, from.end() - (dot ? 1 : 0));
+    return b;
+  }
+  int64_t stride_l = 1, stride_r = 1;
+  for (int64_t j = dot ? 1 : 0; j < std::max(l_nd, r_nd) - 1; ++j) {
+    const int64_t dl = l_nd - 1 - j < 1 ? 1 : ls[l_nd - 1 - j];
+    const int64_t dr = r_nd - 1 - j < 1 ? 1 : rs[r_nd - 1 - j];
+    TORCH_CHECK(dl == dr || dl == 1 || dr == 1, "feature shapes do not broadcast");
+    const int64_t steps = std::max(dl, dr), inner = b.lhs_off.size();
+    std::vector<int64_t> lo(steps * inner), ro(steps * inner);
+    for (int64_t s = 0; s < steps; ++s)
+      for (int64_t i = 0; i < inner; ++i) {
+        lo[s * inner + i] = b.lhs_off[i] + (s < dl ? s : 0) * stride_l;
+        ro[s * inner + i] = b.rhs_off[i] + (s < dr ? s : 0) * stride_r;
+      }
+    b.lhs_off.swap(lo);
+    b.rhs_off.swap(ro);
+    b.feat_shape.insert(b.feat_shape.begin(), steps);
+    b.out_len *= steps;
+    stride_l *= dl;
+    stride_r *= dr;
+  }
+  return b;
+}
+int bcast_op(const std::string &op) {
+  return op == "add" ? GA_BCAST_ADD : op == "sub" ? GA_BCAST_SUB : op == "mul" ? GA_BCAST_MUL
+         : op == "div" ? GA_BCAST_DIV : op == "copy_lhs" ? GA_BCAST_COPY_LHS
+         : op == "copy_rhs" ? GA_BCAST_COPY_RHS : op == "dot" ? GA_BCAST_DOT : -1;
+}
+torch::Tensor offsets_on(const std::vector<int64_t> &table, const torch::Tensor &like) {
+  return torch::tensor(table, at::kLong).to(like.device());
+}
+
+// The reference's general SpMM (SpMMCsrKernel with UseBcast, spmm.cuh:30-71):
+// out[v] = reduce over the in-edges (out-edges with `reverse`) of op(u[src], e[edge])
+// with feature shapes that broadcast; op add | sub | mul | div | copy_lhs | copy_rhs,
+// the operand a copy does not read may be None.  fp32, the general (untuned) kernel.
+torch::Tensor gspmm_bcast(at::optional<torch::Tensor> u, at::optional<torch::Tensor> e,
+                          std::string op, std::string reduce, bool reverse,
+                          const GraphPtr &g) {
+  const int code = bcast_op(op);
+  TORCH_CHECK(code >= 0 && code != GA_BCAST_DOT, "Unsupported SpMM binary operator: ", op);
+  const int r = reduce == "sum" ? GA_SUM : reduce == "max" ? GA_MAX : reduce == "min" ? GA_MIN : -1;
+  TORCH_CHECK(r >= 0, "Unsupported SpMM reducer: ", reduce);
+  const bool use_u = code != GA_BCAST_COPY_RHS, use_e = code != GA_BCAST_COPY_LHS;
+  TORCH_CHECK(!use_u || u.has_value(), "node features are required");
+  TORCH_CHECK(!use_e || e.has_value(), "edge features are required");
+  if (use_u) {
+    check_input(u.value(), "u");
+    TORCH_CHECK(u.value().scalar_type() == at::kFloat, "the general SpMM is float32 only");
+    TORCH_CHECK(u.value().size(0) == g->num_nodes, "u has the wrong number of rows");
+  }
+  if (use_e) {
+    check_input(e.value(), "e");
+    TORCH_CHECK(e.value().scalar_type() == at::kFloat, "the general SpMM is float32 only");
+    TORCH_CHECK(e.value().size(0) == g->num_edges, "e must have one row per edge");
+  }
+  const torch::Tensor &ref = use_u ? u.value() : e.value();
+  std::vector<int64_t> ls = use_u ? u.value().sizes().vec() : e.value().sizes().vec();
+  std::vector<int64_t> rs = use_e ? e.value().sizes().vec() : u.value().sizes().vec();
+  const BcastTables b = bcast_tables(code, ls, rs);
+  std::vector<int64_t> shape{g->num_nodes};
+  shape.insert(shape.end(), b.feat_shape.begin(), b.feat_shape.end());
+  torch::Tensor out = torch::empty(shape, ref.options());
+  torch::Tensor u_off, e_off;
+  if (b.use) {
+    u_off = offsets_on(b.lhs_off, ref);
+    e_off = offsets_on(b.rhs_off, ref);
+  }
+  const auto &side = g->side(reverse);
+  const torch::Tensor &ptr = reverse ? g->out_pointer : g->in_pointer;
+  const torch::Tensor &nbr = reverse ? g->out_node_indices : g->in_node_indices;
+  const torch::Tensor &eid = reverse ? g->out_edge_indices : g->in_edge_indices;
+  check_ga(ga_spmm_csr_bcast(ptr.data_ptr<int>(), nbr.data_ptr<int>(),
+                             side.identity ? nullptr : eid.data_ptr<int>(),
+                             use_u ? u.value().data_ptr<float>() : nullptr,
+                             use_e ? e.value().data_ptr<float>() : nullptr, out.data_ptr<float>(),
+                             nullptr, nullptr, g->num_nodes, g->num_edges,
+                             b.use ? u_off.data_ptr<int64_t>() : nullptr,
+                             b.use ? e_off.data_ptr<int64_t>() : nullptr,
+                             std::max<int64_t>(b.lhs_len, 1), std::max<int64_t>(b.rhs_len, 1),
+                             b.out_len, code, r,
+                             current_stream(ref)),
+           "ga_spmm_csr_bcast");
+  return out;
+}
+
+// The reference's general SDDMM (sddmm.cuh:34-120): out[e] = op(lhs[id_l(e)], rhs[id_r(e)])
+// in edge-id order, each operand on the source nodes ("u"), the edges ("e") or the
+// destination nodes ("v") (selector.h:30-60), feature shapes that broadcast; "dot" sums
+// the products over the last dimension.  fp32, the general (untuned) kernel.
+torch::Tensor gsddmm(torch::Tensor lhs, torch::Tensor rhs, std::string op,
+                     std::string lhs_target, std::string rhs_target, const GraphPtr &g) {
+  const int code = bcast_op(op);
+  TORCH_CHECK(code >= 0, "Unsupported SDDMM binary operator: ", op);
+  check_input(lhs, "lhs");
+  check_input(rhs, "rhs");
+  TORCH_CHECK(lhs.scalar_type() == at::kFloat && rhs.scalar_type() == at::kFloat,
+              "the general SDDMM is float32 only");
+  auto target = [&](const std::string &t, const torch::Tensor &x, const char *name) {
+    const int k = t == "u" ? 0 : t == "e" ? 1 : t == "v" ? 2 : -1;
+    TORCH_CHECK(k >= 0, "targets are 'u' (source), 'e' (edge) or 'v' (destination)");
+    TORCH_CHECK(x.dim() >= 1 && x.size(0) == (k == 1 ? g->num_edges : g->num_nodes), name,
+                " has the wrong number of rows for target '", t, "'");
+    return k;
+  };
+  const int lt = target(lhs_target, lhs, "lhs"), rt = target(rhs_target, rhs, "rhs");
+  TORCH_CHECK(code != GA_BCAST_DOT ||
+                  (lhs.dim() >= 2 && rhs.dim() >= 2 && lhs.size(-1) == rhs.size(-1)),
+              "dot needs operands with the same last dimension");
+  const BcastTables b = bcast_tables(code, lhs.sizes(), rhs.sizes());
+  std::vector<int64_t> shape{g->num_edges};
+  shape.insert(shape.end(), b.feat_shape.begin(), b.feat_shape.end());
+  if (shape.size() == 1) shape.push_back(1);
+  torch::Tensor out = torch::empty(shape, lhs.options());
+  torch::Tensor l_off, r_off;
+  if (b.use) {
+    l_off = offsets_on(b.lhs_off, lhs);
+    r_off = offsets_on(b.rhs_off, lhs);
+  }
+  check_ga(ga_sddmm_bcast(g->COO_src.data_ptr<int64_t>(), g->COO_dst.data_ptr<int64_t>(),
+                          lhs.data_ptr<float>(), rhs.data_ptr<float>(), out.data_ptr<float>(),
+                          g->num_edges, lt, rt, b.use ? l_off.data_ptr<int64_t>() : nullptr,
+                          b.use ? r_off.data_ptr<int64_t>() : nullptr,
+                          std::max<int64_t>(b.lhs_len, 1), std::max<int64_t>(b.rhs_len, 1),
+                          b.out_len, b.reduce_size, code, current_stream(out)),
+           "ga_sddmm_bcast");
+  return out;
+}
+
 // SpMMEdge(x * y) for two per-edge operands without the product tensor: one of
 // them must be a per-edge / per-head fp32 weight; otherwise multiply, then copy_e
 torch::Tensor e_mul_e_sum(torch::Tensor x, torch::Tensor y, const GraphPtr &graph) {
@@ -1114,6 +1273,12 @@ static auto registry =
         .op("my_ops::gsddmm_u_dot_v(Tensor x, Tensor y, " GRAPH_T " g) -> Tensor z", &u_dot_v)
         .op("my_ops::gspmm(Tensor x, Tensor? y, str op, str reduce, " GRAPH_T " g) -> Tensor z",
             &gspmm)
+        .op("my_ops::gspmm_bcast(Tensor? u, Tensor? e, str op, str reduce, bool reverse, " GRAPH_T
+            " g) -> Tensor z",
+            &gspmm_bcast)
+        .op("my_ops::gsddmm(Tensor lhs, Tensor rhs, str op, str lhs_target, str rhs_target, "
+            GRAPH_T " g) -> Tensor z",
+            &gsddmm)
         .op("my_ops::gspmm_e_mul_e_sum(Tensor x, Tensor y, " GRAPH_T " g) -> Tensor z",
             &e_mul_e_sum)
         .op("my_ops::edge_softmax_sum(Tensor x, Tensor m, " GRAPH_T " g) -> Tensor z",

@@ -188,6 +188,55 @@ def test_relation_pair_attention_op(device, bf16):
                     assert not torch.equal(got, want)
 
 
+def test_general_broadcast_forms_through_torchscript(device):
+    """my_ops::gspmm_bcast / my_ops::gsddmm build the offset tables of bcast.cc:19-71 in
+    C++ and run the kernels the Python wrappers run (those are checked against numpy
+    broadcasting in test_gpu_bcast.py): same shapes out, same bits."""
+    from graphiler_amd import ops as pyops
+    torch_boundary.load()
+    rng = np.random.default_rng(33)
+    n = 300
+    src, dst = skewed_graph(rng, n, 1200, 2500)
+    g = prepare_graph(src, dst, n, device=device)
+    sg = torch_boundary.script_graph(g)
+    e = src.shape[0]
+    for u_feat, e_feat in (((4, 1), (1, 8)), ((3,), (1,)), ((2, 3), (3,)), ((5,), (5,)),
+                           ((1, 6), (4, 1)), ((2, 1, 3), (4, 1))):
+        u = _t(rng.standard_normal((n,) + u_feat).astype(np.float32), device)
+        w = _t(rng.uniform(0.5, 2.0, (e,) + e_feat).astype(np.float32), device)
+        for op in ("add", "sub", "mul", "div"):
+            for reduce, reverse in (("sum", False), ("max", False), ("min", True)):
+                got = torch.ops.my_ops.gspmm_bcast(u, w, op, reduce, reverse, sg)
+                want = pyops.gspmm(g, op, reduce, u, w, reverse=reverse)
+                assert got.shape == want.shape and torch.equal(got, want), (op, reduce, u_feat)
+        assert torch.equal(torch.ops.my_ops.gspmm_bcast(u, None, "copy_lhs", "sum", False, sg),
+                           pyops.gspmm(g, "copy_lhs", "sum", u, None))
+        assert torch.equal(torch.ops.my_ops.gspmm_bcast(None, w, "copy_rhs", "max", False, sg),
+                           pyops.gspmm(g, "copy_rhs", "max", None, w))
+    rows = {"u": n, "e": e, "v": n}
+    for lt, rt in (("u", "v"), ("u", "e"), ("e", "v"), ("v", "u"), ("e", "e")):
+        for l_feat, r_feat in (((4,), (4,)), ((3, 1), (1, 5)), ((2, 3), (3,)), ((1,), (6,))):
+            lhs = _t(rng.standard_normal((rows[lt],) + l_feat).astype(np.float32), device)
+            rhs = _t(rng.uniform(0.5, 2.0, (rows[rt],) + r_feat).astype(np.float32), device)
+            for op in ("add", "sub", "mul", "div", "copy_lhs", "copy_rhs"):
+                got = torch.ops.my_ops.gsddmm(lhs, rhs, op, lt, rt, sg)
+                want = pyops.gsddmm(g, op, lhs, rhs, lt, rt)
+                assert got.shape == want.shape and torch.equal(got, want), (op, lt, rt, l_feat)
+        for l_feat, r_feat in (((4, 8), (4, 8)), ((4, 8), (1, 8)), ((16,), (16,)), ((2, 1, 5), (3, 5))):
+            lhs = _t(rng.standard_normal((rows[lt],) + l_feat).astype(np.float32), device)
+            rhs = _t(rng.standard_normal((rows[rt],) + r_feat).astype(np.float32), device)
+            got = torch.ops.my_ops.gsddmm(lhs, rhs, "dot", lt, rt, sg)
+            want = pyops.gsddmm(g, "dot", lhs, rhs, lt, rt)
+            assert got.shape == want.shape and torch.equal(got, want), ("dot", lt, rt, l_feat)
+    x = torch.zeros(n, 3, device=device)
+    with pytest.raises(RuntimeError, match="number of rows"):
+        torch.ops.my_ops.gsddmm(x, x, "add", "e", "v", sg)
+    with pytest.raises(RuntimeError, match="do not broadcast"):
+        torch.ops.my_ops.gsddmm(x, torch.zeros(n, 4, device=device), "add", "u", "v", sg)
+    with pytest.raises(RuntimeError, match="Unsupported SpMM binary operator"):
+        torch.ops.my_ops.gspmm_bcast(x, x, "dot", "sum", False, sg)
+
+
 def test_error_convention(setup, device):
     sg, arr, rng = setup
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
