@@ -113,7 +113,7 @@ struct GatPolicy {
     finish(st, o);
 #pragma unroll
     for (int v = 0; v < VEC; ++v)
-      o[v] = o[v] > 0.0f ? o[v] : (A.act == GA_ACT_ELU ? __expf(o[v]) - 1.0f : (o[v] != o[v] ? o[v] : 0.0f));
+      o[v] = o[v] > 0.0f ? o[v] : (A.act == GA_ACT_ELU ? expm1f(o[v]) : (o[v] != o[v] ? o[v] : 0.0f));
     IO::store(out + row * feat + f0, o, IO::lane(A.stride_shift, feat - f0));
   }
   static __device__ __forceinline__ void emit_empty(const Args &A, out_t *out, int64_t row,

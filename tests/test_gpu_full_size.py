@@ -235,3 +235,158 @@ def test_config5_three_layer_network_layer_by_layer(device):
         assert_close(out.float().cpu().numpy()[sample], ref, TOL_BF16,
                      f"config 5 network, layer {layer + 1} ({k} -> 256), sampled rows")
         x = torch.nn.functional.elu(out)
+
+
+def _hgt_reference(wl, ptr, nbr, eid, h, wk, wq, wv, wa, ratt, rmsg, rpri, skip, heads, d, cast):
+    """The unfused HGT plan (examples/HGT/HGT.py:28-60, one (D x D) block per head) on
+    the oracle; ``cast`` rounds where the device stores tensors of the feature dtype.
+    Returns (K, Q, V, t, out): node projections, the aggregate, the layer output."""
+    n, e, hid = wl.num_nodes, wl.num_edges, heads * d
+    ntp, etp = oracle.type_pointer(wl.ntype, 4), oracle.type_pointer(wl.etype, 10)
+    K = cast(oracle.segment_mm(ntp, h, wk))
+    V = cast(oracle.segment_mm(ntp, h, wv))
+    Q = cast(oracle.segment_mm(ntp, h, wq))
+    k_e = oracle.segment_mm(etp, oracle.gather_rows(wl.src, K), ratt, heads=heads)
+    q_e = oracle.gather_rows(wl.dst, Q)
+    attn = np.einsum("ehd,ehd->eh", k_e.reshape(e, heads, d).astype(np.float64),
+                     q_e.reshape(e, heads, d))
+    del k_e, q_e
+    attn = (attn * rpri[wl.etype] / np.sqrt(d)).astype(np.float32)
+    a = oracle.segment_softmax(ptr, eid, attn)
+    v_e = oracle.segment_mm(etp, oracle.gather_rows(wl.src, V), rmsg, heads=heads)
+    m = (v_e.reshape(e, heads, d) * a[:, :, None]).reshape(e, hid).astype(np.float32)
+    del v_e
+    t = oracle.spmm(ptr, nbr, eid, m, op="copy_e")
+    gate = (1.0 / (1.0 + np.exp(-skip[wl.ntype])))[:, None]
+    return K, Q, V, t, oracle.segment_mm(ntp, cast(t), wa) * gate
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("bf16", [True, False])
+def test_config4_hgt_layer_pair_form_full(device, bf16, monkeypatch):
+    """The path the benchmark times at config 4: ``hgt_layer(fused=True)``, which on this
+    graph (2 M edges, 269,078 (destination, relation) pairs) applies the relation
+    matrices per pair, and ``relation_pair_attention`` on its own, both against the
+    unfused plan evaluated by the oracle on all 2 M edges."""
+    wl = datasets.hgt_hetero()
+    n, heads, d = wl.num_nodes, 8, 16
+    hid = heads * d
+    g = prepare_graph(wl.src, wl.dst, n, device=device, ntype_of=wl.ntype,
+                      num_ntypes=4, etype_of=wl.etype, num_etypes=10)
+    ptr, nbr, eid = _host(g)
+    pairs = g.relation_pairs()
+    key = wl.dst.astype(np.int64) * 10 + wl.etype
+    assert pairs is not None and pairs.num_pairs == len(np.unique(key))
+    assert wl.num_edges >= layers.PAIRS_MIN_EDGES_PER_PAIR * pairs.num_pairs
+    cast = to_bf16_f32 if bf16 else (lambda a: np.asarray(a, dtype=np.float32))
+    tol = TOL_BF16 if bf16 else TOL_F32
+    rng = np.random.default_rng(34)
+    h = cast(rng.standard_normal((n, hid), dtype=np.float32))
+    wk, wq, wv, wa = (cast(datasets.glorot(rng, (4, hid, hid))) for _ in range(4))
+    ratt, rmsg = (cast(datasets.glorot(rng, (10, heads, d, d))) for _ in range(2))
+    rpri = cast(rng.uniform(0.5, 1.5, (10, heads)).astype(np.float32))
+    skip = rng.standard_normal(4).astype(np.float32)
+    K, Q, V, t_ref, out_ref = _hgt_reference(wl, ptr, nbr, eid, h, wk, wq, wv, wa, ratt, rmsg,
+                                             rpri, skip, heads, d, cast)
+    calls = []
+    real = ops.relation_pair_attention
+
+    def counted(*a, **kw):
+        calls.append(1)
+        return real(*a, **kw)
+
+    monkeypatch.setattr(ops, "relation_pair_attention", counted)
+    got = layers.hgt_layer(g, _t(h, device, bf16), _t(wk, device, bf16), _t(wq, device, bf16),
+                           _t(wv, device, bf16), _t(wa, device, bf16), _t(ratt, device, bf16),
+                           _t(rmsg, device, bf16), _t(rpri, device, bf16), _t(skip, device),
+                           heads, fused=True)
+    assert calls == [1], "the layer must take the per-pair form on this graph"
+    assert_close(got.float().cpu().numpy(), out_ref, tol, f"config 4 HGT layer, pairs, bf16={bf16}")
+    # the attention stage alone, on the oracle's own (rounded) K, Q, V
+    t = real(_t(K, device, bf16), _t(Q, device, bf16), _t(V, device, bf16), _t(ratt, device, bf16),
+             _t(rmsg, device, bf16), _t(rpri, device), g, factor=1.0 / np.sqrt(d))
+    assert_close(t.float().cpu().numpy(), t_ref, tol,
+                 f"config 4 relation_pair_attention, bf16={bf16}")
+    # and the per-edge form of the same layer
+    per_edge = layers.hgt_layer(g, _t(h, device, bf16), _t(wk, device, bf16), _t(wq, device, bf16),
+                                _t(wv, device, bf16), _t(wa, device, bf16), _t(ratt, device, bf16),
+                                _t(rmsg, device, bf16), _t(rpri, device, bf16), _t(skip, device),
+                                heads, fused="edges")
+    assert calls == [1]
+    assert_close(per_edge.float().cpu().numpy(), out_ref, tol,
+                 f"config 4 HGT layer, per edge, bf16={bf16}")
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_config3_rgcn_network_with_fused_relu_full(device, bf16):
+    """The calls the benchmark times at config 3: layer 1 with the relu applied by the
+    one-pass kernel to the sums it stores, layer 2 plain on that output."""
+    wl = datasets.rgcn_zipf()
+    n = wl.num_nodes
+    g = prepare_graph(wl.src, wl.dst, n, device=device, etype_of=wl.etype, num_etypes=60)
+    ptr, nbr, eid = _host(g)
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((n, 16), dtype=np.float32)
+    w1, w2 = datasets.glorot(rng, (60, 16, 64)), datasets.glorot(rng, (60, 64, 8))
+    if bf16:
+        x, w1, w2 = to_bf16_f32(x), to_bf16_f32(w1), to_bf16_f32(w2)
+    deg = np.maximum(np.bincount(wl.dst, minlength=n), 1)
+    norm = (1.0 / deg[wl.dst]).astype(np.float32)[:, None]
+    etp = oracle.type_pointer(wl.etype, 60)
+    tol = TOL_BF16 if bf16 else TOL_F32
+
+    def ref_layer(hh, w):
+        msg = oracle.segment_mm(etp, oracle.gather_rows(wl.src, hh), w) * norm
+        return oracle.spmm(ptr, nbr, eid, msg.astype(np.float32), op="copy_e")
+
+    assert ops.typed_spmm_preferred(_t(x, device, bf16), _t(w1, device, bf16))
+    h1 = layers.rgcn_layer(g, _t(x, device, bf16), _t(w1, device, bf16), _t(norm, device),
+                           fused=True, activation="relu")
+    r1 = np.maximum(ref_layer(x, w1), 0)
+    assert_close(h1.float().cpu().numpy(), r1, tol, "config 3 layer 1 with relu in the kernel")
+    assert bool((h1 == 0).any()) and not bool((h1 < 0).any())
+    h2 = layers.rgcn_layer(g, h1, _t(w2, device, bf16), _t(norm, device), fused=True)
+    assert_close(h2.float().cpu().numpy(), ref_layer(h1.float().cpu().numpy(), w2), tol,
+                 "config 3 layer 2 on the device's layer 1")
+    # elu through the same epilogue
+    e1 = layers.rgcn_layer(g, _t(x, device, bf16), _t(w1, device, bf16), _t(norm, device),
+                           fused=True, activation="elu")
+    pre = ref_layer(x, w1).astype(np.float64)
+    assert_close(e1.float().cpu().numpy(), np.where(pre > 0, pre, np.expm1(pre)), tol,
+                 "config 3 layer 1 with elu in the kernel")
+
+
+@pytest.mark.timeout(600)
+def test_config5_network_as_benchmarked(device):
+    """The three calls of the benchmarked network, ``gat_layer(..., fused=True,
+    activation="elu")`` for the hidden layers and no activation on the last one, each on
+    the device's own previous output; sampled destination rows and the heaviest ones."""
+    wl = datasets.gat_rmat_large()
+    n, heads, d = wl.num_nodes, 4, 64
+    deg = np.bincount(wl.dst, minlength=n)
+    g = prepare_graph(wl.src, wl.dst, n, device=device)
+    ptr = g.in_pointer.cpu().numpy()
+    rng = np.random.default_rng(46)
+    sample = np.unique(np.concatenate([rng.integers(0, n, 2000), np.argsort(deg)[-3:], [0, n - 1]]))
+    sub_ptr = np.concatenate([[0], np.cumsum(deg[sample])]).astype(np.int32)
+    sub_nbr = np.concatenate([wl.src[ptr[v]:ptr[v + 1]] for v in sample]).astype(np.int32)
+    x = _t(to_bf16_f32(rng.standard_normal((n, 100), dtype=np.float32)), device, True)
+    for layer, k in enumerate((100, 256, 256)):
+        act = "elu" if layer < 2 else None
+        w = to_bf16_f32(datasets.glorot(rng, (k, heads * d)))
+        a = datasets.glorot(rng, (2, heads, d), fan_in=2 * d, fan_out=1)
+        out = layers.gat_layer(g, x, _t(w, device, True), _t(a, device), heads, 0.2, fused=True,
+                               activation=act)
+        z32 = x.float().cpu().numpy() @ w
+        zh = z32.reshape(n, heads, d)
+        z = to_bf16_f32(z32)
+        # the source term as the pass forms it: from the stored (rounded) rows
+        el = (z.reshape(n, heads, d) * a[0]).sum(-1).astype(np.float32)
+        er = (zh * a[1]).sum(-1).astype(np.float32)
+        ref = oracle.gat_aggregate(sub_ptr, sub_nbr, el, er[sample], z, heads=heads,
+                                   slope=0.2).astype(np.float64)
+        if act:
+            ref = np.where(ref > 0, ref, np.expm1(ref))
+        assert_close(out.float().cpu().numpy()[sample], ref, TOL_BF16,
+                     f"config 5 network as benchmarked, layer {layer + 1} ({k} -> 256, {act})")
+        x = out

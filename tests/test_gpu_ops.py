@@ -801,6 +801,18 @@ def test_gat_aggregate_with_activation(graph, device, heads, dim, bf16, activati
                  TOL_BF16 if bf16 else TOL_F32, f"gat + {activation} on {name}")
     if activation == "relu":
         assert torch.equal(got, torch.relu(ops.gat_aggregate(*args)))
+    elif not bf16:
+        # sums of about 1e-4: exp(o) - 1 would cancel to 1e-3 relative there, F.elu's expm1
+        # does not; every element is held to the size of its row's terms
+        zs = (z * np.float32(1e-4)).astype(np.float32)
+        pre = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er, zs, heads=heads,
+                                   slope=0.2).astype(np.float64)
+        mag = oracle.gat_aggregate(arr.in_pointer, arr.in_node_indices, el, er, np.abs(zs),
+                                   heads=heads, slope=0.2)
+        small = ops.gat_aggregate(_dev(el, device), _dev(er, device), _dev(zs, device), g, 0.2,
+                                  activation="elu")
+        assert_close(small.cpu().numpy().reshape(pre.shape), np.where(pre > 0, pre, np.expm1(pre)),
+                     TOL_F32, f"gat + elu on sums near 1e-4, {name}", mag=mag)
     if dim in (16, 64):          # head widths the source-term variant takes
         a_l = (rng.standard_normal((heads, dim)) / np.sqrt(dim)).astype(np.float32)
         plain = ops.gat_aggregate_from_z(_dev(a_l, device), _dev(er, device), _dev(z, device, bf16), g, 0.2)

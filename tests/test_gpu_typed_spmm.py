@@ -212,6 +212,13 @@ def test_typed_spmm_activation(device, bf16):
         elu = ops.TypedSpMMEdge(x, w, g, row_scale=norm.reshape(-1), activation="elu")
         assert_close(elu.float().cpu().numpy(), F.elu(plain.float()).cpu().numpy(),
                      TOL_BF16 if bf16 else TOL_F32, f"typed elu {k}->{m}")
+        if not bf16:
+            # sums near 1e-4, element by element: expm1, not exp(o) - 1
+            xs = x * 1e-4
+            want = F.elu(ops.TypedSpMMEdge(xs, w, g, row_scale=norm.reshape(-1))).cpu().numpy()
+            got = ops.TypedSpMMEdge(xs, w, g, row_scale=norm.reshape(-1), activation="elu")
+            assert_close(got.cpu().numpy(), want, TOL_F32, f"typed elu near 1e-4 {k}->{m}",
+                         mag=np.abs(want))
         for fused in ("tiles", "pair", False):
             got = layers.rgcn_layer(g, x, w, norm, fused=fused, activation="relu")
             want = torch.relu(layers.rgcn_layer(g, x, w, norm, fused=fused))
