@@ -2,8 +2,8 @@
 """Benchmark of the graph-primitive layer on one MI355X: GAT / RGCN / HGT layer
 forwards at the benchmark configurations, with per-kernel roofline figures.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs c5,c2,c3,c4]
-                    [--no-cpu-baseline] [--calibrate-copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs c5,c2,c3,c4,c1]
+                    [--only KEY[,KEY]] [--no-cpu-baseline] [--markers]
 
 Headline (the JSON line's metric / value / roofline / cpu_baseline): the first
 configuration named in --configs, by default c5 = configs[4], the largest one
@@ -15,16 +15,26 @@ edge softmax -> u_mul_e sum, elu between layers); `value` counts the edges the t
 layers traverse per second.  All inputs are resident in HBM before the timed region.
 
 The other configurations (c2 = configs[1] 1-head fp32 GAT, c3 = configs[2] RGCN
-fp32 and bf16, c4 = configs[3] HGT bf16) are measured in the same run and reported
-as objects under "configs" of the same line: layer time, edges/s and, per operator,
+fp32 and bf16, c4 = configs[3] HGT bf16, c1 = configs[0] the 2-layer GCN that the
+configuration list assigns to the host cores, timed there and on the GPU) are measured
+in the same run and reported as objects under "configs" of the same line: layer time, edges/s and, per operator,
 launch time (HIP events on the launch stream), algorithmic bytes, effective GB/s,
 fraction of the 8 TB/s HBM peak and, for the matrix kernels, TFLOP/s against the
 MFMA peak and against min(MFMA peak, intensity x HBM peak).
 
-Algorithmic bytes credit one gathered row per edge and no cache reuse.  When they
-flow faster than the HBM peak the operator is marked "cache_served" and its fraction
-is taken from the L2 <-> memory traffic that rocprofv3 counted for the same kernel
-(read from profiles/hbm_traffic.md, a separate counter run: not measured here).
+Algorithmic bytes credit one gathered row per edge and no cache reuse.  An operator
+whose gathered table fits the 256 MB Infinity Cache, or whose algorithmic bytes flow
+faster than the HBM peak, is marked "cache_served": its fraction is then taken from the
+L2 <-> fabric traffic that rocprofv3 counted for the operator's own dispatches (read
+from profiles/hbm_traffic.md, separate counter runs of this script with --markers: not
+measured here), and is null when no such count exists.  A count below the bytes the
+operator writes cannot be that operator's and is refused.
+
+--markers brackets every timed operator with an elementwise pass over 1 GiB
+(`x.add(0)`: reads 1 GiB, writes 1 GiB).  In a rocprofv3 trace or counter file the
+dispatches between two such passes are exactly one operator's calls (the line's
+"profile_segments" lists key and number of calls in order), and the passes themselves
+calibrate the counters.
 Prints ONE JSON line.
 """
 import argparse
@@ -38,6 +48,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0                                   # MI355X published HBM3E bandwidth
+INFINITY_CACHE_BYTES = 256 << 20                        # memory-side cache in front of the HBM
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}       # published dense matrix peaks
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.md")
 
@@ -59,22 +70,25 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--configs", default="c5,c2,c3,c4",
-                    help="comma-separated subset of c2,c3,c4,c5; the first one is the headline")
+    ap.add_argument("--configs", default="c5,c2,c3,c4,c1",
+                    help="comma-separated subset of c1,c2,c3,c4,c5; the first one is the headline")
+    ap.add_argument("--only", default="",
+                    help="comma-separated operator keys (c4.hgt_layer, c2.segment_softmax, ...): time "
+                         "only these, skip the network steps and the CPU legs (short profiler runs)")
     ap.add_argument("--reps", type=int, default=30, help="timed calls per operator")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ops", action="store_true",
                     help="time the layers only (shorter kernel traces for profiling)")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run an elementwise copy of 1 GiB (x.add(0)) so that rocprofv3 "
-                         "--pmc counters can be scaled against a kernel of known traffic")
+    ap.add_argument("--markers", "--calibrate-copy", dest="markers", action="store_true",
+                    help="bracket every timed operator with an elementwise pass over 1 GiB (x.add(0)): "
+                         "segment boundaries and counter calibration for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 "
                  "(the path is not sharded across devices)")
     wanted = [c for c in args.configs.split(",") if c]
     for c in wanted:
-        if c not in ("c2", "c3", "c4", "c5"):
+        if c not in ("c1", "c2", "c3", "c4", "c5"):
             sys.exit(f"bench.py: unknown configuration {c!r}")
 
     import numpy as np
@@ -87,46 +101,93 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     traffic = load_traffic()
+    only = {k for k in args.only.split(",") if k}
+    if only:
+        args.no_cpu_baseline = True
+    segments = []                      # (key, calls) of every bracketed operator, in order
+    marker_buf = torch.zeros(1 << 28, dtype=torch.float32, device=dev) if args.markers else None
 
-    def ev_time(fn, reps=None, warmup=3):
+    def marker():
+        if marker_buf is not None:
+            marker_buf.add(0.0)        # reads 1 GiB, writes 1 GiB (the result is dropped)
+
+    def ev_time(fn, reps=None, warmup=3, key=None):
         reps = reps or args.reps
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
+        if key is not None:
+            marker()
         s = torch.cuda.Event(enable_timing=True)
         e = torch.cuda.Event(enable_timing=True)
         s.record()
         for _ in range(reps):
             fn()
         e.record()
+        if key is not None:
+            marker()
+            segments.append([key, reps])
         torch.cuda.synchronize()
         return s.elapsed_time(e) / reps
 
-    def wall_time(fn, steps, warmup):
+    def wall_time(fn, steps, warmup, key=None):
+        """Wall-clock time per call of a network step (None with --only: steps are
+        not operators of their own)."""
+        if only:
+            return None, fn()
         for _ in range(warmup):
             fn()
+        torch.cuda.synchronize()
+        marker()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
             out = fn()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / steps, out
+        dt = time.perf_counter() - t0
+        marker()
+        if key is not None:
+            segments.append([key, steps])
+        return dt * 1e3 / steps, out
 
-    def op_record(key, fn, nbytes, flops=None, mfma=None, reps=None):
-        """Launch time and roofline position of one operator call."""
-        ms = ev_time(fn, reps)
+    def tensor_bytes(out):
+        if isinstance(out, torch.Tensor):
+            return out.numel() * out.element_size()
+        return sum(tensor_bytes(o) for o in out) if isinstance(out, (tuple, list)) else 0
+
+    def op_record(key, fn, nbytes, flops=None, mfma=None, reps=None, gather=None):
+        """Launch time and roofline position of one operator call.  ``gather`` = (bytes of
+        the table the operator gathers rows from, bytes of gathered rows among ``nbytes``);
+        None for an operator that streams."""
+        if only and key not in only:
+            return None
+        written = tensor_bytes(fn())
+        ms = ev_time(fn, reps, key=key)
         gbps = nbytes / ms / 1e6
-        rec = {"ms": round(ms, 4), "algorithmic_bytes": int(nbytes),
-               "effective_GBps": round(gbps, 1), "bound": "hbm"}
+        rec = {"ms": round(ms, 4), "algorithmic_bytes": int(nbytes), "written_bytes": int(written),
+               "effective_GBps": round(gbps, 1), "frac_algorithmic": round(gbps / HBM_PEAK_GBS, 4),
+               "bound": "hbm"}
         moved = traffic.get(key)
+        if moved is not None and moved < 0.98 * written:
+            rec["traffic_refused"] = ("the recorded count (%d B) is below the %d B this operator "
+                                      "writes: not this operator's dispatches" % (moved, written))
+            moved = None
         if moved is not None:
             rec["traffic"] = moved
             rec["traffic_GBps"] = round(moved / ms / 1e6, 1)
-        if gbps > HBM_PEAK_GBS:
+        cached_table = gather is not None and gather[0] <= INFINITY_CACHE_BYTES \
+            and 2 * gather[1] >= nbytes
+        if gbps > HBM_PEAK_GBS or cached_table:
+            # most of the algorithmic bytes are rows gathered from a table that the L2s and
+            # the Infinity Cache hold: bytes over time is not memory bandwidth.  The fraction
+            # is the counted L2 <-> fabric traffic (itself an upper bound of the HBM traffic:
+            # Infinity Cache hits are counted), and never more than the algorithmic figure
             rec["cache_served"] = True
-            rec["frac"] = round(moved / ms / 1e6 / HBM_PEAK_GBS, 4) if moved else None
+            rec["frac"] = round(min(moved, nbytes) / ms / 1e6 / HBM_PEAK_GBS, 4) if moved else None
+            rec["frac_basis"] = "min(counted traffic, algorithmic bytes)" if moved else None
         else:
-            rec["frac"] = round(gbps / HBM_PEAK_GBS, 4)
+            rec["frac"] = rec["frac_algorithmic"]
+            rec["frac_basis"] = "algorithmic bytes"
         if flops:
             peak = MFMA_PEAK_TFLOPS[mfma]
             tf = flops / ms / 1e9
@@ -136,6 +197,25 @@ def main():
                         "ceiling_tflops": round(ceiling, 1),
                         "frac_of_ceiling": round(tf / ceiling, 4)})
         return rec
+
+    def kept(table):
+        return {k: v for k, v in table.items() if v is not None}
+
+    def per_s(count, ms):
+        return None if ms is None else round(count / (ms * 1e-3), 1)
+
+    def r4(ms, div=1):
+        return None if ms is None else round(ms / div, 4)
+
+    def cpu_time(fn, budget_s=10.0, min_reps=3, max_reps=50):
+        """One warm-up pass, then at least ``min_reps`` timed passes (more while they fit
+        ``budget_s``); returns (ms per pass, passes, last result)."""
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while reps < min_reps or (time.perf_counter() - t0 < budget_s and reps < max_reps):
+            out = fn()
+            reps += 1
+        return (time.perf_counter() - t0) * 1e3 / reps, reps, out
 
     def rnd(*shape, dtype=torch.float32, scale=1.0):
         return (torch.randn(*shape, device=dev) * scale).to(dtype)
@@ -150,13 +230,7 @@ def main():
         del a, b
         return round(2 * (1 << 30) / ms / 1e6, 1)
 
-    if args.calibrate_copy:
-        big = torch.zeros(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB
-        for _ in range(3):
-            big2 = big.add(0.0)        # reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del big, big2
-    measured_copy = copy_rate()
+    measured_copy = None if only else copy_rate()
 
     results = {}
     cpu = None
@@ -185,15 +259,37 @@ def main():
         def network():
             x = x0
             for w, a in params:
-                x = layers.gat_layer(g, x, w, a, H, slope, fused=True, activation="elu")
+                # F.elu between the layers, none after the last (examples/GAT/GAT.py:80-84)
+                x = layers.gat_layer(g, x, w, a, H, slope, fused=True,
+                                     activation=None if w is params[-1][0] else "elu")
             return x
 
-        ms_step, out = wall_time(network, args.steps, args.warmup)
+        # HIP events around every launch of the dominant operator inside the timed steps (on
+        # the stream it is launched on): its duration in the network, where the projection
+        # before it has just streamed 1.25 GB through the caches
+        inside = []
+        plain_from_z = ops.gat_aggregate_from_z
+
+        def timed_from_z(*a, **kw):
+            s_ev = torch.cuda.Event(enable_timing=True)
+            e_ev = torch.cuda.Event(enable_timing=True)
+            s_ev.record()
+            r = plain_from_z(*a, **kw)
+            e_ev.record()
+            inside.append((s_ev, e_ev))
+            return r
+
+        ops.gat_aggregate_from_z = timed_from_z
+        try:
+            ms_step, out = wall_time(network, args.steps, args.warmup, key="c5.step")
+        finally:
+            ops.gat_aggregate_from_z = plain_from_z
+        inside = [s_ev.elapsed_time(e_ev) for s_ev, e_ev in inside[-3 * args.steps:]] if not only else []
         rec = {"workload": "configs[4]: 3-layer GAT 100->256->256->256, 4 heads x 64, bf16 features, "
                            "fp32 softmax and accumulation; R-MAT(a=.57,b=.19,c=.19, seed 4) + self loops",
                "num_nodes": N, "num_edges": E, "max_in_degree": max_deg, "dtype": "bf16",
-               "ms_per_step": round(ms_step, 4), "ms_per_layer": round(ms_step / 3, 4),
-               "edges_per_s": round(3 * E / (ms_step * 1e-3), 1)}
+               "ms_per_step": r4(ms_step), "ms_per_layer": r4(ms_step, 3),
+               "edges_per_s": per_s(3 * E, ms_step)}
         z, el, er = layers.gat_project(x0, *params[0], H)
         z1, el1, er1 = layers.gat_project(z, *params[1], H)
         a_l = params[1][1][0].contiguous()
@@ -201,18 +297,19 @@ def main():
         opsr = {}
         opsr["gat_aggregate_from_z"] = op_record(
             "c5.gat_aggregate_from_z", lambda: ops.gat_aggregate_from_z(a_l, er1, z1, g, slope),
-            fused_bytes)
+            fused_bytes, gather=(N * Fw * b, E * Fw * b))
         if not args.no_ops:
             opsr["gat_aggregate"] = op_record(
                 "c5.gat_aggregate", lambda: ops.gat_aggregate(el1, er1, z1, g, slope),
-                4 * (N + 1) + E * (4 + H * 4 + Fw * b) + N * (H * 4 + Fw * b))
+                4 * (N + 1) + E * (4 + H * 4 + Fw * b) + N * (H * 4 + Fw * b),
+                gather=(N * Fw * b, E * Fw * b))
             att = torch.rand(E, H, device=dev)
             opsr["spmm_u_mul_e"] = op_record(
                 "c5.spmm_u_mul_e", lambda: ops.gspmm_src_mul_e_sum(z1, att, [1], False, None, g),
-                4 * (N + 1) + E * (4 + 4 * H + Fw * b) + N * Fw * b)
+                4 * (N + 1) + E * (4 + 4 * H + Fw * b) + N * Fw * b, gather=(N * Fw * b, E * Fw * b))
             opsr["sddmm_u_add_v"] = op_record(
                 "c5.sddmm_u_add_v", lambda: ops.gsddmm_u_add_v_mul_alpha(el1, er1, 1, g),
-                4 * (N + 1) + E * (4 + H * 4 + 4 * H) + N * H * 4)
+                4 * (N + 1) + E * (4 + H * 4 + 4 * H) + N * H * 4, gather=(N * H * 4, E * H * 4))
             lg = rnd(E, H)
             opsr["segment_softmax"] = op_record(
                 "c5.segment_softmax", lambda: ops.SegmentSoftmax(lg, 1, None, g),
@@ -224,9 +321,26 @@ def main():
                     f"c5.project_attn_{k}_256", lambda: layers.gat_project(xin, w, a, H),
                     N * (k + Fw) * b + k * Fw * b + 2 * N * H * 4,
                     2.0 * N * k * Fw + 4.0 * N * Fw, "bf16")
-        rec["ops"] = opsr
-        rec["roofline"] = dict(opsr["gat_aggregate_from_z"], kernel="gat_aggregate_from_z "
-                               "(runs_kernel<GatPolicy<bf16, 8, from z>> + fix-up)")
+        rec["ops"] = opsr = kept(opsr)
+        if "gat_aggregate_from_z" in opsr:
+            roof = dict(opsr["gat_aggregate_from_z"], kernel="gat_aggregate_from_z "
+                        "(runs_kernel<GatPolicy<bf16, 8, from z>> + fix-up)")
+            if inside:
+                # the headline figure is the operator's duration inside the timed network steps;
+                # "ms_back_to_back" keeps the repetitions of the operator on its own (its hot
+                # rows still in the Infinity Cache from the call before)
+                ms_in = sum(inside) / len(inside)
+                roof.update({"ms_back_to_back": roof["ms"], "ms": round(ms_in, 4),
+                             "launches_timed": len(inside),
+                             "effective_GBps": round(fused_bytes / ms_in / 1e6, 1),
+                             "frac": round(fused_bytes / ms_in / 1e6 / HBM_PEAK_GBS, 4),
+                             "frac_algorithmic": round(fused_bytes / ms_in / 1e6 / HBM_PEAK_GBS, 4)})
+                if "traffic" in roof:
+                    roof["traffic_GBps"] = round(roof["traffic"] / ms_in / 1e6, 1)
+            rec["roofline"] = roof
+        if "project_attn_256_256" in opsr:
+            rec["mfma"] = dict(opsr["project_attn_256_256"], kernel="project_attn 256 -> 256 bf16 "
+                               "(wide_mm_kernel, v_mfma_f32_16x16x32_bf16)")
 
         if headline == "c5" and not args.no_cpu_baseline:
             # one hidden layer (256 -> 256) of the same network on the host cores: the fp32
@@ -248,17 +362,16 @@ def main():
                 at = oracle.segment_softmax(ptr, None, lg_, zero_floor=True)
                 return oracle.spmm_sum_f32(ptr, nbr, None, zc, at, op="u_mul_e", heads=H)
 
-            t0 = time.perf_counter()
-            ref = cpu_layer()
-            cpu_ms = (time.perf_counter() - t0) * 1e3
+            cpu_ms, cpu_reps, ref = cpu_time(cpu_layer)
             got = layers.gat_layer(g, z, params[1][0], params[1][1], H, slope).float().cpu().numpy()
             err = float(np.abs(got - ref).max() / np.abs(ref).max())
             cpu = {"value": round(E / (cpu_ms * 1e-3), 1), "unit": "edges/s",
                    "cores": oracle.num_threads(), "kind": "port",
                    "ms_per_layer": round(cpu_ms, 1),
+                   "passes": cpu_reps,
                    "sample": f"one hidden layer (256 -> 256, all {E} edges, 4 heads) of the "
-                             "3-layer network, one pass of the fp32 C port (OpenMP) of the four graph "
-                             "operators + torch-CPU projection",
+                             f"3-layer network: one warm-up pass, then the mean of {cpu_reps} passes of "
+                             "the fp32 C port (OpenMP) of the four graph operators + torch-CPU projection",
                    "max_rel_diff_vs_gpu_bf16": err}
         return rec
 
@@ -276,40 +389,44 @@ def main():
         a_h = datasets.glorot(rng, (2, H, Fw // H), fan_in=2 * Fw, fan_out=1)
         x, w, a = (torch.from_numpy(t).to(dev) for t in (x_h, w_h, a_h))
         ms_step, out = wall_time(lambda: layers.gat_layer(g, x, w, a, H, slope, fused=True),
-                                 max(args.steps, 100), max(args.warmup, 10))
+                                 max(args.steps, 100), max(args.warmup, 10), key="c2.step")
         rec = {"workload": "configs[1]: 1-head GAT layer 602->64 fp32 (dense projection + fused "
                            "chain); R-MAT(a=.57,b=.19,c=.19, seed 1)",
                "num_nodes": N, "num_edges": E, "dtype": "f32",
-               "ms_per_step": round(ms_step, 4), "edges_per_s": round(E / (ms_step * 1e-3), 1)}
+               "ms_per_step": r4(ms_step), "edges_per_s": per_s(E, ms_step)}
         z, el, er = layers.gat_project(x, w, a, H)
+        rows = (N * Fw * b, E * Fw * b)
         opsr = {}
         opsr["gat_aggregate"] = op_record(
             "c2.gat_aggregate", lambda: ops.gat_aggregate(el, er, z, g, slope),
-            4 * (N + 1) + E * (4 + H * b + Fw * b) + N * (H * b + Fw * b), reps=50)
+            4 * (N + 1) + E * (4 + H * b + Fw * b) + N * (H * b + Fw * b), reps=50, gather=rows)
         dense_bytes = 4 * (N * in_dim + in_dim * Fw + N * Fw + 2 * N * H)
         opsr["linear_attn_602_64"] = op_record(
             "c2.linear_attn", lambda: layers.gat_project(x, w, a, H), dense_bytes, reps=50)
-        dms = opsr["linear_attn_602_64"]["ms"]
-        opsr["linear_attn_602_64"]["fp32_equivalent_tflops"] = round(2.0 * N * in_dim * Fw / dms / 1e9, 2)
-        opsr["linear_attn_602_64"]["bf16_piece_mfma_tflops"] = round(12.0 * N * in_dim * Fw / dms / 1e9, 1)
+        if opsr["linear_attn_602_64"] is not None:
+            dms = opsr["linear_attn_602_64"]["ms"]
+            opsr["linear_attn_602_64"]["fp32_equivalent_tflops"] = round(2.0 * N * in_dim * Fw / dms / 1e9, 2)
+            opsr["linear_attn_602_64"]["bf16_piece_mfma_tflops"] = round(12.0 * N * in_dim * Fw / dms / 1e9, 1)
         if not args.no_ops:
             logits = F.leaky_relu_(ops.gsddmm_u_add_v_mul_alpha(el, er, 1, g), slope)
             att = ops.SegmentSoftmax(logits, 1, None, g)
             opsr["sddmm_u_add_v"] = op_record(
                 "c2.sddmm_u_add_v", lambda: ops.gsddmm_u_add_v_mul_alpha(el, er, 1, g),
-                4 * (N + 1) + E * (4 + H * b + 4 * H) + N * H * b, reps=50)
+                4 * (N + 1) + E * (4 + H * b + 4 * H) + N * H * b, reps=50,
+                gather=(N * H * b, E * H * b))
             opsr["segment_softmax"] = op_record(
                 "c2.segment_softmax", lambda: ops.SegmentSoftmax(logits, 1, None, g),
                 4 * (N + 1) + 8 * E * H, reps=50)
             opsr["spmm_u_mul_e"] = op_record(
                 "c2.spmm_u_mul_e", lambda: ops.gspmm_src_mul_e_sum(z, att, [1], False, None, g),
-                4 * (N + 1) + E * (4 + 4 * H + Fw * b) + N * Fw * b, reps=50)
+                4 * (N + 1) + E * (4 + 4 * H + Fw * b) + N * Fw * b, reps=50, gather=rows)
             opsr["spmm_copy_u"] = op_record(
                 "c2.spmm_copy_u", lambda: ops.SpMMSrc(z, [1], False, None, g),
-                4 * (N + 1) + E * (4 + Fw * b) + N * Fw * b, reps=50)
-        rec["ops"] = opsr
-        rec["roofline"] = dict(opsr["gat_aggregate"],
-                               kernel="gat_aggregate (runs_kernel<GatPolicy<float, 4>> + fix-up)")
+                4 * (N + 1) + E * (4 + Fw * b) + N * Fw * b, reps=50, gather=rows)
+        rec["ops"] = opsr = kept(opsr)
+        if "gat_aggregate" in opsr:
+            rec["roofline"] = dict(opsr["gat_aggregate"],
+                                   kernel="gat_aggregate (runs_kernel<GatPolicy<float, 4>> + fix-up)")
         if headline == "c2" and not args.no_cpu_baseline:
             import oracle
             ptr = g.in_pointer.cpu().numpy()
@@ -326,12 +443,7 @@ def main():
                 at = oracle.segment_softmax(ptr, None, lg_, zero_floor=True)
                 return oracle.spmm_sum_f32(ptr, nbr, None, zc, at, op="u_mul_e", heads=H)
 
-            cpu_layer()
-            reps, t0 = 0, time.perf_counter()
-            while reps < 3 or (time.perf_counter() - t0 < 10.0 and reps < 50):
-                ref = cpu_layer()
-                reps += 1
-            cpu_ms = (time.perf_counter() - t0) * 1e3 / reps
+            cpu_ms, reps, ref = cpu_time(cpu_layer)
             got = out.cpu().numpy().reshape(ref.shape)
             cpu = {"value": round(E / (cpu_ms * 1e-3), 1), "unit": "edges/s",
                    "cores": oracle.num_threads(), "kind": "port", "ms_per_layer": round(cpu_ms, 2),
@@ -361,31 +473,34 @@ def main():
                 h1 = layers.rgcn_layer(g, x, w1, norm, fused=True, activation="relu")
                 return layers.rgcn_layer(g, h1, w2, norm, fused=True)
 
-            ms_step, _ = wall_time(network, max(args.steps, 100), max(args.warmup, 10))
-            v = {"dtype": tag, "ms_per_step": round(ms_step, 4), "ms_per_layer": round(ms_step / 2, 4),
-                 "edges_per_s": round(2 * E / (ms_step * 1e-3), 1), "ops": {}}
+            ms_step, _ = wall_time(network, max(args.steps, 100), max(args.warmup, 10),
+                                   key=f"c3.step_{tag}")
+            v = {"dtype": tag, "ms_per_step": r4(ms_step), "ms_per_layer": r4(ms_step, 2),
+                 "edges_per_s": per_s(2 * E, ms_step), "ops": {}}
             h1 = torch.relu(layers.rgcn_layer(g, x, w1, norm, fused=True))
             for (K, M), xin, w in (((16, 64), x, w1), ((64, 8), h1, w2)):
                 lbytes = 4 * (N + 1) + E * (8 + 4 + 4 + K * b) + R * K * M * b + N * M * b
+                rows = (N * K * b, E * K * b)
                 v["ops"][f"rgcn_layer_{K}_{M}"] = op_record(
                     f"c3.rgcn_layer_{K}_{M}_{tag}", lambda: layers.rgcn_layer(g, xin, w, norm, fused=True),
-                    lbytes, 2.0 * E * K * M, tag, reps=50)
+                    lbytes, 2.0 * E * K * M, tag, reps=50, gather=rows)
                 # the same layer by its two implementations: the operator pair over an
                 # (E, M) message tensor, and the single pass over destination tiles
                 v["ops"][f"rgcn_layer_{K}_{M}_two_pass"] = op_record(
                     f"c3.rgcn_layer_{K}_{M}_two_pass_{tag}",
                     lambda: layers.rgcn_layer(g, xin, w, norm, fused="pair"),
-                    lbytes + 2 * E * M * b, 2.0 * E * K * M, tag, reps=50)
+                    lbytes + 2 * E * M * b, 2.0 * E * K * M, tag, reps=50, gather=rows)
                 v["ops"][f"rgcn_layer_{K}_{M}_tiles"] = op_record(
                     f"c3.rgcn_layer_{K}_{M}_tiles_{tag}",
                     lambda: layers.rgcn_layer(g, xin, w, norm, fused="tiles"),
-                    lbytes, 2.0 * E * K * M, tag, reps=50)
+                    lbytes, 2.0 * E * K * M, tag, reps=50, gather=rows)
                 if args.no_ops:
                     continue
                 v["ops"][f"segment_mm_gather_{K}_{M}"] = op_record(
                     f"c3.segment_mm_gather_{K}_{M}_{tag}",
                     lambda: ops.SegmentMMEdgeGather(xin, w, 0, g, row_scale=norm),
-                    E * (8 + 4 + (K + M) * b) + R * K * M * b, 2.0 * E * K * M, tag, reps=50)
+                    E * (8 + 4 + (K + M) * b) + R * K * M * b, 2.0 * E * K * M, tag, reps=50,
+                    gather=rows)
                 xe = rnd(E, K, dtype=dt)
                 v["ops"][f"segment_mm_edge_{K}_{M}"] = op_record(
                     f"c3.segment_mm_edge_{K}_{M}_{tag}", lambda: ops.SegmentMMEdge(xe, w, g),
@@ -394,10 +509,12 @@ def main():
                 v["ops"][f"spmm_copy_e_{M}"] = op_record(
                     f"c3.spmm_copy_e_{M}_{tag}", lambda: ops.SpMMEdge(m, [1], False, None, g),
                     4 * (N + 1) + E * (4 + 4 + M * b) + N * M * b, reps=50)
+            v["ops"] = kept(v["ops"])
             rec["variants"][tag] = v
-        dom = rec["variants"]["f32"]["ops"]["rgcn_layer_16_64"]
-        rec["roofline"] = dict(dom, kernel="rgcn_layer 16->64 fp32 (one pass over destination tiles: "
-                                           "typed product and neighbour sum on the matrix cores)")
+        dom = rec["variants"]["f32"]["ops"].get("rgcn_layer_16_64")
+        if dom is not None:
+            rec["roofline"] = dict(dom, kernel="rgcn_layer 16->64 fp32 (one pass over destination tiles: "
+                                               "typed product and neighbour sum on the matrix cores)")
         return rec
 
     # ------------------------------------------------------------------ c4 ----
@@ -421,11 +538,12 @@ def main():
         def layer():
             return layers.hgt_layer(g, X, wk, wq, wv, wa, ra, rm, rp, skip, H, fused=True)
 
-        ms_step, _ = wall_time(layer, max(args.steps, 50), max(args.warmup, 5))
+        ms_step, _ = wall_time(layer, max(args.steps, 50), max(args.warmup, 5), key="c4.step")
         rec = {"workload": "configs[3]: 1-layer HGT, 4 node types 40k/30k/20k/10k, 10 edge types, 8 heads "
                            "x 16, hidden 128, bf16 with fp32 accumulation; power-law out-degree, seed 3",
                "num_nodes": N, "num_edges": E, "dtype": "bf16",
-               "ms_per_step": round(ms_step, 4), "edges_per_s": round(E / (ms_step * 1e-3), 1)}
+               "ms_per_step": r4(ms_step), "edges_per_s": per_s(E, ms_step)}
+        rows = N * hid * b                   # one (N, 128) bf16 table: 25.6 MB
         # bytes of the layer with its relation products per edge: h in, K/V/Q/t/out node rows,
         # three gathered rows per edge, the transformed values written and read once, scores
         # written and read once
@@ -443,18 +561,20 @@ def main():
         rec["num_pairs"] = P
         rec["relation_products"] = "per (destination, relation) pair" if by_pairs else "per edge"
         opsr = {"hgt_layer": op_record("c4.hgt_layer", layer, pairs_bytes if by_pairs else edges_bytes,
-                                       pairs_flops if by_pairs else edges_flops, "bf16")}
+                                       pairs_flops if by_pairs else edges_flops, "bf16",
+                                       gather=(3 * rows, E * 3 * hid * b))}
         if not args.no_ops:
             opsr["hgt_layer_per_edge"] = op_record(
                 "c4.hgt_layer_per_edge",
                 lambda: layers.hgt_layer(g, X, wk, wq, wv, wa, ra, rm, rp, skip, H, fused="edges"),
-                edges_bytes, edges_flops, "bf16")
+                edges_bytes, edges_flops, "bf16", gather=(3 * rows, E * 3 * hid * b))
             kk, vv, qq = ops.SegmentMMNodeStacked(X, [wk, wv, wq], g)
             opsr["relation_pair_attention"] = op_record(
                 "c4.relation_pair_attention",
                 lambda: ops.relation_pair_attention(kk, qq, vv, ra, rm, rp.float(), g,
                                                     factor=1.0 / D ** 0.5),
-                pairs_bytes - N * hid * b * 6, pairs_flops - 2.0 * N * hid * hid * 4, "bf16")
+                pairs_bytes - N * hid * b * 6, pairs_flops - 2.0 * N * hid * hid * 4, "bf16",
+                gather=(3 * rows, E * 3 * hid * b))
             opsr["segment_mm_node_128_128"] = op_record(
                 "c4.segment_mm_node", lambda: ops.SegmentMMNode(X, wk, g),
                 N * 2 * hid * b + Tn * hid * hid * b, 2.0 * N * hid * hid, "bf16", reps=50)
@@ -464,14 +584,16 @@ def main():
                 N * 4 * hid * b + 3 * Tn * hid * hid * b, 3 * 2.0 * N * hid * hid, "bf16", reps=50)
             opsr["segment_mm_dot_8x16x16"] = op_record(
                 "c4.segment_mm_dot", lambda: ops.SegmentMMEdgeDot(X, ra, 0, X, 1, g),
-                E * (16 + 2 * hid * b + 4 * H) + Te * H * D * D * b, 2.0 * E * H * D * D, "bf16", reps=50)
+                E * (16 + 2 * hid * b + 4 * H) + Te * H * D * D * b, 2.0 * E * H * D * D, "bf16", reps=50,
+                gather=(rows, E * 2 * hid * b))
             opsr["segment_mm_gather_8x16x16"] = op_record(
                 "c4.segment_mm_gather", lambda: ops.SegmentMMEdgeGather(X, rm, 0, g),
-                E * (8 + 2 * hid * b) + Te * H * D * D * b, 2.0 * E * H * D * D, "bf16", reps=50)
+                E * (8 + 2 * hid * b) + Te * H * D * D * b, 2.0 * E * H * D * D, "bf16", reps=50,
+                gather=(rows, E * hid * b))
             q, k = rnd(N, H, D, dtype=dt), rnd(N, H, D, dtype=dt)
             opsr["sddmm_u_dot_v"] = op_record(
                 "c4.sddmm_u_dot_v", lambda: ops.gsddmm_u_dot_v(k, q, g),
-                4 * (N + 1) + E * (4 + 2 * H * D * b + 4 * H), reps=50)
+                4 * (N + 1) + E * (4 + 2 * H * D * b + 4 * H), reps=50, gather=(2 * rows, E * 2 * hid * b))
             lg = rnd(E, H)
             opsr["segment_softmax"] = op_record(
                 "c4.segment_softmax", lambda: ops.SegmentSoftmax(lg, 1, None, g),
@@ -479,21 +601,95 @@ def main():
             att, v = torch.rand(E, H, device=dev), rnd(N, hid, dtype=dt)
             opsr["spmm_u_mul_e"] = op_record(
                 "c4.spmm_u_mul_e", lambda: ops.gspmm_src_mul_e_sum(v, att, [1], False, None, g),
-                4 * (N + 1) + E * (4 + 4 * H + hid * b) + N * hid * b, reps=50)
+                4 * (N + 1) + E * (4 + 4 * H + hid * b) + N * hid * b, reps=50, gather=(rows, E * hid * b))
             ve = rnd(E, hid, dtype=dt)
             opsr["edge_softmax_sum"] = op_record(
                 "c4.edge_softmax_sum", lambda: ops.edge_softmax_sum(lg, ve, g),
                 4 * (N + 1) + E * (4 + 4 + 4 * H + hid * b) + N * hid * b, reps=50)
-        rec["ops"] = opsr
-        rec["roofline"] = dict(opsr["hgt_layer"], kernel="hgt_layer (3 node projections, relation "
-                               "products " + rec["relation_products"] + ", dot-product scores, edge "
-                               "softmax, weighted sum of gathered values, output projection)")
+        rec["ops"] = opsr = kept(opsr)
+        if "hgt_layer" in opsr:
+            rec["roofline"] = dict(opsr["hgt_layer"], kernel="hgt_layer (3 node projections, relation "
+                                   "products " + rec["relation_products"] + ", dot-product scores, edge "
+                                   "softmax, weighted sum of gathered values, output projection)")
+        if "segment_mm_node_qkv_128_3x128" in opsr:
+            rec["mfma"] = dict(opsr["segment_mm_node_qkv_128_3x128"], kernel="K | Q | V projections 128 -> "
+                               "3 x 128 bf16 (wide_mm_kernel, v_mfma_f32_16x16x32_bf16)")
         return rec
 
-    runners = {"c2": run_c2, "c3": run_c3, "c4": run_c4, "c5": run_c5}
+    # ------------------------------------------------------------------ c1 ----
+    def run_c1():
+        """configs[0]: the configuration the list assigns to the host cores (the reference's
+        DGL CPU path, examples/GCN/GCN_DGL.py:11-14; DGL is not installed, so the host leg is
+        the C port of SpMMSrc + torch-CPU products) with the same network on the GPU beside it."""
+        nonlocal cpu
+        wl = datasets.gcn_uniform()                         # seed 0
+        N, E = wl.num_nodes, wl.num_edges
+        g = prepare_graph(wl.src, wl.dst, N, device=dev)
+        g.in_row_of_slot
+        rng = np.random.default_rng(0)
+        x_h = rng.standard_normal((N, 500), dtype=np.float32)
+        w1_h, w2_h = datasets.glorot(rng, (500, 16)), datasets.glorot(rng, (16, 3))
+        deg = np.bincount(wl.dst, minlength=N).astype(np.float32)     # in-degree, self loop included
+        norm_h = (1.0 / np.sqrt(deg)).astype(np.float32)[:, None]     # symmetric normalisation
+        x, w1, w2, norm = (torch.from_numpy(t).to(dev) for t in (x_h, w1_h, w2_h, norm_h))
+
+        def network():
+            h1 = layers.gcn_layer(g, x, w1, norm, norm, relu=True)
+            return layers.gcn_layer(g, h1, w2, norm, norm, relu=False)
+
+        ms_step, out = wall_time(network, max(args.steps, 100), max(args.warmup, 10), key="c1.step")
+        rec = {"workload": "configs[0]: 2-layer GCN 500->16->3 with ReLU, symmetric degree normalisation, "
+                           "fp32; uniform random graph (seed 0) + self loops",
+               "num_nodes": N, "num_edges": E, "dtype": "f32",
+               "ms_per_step": r4(ms_step), "edges_per_s": per_s(2 * E, ms_step)}
+        opsr = {}
+        for F_ in (16, 3):
+            m = rnd(N, F_)
+            opsr[f"spmm_copy_u_{F_}"] = op_record(
+                f"c1.spmm_copy_u_{F_}", lambda: ops.SpMMSrc(m, [1], False, None, g),
+                4 * (N + 1) + E * (4 + F_ * 4) + N * F_ * 4, reps=100, gather=(N * F_ * 4, E * F_ * 4))
+        opsr["linear_500_16"] = op_record(
+            "c1.linear_500_16", lambda: ops.linear(x, w1), 4 * (N * 500 + 500 * 16 + N * 16), reps=100)
+        rec["ops"] = opsr = kept(opsr)
+        if "spmm_copy_u_16" in opsr:
+            rec["roofline"] = dict(opsr["spmm_copy_u_16"],
+                                   kernel="SpMMSrc copy_u sum, F = 16 (runs_kernel<SpmmPolicy<float, 4>> + fix-up)")
+        if not args.no_cpu_baseline:
+            import oracle
+            ptr = g.in_pointer.cpu().numpy()
+            nbr = g.in_node_indices.cpu().numpy()
+            xt, w1t, w2t, nt = (torch.from_numpy(t) for t in (x_h, w1_h, w2_h, norm_h))
+
+            def cpu_network():
+                m1 = (torch.mm(xt, w1t) * nt).numpy()
+                h1 = torch.relu(torch.from_numpy(oracle.spmm_sum_f32(ptr, nbr, None, m1, op="copy_u")) * nt)
+                m2 = (torch.mm(h1, w2t) * nt).numpy()
+                return oracle.spmm_sum_f32(ptr, nbr, None, m2, op="copy_u") * norm_h
+
+            cpu_ms, reps, ref = cpu_time(cpu_network, budget_s=3.0, min_reps=5, max_reps=200)
+            got = out.cpu().numpy()
+            host = {"value": round(2 * E / (cpu_ms * 1e-3), 1), "unit": "edges/s",
+                    "cores": oracle.num_threads(), "torch_threads": torch.get_num_threads(),
+                    "kind": "port", "ms_per_step": round(cpu_ms, 3), "passes": reps,
+                    "sample": f"the whole 2-layer network (2 x {E} edges): one warm-up pass, then the mean "
+                              f"of {reps} passes of the fp32 C port of SpMMSrc (OpenMP) + torch-CPU products",
+                    "max_rel_diff_vs_gpu": float(np.abs(got - ref).max() / np.abs(ref).max())}
+            rec["host_cores"] = host
+            if ms_step is not None:
+                rec["host_ms_over_gpu_ms"] = round(cpu_ms / ms_step, 1)
+            if headline == "c1":
+                cpu = host
+        return rec
+
+    runners = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4, "c5": run_c5}
     for c in wanted:
         results[c] = runners[c]()
         torch.cuda.empty_cache()
+
+    extra = {"profile_segments": segments} if args.markers else {}
+    if only:                    # a profiler run: the operators asked for, nothing else
+        print(json.dumps(dict({"only": sorted(only), "configs": results}, **extra)))
+        return
 
     head = results[headline]
     if headline == "c3":
@@ -502,19 +698,31 @@ def main():
     else:
         ms_step, eps, dtype = head["ms_per_step"], head["edges_per_s"], head["dtype"]
     roof = head["roofline"]
+    by_traffic = bool(roof.get("cache_served")) and roof.get("traffic") is not None
     roofline = {"kernel": roof["kernel"], "bound": "hbm",
-                "achieved": roof.get("traffic_GBps") if roof.get("cache_served") else roof["effective_GBps"],
+                "achieved": round(roof["frac"] * HBM_PEAK_GBS, 1) if by_traffic else roof["effective_GBps"],
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": roof["frac"],
+                "frac_basis": roof.get("frac_basis"),
                 "traffic": roof.get("traffic"),
-                "traffic_source": "profiles/hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
-                                  "separate runs; not measured in this run)",
+                "traffic_source": "profiles/hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over the "
+                                  "operator's own dispatches, separate runs; not measured in this run)",
                 "algorithmic_bytes": roof["algorithmic_bytes"], "launch_ms": roof["ms"],
                 "effective_GBps": roof["effective_GBps"],
                 "cache_served": bool(roof.get("cache_served", False)),
                 "peak_measured_copy_GBps": measured_copy}
+    # the matrix-core figure the metric names: the best-placed MFMA kernel of the headline
+    # configuration (else of any configuration measured in this run)
+    mf = head.get("mfma") or next((results[c]["mfma"] for c in wanted if "mfma" in results[c]), None)
+    if mf is not None:
+        roofline["mfma"] = {"kernel": mf["kernel"], "tflops": mf["mfma_tflops"],
+                            "peak_tflops": mf["mfma_peak_tflops"], "util": mf["mfma_util"],
+                            "ceiling_tflops": mf["ceiling_tflops"],
+                            "frac_of_ceiling": mf["frac_of_ceiling"],
+                            "ceiling": "min(dense bf16 MFMA peak, arithmetic intensity x 8 TB/s)",
+                            "launch_ms": mf["ms"]}
+    metric = {"c1": "GCN", "c2": "GAT", "c5": "GAT", "c3": "RGCN", "c4": "HGT"}[headline]
     line = {
-        "metric": "GAT layer fwd edges/s" if headline in ("c2", "c5") else
-                  ("RGCN layer fwd edges/s" if headline == "c3" else "HGT layer fwd edges/s"),
+        "metric": metric + " layer fwd edges/s",
         "value": eps, "unit": "edges/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step,
@@ -527,6 +735,7 @@ def main():
         "peak_measured_copy_GBps": measured_copy,
         "configs": results,
     }
+    line.update(extra)
     print(json.dumps(line))
 
 

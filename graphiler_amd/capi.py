@@ -81,6 +81,7 @@ SIGNATURES = {
                                    _int, _vp, _sz, _vp]),
     "ga_dot_attention_sum": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
                                     _i64, _i64, _int, _vp, _sz, _vp]),
+    "ga_gat_static_scratch_needed": (_i64, [_i64, _i64, _i64, _int, _int]),
     "ga_gat_aggregate_static": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
                                        _i64, _i64, ctypes.c_float, _int, _vp]),
     "ga_gat_aggregate": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,

@@ -351,7 +351,7 @@ int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const int32_t *nbr, const float *el, const float *er,
                const void *z, void *out, int64_t n_rows, int64_t n_edges,
                int heads, int dim, float slope, float *ws, hipStream_t stream,
-               size_t ws_bytes = SIZE_MAX, int act = GA_ACT_NONE) {
+               size_t ws_bytes = SIZE_MAX, int act = GA_ACT_NONE, size_t *size_only = nullptr) {
   typedef GatPolicy<T, VEC, MODE, SPREAD> P;
   const bool ids_vec = aligned(row_of_slot, 16) && (!nbr || aligned(nbr, 16));
   const int head_lanes = dim / VEC;
@@ -360,7 +360,7 @@ int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
     return GA_EUNSUPPORTED;
   typename P::Args args{nbr, el, er, (const T *)z, heads, dim, slope, ids_vec, head_lanes, 0, act};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges,
-                        heads * dim, ws, stream, ws_bytes);
+                        heads * dim, ws, stream, ws_bytes, size_only);
 }
 
 // The element type and lane layout ga_gat_aggregate runs for a shape, launched
@@ -369,26 +369,27 @@ int gat_aggregate_dispatch(const int32_t *pointer, const int32_t *row_of_slot,
                            const int32_t *nbr, const float *el, const float *er,
                            const void *z, void *out, int64_t n_rows, int64_t n_edges,
                            int heads, int dim, float slope, int dtype, float *ws,
-                           size_t ws_bytes, hipStream_t s, int act = GA_ACT_NONE) {
+                           size_t ws_bytes, hipStream_t s, int act = GA_ACT_NONE,
+                           size_t *size_only = nullptr) {
   const bool vec_ok = aligned(out, 16) && (!z || aligned(z, 16));
   if (dtype == GA_F32) {
     if (vec_ok && dim % 4 == 0)
       return launch_gat<float, 4>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
-                                  heads, dim, slope, ws, s, ws_bytes, act);
+                                  heads, dim, slope, ws, s, ws_bytes, act, size_only);
     if (heads == 1 && dim >= 3 && dim <= 256)   // rows that 16-byte accesses do not tile
       return launch_gat<float, 4, kGatNode, true>(pointer, row_of_slot, nbr, el, er, z, out,
-                                                  n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes, act);
+                                                  n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes, act, size_only);
     return launch_gat<float, 1>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
-                                heads, dim, slope, ws, s, ws_bytes, act);
+                                heads, dim, slope, ws, s, ws_bytes, act, size_only);
   }
   if (vec_ok && dim % 8 == 0)
     return launch_gat<bf16_t, 8>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
-                                 heads, dim, slope, ws, s, ws_bytes, act);
+                                 heads, dim, slope, ws, s, ws_bytes, act, size_only);
   if (heads == 1 && dim >= 3 && dim <= 256)
     return launch_gat<bf16_t, 4, kGatNode, true>(pointer, row_of_slot, nbr, el, er, z, out,
-                                                 n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes, act);
+                                                 n_rows, n_edges, 1, dim, slope, ws, s, ws_bytes, act, size_only);
   return launch_gat<bf16_t, 1>(pointer, row_of_slot, nbr, el, er, z, out, n_rows, n_edges,
-                               heads, dim, slope, ws, s, ws_bytes, act);
+                               heads, dim, slope, ws, s, ws_bytes, act, size_only);
 }
 
 // Argument checks shared by ga_gat_aggregate and ga_gat_aggregate_static
@@ -502,6 +503,22 @@ int ga_gat_aggregate_static(const int32_t *pointer, const int32_t *row_of_slot,
                                             (float *)ws, (size_t)GA_STATIC_SCRATCH_BYTES,
                                             (hipStream_t)stream);
   return lr == GA_EWORKSPACE ? GA_ESCRATCH : lr;
+}
+
+int64_t ga_gat_static_scratch_needed(int64_t n_edges, int64_t heads, int64_t dim, int dtype,
+                                     int rows_16_byte_aligned) {
+  if (n_edges < 0 || heads <= 0 || dim <= 0 || n_edges > 0x7fffffff ||
+      heads * dim > 0x7fffffff || (dtype != GA_F32 && dtype != GA_BF16))
+    return GA_EINVAL;
+  if (n_edges == 0) return 0;
+  // the dispatch itself, asked for the size of the layout it would launch: the two
+  // addresses below only carry the alignment and are never dereferenced
+  const void *row = (const void *)(uintptr_t)(rows_16_byte_aligned ? 16 : (dtype == GA_F32 ? 4 : 2));
+  size_t needed = 0;
+  const int rc = ga::gat_aggregate_dispatch(nullptr, nullptr, nullptr, nullptr, nullptr, row,
+                                            (void *)row, 1, n_edges, (int)heads, (int)dim, 0.0f,
+                                            dtype, nullptr, 0, nullptr, GA_ACT_NONE, &needed);
+  return rc == GA_OK ? (int64_t)needed : (int64_t)rc;
 }
 
 int ga_edge_softmax_sum(const int32_t *pointer, const int32_t *row_of_slot,

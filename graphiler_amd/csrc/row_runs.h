@@ -370,11 +370,13 @@ inline size_t runs_workspace_bytes(int64_t n_edges, int64_t feat,
 // `partial_bytes`: capacity of `partial`.  The launch needs two partial rows per
 // workgroup of the layout actually chosen (never more than runs_workspace_bytes)
 // and returns GA_EWORKSPACE, having launched nothing, when that does not fit.
+// With `size_only` the call only stores that byte count there (host arithmetic,
+// no pointer is read, nothing is launched).
 template <class Policy>
 int launch_runs(typename Policy::Args args, const int32_t *pointer,
                 const int32_t *row_of_slot, void *out, int64_t n_rows,
                 int64_t n_edges, int feat, float *partial, hipStream_t stream,
-                size_t partial_bytes = SIZE_MAX) {
+                size_t partial_bytes = SIZE_MAX, size_t *size_only = nullptr) {
   constexpr int VEC = Policy::kVec;
   constexpr int SF = Policy::kState;
   RunGeom geo;
@@ -395,8 +397,12 @@ int launch_runs(typename Policy::Args args, const int32_t *pointer,
   geo.n_wg = n_wg;
   typedef typename Policy::out_t out_t;
   if (n_wg + row_blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-  if ((size_t)n_wg * 2 * (size_t)geo.lanes_total * SF * sizeof(float) > partial_bytes)
-    return GA_EWORKSPACE;
+  const size_t needed = (size_t)n_wg * 2 * (size_t)geo.lanes_total * SF * sizeof(float);
+  if (size_only) {          // sizing query: report the bytes of this layout, launch nothing
+    *size_only = needed;
+    return GA_OK;
+  }
+  if (needed > partial_bytes) return GA_EWORKSPACE;
   if (n_wg > 0) {
     const size_t lds = (size_t)kBlock * 2 * SF * sizeof(float);
     hipLaunchKernelGGL((runs_kernel<Policy>), dim3((unsigned)(n_wg + row_blocks), ftiles),

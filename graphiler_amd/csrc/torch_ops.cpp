@@ -140,7 +140,7 @@ struct DGLGraph : torch::CustomClassHolder {
     bool identity = false;
     bool ready = false;
   };
-  const Side &side(bool reverse) {
+  Side side(bool reverse) {
     std::lock_guard<std::mutex> lock(mu_);
     Side &s = reverse ? out_side_ : in_side_;
     if (!s.ready) {
@@ -163,8 +163,12 @@ struct DGLGraph : torch::CustomClassHolder {
     int64_t tile_rows = 128;
     bool ready = false;
   };
-  const TypedTiles &typed_tiles() {
-    const Side &in = side(false);
+  // Returned by value (tensor handles are reference counted): a SetEtypePointer that
+  // runs while an operator still uses the layout drops the graph's copy, not the
+  // operator's.  Setters must still not run concurrently with operators on one graph
+  // object: the operator would read the counts and the type pointer of two states.
+  TypedTiles typed_tiles() {
+    const Side in = side(false);
     std::lock_guard<std::mutex> lock(mu_);
     if (!tiles_.ready) {
       TORCH_CHECK(etype_pointer.has_value(), "the graph has no edge type pointer");
@@ -207,8 +211,8 @@ struct DGLGraph : torch::CustomClassHolder {
     bool valid = false;
     bool ready = false;
   };
-  const RelationPairs &relation_pairs() {
-    const Side &in = side(false);
+  RelationPairs relation_pairs() {   // by value, like typed_tiles()
+    const Side in = side(false);
     std::lock_guard<std::mutex> lock(mu_);
     if (!pairs_.ready) {
       pairs_.ready = true;

@@ -56,10 +56,7 @@ def dedup(graph: torch._C.Graph) -> None:
                 known[key] = n.output()
     torch._C._jit_pass_cse(graph)
 
-    def mutated(v) -> bool:
-        return any(u.user.kind().endswith("_") or u.user.kind() == "aten::_set_item"
-                   for u in v.uses())
-
+    mutated = _mutated
     changed = True
     while changed:
         changed = False
@@ -91,6 +88,12 @@ def dedup(graph: torch._C.Graph) -> None:
             else:
                 seen[key] = n
     torch._C._jit_pass_dce(graph)
+
+
+def _mutated(v) -> bool:
+    """True when an in-place operator (aten::*_) or a dictionary store uses ``v``."""
+    return any(u.user.kind().endswith("_") or u.user.kind() == "aten::_set_item"
+               for u in v.uses())
 
 
 class _Rewriter:
@@ -727,6 +730,10 @@ class _Rewriter:
                 groups.setdefault(n.inputsAt(0).unique(), []).append(n)
         changed = False
         for nodes in groups.values():
+            # an input or a result that an in-place operator overwrites somewhere is not
+            # one value over the whole group: such products stay where they are
+            nodes = [n for n in nodes if not (_mutated(n.inputsAt(0)) or _mutated(n.inputsAt(1))
+                                              or _mutated(n.output()))]
             nodes = nodes[:4]
             while len(nodes) >= 2:
                 last = nodes[-1]

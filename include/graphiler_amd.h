@@ -395,9 +395,14 @@ int ga_gat_aggregate(const int32_t *pointer, const int32_t *row_of_slot,
  * file-scope array: every GPU the library runs on keeps it until the process
  * ends).  The call allocates nothing and calls no allocating routine.
  *   - GA_ESCRATCH (nothing launched) when the graph and width need more partial
- *     rows than the buffer holds: 2 rows of heads*dim features (x 1.25 - 1.5 for
- *     the softmax state) per workgroup; 64.3 M edges x 256 bf16 features need
- *     20 MB, 11.6 M edges x 64 fp32 features 4.3 MB.
+ *     rows than the buffer holds: 2 rows of heads*dim features per workgroup, with
+ *     the softmax state beside every feature: x 1.5 for 16-byte lanes of fp32
+ *     (4 features + maximum + denominator per lane), x 1.25 for 16-byte lanes of
+ *     bf16 (8 features), and x 3 for rows that 16-byte accesses do not tile with
+ *     several heads (one feature per lane, each with its own maximum and
+ *     denominator).  64.3 M edges x 256 bf16 features need 20 MB, 11.6 M edges x
+ *     64 fp32 features 4.3 MB.  ga_gat_static_scratch_needed gives the exact
+ *     figure for a shape without touching the device.
  *   - All calls on one GPU share that GPU's buffer: calls that overlap on one
  *     GPU (two streams, two threads) race; calls on one stream are ordered.
  *   - The first call on a device looks the buffer's address up
@@ -410,6 +415,15 @@ int ga_gat_aggregate_static(const int32_t *pointer, const int32_t *row_of_slot,
                             const void *z, void *out, int64_t n_rows, int64_t n_edges,
                             int64_t heads, int64_t dim, float slope, int dtype,
                             ga_stream_t stream);
+
+/* Host arithmetic only (no device call, no pointer read): the bytes of the static
+ * buffer that ga_gat_aggregate_static uses for a graph of n_edges edges and rows of
+ * heads x dim values of `dtype`, stored at 16-byte aligned addresses or not (the
+ * lane layout depends on it).  The call fits when the result is at most
+ * GA_STATIC_SCRATCH_BYTES.  Negative: a GA_E* code for arguments the entry point
+ * would reject.  No counterpart in the reference. */
+int64_t ga_gat_static_scratch_needed(int64_t n_edges, int64_t heads, int64_t dim, int dtype,
+                                     int rows_16_byte_aligned);
 
 /* The same chain with the source term recomputed from the gathered row:
  *   s_i = leaky_relu(<z[nbr[i], h, :], a_l[h, :]> + er[v, h], slope)

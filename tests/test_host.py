@@ -203,3 +203,29 @@ def test_bcast_dot_and_plain_shapes():
     got = [(u.reshape(-1, 16)[b.lhs_offset[k]] * v.reshape(-1, 16)[b.rhs_offset[k]]).sum()
            for k in range(b.out_len)]
     np.testing.assert_allclose(got, (u * v).sum(-1))
+
+
+def test_static_scratch_sizing_query_without_gpu():
+    """ga_gat_static_scratch_needed is host arithmetic: the sizes quoted beside the entry
+    point's declaration, the three state layouts (x 1.5 fp32 lanes of four, x 1.25 bf16
+    lanes of eight, x 3 one feature per lane), never above the workspace bound of
+    ga_gat_aggregate, and the refusal of what the 32 MiB buffer cannot hold."""
+    lib = capi.load()
+    cap = 32 << 20
+    need = lib.ga_gat_static_scratch_needed
+    assert need(0, 1, 64, capi.GA_F32, 1) == 0
+    assert need(-1, 1, 64, capi.GA_F32, 1) == capi.GA_EINVAL
+    assert need(10, 0, 64, capi.GA_F32, 1) == capi.GA_EINVAL
+    assert need(10, 1, 64, 99, 1) == capi.GA_EINVAL
+    c5 = need(64_308_169, 4, 64, capi.GA_BF16, 1)
+    c2 = need(11_600_000, 1, 64, capi.GA_F32, 1)
+    assert 15e6 < c5 <= cap and 3e6 < c2 <= cap
+    e = 4_000_000
+    a4 = need(e, 4, 16, capi.GA_F32, 1)           # lanes of four fp32 features
+    a8 = need(e, 4, 16, capi.GA_BF16, 1)          # lanes of eight bf16 features
+    s1 = need(e, 4, 16, capi.GA_F32, 0)           # unaligned rows, several heads: scalar lanes
+    assert 0 < a8 < a4 < s1            # 6 floats per 4 features, 10 per 8, 3 per feature
+    for heads, dim, dt, al in ((4, 16, capi.GA_F32, 1), (4, 16, capi.GA_BF16, 1), (4, 16, capi.GA_F32, 0),
+                               (1, 17, capi.GA_F32, 1), (3, 5, capi.GA_BF16, 0), (1, 200, capi.GA_BF16, 1)):
+        assert 0 < need(e, heads, dim, dt, al) <= lib.ga_gat_workspace_bytes(e, heads * dim, heads)
+    assert need(2_000_000_000, 1, 4096, capi.GA_F32, 1) > cap

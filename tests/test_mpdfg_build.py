@@ -213,3 +213,37 @@ def test_typed_product_and_dot_fuse_only_without_row_factor_and_heads():
     heads = _DOT_PLAN.replace("WTYPE", "Float(4, 2, 16, 8)").replace("SCALE", "%none")
     assert sorted(_late_fused_kinds(heads)) == ["my_ops::BroadcastDstNode",
                                                 "my_ops::SegmentMMEdgeGather"]
+
+
+def test_stacked_products_skip_operands_overwritten_in_place():
+    """Two SegmentMMNode of one x with an in-place operator on x between them are two
+    products of two different values: they must not become one stacked product placed
+    after the overwrite.  Without the overwrite the same graph does stack."""
+    from types import SimpleNamespace
+
+    from graphiler_amd.mpdfg import passes
+
+    def build(inplace):
+        g = torch._C.Graph()
+        dgl = g.addInput()
+        x, w1, w2 = (g.addInput() for _ in range(3))
+        for v in (x, w1, w2):
+            v.setType(torch._C.TensorType.get())
+        a = g.create("my_ops::SegmentMMNode", [x, w1, dgl], 1)
+        g.appendNode(a)
+        if inplace:
+            m = g.create("aten::relu_", [x], 1)
+            g.appendNode(m)
+        b = g.create("my_ops::SegmentMMNode", [x, w2, dgl], 1)
+        g.appendNode(b)
+        s = g.create("aten::add", [a.output(), b.output(), g.insertConstant(1)], 1)
+        g.appendNode(s)
+        g.registerOutput(s.output())
+        rw = passes._Rewriter(SimpleNamespace(graph=g, residency={}))
+        changed = rw._fuse_stacked_mm()
+        return changed, [n.kind() for n in g.nodes()]
+
+    changed, kinds = build(inplace=False)
+    assert changed and kinds.count("my_ops::SegmentMMNodeStacked") == 1
+    changed, kinds = build(inplace=True)
+    assert not changed and kinds.count("my_ops::SegmentMMNode") == 2

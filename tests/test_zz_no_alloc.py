@@ -66,20 +66,29 @@ def test_static_scratch_matches_workspace_entry_point(device, feat, heads, dtype
             f"call {i}: static-scratch result differs from the workspace entry point"
 
 
-def test_static_scratch_rejects_what_does_not_fit(device):
-    """A graph whose partial rows exceed the buffer is refused before anything is
-    launched: the output keeps its fill value.  Sizes only: the arrays the call would
-    read are far smaller than the counts claim, so a launch would be a bug."""
+def test_static_scratch_sizing_query_matches_the_entry_point(device):
+    """ga_gat_static_scratch_needed (host arithmetic) says exactly when the entry point
+    refuses: on real arrays, a width whose partial rows exceed the buffer gives
+    GA_ESCRATCH with the output untouched, and the widest one that fits runs."""
     lib = capi.load()
-    n, e, feat = 1000, 2_000_000_000, 4096
-    ptr = torch.zeros(n + 1, dtype=torch.int32, device=device)
-    col = torch.zeros(16, dtype=torch.int32, device=device)
-    t = torch.zeros(n, feat, device=device)
-    out = torch.full((n, feat), 7.0, device=device)
-    rc = lib.ga_gat_aggregate_static(ptr.data_ptr(), col.data_ptr(), col.data_ptr(), t.data_ptr(),
-                                     t.data_ptr(), t.data_ptr(), out.data_ptr(), n, e, 1, feat,
-                                     0.2, capi.GA_F32, torch.cuda.current_stream(device).cuda_stream)
-    torch.cuda.synchronize()
-    assert rc == capi.GA_ESCRATCH
-    assert b"static scratch" in lib.ga_error_string(rc)
-    assert bool((out == 7.0).all())
+    wl = datasets.gat_rmat(num_nodes=2_000, n_edges=1_200_000, scale=11, seed=5)
+    g = prepare_graph(wl.src, wl.dst, wl.num_nodes, device=device)
+    cap = 32 << 20
+    heads = 3                       # several heads of an odd width: one feature per lane
+    fits = [d for d in range(1, 4000, 2)
+            if lib.ga_gat_static_scratch_needed(g.num_edges, heads, d, capi.GA_F32, 1) <= cap]
+    assert fits and fits[-1] < 3999, "the sweep must cross the buffer's size"
+    for dim, want in ((fits[-1], capi.GA_OK), (fits[-1] + 2, capi.GA_ESCRATCH)):
+        el, er, z = _inputs(dim, wl.num_nodes, heads * dim, heads, torch.float32, device)
+        out = torch.full_like(z, 7.0)
+        rc = _call("static", g, el, er, z, out, heads, 0.2)
+        assert rc == want, (dim, lib.ga_error_string(rc))
+        if want == capi.GA_OK:
+            ws = torch.empty(lib.ga_gat_workspace_bytes(g.num_edges, heads * dim, heads),
+                             dtype=torch.uint8, device=device)
+            ref = torch.empty_like(z)
+            assert _call("workspace", g, el, er, z, ref, heads, 0.2, ws) == capi.GA_OK
+            assert torch.equal(out, ref)
+        else:
+            assert b"static scratch" in lib.ga_error_string(rc)
+            assert bool((out == 7.0).all())
