@@ -204,6 +204,22 @@ template <> struct BufLoad<1> {
   }
 };
 
+// ---- activations applied to fp32 rows before they are rounded and stored ----
+
+// elu with alpha = 1 (torch.nn.functional.elu computes expm1 for x <= 0).  exp(x) - 1
+// loses its leading digits near zero, so a short series takes over above -1/8: its
+// first dropped term is x^7 / 5040, below 2^-24 |x| there; below -1/8 the result is at
+// least 0.117 in magnitude and the rounding of exp (about 1e-7) is under 1e-6 of it.
+__device__ __forceinline__ float elu(float x) {
+  const float e = __expf(x) - 1.0f;
+  const float p = x * (1.0f + x * (0.5f + x * (1.0f / 6 + x * (1.0f / 24 + x * (1.0f / 120 + x * (1.0f / 720))))));
+  const float neg = x > -0.125f ? p : e;
+  return x > 0.0f ? x : neg;          // NaN: the comparisons fail, neg = e = NaN
+}
+__device__ __forceinline__ float relu_keep_nan(float x) {
+  return x > 0.0f ? x : (x != x ? x : 0.0f);
+}
+
 // ---- host side -----------------------------------------------------------
 
 inline int ilog2_floor(uint64_t x) {

@@ -56,7 +56,13 @@ __device__ __forceinline__ float lanes_sum(float v, int lanes) {
 
 // SPREAD: the lane's features lie a lane-group width apart (rows that 16-byte
 // accesses do not tile); they share the lane's one (m, l) pair, i.e. one head.
-template <typename T, int VEC, int MODE = kGatNode, bool SPREAD = false>
+// ACT: the activation compiled into the row store (GA_ACT_RELU / GA_ACT_ELU), or
+// kActRuntime = the one named by Args::act (the less common lane layouts; one build
+// for all three).  The compiled-in forms keep the dead branches out of the kernel:
+// the store sits at five places of the run loop, under divergence, so its length is
+// paid once per closed row and wavefront, not per element.
+constexpr int kActRuntime = -1;
+template <typename T, int VEC, int MODE = kGatNode, bool SPREAD = false, int ACT = kActRuntime>
 struct GatPolicy {
   static constexpr bool EDGE = MODE == kGatEdge;
   typedef T out_t;
@@ -102,7 +108,8 @@ struct GatPolicy {
   }
   static __device__ __forceinline__ void emit(const Args &A, out_t *out, int64_t row, int feat,
                                               int f0, const float (&st)[kState]) {
-    if (A.act == GA_ACT_NONE) {
+    const int act = ACT == kActRuntime ? A.act : ACT;
+    if (act == GA_ACT_NONE) {
       emit_row<GatPolicy>(out, row, feat, f0, st, A.stride_shift);
       return;
     }
@@ -112,8 +119,7 @@ struct GatPolicy {
     float o[VEC];
     finish(st, o);
 #pragma unroll
-    for (int v = 0; v < VEC; ++v)
-      o[v] = o[v] > 0.0f ? o[v] : (A.act == GA_ACT_ELU ? expm1f(o[v]) : (o[v] != o[v] ? o[v] : 0.0f));
+    for (int v = 0; v < VEC; ++v) o[v] = act == GA_ACT_ELU ? elu(o[v]) : relu_keep_nan(o[v]);
     IO::store(out + row * feat + f0, o, IO::lane(A.stride_shift, feat - f0));
   }
   static __device__ __forceinline__ void emit_empty(const Args &A, out_t *out, int64_t row,
@@ -346,13 +352,28 @@ int launch_dot_attn(const int32_t *pointer, const int32_t *row_of_slot, const in
                         stream, ws_bytes);
 }
 
-template <typename T, int VEC, int MODE = kGatNode, bool SPREAD = false>
+template <typename T, int VEC, int MODE = kGatNode, bool SPREAD = false, int ACT = kActRuntime>
 int launch_gat(const int32_t *pointer, const int32_t *row_of_slot,
                const int32_t *nbr, const float *el, const float *er,
                const void *z, void *out, int64_t n_rows, int64_t n_edges,
                int heads, int dim, float slope, float *ws, hipStream_t stream,
                size_t ws_bytes = SIZE_MAX, int act = GA_ACT_NONE, size_t *size_only = nullptr) {
-  typedef GatPolicy<T, VEC, MODE, SPREAD> P;
+  // the 16-byte lane layouts of the node forms (every benchmarked shape) get a build per
+  // activation; everything else reads it from the arguments
+  if constexpr (ACT == kActRuntime && !SPREAD && MODE != kGatEdge && VEC > 1) {
+    if (act == GA_ACT_NONE)
+      return launch_gat<T, VEC, MODE, SPREAD, GA_ACT_NONE>(pointer, row_of_slot, nbr, el, er, z, out,
+                                                           n_rows, n_edges, heads, dim, slope, ws,
+                                                           stream, ws_bytes, act, size_only);
+    if (act == GA_ACT_RELU)
+      return launch_gat<T, VEC, MODE, SPREAD, GA_ACT_RELU>(pointer, row_of_slot, nbr, el, er, z, out,
+                                                           n_rows, n_edges, heads, dim, slope, ws,
+                                                           stream, ws_bytes, act, size_only);
+    return launch_gat<T, VEC, MODE, SPREAD, GA_ACT_ELU>(pointer, row_of_slot, nbr, el, er, z, out,
+                                                        n_rows, n_edges, heads, dim, slope, ws, stream,
+                                                        ws_bytes, act, size_only);
+  }
+  typedef GatPolicy<T, VEC, MODE, SPREAD, ACT> P;
   const bool ids_vec = aligned(row_of_slot, 16) && (!nbr || aligned(nbr, 16));
   const int head_lanes = dim / VEC;
   if (MODE == kGatFromZ &&

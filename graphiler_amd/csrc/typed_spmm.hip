@@ -348,7 +348,7 @@ __device__ __forceinline__ bool is_finite(float v) {
 }
 
 __device__ __forceinline__ float activated(float o, int act) {
-  return o > 0.0f ? o : (act == GA_ACT_ELU ? expm1f(o) : (o != o ? o : 0.0f));
+  return act == GA_ACT_ELU ? elu(o) : relu_keep_nan(o);
 }
 
 __device__ __forceinline__ void store_row4(float *p, const float4 &v) {
