@@ -77,6 +77,10 @@ def main():
                          "only these, skip the network steps and the CPU legs (short profiler runs)")
     ap.add_argument("--reps", type=int, default=30, help="timed calls per operator")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--gather-ceiling", action="store_true",
+                    help="configs[4] only: also run its aggregation kernels on graphs with the same "
+                         "destinations and uniformly random sources over tables of several sizes (HBM, "
+                         "Infinity Cache, L2): what the memory system gives a gather of 512-byte rows")
     ap.add_argument("--no-ops", action="store_true",
                     help="time the layers only (shorter kernel traces for profiling)")
     ap.add_argument("--markers", "--calibrate-copy", dest="markers", action="store_true",
@@ -342,6 +346,27 @@ def main():
         if "project_attn_256_256" in opsr:
             rec["mfma"] = dict(opsr["project_attn_256_256"], kernel="project_attn 256 -> 256 bf16 "
                                "(wide_mm_kernel, v_mfma_f32_16x16x32_bf16)")
+
+        if args.gather_ceiling and not only:
+            # the same destinations, sources drawn uniformly from the first K rows of z: K = N
+            # misses every cache (the random-row rate of the HBM), 2^17 rows = 67 MB stay in the
+            # Infinity Cache, 2^13 rows = 4 MB in an L2 (what the kernel's own instructions allow)
+            ceil = {}
+            crng = np.random.default_rng(44)
+            for K in (N, 1 << 17, 1 << 13):
+                gk = prepare_graph(crng.integers(0, K, E), wl.dst, N, device=dev)
+                gk.in_row_of_slot
+                t_z = ev_time(lambda: ops.gat_aggregate_from_z(a_l, er1, z1, gk, slope), 10)
+                t_c = ev_time(lambda: ops.SpMMSrc(z1, [1], False, None, gk), 10)
+                ceil[f"uniform_sources_over_{K}_rows"] = {
+                    "table_MB": round(K * Fw * b / 1e6, 1),
+                    "gat_aggregate_from_z_ms": round(t_z, 4),
+                    "gat_aggregate_from_z_row_GBps": round(E * Fw * b / t_z / 1e6, 1),
+                    "spmm_copy_u_ms": round(t_c, 4),
+                    "spmm_copy_u_row_GBps": round(E * Fw * b / t_c / 1e6, 1)}
+                del gk
+                torch.cuda.empty_cache()
+            rec["gather_ceiling"] = ceil
 
         if headline == "c5" and not args.no_cpu_baseline:
             # one hidden layer (256 -> 256) of the same network on the host cores: the fp32
