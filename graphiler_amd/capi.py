@@ -64,7 +64,9 @@ SIGNATURES = {
                                   _vp, _sz, _vp]),
     "ga_segment_mm": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                              _int, _vp]),
+    "ga_segment_mm_gated": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
     "ga_transpose_scale_blocks": (_int, [_vp, _vp, ctypes.c_float, _vp, _i64, _i64, _int, _vp]),
+    "ga_transpose_scale_blocks_as": (_int, [_vp, _vp, _int, ctypes.c_float, _vp, _i64, _i64, _int, _vp]),
     "ga_segment_mm_stacked": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                      _int, _vp]),
     "ga_segment_mm_gather": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,

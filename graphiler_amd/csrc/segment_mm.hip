@@ -1002,7 +1002,8 @@ namespace {
 // wide_mm.hip reads X once for all of `n_w` weight tensors.  GA_EUNSUPPORTED: not its shape.
 int wide_typed(const int32_t *type_pointer, int64_t n_types, const void *X,
                const void *const *W, void *const *Y, int n_w, int64_t rows, int64_t K,
-               int64_t M, const float *row_scale, hipStream_t s) {
+               int64_t M, const float *row_scale, hipStream_t s, const float *type_gate = nullptr,
+               bool gate_sigmoid = false) {
   if (M % kWideGroupCols != 0 || n_types > 64) return GA_EUNSUPPORTED;
   const int per_w = (int)(M / kWideGroupCols);
   if (!wide_mm_fits((int)K, n_w * per_w)) return GA_EUNSUPPORTED;
@@ -1014,6 +1015,8 @@ int wide_typed(const int32_t *type_pointer, int64_t n_types, const void *X,
   p.K = (int)K;
   p.n_groups = n_w * per_w;
   p.row_scale = row_scale;
+  p.type_gate = type_gate;
+  p.gate_sigmoid = gate_sigmoid;
   for (int w = 0; w < n_w; ++w)
     for (int c = 0; c < per_w; ++c) {
       const int g = w * per_w + c;
@@ -1205,41 +1208,56 @@ extern "C" int ga_project_attn(const void *X, const void *W, const float *a_l,
 namespace ga {
 namespace {
 // out[b][j][i] = W[b][i][j] * scale[b] * factor over square blocks of D x D values
-template <typename T>
+template <typename T, typename S>
 __global__ __launch_bounds__(kBlock) void transpose_scale_blocks_kernel(
-    const T *__restrict__ W, const float *__restrict__ scale, float factor, T *__restrict__ out,
+    const T *__restrict__ W, const S *__restrict__ scale, float factor, T *__restrict__ out,
     int D, int64_t total) {
   const int64_t o = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (o >= total) return;
   const int i = (int)(o % D), j = (int)(o / D % D);
   const int64_t b = o / ((int64_t)D * D);
-  const float v = elem_to_f32(W[(b * D + i) * D + j]) * (scale ? scale[b] : 1.0f) * factor;
+  const float v = elem_to_f32(W[(b * D + i) * D + j]) * (scale ? elem_to_f32(scale[b]) : 1.0f) * factor;
   f32_to_elem(v, out[o]);
 }
 }  // namespace
 }  // namespace ga
 
-extern "C" int ga_transpose_scale_blocks(const void *W, const float *scale, float factor,
-                                         void *out, int64_t n_blocks, int64_t D, int dtype,
-                                         ga_stream_t stream) {
+extern "C" int ga_transpose_scale_blocks_as(const void *W, const void *scale, int scale_dtype,
+                                            float factor, void *out, int64_t n_blocks, int64_t D,
+                                            int dtype, ga_stream_t stream) {
   using namespace ga;
   if (n_blocks < 0 || D <= 0 || D > 0x7fff) return GA_EINVAL;
   if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  if (scale_dtype != GA_F32 && scale_dtype != GA_BF16) return GA_EINVAL;
   const int64_t total = n_blocks * D * D;
   if (total == 0) return GA_OK;
   if (!W || !out || W == out) return GA_EINVAL;
   const size_t esz = dtype == GA_F32 ? 4 : 2;
-  if (!aligned(W, esz) || !aligned(out, esz) || (scale && !aligned(scale, 4))) return GA_EALIGN;
+  if (!aligned(W, esz) || !aligned(out, esz) || (scale && !aligned(scale, scale_dtype == GA_F32 ? 4 : 2)))
+    return GA_EALIGN;
   const int64_t blocks = (total + kBlock - 1) / kBlock;
   if (blocks > 0x7fffffff) return GA_EUNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == GA_F32)
-    hipLaunchKernelGGL(transpose_scale_blocks_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0,
-                       s, (const float *)W, scale, factor, (float *)out, (int)D, total);
+  const dim3 grid((unsigned)blocks), block(kBlock);
+  if (dtype == GA_F32 && scale_dtype == GA_F32)
+    hipLaunchKernelGGL((transpose_scale_blocks_kernel<float, float>), grid, block, 0, s, (const float *)W,
+                       (const float *)scale, factor, (float *)out, (int)D, total);
+  else if (dtype == GA_F32)
+    hipLaunchKernelGGL((transpose_scale_blocks_kernel<float, bf16_t>), grid, block, 0, s, (const float *)W,
+                       (const bf16_t *)scale, factor, (float *)out, (int)D, total);
+  else if (scale_dtype == GA_F32)
+    hipLaunchKernelGGL((transpose_scale_blocks_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t *)W,
+                       (const float *)scale, factor, (bf16_t *)out, (int)D, total);
   else
-    hipLaunchKernelGGL(transpose_scale_blocks_kernel<bf16_t>, dim3((unsigned)blocks), dim3(kBlock),
-                       0, s, (const bf16_t *)W, scale, factor, (bf16_t *)out, (int)D, total);
+    hipLaunchKernelGGL((transpose_scale_blocks_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t *)W,
+                       (const bf16_t *)scale, factor, (bf16_t *)out, (int)D, total);
   return launch_status();
+}
+
+extern "C" int ga_transpose_scale_blocks(const void *W, const float *scale, float factor,
+                                         void *out, int64_t n_blocks, int64_t D, int dtype,
+                                         ga_stream_t stream) {
+  return ga_transpose_scale_blocks_as(W, scale, GA_F32, factor, out, n_blocks, D, dtype, stream);
 }
 
 extern "C" int ga_segment_mm(const int32_t *type_pointer, int64_t n_types,
@@ -1286,6 +1304,22 @@ extern "C" int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_type
     if (rc != GA_OK) return rc;
   }
   return GA_OK;
+}
+
+extern "C" int ga_segment_mm_gated(const int32_t *type_pointer, int64_t n_types, const void *X,
+                                   const void *W, void *Y, const float *gate, int gate_sigmoid,
+                                   int64_t rows, int64_t K, int64_t M, int dtype,
+                                   ga_stream_t stream) {
+  using namespace ga;
+  const int bad = check_mm_args(n_types, rows, 1, K, M, dtype);
+  if (bad != GA_OK) return bad;
+  if (rows == 0 || n_types == 0) return GA_OK;
+  if (!type_pointer || !X || !W || !Y || !gate) return GA_EINVAL;
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!aligned(X, esz) || !aligned(W, esz) || !aligned(Y, esz) || !aligned(gate, 4)) return GA_EALIGN;
+  if (dtype != GA_BF16) return GA_EUNSUPPORTED;
+  return wide_typed(type_pointer, n_types, X, &W, &Y, 1, rows, K, M, nullptr, (hipStream_t)stream,
+                    gate, gate_sigmoid != 0);
 }
 
 extern "C" int ga_segment_mm_gather(const int32_t *type_pointer, int64_t n_types,

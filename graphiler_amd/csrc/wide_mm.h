@@ -28,6 +28,8 @@ struct WideMm {
   const float *a_l[kWideMaxGroups], *a_r[kWideMaxGroups];
   float *el[kWideMaxGroups], *er[kWideMaxGroups];
   const float *row_scale;     // Y[r, :] of every group times row_scale[r]; null: 1 (not with a_l / a_r)
+  const float *type_gate;     // Y[r, :] times g(type_gate[type(r)]); null: 1 (not with a_l / a_r)
+  bool gate_sigmoid;          // g = 1 / (1 + exp(-x)) instead of the identity
   int64_t ldd;                // heads per row of el / er
   int dph;                    // columns per head: 32, 64 or 128
   bool w_wide;                // set by wide_mm_launch: rows of every W are 16-byte aligned

@@ -123,6 +123,12 @@ __global__ __launch_bounds__(kWideBlock) void wide_mm_kernel(WideMm p, int chunk
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int n = lane & 15, q = lane >> 4;
+  // factor of every row of this workgroup's type (HGT's sigmoid(skip[type]) gate)
+  float gate = 1.0f;
+  if (!ATTN && p.type_gate) {
+    const float v = p.type_gate[type];
+    gate = p.gate_sigmoid ? 1.0f / (1.0f + __expf(-v)) : v;
+  }
 
   // halves (4 elements) of this lane's k fragments that lie inside a row: bits 2 f, 2 f + 1
   unsigned kmask = 0;
@@ -181,7 +187,7 @@ __global__ __launch_bounds__(kWideBlock) void wide_mm_kernel(WideMm p, int chunk
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = rel + 16 * t + 4 * q + i;
-        rs[t][i] = !ATTN && p.row_scale ? p.row_scale[row0 + (r < nrows ? r : nrows - 1)] : 1.0f;
+        rs[t][i] = !ATTN && p.row_scale ? gate * p.row_scale[row0 + (r < nrows ? r : nrows - 1)] : gate;
       }
 #pragma unroll 1
     for (int g = 0; g < NG; ++g) {
@@ -208,7 +214,7 @@ __global__ __launch_bounds__(kWideBlock) void wide_mm_kernel(WideMm p, int chunk
         }
       }
       // lane (n, q) holds rows rel + 16 t + 4 q + i, columns 8 n .. 8 n + 7 of the group
-      if (!ATTN && p.row_scale) {
+      if (!ATTN && (p.row_scale || p.type_gate)) {
 #pragma unroll
         for (int t = 0; t < TW; ++t)
 #pragma unroll
@@ -362,6 +368,7 @@ int wide_mm_launch(const WideMm &p, hipStream_t s) {
   if (p.rows <= 0) return GA_OK;
   if (p.rows > 0x7fffffff || !aligned(p.X, p.K % 8 == 0 ? 16 : 8)) return GA_EUNSUPPORTED;
   if (p.row_scale && (!aligned(p.row_scale, 4) || p.a_l[0])) return GA_EUNSUPPORTED;
+  if (p.type_gate && (!aligned(p.type_gate, 4) || p.a_l[0])) return GA_EUNSUPPORTED;
   const bool attn = p.a_l[0] != nullptr;
   if (attn && p.dph != 32 && p.dph != 64 && p.dph != 128) return GA_EUNSUPPORTED;
   for (int g = 0; g < p.n_groups; ++g) {

@@ -179,8 +179,10 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
         if pairs is not None and (fused == "pairs"
                                   or e >= PAIRS_MIN_EDGES_PER_PAIR * pairs.num_pairs):
             try:
+                pri = relation_pri if relation_pri.dtype in (torch.float32, torch.bfloat16) \
+                    else relation_pri.float()
                 t = ops.relation_pair_attention(k, q, v, relation_att, relation_msg,
-                                                relation_pri.float().contiguous(), g,
+                                                pri.contiguous(), g,
                                                 factor=1.0 / (d ** 0.5))
             except capi.GraphilerError as err:      # head width outside the typed product
                 if err.code != capi.GA_EUNSUPPORTED or fused == "pairs":
@@ -199,8 +201,8 @@ def hgt_layer(g: DGLGraph, h, k_weight, q_weight, v_weight, a_weight,
         a = ops.SegmentSoftmax(attn.contiguous(), 1, None, g)      # (E, heads) fp32
         m = (v_e.view(e, heads, d).float() * a.unsqueeze(-1)).to(h.dtype).view(e, hidden)
         t = ops.SpMMEdge(m, [1], False, None, g)
+    if fused:       # the gate goes into the product's epilogue, sigmoid and copy to the nodes included
+        return ops.SegmentMMNodeGated(t, a_weight, skip.float().contiguous(), g, sigmoid=True)
     alpha = ops.BroadcastNodeType(torch.sigmoid(skip.float()).unsqueeze(1), g)
-    if fused:       # the gate goes into the product's epilogue
-        return ops.SegmentMMNode(t, a_weight, g, row_scale=alpha)
     out = ops.SegmentMMNode(t, a_weight, g)
     return (out.float() * alpha).to(h.dtype)

@@ -475,6 +475,37 @@ def SegmentMMNode(features, weights, graph: DGLGraph, row_scale=None) -> torch.T
                        graph.num_ntypes, graph.num_nodes, row_scale)
 
 
+def SegmentMMNodeGated(features, weights, gate, graph: DGLGraph, sigmoid: bool = True) -> torch.Tensor:
+    """``SegmentMMNode(features, weights) * g(BroadcastNodeType(gate))`` with g the sigmoid
+    (or the identity): the output projection of an HGT layer with its per-node-type gate
+    (examples/HGT/HGT.py:58-60).  ``gate`` (T,) fp32.  The factor is applied to the fp32 sums
+    in the product's kernel where that kernel takes it (bf16, wide outputs); otherwise it is
+    formed per row first and goes in as ``row_scale`` of SegmentMMNode."""
+    _check_input(features, "features")
+    _check_input(weights, "weights")
+    _check_input(gate, "gate")
+    if graph.ntype_pointer is None:
+        raise RuntimeError("the graph has no type pointer for this operator")
+    if gate.dtype != torch.float32 or gate.numel() != graph.num_ntypes:
+        raise RuntimeError("gate must be one float32 per node type")
+    if features.dtype == torch.bfloat16 and weights.dtype == torch.bfloat16 and weights.dim() == 3 \
+            and int(weights.shape[0]) == graph.num_ntypes and features.dim() == 2 \
+            and int(features.shape[0]) == graph.num_nodes \
+            and int(features.shape[1]) == int(weights.shape[1]):
+        K, M = int(weights.shape[1]), int(weights.shape[2])
+        out = torch.empty((graph.num_nodes, M), dtype=features.dtype, device=features.device)
+        rc = capi.load().ga_segment_mm_gated(
+            graph.ntype_pointer.data_ptr(), graph.num_ntypes, features.data_ptr(),
+            weights.data_ptr(), out.data_ptr(), gate.data_ptr(), 1 if sigmoid else 0,
+            graph.num_nodes, K, M, capi.GA_BF16, _stream(out))
+        if rc != capi.GA_EUNSUPPORTED:
+            capi.check(rc, "ga_segment_mm_gated")
+            return out
+    factor = torch.sigmoid(gate) if sigmoid else gate
+    alpha = BroadcastNodeType(factor.reshape(-1, 1).contiguous(), graph)
+    return SegmentMMNode(features, weights, graph, row_scale=alpha)
+
+
 def SegmentMMNodeStacked(features, weights: Sequence[torch.Tensor], graph: DGLGraph):
     """``[SegmentMMNode(features, w, graph) for w in weights]`` (1 to 4 weight tensors
     of one shape (T, K, M)) with the rows of ``features`` read once: the K, Q and V
@@ -875,7 +906,7 @@ def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
       out[v]      = sum_e a[e] * (v[src] @ M[t])      = sum_{pairs (v, t)} (sum_{e in pair} a[e] * v[src]) @ M[t]
 
     with a = softmax of the scores over the in-edges of v.  k, q, v (N, H*D);
-    relation_att, relation_msg (T, H, D, D); relation_scale (T, H) fp32 (the prior)
+    relation_att, relation_msg (T, H, D, D); relation_scale (T, H) fp32 or bf16 (the prior)
     or None, ``factor`` a further constant on the scores (1 / sqrt(D)): s = scale * factor.  The typed products run over P pairs, the scores are a
     plain dot product per edge and the weighted sum gathers rows of v: no (E, H*D)
     tensor is written.  Returns (N, H*D).  Raises GraphilerError(GA_EUNSUPPORTED) for
@@ -902,14 +933,17 @@ def relation_pair_attention(k, q, v, relation_att, relation_msg, relation_scale,
     lib, stream, dev, P = capi.load(), _stream(k), k.device, pairs.num_pairs
     if relation_scale is not None:
         _check_input(relation_scale, "relation_scale")
-        if tuple(relation_scale.shape) != (n_types, heads) or relation_scale.dtype != torch.float32:
-            raise RuntimeError("relation_scale must be (edge types, heads) float32")
+        if tuple(relation_scale.shape) != (n_types, heads) \
+                or relation_scale.dtype not in (torch.float32, torch.bfloat16):
+            raise RuntimeError("relation_scale must be (edge types, heads) float32 or bfloat16")
     # the matrices as the query side needs them: transposed, times the scale (an fp32
     # product rounded once to the features' dtype)
     att_t = torch.empty_like(relation_att)
-    capi.check(lib.ga_transpose_scale_blocks(
-        relation_att.data_ptr(), _ptr(relation_scale), float(factor), att_t.data_ptr(), n_types * heads, d,
-        dt, stream), "ga_transpose_scale_blocks")
+    scale_dt = capi.GA_BF16 if relation_scale is not None and relation_scale.dtype == torch.bfloat16 \
+        else capi.GA_F32
+    capi.check(lib.ga_transpose_scale_blocks_as(
+        relation_att.data_ptr(), _ptr(relation_scale), scale_dt, float(factor), att_t.data_ptr(),
+        n_types * heads, d, dt, stream), "ga_transpose_scale_blocks_as")
 
     def typed_rows(x, index, w):        # row r = x[index[r]] @ w[relation of pair by_type[r]]
         y = torch.empty((P, hid), dtype=x.dtype, device=dev)

@@ -315,6 +315,18 @@ int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_types, const vo
                           const void *const *W, void *const *Y, int64_t n_weights,
                           int64_t rows, int64_t K, int64_t M, int dtype, ga_stream_t stream);
 
+/* Y[r] = (X[r] @ W[type(r)]) * g(gate[type(r)]), g the identity or, with gate_sigmoid != 0,
+ * 1 / (1 + exp(-x)): SegmentMMNode (segment_mm.cu:23-27) with the per-node-type gate of
+ * examples/HGT/HGT.py:58-60 (`trans_out * sigmoid(skip[ntype])`) applied to the fp32 sums
+ * before they are rounded, so that neither the sigmoid, nor its copy to the nodes
+ * (BroadcastNodeType, broadcast.cu:67-72), nor the multiplication is a pass of its own.
+ * gate: (n_types,) fp32.  bf16 shapes of the wide kernel only (see ga_segment_mm_stacked);
+ * GA_EUNSUPPORTED, having launched nothing, otherwise: the caller then forms the per-row
+ * factor itself and passes it as row_scale of ga_segment_mm_gather. */
+int ga_segment_mm_gated(const int32_t *type_pointer, int64_t n_types, const void *X,
+                        const void *W, void *Y, const float *gate, int gate_sigmoid,
+                        int64_t rows, int64_t K, int64_t M, int dtype, ga_stream_t stream);
+
 /* out[b, j, i] = W[b, i, j] * scale[b] * factor over n_blocks square D x D blocks (scale
  * NULL: 1), computed in fp32 and rounded once to `dtype`: the relation matrices of
  * examples/HGT/HGT.py:39-45 transposed and carrying `relation_pri / sqrt(D)`, as the query
@@ -322,6 +334,11 @@ int ga_segment_mm_stacked(const int32_t *type_pointer, int64_t n_types, const vo
  * (ga_dot_attention_sum).  out must not be W. */
 int ga_transpose_scale_blocks(const void *W, const float *scale, float factor, void *out,
                               int64_t n_blocks, int64_t D, int dtype, ga_stream_t stream);
+/* The same with `scale` stored as scale_dtype (GA_F32 or GA_BF16): a prior kept in the
+ * model's bf16 needs no conversion pass of its own (bf16 -> fp32 is exact). */
+int ga_transpose_scale_blocks_as(const void *W, const void *scale, int scale_dtype, float factor,
+                                 void *out, int64_t n_blocks, int64_t D, int dtype,
+                                 ga_stream_t stream);
 
 /* Per-edge typed linear whose operand lives on the nodes, without the per-edge
  * copy: Y[r] = X[x_index[r]] @ W[type(r)] (x_index NULL: X[r]).  Replaces the

@@ -134,6 +134,45 @@ def test_node_product_with_row_factor(device, K, M, bf16):
                           row_scale=_dev(scale[:-1], device))
 
 
+@pytest.mark.parametrize("K,M,bf16", [(128, 128, True), (256, 256, True), (100, 128, True),
+                                      (64, 384, True), (102, 128, True), (128, 64, True),
+                                      (20, 24, False), (128, 128, False)])
+@pytest.mark.parametrize("sigmoid", [True, False])
+def test_node_product_with_type_gate(device, K, M, bf16, sigmoid):
+    """ops.SegmentMMNodeGated: the per-node-type gate of an HGT layer's output projection
+    (sigmoid(skip[ntype]), examples/HGT/HGT.py:58-60) applied inside the product where the
+    wide kernel takes the shape, as a row factor elsewhere; against the oracle's product
+    times the gate, and against the same gate handed over per row."""
+    from graphiler_amd import prepare_graph
+    rng = np.random.default_rng(K * 3 + M + int(sigmoid))
+    tn = len(COUNTS)
+    ntype = np.repeat(np.arange(tn), COUNTS)
+    n = ntype.shape[0]
+    src, dst = rng.integers(0, n, 2000), rng.integers(0, n, 2000)
+    g = prepare_graph(src, dst, n, device=device, ntype_of=ntype, num_ntypes=tn)
+    tp = np.concatenate([[0], np.cumsum(COUNTS)]).astype(np.int32)
+    x = rng.standard_normal((n, K), dtype=np.float32)
+    w = (rng.standard_normal((tn, K, M)) / np.sqrt(K)).astype(np.float32)
+    if bf16:
+        x, w = to_bf16_f32(x), to_bf16_f32(w)
+    gate = rng.uniform(-3.0, 3.0, tn).astype(np.float32)
+    factor = (1.0 / (1.0 + np.exp(-gate.astype(np.float64)))) if sigmoid else gate.astype(np.float64)
+    got = ops.SegmentMMNodeGated(_dev(x, device, bf16), _dev(w, device, bf16), _dev(gate, device), g,
+                                 sigmoid=sigmoid)
+    assert got.dtype == (torch.bfloat16 if bf16 else torch.float32) and got.shape == (n, M)
+    ref = oracle.segment_mm(tp, x, w) * factor[ntype][:, None]
+    assert_close(got.float().cpu().numpy(), ref, TOL_BF16 if bf16 else TOL_F32,
+                 f"gated node product K={K} M={M} sigmoid={sigmoid}",
+                 mag=oracle.segment_mm(tp, np.abs(x), np.abs(w)) * np.abs(factor)[ntype][:, None])
+    per_row = ops.SegmentMMNode(_dev(x, device, bf16), _dev(w, device, bf16), g,
+                                row_scale=_dev(factor[ntype].astype(np.float32), device))
+    # the two differ by the rounding of the factor only (fp32 sigmoid in the kernel)
+    assert_close(got.float().cpu().numpy(), per_row.float().cpu().numpy(),
+                 8e-3 if bf16 else TOL_F32, "gate inside the product against the gate per row")
+    with pytest.raises(RuntimeError):
+        ops.SegmentMMNodeGated(_dev(x, device, bf16), _dev(w, device, bf16), _dev(gate[:-1], device), g)
+
+
 @pytest.mark.parametrize("rows,K,M,heads", [
     (1500, 256, 256, 4), (1500, 256, 256, 2), (1500, 256, 256, 8),   # heads of 64, 128, 32 columns
     (777, 128, 128, 1), (777, 128, 128, 4), (333, 64, 384, 3), (255, 32, 512, 8),
