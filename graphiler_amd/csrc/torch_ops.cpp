@@ -696,6 +696,38 @@ torch::Tensor SegmentMMNodeScaled(torch::Tensor features, torch::Tensor weights,
   }
   return SegmentMMNode(features, weights, graph) * row_scale;
 }
+torch::Tensor BroadcastNodeType(torch::Tensor features, const GraphPtr &graph);
+// SegmentMMNode(features, weights) * g(BroadcastNodeType(gate.unsqueeze(1))) with g the
+// sigmoid (or the identity): the output projection of examples/HGT/HGT.py:58-60 with its
+// per-node-type gate.  The product's kernel takes the per-type factor where it runs the
+// shape (ga_segment_mm_gated: bf16, wide outputs); otherwise the factor is formed per row
+// and handed to SegmentMMNodeScaled.
+torch::Tensor SegmentMMNodeGated(torch::Tensor features, torch::Tensor weights, torch::Tensor gate,
+                                 bool sigmoid, const GraphPtr &graph) {
+  TORCH_CHECK(gate.dim() == 1 && gate.size(0) == graph->num_ntypes,
+              "gate must have one entry per node type");
+  if (features.is_cuda() && features.scalar_type() == at::kBFloat16 &&
+      weights.scalar_type() == at::kBFloat16 && features.dim() == 2 && weights.dim() == 3 &&
+      features.size(0) == graph->num_nodes && weights.size(0) == graph->num_ntypes &&
+      features.size(1) == weights.size(1) && gate.is_floating_point() &&
+      graph->ntype_pointer.has_value()) {
+    check_input(features, "features");
+    check_input(weights, "weights");
+    torch::Tensor g32 = gate.to(at::kFloat).contiguous();
+    check_input(g32, "gate");
+    torch::Tensor out = torch::empty({graph->num_nodes, weights.size(2)}, features.options());
+    const int rc = ga_segment_mm_gated(
+        graph->ntype_pointer.value().data_ptr<int>(), graph->num_ntypes, features.data_ptr(),
+        weights.data_ptr(), out.data_ptr(), g32.data_ptr<float>(), sigmoid ? 1 : 0,
+        graph->num_nodes, weights.size(1), weights.size(2), GA_BF16, current_stream(out));
+    if (rc != GA_EUNSUPPORTED) {
+      check_ga(rc, "ga_segment_mm_gated");
+      return out;
+    }
+  }
+  torch::Tensor factor = sigmoid ? torch::sigmoid(gate) : gate;
+  return SegmentMMNodeScaled(features, weights, BroadcastNodeType(factor.unsqueeze(1), graph), graph);
+}
 // segment_mm.cu:29-33
 torch::Tensor SegmentMMEdge(torch::Tensor features, torch::Tensor weights,
                             const GraphPtr &graph) {
@@ -1298,6 +1330,9 @@ static auto registry =
         .op("my_ops::SegmentMMNodeScaled(Tensor x, Tensor w, Tensor row_scale, " GRAPH_T
             " g) -> Tensor z",
             &SegmentMMNodeScaled)
+        .op("my_ops::SegmentMMNodeGated(Tensor x, Tensor w, Tensor gate, bool sigmoid, " GRAPH_T
+            " g) -> Tensor z",
+            &SegmentMMNodeGated)
         .op("my_ops::SegmentMMEdgeDot(Tensor x, Tensor w, int endpoint, Tensor q, "
             "int q_endpoint, Tensor? scale, " GRAPH_T " g) -> Tensor z",
             &SegmentMMEdgeDot)

@@ -511,6 +511,9 @@ class _Rewriter:
             if n.kind() == "aten::mul":
                 changed |= self._fuse_node_scale(n)
         for n in list(self.G.nodes()):
+            if n.kind() == "my_ops::SegmentMMNodeScaled":
+                changed |= self._fuse_type_gate(n)
+        for n in list(self.G.nodes()):
             if n.kind() == "my_ops::edge_softmax_sum":
                 changed |= self._fuse_pair_attention(n)
         changed |= self._fuse_stacked_mm()
@@ -717,6 +720,32 @@ class _Rewriter:
                 mm.destroy()
                 return True
         return False
+
+    def _fuse_type_gate(self, n) -> bool:
+        """SegmentMMNodeScaled(x, w, BroadcastNodeType(unsqueeze([sigmoid](s), 1))) ->
+        SegmentMMNodeGated(x, w, s, sigmoid): a factor that is one number per node type
+        needs neither the sigmoid nor its copy to the nodes as operators of their own
+        (HGT's `trans_out * sigmoid(skip)[ntype]`)."""
+        bc = n.inputsAt(2).node()
+        if bc.kind() != "my_ops::BroadcastNodeType" or not self.single_use(n.inputsAt(2)):
+            return False
+        un = bc.inputsAt(0).node()
+        if un.kind() != "aten::unsqueeze" or self.const_of(un.inputsAt(1)) not in (1, -1) \
+                or not self.single_use(bc.inputsAt(0)):
+            return False
+        gate, sig = un.inputsAt(0), None
+        if gate.node().kind() == "aten::sigmoid" and self.single_use(gate) and not _mutated(gate):
+            sig = gate.node()
+            gate = sig.inputsAt(0)
+        if self.where(gate) != NTYPE or _mutated(gate):
+            return False
+        out = self.make("my_ops::SegmentMMNodeGated",
+                        [n.inputsAt(0), n.inputsAt(1), gate, self.const(sig is not None, n),
+                         self.dglgraph], n, NODE)
+        n.output().replaceAllUsesWith(out)
+        for dead in (n, bc, un) + ((sig,) if sig is not None else ()):
+            dead.destroy()
+        return True
 
     def _fuse_stacked_mm(self) -> bool:
         """Two to four SegmentMMNode(x, w_i) of one x -> SegmentMMNodeStacked(x, [w_i]):

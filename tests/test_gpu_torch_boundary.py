@@ -293,6 +293,21 @@ def test_typed_sum_and_stacked_products_through_torchscript(device):
             assert got.dtype == want.dtype and got.shape == want.shape
             assert_close(got.float().cpu().numpy(), want.float().cpu().numpy(),
                          2e-2 if dt == torch.bfloat16 else 2 * TOL_F32, f"SegmentMMNodeScaled {dt}")
+    # ... and with a gate per node type (HGT's sigmoid(skip)): in the kernel for the wide
+    # bf16 shape, through the per-row factor otherwise -- the ctypes wrapper does the same
+    gate = torch.randn(tn, device=device)
+    for w, dt in ((ws[0], torch.bfloat16), (ws[0].float(), torch.float32)):
+        hh = h.to(dt)
+        for sig in (True, False):
+            got = ops.SegmentMMNodeGated(hh, w, gate, sig, sg)
+            fac = (torch.sigmoid(gate) if sig else gate)[g.ntype_COO][:, None]
+            want = ops.SegmentMMNode(hh, w, sg).float() * fac
+            assert got.dtype == dt and got.shape == want.shape
+            assert_close(got.float().cpu().numpy(), want.cpu().numpy(),
+                         2e-2 if dt == torch.bfloat16 else 2 * TOL_F32, f"SegmentMMNodeGated {dt} {sig}")
+            mirror = pyops.SegmentMMNodeGated(hh, w, gate, g, sigmoid=sig)
+            assert torch.equal(got.view(torch.int16 if dt == torch.bfloat16 else torch.int32),
+                               mirror.view(torch.int16 if dt == torch.bfloat16 else torch.int32))
     mixed = [ws[0], ws[1][:, :, :64].contiguous()]          # different shapes: one product each
     outs = ops.SegmentMMNodeStacked(h, mixed, sg)
     assert outs[1].shape == (n, 64)

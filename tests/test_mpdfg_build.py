@@ -74,7 +74,10 @@ def test_level2_fuses_into_graph_operators():
     ours = [x for x in k if x.startswith("my_ops::")]
     # K, V, Q in one pass over h; the output projection takes the gate as its row factor
     assert ours.count("my_ops::SegmentMMNodeStacked") == 1 and ours.count("my_ops::SegmentMMNode") == 0
-    assert ours.count("my_ops::SegmentMMNodeScaled") == 1 and "aten::mul" not in ours
+    # ... and takes the gate per node type: no sigmoid, no copy of it to the nodes, no product
+    assert ours == ["my_ops::SegmentMMNodeStacked", "my_ops::relation_pair_attention",
+                    "my_ops::SegmentMMNodeGated"]
+    assert not any(x in k for x in ("aten::mul", "aten::sigmoid", "aten::unsqueeze"))
     # scores, softmax and weighted sum of transformed values as one operator (it picks the
     # per-pair or the per-edge form from the graph it is given)
     assert ours.count("my_ops::relation_pair_attention") == 1 and "aten::div" not in ours
