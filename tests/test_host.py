@@ -1,4 +1,5 @@
 """Host-side logic and C-ABI surface (runs without a GPU)."""
+import ctypes
 import os
 import re
 
@@ -229,3 +230,26 @@ def test_static_scratch_sizing_query_without_gpu():
                                (1, 17, capi.GA_F32, 1), (3, 5, capi.GA_BF16, 0), (1, 200, capi.GA_BF16, 1)):
         assert 0 < need(e, heads, dim, dt, al) <= lib.ga_gat_workspace_bytes(e, heads * dim, heads)
     assert need(2_000_000_000, 1, 4096, capi.GA_F32, 1) > cap
+
+
+def test_new_entry_points_reject_bad_arguments_without_gpu():
+    """ga_segment_mm_gated and ga_transpose_scale_blocks_as validate before any launch."""
+    lib = capi.load()
+    one = ctypes.c_void_p(256)          # an aligned, never dereferenced address
+    # empty problems are fine whatever the pointers
+    assert lib.ga_segment_mm_gated(None, 4, None, None, None, None, 1, 0, 128, 128, capi.GA_BF16, None) == capi.GA_OK
+    assert lib.ga_segment_mm_gated(None, 0, None, None, None, None, 1, 10, 128, 128, capi.GA_BF16, None) == capi.GA_OK
+    # a missing gate, a bad dtype, a bad shape
+    assert lib.ga_segment_mm_gated(one, 4, one, one, one, None, 1, 10, 128, 128, capi.GA_BF16, None) == capi.GA_EINVAL
+    assert lib.ga_segment_mm_gated(one, 4, one, one, one, one, 1, 10, 128, 128, 7, None) == capi.GA_EINVAL
+    assert lib.ga_segment_mm_gated(one, 4, one, one, one, one, 1, 10, 0, 128, capi.GA_BF16, None) == capi.GA_EINVAL
+    # fp32, or a width the wide kernel does not take: the caller forms the per-row factor
+    assert lib.ga_segment_mm_gated(one, 4, one, one, one, one, 1, 10, 128, 128, capi.GA_F32, None) == capi.GA_EUNSUPPORTED
+    assert lib.ga_segment_mm_gated(one, 4, one, one, one, one, 1, 10, 128, 64, capi.GA_BF16, None) == capi.GA_EUNSUPPORTED
+    odd = ctypes.c_void_p(258)
+    assert lib.ga_segment_mm_gated(one, 4, one, one, one, odd, 1, 10, 128, 128, capi.GA_BF16, None) == capi.GA_EALIGN
+    tsb = lib.ga_transpose_scale_blocks_as
+    assert tsb(None, None, capi.GA_F32, 1.0, None, 0, 16, capi.GA_BF16, None) == capi.GA_OK
+    assert tsb(one, None, 9, 1.0, ctypes.c_void_p(512), 4, 16, capi.GA_BF16, None) == capi.GA_EINVAL
+    assert tsb(one, None, capi.GA_F32, 1.0, one, 4, 16, capi.GA_BF16, None) == capi.GA_EINVAL      # in place
+    assert tsb(one, ctypes.c_void_p(257), capi.GA_BF16, 1.0, ctypes.c_void_p(512), 4, 16, capi.GA_BF16, None) == capi.GA_EALIGN
