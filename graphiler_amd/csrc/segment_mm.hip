@@ -955,7 +955,9 @@ int launch_fold(const int32_t *tp, int n_types, const T *X, const T *W, T *Y,
       if (rc != GA_EUNSUPPORTED || fused) return rc;
     }
   }
-  if (fused) return GA_EUNSUPPORTED;   // only the exact-shape kernel gathers
+  // only the exact-shape kernel gathers, and only it takes a row factor: a call that
+  // carries one must not come back "done" from a kernel that ignores it
+  if (fused || ext.row_scale) return GA_EUNSUPPORTED;
   const size_t lds = (size_t)MM::tile_elems(g.KB, g.MB) * sizeof(T);
   if (lds > (size_t)kMaxLdsOptIn) return GA_EUNSUPPORTED;
   const int mbp = MM::mb_pad(g.MB);

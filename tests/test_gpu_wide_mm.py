@@ -103,9 +103,16 @@ def test_stacked_operator_and_hgt_projections(device):
         ops.SegmentMMNodeStacked(h, [], g)
 
 
-@pytest.mark.parametrize("K,M,bf16", [(128, 128, True), (256, 256, True), (100, 128, True),
-                                      (64, 384, True), (102, 128, True), (128, 64, True),
-                                      (20, 24, False), (128, 128, False)])
+# shapes of the wide kernel, of the exact-shape tile kernel, and of the generic tile kernel
+# (more than 8 column blocks or k blocks: fp32 M = 256 / 384, fp32 K = 256, bf16 K = 136 with
+# three column groups), which takes no factor: the call must fall back, not drop it
+FACTOR_SHAPES = [(128, 128, True), (256, 256, True), (100, 128, True), (64, 384, True),
+                 (102, 128, True), (128, 64, True), (20, 24, False), (128, 128, False),
+                 (16, 256, False), (32, 384, False), (256, 64, False), (136, 384, True),
+                 (100, 384, True)]
+
+
+@pytest.mark.parametrize("K,M,bf16", FACTOR_SHAPES)
 def test_node_product_with_row_factor(device, K, M, bf16):
     """ops.SegmentMMNode(..., row_scale): the factor multiplies the fp32 sums (wide kernel,
     tile kernels, and shapes where it is applied afterwards)."""
@@ -134,9 +141,7 @@ def test_node_product_with_row_factor(device, K, M, bf16):
                           row_scale=_dev(scale[:-1], device))
 
 
-@pytest.mark.parametrize("K,M,bf16", [(128, 128, True), (256, 256, True), (100, 128, True),
-                                      (64, 384, True), (102, 128, True), (128, 64, True),
-                                      (20, 24, False), (128, 128, False)])
+@pytest.mark.parametrize("K,M,bf16", FACTOR_SHAPES)
 @pytest.mark.parametrize("sigmoid", [True, False])
 def test_node_product_with_type_gate(device, K, M, bf16, sigmoid):
     """ops.SegmentMMNodeGated: the per-node-type gate of an HGT layer's output projection
