@@ -191,6 +191,14 @@ class DGLGraph:
         return self._cache[key]
 
     @property
+    def max_in_degree(self) -> int:
+        """Largest number of in-edges of a node (one reduction and host read, then cached)."""
+        if "max_in_degree" not in self._cache:
+            self._cache["max_in_degree"] = int(torch.diff(self.in_pointer).max().item()) \
+                if self.num_nodes > 0 else 0
+        return self._cache["max_in_degree"]
+
+    @property
     def in_eid_is_identity(self) -> bool:
         """True when edge ids already are in-adjacency slot numbers."""
         return self._identity("in_ident", self.in_edge_indices)

@@ -105,8 +105,9 @@ def rgcn_layer(g: DGLGraph, h, weight, norm, fused=True, activation=None):
     ``fused=True``: the typed product reads the source rows through the COO column
     and applies the norm to the rows it produces, then the neighbour sum (two
     passes over an (E, M) message tensor); for the small products where it is the
-    faster one (ops.typed_spmm_preferred: 16 -> 64, 64 -> 8, ...), the single pass
-    of ``fused="tiles"``.
+    faster one (ops.typed_spmm_preferred: 16 -> 64, 64 -> 8, ...; fp32 only on graphs
+    without very large in-degrees, where its one accumulator per destination would
+    lose accuracy), the single pass of ``fused="tiles"``.
     ``fused="pair"``: always the two passes.
     ``fused="tiles"``: ops.TypedSpMMEdge, one pass without the message tensor
     (K in 16, 32, 48, 64; M in 8, 16, 32, 64).
@@ -118,7 +119,7 @@ def rgcn_layer(g: DGLGraph, h, weight, norm, fused=True, activation=None):
     if activation not in (None, "relu", "elu"):
         raise RuntimeError("activation must be None, 'relu' or 'elu'")
     if fused == "tiles" or (fused is True and h.dim() == 2
-                            and ops.typed_spmm_preferred(h, weight)):
+                            and ops.typed_spmm_preferred(h, weight, g)):
         return ops.TypedSpMMEdge(h, weight, g, row_scale=norm.float().contiguous(),
                                  activation=activation)
     if fused:

@@ -639,11 +639,25 @@ def typed_spmm_supported(features, weights) -> bool:
         and get_feat_dim(features) == int(weights.shape[1])
 
 
-def typed_spmm_preferred(features, weights) -> bool:
+# The one-pass kernel adds the messages of a destination chunk after chunk into one fp32
+# accumulator: its rounding error grows with the in-degree (2.5e-6 of the sum at 4,000
+# in-edges of one sign, 6.4e-6 at 16,000, 2.2e-5 at 256,000), where the run-wise sums of
+# SpMMEdge stay at 3e-7.  Above this in-degree fp32 layers take the operator pair.
+TYPED_SPMM_MAX_IN_DEGREE_F32 = 8192
+
+
+def typed_spmm_preferred(features, weights, graph: Optional[DGLGraph] = None) -> bool:
     """Shapes at which the one-pass kernel beats SegmentMMEdgeGather + SpMMEdge: the
-    small products (K * M up to 2048; at 64 x 64 the pair is the faster one)."""
-    return typed_spmm_supported(features, weights) \
-        and int(weights.shape[1]) * int(weights.shape[2]) <= 2048
+    small products (K * M up to 2048; at 64 x 64 the pair is the faster one) -- and, for
+    fp32 on a given graph, only while no node has more than
+    ``TYPED_SPMM_MAX_IN_DEGREE_F32`` in-edges (accuracy, see above)."""
+    if not typed_spmm_supported(features, weights) \
+            or int(weights.shape[1]) * int(weights.shape[2]) > 2048:
+        return False
+    if graph is not None and features.dtype == torch.float32 \
+            and graph.max_in_degree > TYPED_SPMM_MAX_IN_DEGREE_F32:
+        return False
+    return True
 
 
 def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None,

@@ -193,6 +193,45 @@ def test_rgcn_layer_paths_agree(device):
                      2 * TOL_F32, f"{k} -> {m} against unfused")
 
 
+def test_rgcn_layer_on_a_hub_keeps_fp32_accuracy(device):
+    """A destination with 60,000 in-edges whose messages all have one sign: the one-pass
+    kernel adds them chunk after chunk into one accumulator and drifts with the in-degree,
+    so the fp32 layer (and the TorchScript operator) must take the operator pair, whose
+    run-wise sums hold the 1e-5 element by element; bf16 keeps the single pass."""
+    from graphiler_amd import torch_boundary
+    rng = np.random.default_rng(77)
+    n, r, hub = 400, 5, 60_000
+    e = hub + 3000
+    src = rng.integers(0, n, e)
+    dst = rng.integers(0, n, e)
+    dst[:hub] = 11
+    etype = rng.integers(0, r, e)
+    src, dst, etype, _ = sort_edges_by_type(src, dst, etype)
+    g = prepare_graph(src, dst, n, device=device, etype_of=etype, num_etypes=r)
+    arr = build_graph_arrays(src, dst, n)
+    assert g.max_in_degree >= hub > ops.TYPED_SPMM_MAX_IN_DEGREE_F32
+    x = np.abs(rng.standard_normal((n, 16), dtype=np.float32))
+    w = np.abs(rng.standard_normal((r, 16, 64)) / 4).astype(np.float32)
+    norm = rng.uniform(0.5, 1.0, (e, 1)).astype(np.float32)
+    etp = oracle.type_pointer(etype, r)
+    msg = (oracle.segment_mm(etp, oracle.gather_rows(src, x), w) * norm).astype(np.float32)
+    ref = oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices, msg, op="copy_e")
+    dx, dw, dn = _dev(x, device), _dev(w, device), _dev(norm, device)
+    assert not ops.typed_spmm_preferred(dx, dw, g) and ops.typed_spmm_preferred(dx, dw)
+    got = layers.rgcn_layer(g, dx, dw, dn, fused=True)
+    assert_close(got.cpu().numpy(), ref, TOL_F32, "fp32 RGCN layer with a 60,000-edge row", mag=ref)
+    assert torch.equal(got, layers.rgcn_layer(g, dx, dw, dn, fused="pair"))
+    torch_boundary.load()
+    scripted = torch.ops.my_ops.TypedSpMMEdge(dx, dw, dn, torch_boundary.script_graph(g))
+    assert_close(scripted.cpu().numpy(), ref, TOL_F32, "my_ops::TypedSpMMEdge with a 60,000-edge row",
+                 mag=ref)
+    # bf16 (2e-2): the single pass stays
+    xb, wb = dx.bfloat16(), dw.bfloat16()
+    assert ops.typed_spmm_preferred(xb, wb, g)
+    assert torch.equal(layers.rgcn_layer(g, xb, wb, dn, fused=True),
+                       layers.rgcn_layer(g, xb, wb, dn, fused="tiles"))
+
+
 @pytest.mark.parametrize("bf16", [False, True], ids=["f32", "bf16"])
 def test_typed_spmm_activation(device, bf16):
     """The activation applied to the fp32 sums inside the kernel against the same
