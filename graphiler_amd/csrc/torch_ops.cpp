@@ -708,7 +708,10 @@ torch::Tensor SegmentMMNodeGated(torch::Tensor features, torch::Tensor weights, 
                                  bool sigmoid, const GraphPtr &graph) {
   TORCH_CHECK(gate.dim() == 1 && gate.size(0) == graph->num_ntypes,
               "gate must have one entry per node type");
+  // (a gate that would promote the product, e.g. fp32 on bf16 features, keeps the
+  // meaning of the expression: it multiplies the result afterwards, below)
   if (features.is_cuda() && features.scalar_type() == at::kBFloat16 &&
+      at::promote_types(features.scalar_type(), gate.scalar_type()) == features.scalar_type() &&
       weights.scalar_type() == at::kBFloat16 && features.dim() == 2 && weights.dim() == 3 &&
       features.size(0) == graph->num_nodes && weights.size(0) == graph->num_ntypes &&
       features.size(1) == weights.size(1) && gate.is_floating_point() &&
@@ -804,22 +807,36 @@ const torch::Tensor &endpoint_column(const GraphPtr &graph, int64_t which) {
 // row_scale: an (E,) / (E, 1) fp32 tensor multiplies row e of the result (the
 // per-edge norm of examples/RGCN/RGCN.py:29); any other shape multiplies the
 // result afterwards with ATen's broadcasting
+// A factor of `product * factor` that a kernel can apply to its fp32 sums without changing
+// what the expression means: one value per row ((rows,) or (rows, 1)) of a floating dtype
+// that does not promote the product (bf16 features times an fp32 factor is an fp32 tensor
+// in eager PyTorch, and stays one here: such a factor multiplies the result afterwards).
+// Returns the factor as contiguous fp32, or an undefined tensor.
+torch::Tensor kernel_row_factor(const at::optional<torch::Tensor> &row_scale, int64_t rows,
+                                const torch::Tensor &features) {
+  if (!row_scale.has_value()) return torch::Tensor();
+  const torch::Tensor &r = row_scale.value();
+  if (!r.is_cuda() || !r.is_floating_point() || r.numel() != rows || r.dim() < 1 || r.dim() > 2 ||
+      r.size(0) != rows ||
+      at::promote_types(features.scalar_type(), r.scalar_type()) != features.scalar_type())
+    return torch::Tensor();
+  return r.to(at::kFloat).contiguous();
+}
+// The same factor as an operand of `out * factor` (one value per row broadcasts over the row).
+torch::Tensor as_row_operand(const torch::Tensor &r, int64_t rows) {
+  return r.dim() == 1 && r.size(0) == rows ? r.unsqueeze(1) : r;
+}
+
 torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
                                   int64_t endpoint, at::optional<torch::Tensor> row_scale,
                                   const GraphPtr &graph) {
   const MmShape s = edge_mm_shape(features, weights, graph);
   const torch::Tensor &index = endpoint_column(graph, endpoint);
   torch::Tensor out = torch::empty({graph->num_edges, s.heads * s.M}, features.options());
-  const float *rs = nullptr;
+  const torch::Tensor factor = kernel_row_factor(row_scale, graph->num_edges, features);
+  const float *rs = factor.defined() ? factor.data_ptr<float>() : nullptr;
   torch::Tensor late;            // a factor the kernel does not take
-  if (row_scale.has_value()) {
-    const torch::Tensor &r = row_scale.value();
-    if (r.is_cuda() && r.is_contiguous() && r.scalar_type() == at::kFloat &&
-        r.numel() == graph->num_edges && r.dim() <= 2 && r.size(0) == graph->num_edges)
-      rs = r.data_ptr<float>();
-    else
-      late = r;
-  }
+  if (row_scale.has_value() && !rs) late = as_row_operand(row_scale.value(), graph->num_edges);
   const int rc = ga_segment_mm_gather(
       graph->etype_pointer.value().data_ptr<int>(), graph->num_etypes, features.data_ptr(),
       index.data_ptr<int64_t>(), weights.data_ptr(), out.data_ptr(), nullptr, nullptr,
@@ -827,7 +844,7 @@ torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
   if (rc == GA_EUNSUPPORTED) {     // shape outside the matrix-core tile
     out = segment_mm(gather(features, index), weights, graph->etype_pointer,
                      graph->num_etypes, graph->num_edges);
-    if (rs) late = row_scale.value();
+    if (rs) late = as_row_operand(row_scale.value(), graph->num_edges);
   } else {
     check_ga(rc, "ga_segment_mm_gather");
   }
@@ -841,16 +858,9 @@ torch::Tensor SegmentMMEdgeGather(torch::Tensor features, torch::Tensor weights,
 torch::Tensor TypedSpMMEdge(torch::Tensor features, torch::Tensor weights,
                             at::optional<torch::Tensor> row_scale, const GraphPtr &graph) {
   const MmShape s = edge_mm_shape(features, weights, graph);
-  const float *rs = nullptr;
-  bool plain_scale = !row_scale.has_value();
-  if (row_scale.has_value()) {
-    const torch::Tensor &r = row_scale.value();
-    if (r.is_cuda() && r.is_contiguous() && r.scalar_type() == at::kFloat &&
-        r.numel() == graph->num_edges && r.dim() <= 2 && r.size(0) == graph->num_edges) {
-      rs = r.data_ptr<float>();
-      plain_scale = true;
-    }
-  }
+  const torch::Tensor factor = kernel_row_factor(row_scale, graph->num_edges, features);
+  const float *rs = factor.defined() ? factor.data_ptr<float>() : nullptr;
+  const bool plain_scale = !row_scale.has_value() || rs;
   const bool cols_ok = s.M == 8 || s.M == 16 || s.M == 32 || s.M == 64;
   // fp32: the one pass keeps one accumulator per destination, whose rounding error grows
   // with the in-degree (6e-6 of the sum at 16,000 in-edges of one sign); beyond 8192 the

@@ -295,19 +295,36 @@ def test_typed_sum_and_stacked_products_through_torchscript(device):
                          2e-2 if dt == torch.bfloat16 else 2 * TOL_F32, f"SegmentMMNodeScaled {dt}")
     # ... and with a gate per node type (HGT's sigmoid(skip)): in the kernel for the wide
     # bf16 shape, through the per-row factor otherwise -- the ctypes wrapper does the same
-    gate = torch.randn(tn, device=device)
     for w, dt in ((ws[0], torch.bfloat16), (ws[0].float(), torch.float32)):
         hh = h.to(dt)
+        gate = torch.randn(tn, device=device).to(dt)       # a gate of the model's dtype
         for sig in (True, False):
             got = ops.SegmentMMNodeGated(hh, w, gate, sig, sg)
-            fac = (torch.sigmoid(gate) if sig else gate)[g.ntype_COO][:, None]
+            fac = (torch.sigmoid(gate.float()) if sig else gate.float())[g.ntype_COO][:, None]
             want = ops.SegmentMMNode(hh, w, sg).float() * fac
             assert got.dtype == dt and got.shape == want.shape
             assert_close(got.float().cpu().numpy(), want.cpu().numpy(),
                          2e-2 if dt == torch.bfloat16 else 2 * TOL_F32, f"SegmentMMNodeGated {dt} {sig}")
-            mirror = pyops.SegmentMMNodeGated(hh, w, gate, g, sigmoid=sig)
+            mirror = pyops.SegmentMMNodeGated(hh, w, gate.float(), g, sigmoid=sig)
             assert torch.equal(got.view(torch.int16 if dt == torch.bfloat16 else torch.int32),
                                mirror.view(torch.int16 if dt == torch.bfloat16 else torch.int32))
+    # a factor that promotes the product keeps the meaning of `product * factor`: fp32 out
+    wide = ops.SegmentMMNodeGated(h, ws[0], torch.randn(tn, device=device), True, sg)
+    assert wide.dtype == torch.float32
+    e_all = g.num_edges
+    for m_cols in (64, 256):        # a width the gathered product's kernel takes, and one it does not
+        w_e = _t(datasets.glorot(rng, (r, 128, m_cols)), device).bfloat16()
+        plain = ops.SegmentMMEdgeGather(h, w_e, 0, None, sg)
+        s32 = torch.rand(e_all, 1, device=device) + 0.5
+        same = ops.SegmentMMEdgeGather(h, w_e, 0, s32.bfloat16(), sg)
+        promoted = ops.SegmentMMEdgeGather(h, w_e, 0, s32, sg)
+        assert plain.dtype == same.dtype == torch.bfloat16 and promoted.dtype == torch.float32
+        assert_close(promoted.cpu().numpy(), (plain.float() * s32).cpu().numpy(), 2 * TOL_F32,
+                     f"gathered product times an fp32 factor, {m_cols} columns")
+        assert_close(same.float().cpu().numpy(), (plain.float() * s32.bfloat16().float()).cpu().numpy(), 2e-2,
+                     f"gathered product times a bf16 factor, {m_cols} columns")
+        flat = ops.SegmentMMEdgeGather(h, w_e, 0, s32.bfloat16().reshape(-1), sg)     # (E,): per row too
+        assert torch.equal(flat.view(torch.int16), same.view(torch.int16))
     mixed = [ws[0], ws[1][:, :, :64].contiguous()]          # different shapes: one product each
     outs = ops.SegmentMMNodeStacked(h, mixed, sg)
     assert outs[1].shape == (n, 64)
