@@ -42,9 +42,9 @@ def gat_project(h, fc_weight, attn_weight, heads: int = 1):
     z = torch.mm(h, fc_weight)                               # (N, H*D)
     # per-head dot products as two skinny GEMMs with block-diagonal (H*D, H)
     # matrices: the reference's mm(z2, attn_weight) after its split pass
-    el = torch.mm(z, _head_blocks(attn_weight[0]))           # (N, H)
-    er = torch.mm(z, _head_blocks(attn_weight[1]))
-    return z, el, er
+    el = torch.mm(z, _head_blocks(attn_weight[0].to(z.dtype)))           # (N, H)
+    er = torch.mm(z, _head_blocks(attn_weight[1].to(z.dtype)))
+    return z, el.float(), er.float()                         # fp32 terms, as the kernel returns them
 
 
 def _head_blocks(a: torch.Tensor) -> torch.Tensor:
