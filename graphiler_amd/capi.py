@@ -36,6 +36,9 @@ SIGNATURES = {
     "ga_spmm_workspace_bytes": (_sz, [_i64, _i64]),
     "ga_spmm_csr": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                            _i64, _int, _int, _int, _vp, _sz, _vp]),
+    "ga_spmm_scaled_workspace_bytes": (_sz, [_i64, _i64]),
+    "ga_spmm_csr_scaled": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64,
+                                  _int, _int, _vp, _sz, _vp]),
     "ga_spmm_arg_workspace_bytes": (_sz, [_i64, _i64]),
     "ga_spmm_csr_arg": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
                                _i64, _i64, _int, _int, _int, _vp, _sz, _vp]),
@@ -74,6 +77,7 @@ SIGNATURES = {
     "ga_gather_rows": (_int, [_vp, _int, _vp, _vp, _i64, _i64, _vp]),
     "ga_linear_attn": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                               _i64, _vp]),
+    "ga_linear_rows_scaled": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "ga_project_attn": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                                _i64, _int, _vp]),
     "ga_gat_workspace_bytes": (_sz, [_i64, _i64, _i64]),

@@ -94,7 +94,7 @@ linear_attn_kernel(
     const float *__restrict__ X, const float *__restrict__ W,
     const float *__restrict__ a_l, const float *__restrict__ a_r,
     float *__restrict__ Z, float *__restrict__ el, float *__restrict__ er,
-    int64_t rows, int K, int M, int heads) {
+    const float *__restrict__ row_scale, int64_t rows, int K, int M, int heads) {
   using xvec_t = typename XVec<VK>::type;
   __shared__ __attribute__((aligned(16))) float xs[kWgRows * kXs];   // wave-private rows, one buffer
   __shared__ __attribute__((aligned(16))) uint32_t wb[2][3][kPassCols * kWb];
@@ -240,6 +240,17 @@ linear_attn_kernel(
   if (sl < n_slices) step(sl, sb);
 
   // epilogue: lane holds rows wrow0 + t*16 + 4*lk + r, column col0 + cb*16 + lr
+  // the row factors of the plain projection, all requested before the first store
+  float rsv[kRT][4];
+  if (!HAS_ATTN) {
+#pragma unroll
+    for (int t = 0; t < kRT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int64_t row = wrow0 + t * 16 + lk * 4 + r;
+        rsv[t][r] = row_scale && row < rows ? row_scale[row] : 1.0f;
+      }
+  }
   float al[kCB], ar[kCB];
   const int dph = M / heads;
   const int bph = dph >> 4;                              // column blocks per head
@@ -257,6 +268,10 @@ linear_attn_kernel(
     for (int r = 0; r < 4; ++r) {
       const int64_t row = wrow0 + t * 16 + lk * 4 + r;
       const bool live = row < rows;
+      if (!HAS_ATTN && row_scale) {                      // the plain projection only
+#pragma unroll
+        for (int cb = 0; cb < kCB; ++cb) acc[t][cb][r] *= rsv[t][r];
+      }
 #pragma unroll
       for (int cb = 0; cb < kCB; ++cb) {
         const int c = col0 + cb * 16 + lr;
@@ -294,11 +309,11 @@ linear_attn_kernel(
 }  // namespace
 }  // namespace ga
 
-extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
-                              const float *a_r, float *Z, float *el, float *er,
-                              int64_t rows, int64_t K, int64_t M, int64_t heads,
-                              ga_stream_t stream) {
-  using namespace ga;
+namespace ga {
+namespace {
+int launch_linear(const float *X, const float *W, const float *a_l, const float *a_r, float *Z,
+                  float *el, float *er, const float *row_scale, int64_t rows, int64_t K,
+                  int64_t M, int64_t heads, ga_stream_t stream) {
   if (rows < 0 || K <= 0 || M <= 0 || heads <= 0 || M % heads) return GA_EINVAL;
   if (rows > 0x7fffffff || K > 0x7fffffff || M > 0x7fffffff) return GA_EINVAL;
   if (rows == 0) return GA_OK;
@@ -307,7 +322,9 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
   if (K > (1 << 22) || K * M >= ((int64_t)1 << 30)) return GA_EUNSUPPORTED;
   const bool attn = el != nullptr || er != nullptr;
   if (attn && (!el || !er || !a_l || !a_r)) return GA_EINVAL;
-  if (!aligned(X, 4) || !aligned(W, 4) || !aligned(Z, 4)) return GA_EALIGN;
+  if (attn && row_scale) return GA_EINVAL;
+  if (!aligned(X, 4) || !aligned(W, 4) || !aligned(Z, 4) || (row_scale && !aligned(row_scale, 4)))
+    return GA_EALIGN;
   const int vk = (K % 4 == 0 && aligned(X, 16)) ? 4 : ((K % 2 == 0 && aligned(X, 8)) ? 2 : 1);
   const int64_t dph = M / heads;
   if (attn && !(dph == 16 || dph == 32 || dph == 64)) return GA_EUNSUPPORTED;
@@ -317,8 +334,8 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
   hipStream_t s = (hipStream_t)stream;
 #define GA_LAUNCH_LINEAR(ATTN, VK, WAVES)                                          \
   hipLaunchKernelGGL((linear_attn_kernel<ATTN, VK, WAVES>), dim3((unsigned)gx, (unsigned)gy), \
-                     dim3(kBlock), 0, s, X, W, a_l, a_r, Z, el, er, rows, (int)K,   \
-                     (int)M, (int)heads)
+                     dim3(kBlock), 0, s, X, W, a_l, a_r, Z, el, er, row_scale, rows, \
+                     (int)K, (int)M, (int)heads)
 #define GA_LAUNCH_LINEAR_VK(ATTN, WAVES)                 \
   do {                                                   \
     if (vk == 4) GA_LAUNCH_LINEAR(ATTN, 4, WAVES);       \
@@ -343,4 +360,20 @@ extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
 #undef GA_LAUNCH_LINEAR_VK
 #undef GA_LAUNCH_LINEAR
   return launch_status();
+}
+}  // namespace
+}  // namespace ga
+
+extern "C" int ga_linear_attn(const float *X, const float *W, const float *a_l,
+                              const float *a_r, float *Z, float *el, float *er,
+                              int64_t rows, int64_t K, int64_t M, int64_t heads,
+                              ga_stream_t stream) {
+  return ga::launch_linear(X, W, a_l, a_r, Z, el, er, nullptr, rows, K, M, heads, stream);
+}
+
+extern "C" int ga_linear_rows_scaled(const float *X, const float *W, const float *row_scale,
+                                     float *Z, int64_t rows, int64_t K, int64_t M,
+                                     ga_stream_t stream) {
+  return ga::launch_linear(X, W, nullptr, nullptr, Z, nullptr, nullptr, row_scale, rows, K, M, 1,
+                           stream);
 }

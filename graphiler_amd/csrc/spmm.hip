@@ -44,12 +44,23 @@ __device__ __forceinline__ float bin_apply(float x, float w) {
 // Row-reduction policy of the SpMM: the state is the VEC running reductions.
 // SPREAD: the lane's features lie a lane-group width apart (rows that 16-byte
 // accesses do not tile); all of them must share the edge datum, i.e. one head.
-template <typename T, int VEC, int RED, int BOP, bool SPREAD = false>
+// EPI: a finished row is multiplied by its entry of Args::row_scale (when given) and
+// passes through Args::act before it is stored -- a GCN layer's destination norm and
+// relu (examples/GCN/GCN.py:26) without a pass of their own; rows without edges too
+// (0 * scale, so a non-finite scale shows as it does in the separate multiplication).
+// The factor travels in one more float of state, fetched beside the gathers of the
+// row's slots: read when the row is stored, it would put a load's latency in front of
+// every store of the walk.
+// ACT (EPI only): the activation, fixed at compile time -- the store sits inside the
+// walk over the slots, once per unrolled position, and a choice made there at run time
+// triples the loop's code.
+template <typename T, int VEC, int RED, int BOP, bool SPREAD = false, bool EPI = false,
+          int ACT = GA_ACT_NONE>
 struct SpmmPolicy {
   static constexpr bool HASW = BOP != 0;
   typedef T out_t;
   static constexpr int kVec = VEC;
-  static constexpr int kState = VEC;
+  static constexpr int kState = VEC + (EPI ? 1 : 0);
   static constexpr bool kSpread = SPREAD;
   struct Args {
     const int32_t *gidx;  // row of `u` gathered per slot (neighbour id, or edge
@@ -61,34 +72,64 @@ struct SpmmPolicy {
     int dph;
     bool ids_vec;   // row_of_slot, gidx and eid (where given) are 16-byte aligned
     int stride_shift;   // SPREAD: log2 of the lanes per group, set by the launcher
+    const float *row_scale;   // EPI: factor per output row, or nullptr
   };
-  static __device__ __forceinline__ void init(float (&st)[VEC]) {
+  static __device__ __forceinline__ void init(float (&st)[kState]) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) st[v] = red_init<RED>();
+    if constexpr (EPI) st[VEC] = 1.0f;
   }
-  static __device__ __forceinline__ void merge(float (&dst)[VEC], const float *src) {
+  // o <- act(o * f); f is 1 (an exact product) without Args::row_scale
+  static __device__ __forceinline__ void epilogue(float f, float (&o)[VEC]) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const float x = o[v] * f;
+      o[v] = ACT == GA_ACT_NONE ? x : (ACT == GA_ACT_ELU ? elu(x) : relu_keep_nan(x));
+    }
+  }
+  static __device__ __forceinline__ void merge(float (&dst)[kState], const float *src) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) dst[v] = red_apply<RED>(dst[v], src[v]);
+    if constexpr (EPI) dst[VEC] = src[VEC];   // every piece of a row carries the row's factor
   }
-  static __device__ __forceinline__ void finish(const float (&st)[VEC], float (&o)[VEC]) {
+  static __device__ __forceinline__ void finish(const float (&st)[kState], float (&o)[VEC]) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) o[v] = st[v];
   }
-  static __device__ __forceinline__ void empty_row(float (&o)[VEC]) { init(o); }
+  static __device__ __forceinline__ void empty_row(float (&o)[VEC]) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o[v] = red_init<RED>();
+  }
   static __device__ __forceinline__ void emit(const Args &A, out_t *out, int64_t row, int feat,
                                               int f0, const float (&st)[kState]) {
-    emit_row<SpmmPolicy>(out, row, feat, f0, st, A.stride_shift);
+    if constexpr (EPI) {
+      typedef RowIO<T, VEC, SPREAD> IO;
+      float o[VEC];
+      finish(st, o);
+      epilogue(st[VEC], o);
+      IO::store(out + row * feat + f0, o, IO::lane(A.stride_shift, feat - f0));
+    } else {
+      emit_row<SpmmPolicy>(out, row, feat, f0, st, A.stride_shift);
+    }
   }
   static __device__ __forceinline__ void emit_empty(const Args &A, out_t *out, int64_t row,
                                                     int feat, int f0) {
-    emit_empty_row<SpmmPolicy>(out, row, feat, f0, A.stride_shift);
+    if constexpr (EPI) {
+      typedef RowIO<T, VEC, SPREAD> IO;
+      float o[VEC];
+      empty_row(o);
+      epilogue(A.row_scale ? A.row_scale[row] : 1.0f, o);
+      IO::store(out + row * feat + f0, o, IO::lane(A.stride_shift, feat - f0));
+    } else {
+      emit_empty_row<SpmmPolicy>(out, row, feat, f0, A.stride_shift);
+    }
   }
 
   template <class Close>
   static __device__ __forceinline__ void walk(const Args &A,
                                               const int32_t *__restrict__ row_of_slot,
                                               int64_t a, int64_t b, int f0, int feat,
-                                              float (&st)[VEC], int &cur,
+                                              float (&st)[kState], int &cur,
                                               Close &&close_segment) {
     typedef RowIO<T, VEC, SPREAD> IO;
     const typename IO::lane_t ln = IO::lane(A.stride_shift, feat - f0);
@@ -116,6 +157,11 @@ struct SpmmPolicy {
       }
 #pragma unroll
       for (int t = 0; t < kUnroll; ++t) x[t] = IO::load(A.u + (int64_t)g[t] * feat + f0, ln);
+      float rs[kUnroll];
+      if constexpr (EPI) {
+#pragma unroll
+        for (int t = 0; t < kUnroll; ++t) rs[t] = A.row_scale ? A.row_scale[r[t]] : 1.0f;
+      }
 #pragma unroll
       for (int t = 0; t < kUnroll; ++t) {
         if (j + t < b) {
@@ -129,23 +175,26 @@ struct SpmmPolicy {
 #pragma unroll
           for (int v = 0; v < VEC; ++v)
             st[v] = red_apply<RED>(st[v], bin_apply<BOP>(xf[v], ww[t]));
+          if constexpr (EPI) st[VEC] = rs[t];
         }
       }
     }
   }
 };
 
-template <typename T, int VEC, int RED, int BOP, bool SPREAD>
+template <typename T, int VEC, int RED, int BOP, bool SPREAD, bool EPI = false,
+          int ACT = GA_ACT_NONE>
 int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
                 const int32_t *gidx, const int32_t *eid, const void *u,
                 const float *w, void *out, int64_t n_rows, int64_t n_edges,
-                int feat, int heads, float *partial, hipStream_t stream) {
-  typedef SpmmPolicy<T, VEC, RED, BOP, SPREAD> P;
+                int feat, int heads, float *partial, hipStream_t stream,
+                const float *row_scale = nullptr, size_t partial_bytes = SIZE_MAX) {
+  typedef SpmmPolicy<T, VEC, RED, BOP, SPREAD, EPI, ACT> P;
   const bool ids_vec = aligned(row_of_slot, 16) && (!gidx || aligned(gidx, 16)) &&
                        (!eid || aligned(eid, 16));
-  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads, ids_vec, 0};
+  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads, ids_vec, 0, row_scale};
   return launch_runs<P>(args, pointer, row_of_slot, out, n_rows, n_edges, feat,
-                        partial, stream);
+                        partial, stream, partial_bytes);
 }
 
 // max / min with the position of the extremum (the reference's generic kernel,
@@ -438,6 +487,61 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
   return ga::pick_red<ga::bf16_t, 1>(reduce, bop, pointer, row_of_slot, gidx,
                                      eid, u, w, out, n_rows, n_edges, (int)feat,
                                      (int)heads, partial, s);
+}
+
+size_t ga_spmm_scaled_workspace_bytes(int64_t n_edges, int64_t feat) {
+  // a float of state per lane beside its features: at most twice the plain sum's
+  return ga::runs_workspace_bytes(n_edges, feat, 2);
+}
+
+int ga_spmm_csr_scaled(const int32_t *pointer, const int32_t *row_of_slot,
+                       const int32_t *nbr, const int32_t *eid, const void *u, void *out,
+                       const float *row_scale, int activation, int64_t n_rows,
+                       int64_t n_edges, int64_t feat, int op, int dtype, void *workspace,
+                       size_t workspace_bytes, ga_stream_t stream) {
+  if (n_rows < 0 || n_edges < 0 || feat <= 0) return GA_EINVAL;
+  if (n_rows > 0x7fffffff || n_edges > 0x7fffffff || feat > 0x7fffffff) return GA_EINVAL;
+  if (op != GA_COPY_U && op != GA_COPY_E) return GA_EINVAL;
+  if (activation < GA_ACT_NONE || activation > GA_ACT_ELU) return GA_EINVAL;
+  if (dtype != GA_F32 && dtype != GA_BF16) return GA_EINVAL;
+  if (n_rows == 0) return GA_OK;
+  if (!pointer || !out) return GA_EINVAL;
+  if (n_edges > 0) {
+    if (!row_of_slot || !u) return GA_EINVAL;
+    if (op == GA_COPY_U && !nbr) return GA_EINVAL;
+    if (ga_spmm_scaled_workspace_bytes(n_edges, feat) > workspace_bytes || !workspace)
+      return GA_EWORKSPACE;
+    if (!ga::aligned(workspace, 16)) return GA_EWORKSPACE;
+  }
+  const size_t esz = dtype == GA_F32 ? 4 : 2;
+  if (!ga::aligned(out, esz) || (u && !ga::aligned(u, esz)) ||
+      (row_scale && !ga::aligned(row_scale, 4)))
+    return GA_EALIGN;
+  const int32_t *gidx = op == GA_COPY_E ? eid : nbr;
+  const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
+  hipStream_t s = (hipStream_t)stream;
+  float *partial = (float *)workspace;
+  const bool spread_ok = feat >= 3 && feat <= 256;
+#define GA_SPMM_EPI_ACT(T, VEC, SPREAD, ACT)                                             \
+  return ga::launch_spmm<T, VEC, GA_SUM, 0, SPREAD, true, ACT>(                         \
+      pointer, row_of_slot, gidx, eid, u, nullptr, out, n_rows, n_edges, (int)feat, 1, \
+      partial, s, row_scale, workspace_bytes)
+#define GA_SPMM_EPI(T, VEC, SPREAD)                                        \
+  do {                                                                     \
+    if (activation == GA_ACT_RELU) GA_SPMM_EPI_ACT(T, VEC, SPREAD, GA_ACT_RELU); \
+    if (activation == GA_ACT_ELU) GA_SPMM_EPI_ACT(T, VEC, SPREAD, GA_ACT_ELU);   \
+    GA_SPMM_EPI_ACT(T, VEC, SPREAD, GA_ACT_NONE);                          \
+  } while (0)
+  if (dtype == GA_F32) {
+    if (vec_ok && feat % 4 == 0) GA_SPMM_EPI(float, 4, false);
+    if (spread_ok) GA_SPMM_EPI(float, 4, true);
+    GA_SPMM_EPI(float, 1, false);
+  }
+  if (vec_ok && feat % 8 == 0) GA_SPMM_EPI(ga::bf16_t, 8, false);
+  if (spread_ok) GA_SPMM_EPI(ga::bf16_t, 4, true);
+  GA_SPMM_EPI(ga::bf16_t, 1, false);
+#undef GA_SPMM_EPI
+#undef GA_SPMM_EPI_ACT
 }
 
 size_t ga_spmm_arg_workspace_bytes(int64_t n_edges, int64_t feat) {

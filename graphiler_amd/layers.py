@@ -23,7 +23,17 @@ def gcn_layer(g: DGLGraph, h: torch.Tensor, weight: torch.Tensor,
               relu: bool = True) -> torch.Tensor:
     """examples/GCN/GCN.py:21-27,39: h' = act(SpMMSrc((h @ W) * norm_src)),
     optionally scaled by ``norm_dst`` for the symmetric normalisation."""
-    m = ops.linear(h, weight) * norm_src
+    if norm_src.dtype != torch.float32 or (norm_dst is not None and norm_dst.dtype != torch.float32):
+        m = ops.linear(h, weight) * norm_src
+        out = ops.SpMMSrc(m, [1], False, None, g)
+        if norm_dst is not None:
+            out = out * norm_dst
+        return torch.relu(out) if relu else out
+    # the norms and the relu ride on the rows the two kernels store
+    m = ops.linear(h, weight, row_scale=norm_src.contiguous())
+    if ops.spmm_tail_preferred(m, g):
+        return ops.spmm_scaled(m, g, row_scale=None if norm_dst is None else norm_dst.contiguous(),
+                               activation="relu" if relu else None)
     out = ops.SpMMSrc(m, [1], False, None, g)
     if norm_dst is not None:
         out = out * norm_dst

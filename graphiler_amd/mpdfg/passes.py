@@ -517,7 +517,57 @@ class _Rewriter:
             if n.kind() == "my_ops::edge_softmax_sum":
                 changed |= self._fuse_pair_attention(n)
         changed |= self._fuse_stacked_mm()
+        # last: only the sums no other rewrite has taken
+        for n in list(self.G.nodes()):
+            if n.kind() in ("aten::relu", "aten::elu"):
+                changed |= self._fuse_spmm_tail(n)
+        for n in list(self.G.nodes()):
+            if n.kind() == "aten::mul":
+                changed |= self._fuse_spmm_tail(n)
         return changed
+
+    def _fuse_spmm_tail(self, n) -> bool:
+        """relu | elu (SpMMSrc | SpMMEdge (x) [* s]) and SpMMSrc | SpMMEdge (x) * s, s
+        a per-node tensor -> SpMMScaled(x, s, activation, edge_rows): what follows the
+        sum row by row is applied where the sum is stored (GCN's
+        `torch.relu(torch.sum(mailbox, 1))`).  The operator multiplies afterwards when
+        s is not one fp32 number per row."""
+        act, tail, top = 0, [], n.inputsAt(0)
+        if n.kind() == "aten::relu":
+            act = 1
+        elif n.kind() == "aten::elu":
+            if any(self.const_of(n.inputsAt(i)) not in (1, 1.0) for i in (1, 2, 3)):
+                return False
+            act = 2
+        if act:
+            if not self.single_use(top) or _mutated(top):
+                return False
+            mul = top.node() if top.node().kind() == "aten::mul" else None
+        else:
+            mul = n
+        scale, summed = None, top
+        if mul is not None:
+            for a, b in ((mul.inputsAt(0), mul.inputsAt(1)), (mul.inputsAt(1), mul.inputsAt(0))):
+                if a.node().kind() in ("my_ops::SpMMSrc", "my_ops::SpMMEdge") and \
+                        isinstance(b.type(), torch._C.TensorType) and self.where(b) == NODE:
+                    scale, summed = b, a
+                    break
+            else:
+                return False
+            if mul is not n:
+                tail.append(mul)
+        sp = summed.node()
+        if sp.kind() not in ("my_ops::SpMMSrc", "my_ops::SpMMEdge") or \
+                not self.single_use(summed) or _mutated(summed):
+            return False
+        out = self.make("my_ops::SpMMScaled",
+                        [sp.inputsAt(0), scale if scale is not None else self.const(None, n),
+                         self.const(act, n), self.const(sp.kind().endswith("Edge"), n),
+                         self.dglgraph], n, NODE)
+        n.output().replaceAllUsesWith(out)
+        for dead in [n] + tail + [sp]:
+            dead.destroy()
+        return True
 
     def _fuse_gather_mm(self, n) -> bool:
         """SegmentMMEdge(BroadcastSrcNode | BroadcastDstNode (x), w) ->

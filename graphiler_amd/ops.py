@@ -159,6 +159,53 @@ def SpMMEdge(features, dims: Sequence[int], keep_dim: bool, dtype,
     return spmm(graph, "copy_e", "sum", features)
 
 
+# Below this size of the (N, feat) result a row factor / activation in the sum's store
+# pays only for rows that 16-byte accesses tile: measured on 19,717 nodes, the store of
+# the 3-wide sum with the tail costs 8 us more than the sum alone, the two small
+# elementwise kernels it replaces 3 us; from 232,965 nodes on the tail in the store wins
+# for every width (4-8 % of the sum).
+SPMM_TAIL_MIN_BYTES = 8 << 20
+
+
+def spmm_tail_preferred(features, graph: DGLGraph) -> bool:
+    """Whether ``spmm_scaled`` beats the sum followed by elementwise operators."""
+    row_bytes = get_feat_dim(features) * features.element_size()
+    return row_bytes % 16 == 0 or graph.num_nodes * row_bytes >= SPMM_TAIL_MIN_BYTES
+
+
+def spmm_scaled(features, graph: DGLGraph, row_scale=None, activation=None,
+                edge_rows: bool = False) -> torch.Tensor:
+    """SpMMSrc (``edge_rows``: SpMMEdge) with the row-wise tail of a layer applied
+    where the sums are stored: out[v] = act(row_scale[v] * sum over in-edges), the
+    reduce of examples/GCN/GCN.py:26 (``torch.relu(torch.sum(mailbox, 1))``) with
+    an optional destination-side norm.  row_scale: (N,) or (N, 1) fp32 or None;
+    activation: None | "relu" | "elu".  Bit for bit what the separate operators
+    give (sum, multiplication in fp32, activation, one rounding to the storage type)."""
+    _check_input(features, "features")
+    dt = _feat_dtype(features, "features")
+    act = _activation(activation)
+    n = graph.num_nodes
+    if features.shape[0] != (graph.num_edges if edge_rows else n):
+        raise RuntimeError("features have the wrong number of rows")
+    if row_scale is not None:
+        _check_input(row_scale, "row_scale")
+        if row_scale.dtype != torch.float32 or row_scale.numel() != n \
+                or row_scale.shape[0] != n:
+            raise RuntimeError("row_scale must be (N,) or (N, 1) float32")
+    feat = get_feat_dim(features)
+    out = torch.empty(_out_shape(n, features), dtype=features.dtype, device=features.device)
+    lib = capi.load()
+    ws = graph.workspace(lib.ga_spmm_scaled_workspace_bytes(graph.num_edges, feat))
+    capi.check(lib.ga_spmm_csr_scaled(
+        graph.in_pointer.data_ptr(), graph.in_row_of_slot.data_ptr(),
+        graph.in_node_indices.data_ptr(),
+        None if graph.in_eid_is_identity else graph.in_edge_indices.data_ptr(),
+        features.data_ptr(), out.data_ptr(), _ptr(row_scale), act, n, graph.num_edges, feat,
+        capi.GA_COPY_E if edge_rows else capi.GA_COPY_U, dt, ws.data_ptr(), ws.numel(),
+        _stream(features)), "ga_spmm_csr_scaled")
+    return out
+
+
 def gspmm_src_mul_e_sum(ufeature, efeature, dims: Sequence[int], keep_dim: bool,
                         dtype, graph: DGLGraph) -> torch.Tensor:
     """spmm.cu:286-320: out[v] = sum over in-edges of ufeature[src] * efeature[e]."""
@@ -1022,15 +1069,33 @@ LINEAR_MAX_COLS = 64
 LINEAR_MIN_ROWS = 16384
 
 
-def linear(x, weight):
+def linear(x, weight, row_scale=None):
     """x @ weight for a (rows, K) node feature matrix and a (K, M) weight: the
     dense operator in front of the graph operators of a layer
-    (examples/GCN/GCN.py:39 ``torch.mm(feature, self.weight)``)."""
+    (examples/GCN/GCN.py:39 ``torch.mm(feature, self.weight)``).  ``row_scale``
+    ((rows,) or (rows, 1) fp32): a factor per row of the product, the source-side
+    norm of the GCN message (GCN.py:22-23), applied by the library's kernel to the
+    rows it stores and by a multiplication afterwards on the ``torch.mm`` route."""
+    if row_scale is not None and (row_scale.dtype != torch.float32
+                                  or row_scale.numel() != x.shape[0]
+                                  or row_scale.shape[0] != x.shape[0]):
+        raise RuntimeError("row_scale must be (rows,) or (rows, 1) float32")
     if (x.dtype == torch.float32 and weight.dtype == torch.float32 and x.dim() == 2
             and weight.dim() == 2 and x.is_cuda and x.is_contiguous() and weight.is_contiguous()
             and weight.shape[1] <= LINEAR_MAX_COLS and x.shape[0] >= LINEAR_MIN_ROWS):
-        return linear_attn(x, weight)
-    return torch.mm(x, weight)
+        if row_scale is None:
+            return linear_attn(x, weight)
+        _check_input(row_scale, "row_scale")
+        if int(weight.shape[0]) != int(x.shape[1]):
+            raise RuntimeError("weight must be (K, M)")
+        z = torch.empty((x.shape[0], weight.shape[1]), dtype=x.dtype, device=x.device)
+        capi.check(capi.load().ga_linear_rows_scaled(
+            x.data_ptr(), weight.data_ptr(), row_scale.data_ptr(), z.data_ptr(),
+            int(x.shape[0]), int(x.shape[1]), int(weight.shape[1]), _stream(x)),
+            "ga_linear_rows_scaled")
+        return z
+    z = torch.mm(x, weight)
+    return z if row_scale is None else z * row_scale.view(-1, 1).to(z.dtype)
 
 
 def linear_attn(x, weight, a_l=None, a_r=None):

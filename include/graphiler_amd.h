@@ -115,6 +115,24 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
                 int64_t feat, int64_t heads, int op, int reduce, int dtype,
                 void *workspace, size_t workspace_bytes, ga_stream_t stream);
 
+/* Sum SpMM of copied rows (GA_COPY_U or GA_COPY_E) with the row-wise tail of a GCN
+ * layer in its store: out[v, :] = act(row_scale[v] * sum_i msg_i), i.e. SpMMSrc
+ * (spmm.cu:375-389) followed by the destination-side normalisation and the relu of
+ * examples/GCN/GCN.py:26 (`torch.relu(torch.sum(mailbox, 1))`) without a pass over
+ * the (n_rows, feat) result for either.  row_scale (n_rows) fp32 or NULL (no
+ * factor); activation one of ga_activation, applied to the fp32 value before it is
+ * rounded.  Rows without edges get act(row_scale[v] * 0).  Everything else as
+ * ga_spmm_csr; with row_scale == NULL and GA_ACT_NONE the result is that of
+ * ga_spmm_csr, bit for bit.  workspace: ga_spmm_scaled_workspace_bytes() bytes,
+ * 16-byte aligned (the factor travels with the partial sums of a row).
+ */
+size_t ga_spmm_scaled_workspace_bytes(int64_t n_edges, int64_t feat);
+int ga_spmm_csr_scaled(const int32_t *pointer, const int32_t *row_of_slot,
+                       const int32_t *nbr, const int32_t *eid, const void *u, void *out,
+                       const float *row_scale, int activation, int64_t n_rows,
+                       int64_t n_edges, int64_t feat, int op, int dtype, void *workspace,
+                       size_t workspace_bytes, ga_stream_t stream);
+
 /* SpMM with max / min and the position of each extremum: the arg_u / arg_e
  * outputs of the reference's generic kernel (SpMMCsrKernel, spmm.cuh:30-71,
  * reducers functor.cuh:148-213: strict comparison, so the first extremum in
@@ -534,6 +552,16 @@ int ga_linear_attn(const float *X, const float *W, const float *a_l,
                    const float *a_r, float *Z, float *el, float *er,
                    int64_t rows, int64_t K, int64_t M, int64_t heads,
                    ga_stream_t stream);
+
+/* The plain projection with a factor per row: Z[n, :] = (X[n, :] @ W) * row_scale[n]
+ * (row_scale (rows) fp32, NULL for none) -- the projection of examples/GCN/GCN.py:39
+ * together with the source-side norm of the message (`edges.src['h'] * norm`,
+ * GCN.py:22-23), which multiplies exactly these rows.  The product is rounded to
+ * fp32 first and then multiplied, as the two separate operators do.  Limits as
+ * ga_linear_attn.
+ */
+int ga_linear_rows_scaled(const float *X, const float *W, const float *row_scale, float *Z,
+                          int64_t rows, int64_t K, int64_t M, ga_stream_t stream);
 
 /* The same projection with the attention terms for fp32 or bf16 storage (fp32
  * accumulation; el / er are fp32 and are taken from the accumulators, before Z

@@ -9,7 +9,7 @@ import oracle
 from graphiler_amd.examples import udf as U
 from graphiler_amd import prepare_graph
 from graphiler_amd.graph import build_graph_arrays
-from graphiler_amd.mpdfg import GraphData, mpdfg_builder, update_all
+from graphiler_amd.mpdfg import GraphData, NodeBatchDummy, mpdfg_builder, update_all
 from helpers import TOL_F32, assert_close
 
 pytestmark = pytest.mark.gpu
@@ -39,6 +39,35 @@ def test_gcn_plan(device, level):
     want = np.maximum(oracle.spmm(arr.in_pointer, arr.in_node_indices, arr.in_edge_indices,
                                   (h * deg ** -0.5).astype(np.float32), op="copy_u"), 0)
     assert_close(g.ndata['h'].cpu().numpy(), want, TOL_F32, f"GCN plan level {level}")
+
+
+def gcn_both_norms_reduce(nodes: NodeBatchDummy):
+    summed = torch.sum(nodes.mailbox['m'], dim=1)
+    return {'h': torch.nn.functional.elu(summed * nodes.data['norm'])}
+
+
+@pytest.mark.parametrize("level", [0, 1, 2])
+@pytest.mark.parametrize("width", [16, 3])
+def test_gcn_plan_with_both_norms(device, level, width):
+    """A destination-side norm and elu after the sum (the symmetric normalisation of a
+    graph convolution): at level 2 both are arguments of the sum operator."""
+    rng = np.random.default_rng(26 + width)
+    n, src, dst = _homo(rng)
+    g = GraphData(prepare_graph(src, dst, n, device))
+    h = rng.standard_normal((n, width), dtype=np.float32)
+    deg = rng.integers(1, 9, (n, 1)).astype(np.float32)
+    norm = rng.uniform(-1.0, 1.0, (n, 1)).astype(np.float32)
+    g.ndata['h'], g.ndata['degree'], g.ndata['norm'] = _t(h, device), _t(deg, device), _t(norm, device)
+    plan = mpdfg_builder(U.gcn_message, gcn_both_norms_reduce, opt_level=level)
+    assert ("my_ops::SpMMScaled" in plan.op_kinds()) == (level == 2)
+    update_all(g, plan)
+    arr = build_graph_arrays(src, dst, n)
+    hs = (h * deg ** -0.5).astype(np.float32)
+    adj = (arr.in_pointer, arr.in_node_indices, arr.in_edge_indices)
+    want = oracle.spmm(*adj, hs, op="copy_u").astype(np.float64) * norm
+    want = np.where(want > 0, want, np.expm1(np.minimum(want, 0)))
+    assert_close(g.ndata['h'].cpu().numpy(), want, TOL_F32, f"GCN plan with both norms, level {level}",
+                 mag=oracle.spmm(*adj, np.abs(hs), op="copy_u") * np.abs(norm))
 
 
 @pytest.mark.parametrize("level,width", [(0, 32), (1, 32), (2, 32), (2, 64), (2, 24)])

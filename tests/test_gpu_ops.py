@@ -108,6 +108,70 @@ def test_spmm_copy_sum_f32(graph, device, feat, op):
     assert not got[empty].any()
 
 
+@pytest.mark.parametrize("feat", [1, 3, 16, 40, 64, 602])
+@pytest.mark.parametrize("op", ["copy_u", "copy_e"])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_spmm_scaled_is_the_separate_operators(graph, device, feat, op, bf16):
+    """Sum, row factor and activation in the store of the sum: against the oracle's sum
+    scaled and activated in float64, and bit for bit against SpMMSrc / SpMMEdge followed
+    by the multiplication and the activation in fp32 (one rounding at the end)."""
+    name, g, arr = graph
+    rng = np.random.default_rng(feat * 3 + bf16)
+    n = arr.num_nodes
+    rows = n if op == "copy_u" else arr.COO_src.shape[0]
+    # a mean away from 0: the 4000-edge row's sum must not cancel to nothing
+    x = rng.standard_normal((rows, feat), dtype=np.float32) + np.float32(0.3)
+    if bf16:
+        x = to_bf16_f32(x)
+    scale = rng.uniform(-1.5, 1.5, (n, 1)).astype(np.float32)
+    xd, sd = _dev(x, device, bf16), _dev(scale, device)
+    adj = (arr.in_pointer, arr.in_node_indices, arr.in_edge_indices)
+    ref = oracle.spmm(*adj, x, op=op).astype(np.float64)
+    mag = oracle.spmm(*adj, np.abs(x), op=op)
+    plain = (ops.SpMMSrc if op == "copy_u" else ops.SpMMEdge)(xd, [1], False, None, g)
+    for act in (None, "relu", "elu"):
+        for sc in (None, sd, sd.view(-1)):
+            got = ops.spmm_scaled(xd, g, row_scale=sc, activation=act, edge_rows=op == "copy_e")
+            assert got.dtype == xd.dtype and got.shape == (n, feat)
+            want = ref if sc is None else ref * scale
+            if act == "relu":
+                want = np.maximum(want, 0)
+            elif act == "elu":
+                want = np.where(want > 0, want, np.expm1(np.minimum(want, 0)))
+            assert_close(got.float().cpu().numpy(), want, TOL_BF16 if bf16 else TOL_F32,
+                         f"spmm_scaled {op} {name} F={feat} act={act} scale={sc is not None}",
+                         mag=mag * (1 if sc is None else np.abs(scale)))
+            # the device's elu is a polynomial near 0, not torch's expm1; a bf16 sum that
+            # is scaled is rounded once here and twice by the separate operators
+            if act != "elu" and not (bf16 and sc is not None):
+                sep = plain if sc is None else plain * sd
+                sep = torch.relu(sep) if act == "relu" else sep
+                assert torch.equal(got, sep), f"{op} {name} F={feat} act={act}"
+    # no factor, no activation: the plain operator
+    assert torch.equal(ops.spmm_scaled(xd, g, edge_rows=op == "copy_e"),
+                       (ops.SpMMSrc if op == "copy_u" else ops.SpMMEdge)(xd, [1], False, None, g))
+
+
+def test_spmm_scaled_non_finite_factor_and_arguments(device):
+    """A row without edges is 0 * factor: an infinite factor (degree 0 to the power -1/2)
+    shows as NaN there, as it does after the separate multiplication."""
+    src, dst = np.array([0, 1, 1], np.int64), np.array([1, 0, 0], np.int64)
+    g = prepare_graph(src, dst, 3, device=device)
+    x = torch.ones(3, 4, device=device)
+    scale = torch.tensor([2.0, float("inf"), float("inf")], device=device)
+    got = ops.spmm_scaled(x, g, row_scale=scale, activation="relu").cpu().numpy()
+    assert np.array_equal(got[0], np.full(4, 4.0, np.float32))
+    assert np.isposinf(got[1]).all() and np.isnan(got[2]).all()
+    with pytest.raises(RuntimeError, match="row_scale"):
+        ops.spmm_scaled(x, g, row_scale=scale[:2])
+    with pytest.raises(RuntimeError, match="row_scale"):
+        ops.spmm_scaled(x, g, row_scale=scale.double())
+    with pytest.raises(RuntimeError, match="activation"):
+        ops.spmm_scaled(x, g, activation="tanh")
+    with pytest.raises(RuntimeError, match="rows"):
+        ops.spmm_scaled(x[:2], g)
+
+
 @pytest.mark.parametrize("feat,heads", [(1, 1), (5, 1), (64, 1), (64, 4),
                                         (128, 8), (256, 4), (12, 3)])
 @pytest.mark.parametrize("reverse", [False, True])
@@ -1168,6 +1232,29 @@ def test_linear_dispatch(device, rows, K, M):
     own = rows >= ops.LINEAR_MIN_ROWS and M <= ops.LINEAR_MAX_COLS
     same = np.array_equal(got.cpu().numpy(), ops.linear_attn(_dev(x, device), _dev(w, device)).cpu().numpy())
     assert same or not own
+
+
+@pytest.mark.parametrize("rows,K,M", [(20000, 50, 64), (16500, 500, 16), (17000, 37, 3),
+                                      (1000, 50, 64), (20000, 50, 128)])
+def test_linear_with_row_factor(device, rows, K, M):
+    """The factor per row in the projection's store is the product rounded to fp32 and
+    then multiplied: bit for bit ``linear(x, w) * s``, on the kernel's shapes and on the
+    vendor GEMM's."""
+    rng = np.random.default_rng(rows + K + M)
+    x = _dev(rng.standard_normal((rows, K), dtype=np.float32), device)
+    w = _dev(datasets.glorot(rng, (K, M)), device)
+    s = _dev(rng.uniform(0.1, 2.0, (rows, 1)).astype(np.float32), device)
+    s[5] = float("nan")
+    want = ops.linear(x, w) * s
+    for sc in (s, s.view(-1)):
+        got = ops.linear(x, w, row_scale=sc)
+        assert got.shape == (rows, M)
+        assert torch.equal(torch.nan_to_num(got, nan=7.0), torch.nan_to_num(want, nan=7.0))
+    assert torch.isnan(got[5]).all()
+    with pytest.raises(RuntimeError, match="row_scale"):
+        ops.linear(x, w, row_scale=s[:-1])
+    with pytest.raises(RuntimeError, match="row_scale"):
+        ops.linear(x, w, row_scale=s.double())
 
 
 @pytest.mark.parametrize("offset", [1, 2, 3, 4])

@@ -329,3 +329,40 @@ def test_typed_sum_and_stacked_products_through_torchscript(device):
     outs = ops.SegmentMMNodeStacked(h, mixed, sg)
     assert outs[1].shape == (n, 64)
     assert torch.equal(outs[1].view(torch.int16), ops.SegmentMMNode(h, mixed[1], sg).view(torch.int16))
+
+
+def test_sum_with_row_wise_tail(setup, device):
+    """my_ops::SpMMScaled = act(SpMMSrc | SpMMEdge (x) * s): in the sum's store for an
+    fp32 (N, 1) factor on fp32 features, by torch's own multiplication (broadcasting and
+    promotion included) for any other factor -- the same values and dtype as the three
+    separate operators either way."""
+    sg, arr, rng = setup
+    ops = torch.ops.my_ops
+    n, e = arr.num_nodes, arr.COO_src.shape[0]
+    for edge_rows, rows in ((False, n), (True, e)):
+        plain_op = ops.SpMMEdge if edge_rows else ops.SpMMSrc
+        for dt in (torch.float32, torch.bfloat16):
+            x = _t(rng.standard_normal((rows, 24), dtype=np.float32) + np.float32(0.2), device).to(dt)
+            plain = plain_op(x, [1], False, None, sg)
+            factors = (None, torch.rand(n, 1, device=device) - 0.4,                   # per row
+                       (torch.rand(n, 1, device=device) - 0.4).to(dt),
+                       torch.rand(24, device=device), torch.rand(n, 24, device=device).double())
+            for fac in factors:
+                for act, fn in ((0, lambda t: t), (1, torch.relu), (2, torch.nn.functional.elu)):
+                    got = ops.SpMMScaled(x, fac, act, edge_rows, sg)
+                    want = fn(plain if fac is None else plain * fac)
+                    assert got.dtype == want.dtype and got.shape == want.shape, (dt, fac, act)
+                    tol = 2e-2 if want.dtype == torch.bfloat16 else 2 * TOL_F32
+                    assert_close(got.double().cpu().numpy(), want.double().cpu().numpy(), tol,
+                                 f"SpMMScaled {dt} act {act} edge_rows {edge_rows}")
+            # three-dimensional features: a factor per row is (N, 1, 1)
+            x3 = x.view(rows, 4, 6)
+            fac3 = torch.rand(n, 1, 1, device=device)
+            got = ops.SpMMScaled(x3, fac3, 1, edge_rows, sg)
+            want = torch.relu(plain_op(x3, [1], False, None, sg) * fac3)
+            assert got.shape == (n, 4, 6) and got.dtype == want.dtype
+            assert_close(got.float().cpu().numpy(), want.float().cpu().numpy(), 2 * TOL_F32, "3-d features")
+    with pytest.raises(RuntimeError, match="activation"):
+        ops.SpMMScaled(x, None, 3, True, sg)
+    with pytest.raises(RuntimeError, match="rows"):
+        ops.SpMMScaled(x, None, 0, False, sg)

@@ -253,3 +253,27 @@ def test_new_entry_points_reject_bad_arguments_without_gpu():
     assert tsb(one, None, 9, 1.0, ctypes.c_void_p(512), 4, 16, capi.GA_BF16, None) == capi.GA_EINVAL
     assert tsb(one, None, capi.GA_F32, 1.0, one, 4, 16, capi.GA_BF16, None) == capi.GA_EINVAL      # in place
     assert tsb(one, ctypes.c_void_p(257), capi.GA_BF16, 1.0, ctypes.c_void_p(512), 4, 16, capi.GA_BF16, None) == capi.GA_EALIGN
+
+
+def test_scaled_sum_and_projection_reject_bad_arguments_without_gpu():
+    """ga_spmm_csr_scaled and ga_linear_rows_scaled validate before any launch."""
+    lib = capi.load()
+    one, odd = ctypes.c_void_p(256), ctypes.c_void_p(258)
+    sp = lib.ga_spmm_csr_scaled
+    # (pointer, row_of_slot, nbr, eid, u, out, row_scale, activation, n_rows, n_edges, feat, op,
+    #  dtype, workspace, workspace_bytes, stream)
+    assert sp(None, None, None, None, None, None, None, 0, 0, 0, 8, capi.GA_COPY_U, capi.GA_F32, None, 0, None) == capi.GA_OK
+    assert sp(one, one, one, None, one, one, None, 3, 4, 4, 8, capi.GA_COPY_U, capi.GA_F32, one, 1 << 20, None) == capi.GA_EINVAL   # activation
+    assert sp(one, one, one, None, one, one, None, 0, 4, 4, 8, capi.GA_U_MUL_E, capi.GA_F32, one, 1 << 20, None) == capi.GA_EINVAL  # copies only
+    assert sp(one, one, one, None, one, one, None, 0, 4, 4, 0, capi.GA_COPY_U, capi.GA_F32, one, 1 << 20, None) == capi.GA_EINVAL   # feat
+    assert sp(one, one, one, None, one, one, None, 0, 4, 4, 8, capi.GA_COPY_U, 5, one, 1 << 20, None) == capi.GA_EINVAL             # dtype
+    assert sp(one, one, None, None, one, one, None, 0, 4, 4, 8, capi.GA_COPY_U, capi.GA_F32, one, 1 << 20, None) == capi.GA_EINVAL  # no neighbours
+    assert sp(one, one, one, None, one, one, None, 0, 4, 4, 8, capi.GA_COPY_U, capi.GA_F32, one, 16, None) == capi.GA_EWORKSPACE
+    assert sp(one, one, one, None, one, one, odd, 0, 4, 4, 8, capi.GA_COPY_U, capi.GA_F32, one, 1 << 20, None) == capi.GA_EALIGN
+    lin = lib.ga_linear_rows_scaled
+    # (X, W, row_scale, Z, rows, K, M, stream)
+    assert lin(None, None, None, None, 0, 8, 8, None) == capi.GA_OK
+    assert lin(one, one, one, one, 4, 0, 8, None) == capi.GA_EINVAL
+    assert lin(one, one, one, None, 4, 8, 8, None) == capi.GA_EINVAL
+    assert lin(one, one, odd, one, 4, 8, 8, None) == capi.GA_EALIGN
+    assert lin(one, one, one, one, 4, 1 << 23, 8, None) == capi.GA_EUNSUPPORTED

@@ -58,7 +58,9 @@ def test_level1_moves_dense_work_to_the_nodes():
 
 def test_level2_fuses_into_graph_operators():
     _, k = _kinds("gcn", 2)
-    assert "my_ops::SpMMSrc" in k and not any(x.startswith("my_ops::Broadcast") for x in k)
+    # the relu of the reduce function rides on the sum's store
+    assert [x for x in k if x.startswith("my_ops::")] == ["my_ops::SpMMScaled"]
+    assert "aten::relu" not in k
     _, k = _kinds("gat", 2)
     ours = [x for x in k if x.startswith("my_ops::")]
     assert ours == ["my_ops::gat_project", "my_ops::gat_aggregate"]    # two kernels end to end
@@ -140,6 +142,57 @@ def test_value_numbering_keeps_reads_that_are_overwritten_apart():
             assert [u.user.kind() for u in target.output().uses()] == ["aten::relu_"]
     assert len(reads) >= 2 or not any(r.inputsAt(0).node().kind() == "my_ops::BroadcastSrcNode"
                                       for r in inplace)
+
+
+def gcn_both_norms_reduce(nodes: NodeBatchDummy):
+    summed = torch.sum(nodes.mailbox['m'], dim=1)
+    return {'h': torch.nn.functional.elu(summed * nodes.data['norm'])}
+
+
+def gcn_scaled_reduce(nodes: NodeBatchDummy):
+    return {'h': nodes.data['norm'] * torch.sum(nodes.mailbox['m'], dim=1)}
+
+
+def gcn_other_elu_reduce(nodes: NodeBatchDummy):
+    return {'h': torch.nn.functional.elu(torch.sum(nodes.mailbox['m'], dim=1), 0.5)}
+
+
+def gcn_sum_read_twice_reduce(nodes: NodeBatchDummy):
+    summed = torch.sum(nodes.mailbox['m'], dim=1)
+    return {'h': torch.relu(summed), 'raw': summed}
+
+
+def gcn_inplace_reduce(nodes: NodeBatchDummy):
+    return {'h': torch.relu_(torch.sum(nodes.mailbox['m'], dim=1))}
+
+
+def _ours(reduce, level=2):
+    plan = mpdfg_builder(U.gcn_message, reduce, opt_level=level)
+    plan.forward
+    return plan, [k for k in plan.op_kinds() if k.startswith(("my_ops::", "aten::"))]
+
+
+def test_row_wise_tail_of_a_sum_joins_the_sum():
+    """A destination-side factor and the activation after a neighbour sum become
+    arguments of the sum; anything the operator cannot reproduce stays as it is."""
+    plan, k = _ours(gcn_both_norms_reduce)
+    assert "my_ops::SpMMScaled" in k and "aten::elu" not in k and "my_ops::SpMMSrc" not in k
+    assert k.count("aten::mul") == 1                        # the message's own factor only
+    node = [n for n in plan.graph.nodes() if n.kind() == "my_ops::SpMMScaled"][0]
+    assert node.inputsAt(1).node().kind() == "aten::__getitem__"       # the stored norm
+    assert node.inputsAt(2).toIValue() == 2 and node.inputsAt(3).toIValue() is False
+    plan, k = _ours(gcn_scaled_reduce)
+    assert "my_ops::SpMMScaled" in k and k.count("aten::mul") == 1
+    node = [n for n in plan.graph.nodes() if n.kind() == "my_ops::SpMMScaled"][0]
+    assert node.inputsAt(2).toIValue() == 0
+    _, k = _ours(gcn_other_elu_reduce)                      # alpha = 0.5: not the operator's elu
+    assert "my_ops::SpMMSrc" in k and "aten::elu" in k and "my_ops::SpMMScaled" not in k
+    _, k = _ours(gcn_sum_read_twice_reduce)                 # the plain sum is an output too
+    assert "my_ops::SpMMSrc" in k and "aten::relu" in k and "my_ops::SpMMScaled" not in k
+    _, k = _ours(gcn_inplace_reduce)                        # relu_ is left alone
+    assert "my_ops::SpMMSrc" in k and "aten::relu_" in k
+    _, k = _ours(gcn_both_norms_reduce, level=1)            # level 1 does not fuse
+    assert "my_ops::SpMMScaled" not in k
 
 
 def bad_reduce(nodes: NodeBatchDummy):
