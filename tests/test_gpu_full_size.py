@@ -390,3 +390,75 @@ def test_config5_network_as_benchmarked(device):
         assert_close(out.float().cpu().numpy()[sample], ref, TOL_BF16,
                      f"config 5 network as benchmarked, layer {layer + 1} ({k} -> 256, {act})")
         x = out
+
+
+@pytest.mark.timeout(600)
+def test_tensors_beyond_two_to_the_31_elements(device):
+    """Per-edge tensors of config 5's graph with 40 features: 2.57 G elements, 10.3 GB --
+    every offset past 2^31 elements / 2^32 bytes.  References are torch's own indexing
+    and float64 scatter-adds on the GPU (independent kernels)."""
+    wl = datasets.gat_rmat_large()
+    n, e, feat = wl.num_nodes, wl.num_edges, 40
+    assert e * feat > 2 ** 31
+    g = prepare_graph(wl.src, wl.dst, n, device=device)
+    src, dst = _t(wl.src, device), _t(wl.dst, device)
+    gen = torch.Generator(device=device).manual_seed(3)
+    x = torch.randn(n, feat, device=device, generator=gen)
+    y = torch.randn(n, feat, device=device, generator=gen)
+
+    def summed(rows):           # float64 scatter-add by destination
+        return torch.zeros(n, feat, device=device, dtype=torch.float64).index_add_(0, dst, rows.double())
+
+    assert torch.equal(ops.BroadcastSrcNode(x, g), x[src])
+    assert torch.equal(ops.BroadcastDstNode(x, g), x[dst])
+    m = ops.gsddmm_u_add_v_mul_alpha(x, y, 1, g)                    # (E, 40): the per-edge tensor below
+    want = x[src]
+    want += y[dst]
+    assert m.shape == (e, feat) and torch.equal(m, want)
+    want = x[src]
+    want *= m
+    assert torch.equal(ops.gsddmm(g, "mul", x, m, "u", "e"), want)
+    del want
+    got = ops.SpMMEdge(m, [1], False, None, g)
+    ref, mag = summed(m), summed(m.abs())
+    assert float(((got - ref).abs() / mag.clamp_min(1e-30)).max()) <= TOL_F32, "SpMMEdge"
+    assert torch.equal(ops.spmm_scaled(m, g, activation="relu", edge_rows=True), torch.relu(got))
+    del got, ref, mag
+    w = torch.rand(e, 1, device=device, generator=gen)
+    got = ops.gspmm_src_mul_e_sum(x, w, [1], False, None, g)
+    xw = x[src] * w
+    assert float(((got - summed(xw)).abs() / summed(xw.abs()).clamp_min(1e-30)).max()) <= TOL_F32, "u_mul_e"
+    del xw, got
+    sm = ops.SegmentSoftmax(m, 1, None, g)                          # 40 heads: the 64-lane-head layout
+    deg = torch.bincount(dst, minlength=n)
+    sums = summed(sm)[deg > 0]
+    assert float((sums - 1).abs().max()) <= 2e-5
+    ptr = g.in_pointer.long()
+    for v in (0, 1, int(deg.argmax()), n - 1, n // 2, 12345, 2_000_000):
+        a, b = int(ptr[v]), int(ptr[v + 1])
+        if b > a:
+            assert torch.allclose(sm[a:b], torch.softmax(m[a:b].double(), 0).float(), rtol=2e-5, atol=1e-9)
+    del sm, sums
+    logit = torch.randn(e, 8, device=device, generator=gen)         # 8 heads x 5
+    got = ops.edge_softmax_sum(logit, m, g)
+    att = ops.SegmentSoftmax(logit, 1, None, g)
+    ref = summed((m.view(e, 8, 5) * att.unsqueeze(-1)).view(e, feat))
+    assert float((got - ref).abs().max()) <= TOL_F32 * float(ref.abs().max()), "edge_softmax_sum"
+    del got, ref, att, logit, m
+    torch.cuda.empty_cache()
+    # typed products: (E, 32) @ (T, 32, 40) -> (E, 40)
+    from graphiler_amd.graph import sort_edges_by_type
+    n_types = 4
+    et = np.sort(np.random.default_rng(5).integers(0, n_types, e))
+    s2, d2, et2, _ = sort_edges_by_type(wl.src, wl.dst, et)
+    gt = prepare_graph(s2, d2, n, device=device, etype_of=et2, num_etypes=n_types)
+    xe = torch.randn(e, 32, device=device, generator=gen)
+    xn = torch.randn(n, 32, device=device, generator=gen)
+    wt = torch.randn(n_types, 32, feat, device=device, generator=gen) / 6
+    per_edge, gathered = ops.SegmentMMEdge(xe, wt, gt), ops.SegmentMMEdgeGather(xn, wt, 0, gt)
+    tp, s2d = gt.etype_pointer.cpu().numpy(), _t(s2, device)
+    for t in range(n_types):
+        a, b = int(tp[t]), int(tp[t + 1])
+        for got, rows in ((per_edge, xe[a:b]), (gathered, xn[s2d[a:b]])):
+            ref = torch.mm(rows.double(), wt[t].double())
+            assert float((got[a:b] - ref).abs().max()) <= TOL_F32 * float(ref.abs().max()), f"typed product {t}"
