@@ -717,7 +717,12 @@ def TypedSpMMEdge(features, weights, graph: DGLGraph, row_scale=None,
     ``row_scale`` (E,) or
     (E, 1) fp32.  The additions of a row happen in the order of the prepared layout
     (by relation, then adjacency order), the same in every call.  ``activation``
-    ("relu" | "elu"): applied to the fp32 sums before they are stored."""
+    ("relu" | "elu"): applied to the fp32 sums before they are stored.
+    This is the kernel itself, whatever the graph: a destination's messages go into one
+    fp32 accumulator, so the rounding error of its sum grows with its in-degree (relative
+    to the sum of magnitudes 3e-7 at 1,000 in-edges, 6e-6 at 16,000, 1.1e-5 at 40,000);
+    ``typed_spmm_preferred(features, weights, graph)`` is the rule the layer, the
+    TorchScript operator and the compiled plans apply before they take it."""
     _check_input(features, "features")
     _check_input(weights, "weights")
     dt = _feat_dtype(features, "features")
