@@ -197,6 +197,284 @@ int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
                         partial, stream, partial_bytes);
 }
 
+// ---- sums of rows of at most four features: one lane per slot -----------------
+// With one lane per row a lane group of the run schedule is a single lane: every
+// lane walks a run of its own, so a wave instruction reads 64 separate pieces of the
+// slot-indexed columns and nothing of the walk coalesces (copy_u with one feature on
+// 11.6 M edges: 129 us for 93 MB).  Here a lane owns one SLOT: the wavefront reads 64
+// consecutive slots of the columns with one access each, gathers their rows (a lane
+// holds the row's one to four features), and adds up the slots of each row with a
+// segmented scan over the lanes -- rows are sorted, so lanes with equal row ids at
+// distance d have that id in between, and the scan stops at the first distance at
+// which no lane finds its own row.  A wavefront owns 2^k consecutive chunks of 64
+// slots; the segment that runs into the next chunk is carried in a register.  The
+// first and the last segment of a wavefront's range may be pieces of a longer row:
+// they take the route of the run schedule -- the four wavefronts of a workgroup chain
+// their pieces through LDS, and what crosses the workgroup's slot range leaves the
+// same two partial states per workgroup that runs_kernel leaves, so the second
+// kernel is runs_fixup_kernel of the one-lane-per-row layout, unchanged.  Additions
+// of a row happen in the scan's tree order, fixed by the slot positions.
+constexpr int kSlotUnroll = 4;   // chunks whose loads are in flight together
+
+// One step of the segmented scan inside rows of 16 lanes: a lane whose neighbour OFF
+// lanes down (in its row of lanes) holds the same key adds that neighbour's sums.  Lanes
+// without such a neighbour see the key -3, which no slot has.
+template <int OFF>
+__device__ __forceinline__ void slots_scan16(int key, float (&acc)[4], int feat) {
+  const int pk = __builtin_amdgcn_update_dpp(-3, key, 0x110 + OFF, 0xF, 0xF, false);   // row_shr:OFF
+  const bool hit = pk == key;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    if (v < feat) {                          // uniform
+      const float pv = __int_as_float(__builtin_amdgcn_update_dpp(
+          0, __float_as_int(acc[v]), 0x110 + OFF, 0xF, 0xF, false));
+      if (hit) acc[v] += pv;
+    }
+  }
+}
+// The lanes of row ROW whose key is that of the last lane of the row before add that
+// lane's (already complete) sums.
+template <int ROW>
+__device__ __forceinline__ void slots_row_carry(int key, float (&acc)[4], int feat, int lane) {
+  const int ck = __builtin_amdgcn_readlane(key, 16 * ROW - 1);
+  const bool hit = (lane >> 4) == ROW && key == ck;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    if (v < feat) {
+      const float cv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc[v]), 16 * ROW - 1));
+      if (hit) acc[v] += cv;
+    }
+  }
+}
+
+template <class P, int BOP>
+__global__ __launch_bounds__(kBlock) void slots_kernel(
+    typename P::Args args, const int32_t *__restrict__ pointer,
+    const int32_t *__restrict__ row_of_slot, typename P::out_t *__restrict__ out,
+    float *__restrict__ partial, RunGeom geo) {
+  typedef typename P::out_t T;
+  typedef RowIO<T, 4, true> IO;
+  constexpr int SF = P::kState;          // 4 sums (+ the row factor)
+  constexpr bool EPI = SF > 4;
+  constexpr bool HASW = BOP != 0;
+  constexpr int kWaves = kBlock / kWave;
+  if ((int64_t)blockIdx.x >= geo.n_wg) {   // rows without edges, one lane per row
+    const int64_t row = ((int64_t)blockIdx.x - geo.n_wg) * kBlock + threadIdx.x;
+    if (row < geo.n_rows && pointer[row] == pointer[row + 1])
+      P::emit_empty(args, out, row, geo.feat, 0);
+    return;
+  }
+  __shared__ float piece[kWaves][2][SF];   // [wavefront][A | B][state]
+  __shared__ RunFlags flags[kWaves];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int feat = geo.feat;
+  const typename IO::lane_t ln = IO::lane(0, feat);
+  const int wg_shift = geo.run_shift + 8;
+  const int64_t wave_slots = (int64_t)1 << (wg_shift - 2);
+  const int64_t wa = ((int64_t)blockIdx.x << wg_shift) + wave * wave_slots;
+  const int64_t wb = min(wa + wave_slots, geo.n_edges);
+  if (lane == 0) {
+    flags[wave].has_a = flags[wave].a_open = flags[wave].has_b = 0;
+    flags[wave].row_a = flags[wave].row_b = 0;
+  }
+  if (wa < wb) {
+    const int first_key = row_of_slot[wa];
+    const bool first_open = wa > 0 && row_of_slot[wa - 1] == first_key;
+    int carry_key = -1;                    // row of the segment that runs on from the last chunk
+    float carry[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float carry_scale = 1.0f;
+    // the slot-indexed columns of kSlotUnroll chunks; those of the next round are
+    // requested before the current round's sums, so they arrive meanwhile
+    struct Ids {
+      int r[kSlotUnroll], rn[kSlotUnroll];
+      int64_t g[kSlotUnroll], e[kSlotUnroll];
+    };
+    auto load_ids = [&](int64_t j0, Ids &I) {
+#pragma unroll
+      for (int c = 0; c < kSlotUnroll; ++c) {
+        const int64_t j = j0 + c * kWave + lane;
+        const int64_t jc = j < wb ? j : wb - 1;
+        I.r[c] = row_of_slot[jc];
+        I.rn[c] = jc + 1 < geo.n_edges ? row_of_slot[jc + 1] : -1;
+        I.g[c] = args.gidx ? (int64_t)args.gidx[jc] : jc;
+        if (HASW) I.e[c] = args.eid ? (int64_t)args.eid[jc] : jc;
+      }
+    };
+    Ids cur;
+    load_ids(wa, cur);
+    for (int64_t j0 = wa; j0 < wb; j0 += kSlotUnroll * kWave) {
+      float val[kSlotUnroll][4], rs[kSlotUnroll];
+      typename IO::raw_t x[kSlotUnroll];
+#pragma unroll
+      for (int c = 0; c < kSlotUnroll; ++c) {
+        x[c] = IO::load(args.u + cur.g[c] * feat, ln);
+        if (EPI) rs[c] = args.row_scale ? args.row_scale[cur.r[c]] : 1.0f;
+        if (HASW) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int h = min(v / args.dph, args.heads - 1);   // dead features: any valid weight
+            val[c][v] = args.w[cur.e[c] * args.heads + h];
+          }
+        }
+      }
+      int r[kSlotUnroll], rn[kSlotUnroll];
+#pragma unroll
+      for (int c = 0; c < kSlotUnroll; ++c) {
+        r[c] = cur.r[c];
+        rn[c] = cur.rn[c];
+      }
+      if (j0 + kSlotUnroll * kWave < wb) load_ids(j0 + kSlotUnroll * kWave, cur);
+#pragma unroll
+      for (int c = 0; c < kSlotUnroll; ++c) {
+        const int64_t c0 = j0 + c * kWave;   // uniform
+        if (c0 >= wb) break;
+        const bool valid = c0 + lane < wb;
+        float xf[4];
+        IO::widen(x[c], xf);
+        int key = valid ? r[c] : -2;         // lanes past the range: a row id no slot has
+        float acc[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const float m = HASW ? bin_apply<BOP>(xf[v], val[c][v]) : xf[v];
+          acc[v] = valid ? m : 0.0f;
+        }
+        if (lane == 0 && key == carry_key) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[v] = carry[v] + acc[v];
+        }
+        // inclusive segmented sum over the lanes: inside each row of 16 lanes with
+        // DPP shifts, then the total at the end of a row of lanes goes to the lanes of
+        // the next one that continue its segment (through a scalar register)
+        slots_scan16<1>(key, acc, feat);
+        slots_scan16<2>(key, acc, feat);
+        slots_scan16<4>(key, acc, feat);
+        slots_scan16<8>(key, acc, feat);
+        slots_row_carry<1>(key, acc, feat, lane);
+        slots_row_carry<2>(key, acc, feat, lane);
+        slots_row_carry<3>(key, acc, feat, lane);
+        const bool is_end = valid && rn[c] != key;
+        if (is_end) {
+          float st[SF];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) st[v] = acc[v];
+          if (EPI) st[4] = rs[c];
+          if (key == first_key && first_open) {   // the piece of a row that began before this range
+#pragma unroll
+            for (int i = 0; i < SF; ++i) piece[wave][0][i] = st[i];
+            flags[wave].has_a = 1;
+            flags[wave].row_a = key;
+          } else {
+            P::emit(args, out, key, feat, 0, st);
+          }
+        }
+        // the segment of the last slot runs on into the next chunk (or past the range)
+        const int last = (int)min((int64_t)kWave - 1, wb - 1 - c0);   // uniform
+        const bool open = !__builtin_amdgcn_readlane((int)is_end, last);
+        carry_key = open ? __builtin_amdgcn_readlane(key, last) : -1;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          carry[v] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc[v]), last));
+        if (EPI) carry_scale = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rs[c]), last));
+      }
+    }
+    if (carry_key != -1 && lane == 0) {      // the range ends inside a row
+      const bool through = carry_key == first_key && first_open;   // ... that also began before it
+      float *dst = piece[wave][through ? 0 : 1];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) dst[v] = carry[v];
+      if (EPI) dst[4] = carry_scale;
+      if (through) {
+        flags[wave].has_a = flags[wave].a_open = 1;
+        flags[wave].row_a = carry_key;
+      } else {
+        flags[wave].has_b = 1;
+        flags[wave].row_b = carry_key;
+      }
+    }
+  }
+  __syncthreads();
+  if (lane != 0 || wa >= wb) return;
+  // the pieces of the workgroup's wavefronts, chained as runs_kernel chains its runs
+  auto chain_into = [&](int i, float (&acc)[SF]) -> bool {
+    int j = i - 1;
+    while (j >= 0 && flags[j].has_a && flags[j].a_open) --j;
+    const bool starts_inside = j >= 0;
+    if (starts_inside) {
+#pragma unroll
+      for (int q = 0; q < SF; ++q) acc[q] = piece[j][1][q];
+    } else {
+      P::init(acc);
+    }
+    for (int g = j + 1; g <= i; ++g) P::merge(acc, piece[g][0]);
+    return starts_inside;
+  };
+  float *const gp = partial + (int64_t)blockIdx.x * 2 * SF;
+  const int64_t slots_left = geo.n_edges - ((int64_t)blockIdx.x << wg_shift);
+  const int last_wave = (int)min((int64_t)kWaves, (slots_left + wave_slots - 1) / wave_slots) - 1;
+  const bool has_a = flags[wave].has_a, a_open = flags[wave].a_open, has_b = flags[wave].has_b;
+  if (has_a && !a_open) {
+    float acc[SF];
+    if (chain_into(wave, acc)) {
+      P::emit(args, out, flags[wave].row_a, feat, 0, acc);
+    } else {
+#pragma unroll
+      for (int q = 0; q < SF; ++q) gp[q] = acc[q];
+    }
+  }
+  if (wave == last_wave) {
+    if (has_b) {
+#pragma unroll
+      for (int q = 0; q < SF; ++q) gp[SF + q] = piece[wave][1][q];
+    } else if (has_a && a_open) {
+      float acc[SF];
+      const bool inside = chain_into(wave, acc);
+      float *p = gp + (inside ? SF : 0);
+#pragma unroll
+      for (int q = 0; q < SF; ++q) p[q] = acc[q];
+    }
+  }
+}
+
+// Slots per workgroup: 256 << run_shift -- one chunk per wavefront on small graphs,
+// up to 16 on large ones (measured on 11.6 M edges, one feature, us by slots per
+// workgroup: 256: 189, 512: 129, 1024: 97, 2048: 93, 4096: 95, 8192: 98, 16384: 120);
+// never fewer slots than four runs of the run schedule, whose workspace bound the
+// caller sized.
+template <typename T, int BOP, bool EPI = false, int ACT = GA_ACT_NONE>
+int launch_spmm_slots(const int32_t *pointer, const int32_t *row_of_slot, const int32_t *gidx,
+                      const int32_t *eid, const void *u, const float *w, void *out,
+                      int64_t n_rows, int64_t n_edges, int feat, int heads, float *partial,
+                      hipStream_t stream, const float *row_scale = nullptr,
+                      size_t partial_bytes = SIZE_MAX) {
+  typedef SpmmPolicy<T, 4, GA_SUM, BOP, true, EPI, ACT> P;
+  constexpr int SF = P::kState;
+  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads, false, 0, row_scale};
+  RunGeom geo;
+  int wg_shift = ilog2_ceil((uint64_t)((n_edges + 8191) / 8192));
+  const int floor_shift = std::max(8, run_shift_for(n_edges, feat) + 2);
+  wg_shift = std::min(std::max(wg_shift, floor_shift), std::max(12, floor_shift));
+  geo.run_shift = wg_shift - 8;
+  geo.tpr_shift = 0;
+  geo.lanes_total = 1;
+  geo.feat = feat;
+  geo.n_edges = n_edges;
+  geo.n_rows = n_rows;
+  const int64_t n_wg = (n_edges + ((int64_t)1 << wg_shift) - 1) >> wg_shift;
+  geo.n_runs = n_wg * kBlock;
+  geo.n_wg = n_wg;
+  const int64_t row_blocks = (n_rows + kBlock - 1) / kBlock;
+  if (n_wg + row_blocks > 0x7fffffff) return GA_EUNSUPPORTED;
+  if ((size_t)n_wg * 2 * SF * sizeof(float) > partial_bytes) return GA_EWORKSPACE;
+  hipLaunchKernelGGL((slots_kernel<P, BOP>), dim3((unsigned)(n_wg + row_blocks)), dim3(kBlock), 0,
+                     stream, args, pointer, row_of_slot, (T *)out, partial, geo);
+  const int64_t fix_blocks = (n_wg + kBlock - 1) / kBlock;
+  hipLaunchKernelGGL((runs_fixup_kernel<P>), dim3((unsigned)fix_blocks), dim3(kBlock),
+                     (size_t)kBlock * SF * sizeof(float), stream, args, pointer, row_of_slot,
+                     partial, (T *)out, geo, n_wg, (int)fix_blocks);
+  return launch_status();
+}
+
 // max / min with the position of the extremum (the reference's generic kernel,
 // spmm.cuh:30-71 with functor.cuh:148-213): beside each running extremum the
 // state keeps the SLOT that produced it, so "first extremum in slot order wins"
@@ -460,6 +738,25 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
   const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
   hipStream_t s = (hipStream_t)stream;
   float *partial = (float *)workspace;
+  // sums of rows of up to four features: one lane per slot
+  if (reduce == GA_SUM && feat <= 4 && n_edges > 0) {
+#define GA_SPMM_SLOTS(T, B)                                                                  \
+  return ga::launch_spmm_slots<T, B>(pointer, row_of_slot, gidx, eid, u, w, out, n_rows,     \
+                                     n_edges, (int)feat, (int)heads, partial, s, nullptr,    \
+                                     workspace_bytes)
+#define GA_SPMM_SLOTS_T(T)                                  \
+  switch (bop) {                                            \
+    case GA_U_MUL_E: GA_SPMM_SLOTS(T, GA_U_MUL_E);          \
+    case GA_U_ADD_E: GA_SPMM_SLOTS(T, GA_U_ADD_E);          \
+    case GA_U_SUB_E: GA_SPMM_SLOTS(T, GA_U_SUB_E);          \
+    case GA_U_DIV_E: GA_SPMM_SLOTS(T, GA_U_DIV_E);          \
+    default: GA_SPMM_SLOTS(T, 0);                           \
+  }
+    if (dtype == GA_F32) GA_SPMM_SLOTS_T(float)
+    GA_SPMM_SLOTS_T(ga::bf16_t)
+#undef GA_SPMM_SLOTS_T
+#undef GA_SPMM_SLOTS
+  }
   // rows that 16-byte accesses do not tile: four features per lane, a lane-group
   // width apart, when all of a row shares the edge datum (one head, or none read)
   const bool spread_ok = (!hasw || heads == 1) && feat >= 3 && feat <= 256;
@@ -521,6 +818,22 @@ int ga_spmm_csr_scaled(const int32_t *pointer, const int32_t *row_of_slot,
   const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
   hipStream_t s = (hipStream_t)stream;
   float *partial = (float *)workspace;
+  if (feat <= 4 && n_edges > 0) {                        // one lane per slot
+#define GA_SPMM_SLOTS_EPI(T, ACT)                                                            \
+  return ga::launch_spmm_slots<T, 0, true, ACT>(pointer, row_of_slot, gidx, eid, u, nullptr, \
+                                                out, n_rows, n_edges, (int)feat, 1, partial, \
+                                                s, row_scale, workspace_bytes)
+#define GA_SPMM_SLOTS_EPI_T(T)                                        \
+  do {                                                                \
+    if (activation == GA_ACT_RELU) GA_SPMM_SLOTS_EPI(T, GA_ACT_RELU); \
+    if (activation == GA_ACT_ELU) GA_SPMM_SLOTS_EPI(T, GA_ACT_ELU);   \
+    GA_SPMM_SLOTS_EPI(T, GA_ACT_NONE);                                \
+  } while (0)
+    if (dtype == GA_F32) GA_SPMM_SLOTS_EPI_T(float);
+    GA_SPMM_SLOTS_EPI_T(ga::bf16_t);
+#undef GA_SPMM_SLOTS_EPI_T
+#undef GA_SPMM_SLOTS_EPI
+  }
   const bool spread_ok = feat >= 3 && feat <= 256;
 #define GA_SPMM_EPI_ACT(T, VEC, SPREAD, ACT)                                             \
   return ga::launch_spmm<T, VEC, GA_SUM, 0, SPREAD, true, ACT>(                         \

@@ -159,18 +159,20 @@ def SpMMEdge(features, dims: Sequence[int], keep_dim: bool, dtype,
     return spmm(graph, "copy_e", "sum", features)
 
 
-# Below this size of the (N, feat) result a row factor / activation in the sum's store
-# pays only for rows that 16-byte accesses tile: measured on 19,717 nodes, the store of
-# the 3-wide sum with the tail costs 8 us more than the sum alone, the two small
-# elementwise kernels it replaces 3 us; from 232,965 nodes on the tail in the store wins
-# for every width (4-8 % of the sum).
+# A row factor / activation in the sum's store is free for rows of up to four features
+# (one lane per slot) and for rows that 16-byte accesses tile.  For the other widths (the
+# one-feature-per-lane layout of the run schedule) it pays from a result of this size on:
+# measured on 19,717 nodes, the 5- or 7-wide sum with the tail takes 31-34 us against
+# 26-27 us for the sum and two elementwise kernels; from 232,965 nodes on the tail in
+# the store wins for every width (4-8 % of the sum).
 SPMM_TAIL_MIN_BYTES = 8 << 20
 
 
 def spmm_tail_preferred(features, graph: DGLGraph) -> bool:
     """Whether ``spmm_scaled`` beats the sum followed by elementwise operators."""
-    row_bytes = get_feat_dim(features) * features.element_size()
-    return row_bytes % 16 == 0 or graph.num_nodes * row_bytes >= SPMM_TAIL_MIN_BYTES
+    feat = get_feat_dim(features)
+    row_bytes = feat * features.element_size()
+    return feat <= 4 or row_bytes % 16 == 0 or graph.num_nodes * row_bytes >= SPMM_TAIL_MIN_BYTES
 
 
 def spmm_scaled(features, graph: DGLGraph, row_scale=None, activation=None,

@@ -152,6 +152,46 @@ def test_spmm_scaled_is_the_separate_operators(graph, device, feat, op, bf16):
                        (ops.SpMMSrc if op == "copy_u" else ops.SpMMEdge)(xd, [1], False, None, g))
 
 
+@pytest.mark.parametrize("feat", [1, 2, 3, 4])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_narrow_sums_with_a_row_across_many_workgroups(device, feat, bf16):
+    """Rows of at most four features take the one-lane-per-slot kernel; a destination
+    with 380,000 in-edges spans hundreds of its workgroups (the cooperative fold of the
+    second kernel), next to short rows, rows without edges and a shuffled edge order."""
+    rng = np.random.default_rng(40 + feat)
+    n, e = 3000, 400_000
+    src = rng.integers(0, n, e)
+    dst = rng.integers(0, n // 2, e)                 # the upper half has no in-edges
+    dst[rng.permutation(e)[:380_000]] = 17
+    g = prepare_graph(src, dst, n, device=device)
+    arr = build_graph_arrays(src, dst, n)
+    assert not g.in_eid_is_identity
+    x = rng.standard_normal((n, feat), dtype=np.float32) + np.float32(0.25)
+    m = rng.standard_normal((e, feat), dtype=np.float32) + np.float32(0.25)
+    w = rng.uniform(0.5, 1.5, (e, 1)).astype(np.float32)
+    if bf16:
+        x, m = to_bf16_f32(x), to_bf16_f32(m)
+    xd, md, wd = _dev(x, device, bf16), _dev(m, device, bf16), _dev(w, device)
+    adj = (arr.in_pointer, arr.in_node_indices, arr.in_edge_indices)
+    tol = TOL_BF16 if bf16 else TOL_F32
+    cases = (("copy_u", lambda: ops.SpMMSrc(xd, [1], False, None, g), (x, None)),
+             ("copy_e", lambda: ops.SpMMEdge(md, [1], False, None, g), (m, None)),
+             ("u_mul_e", lambda: ops.gspmm_src_mul_e_sum(xd, wd, [1], False, None, g), (x, w)),
+             ("u_div_e", lambda: ops.spmm(g, "u_div_e", "sum", xd, wd), (x, w)))
+    for op, fn, (u, ww) in cases:
+        got = fn()
+        assert got.dtype == xd.dtype and got.shape == (n, feat)
+        ref = oracle.spmm(*adj, u, ww, op=op)
+        mag = oracle.spmm(*adj, np.abs(u), ww, op=op)
+        assert_close(got.float().cpu().numpy(), ref, tol, f"{op} F={feat} bf16={bf16}", mag=mag)
+        assert not got[n // 2:].any()               # rows without in-edges
+        assert torch.equal(got, fn())               # the same bits every time
+    got = ops.spmm_scaled(xd, g, row_scale=_dev(np.full((n, 1), 0.5, np.float32), device), activation="relu")
+    want = np.maximum(oracle.spmm(*adj, x, op="copy_u") * 0.5, 0)
+    assert_close(got.float().cpu().numpy(), want, tol, f"scaled F={feat} bf16={bf16}",
+                 mag=oracle.spmm(*adj, np.abs(x), op="copy_u") * 0.5)
+
+
 def test_spmm_scaled_non_finite_factor_and_arguments(device):
     """A row without edges is 0 * factor: an infinite factor (degree 0 to the power -1/2)
     shows as NaN there, as it does after the separate multiplication."""
