@@ -197,57 +197,72 @@ int launch_spmm(const int32_t *pointer, const int32_t *row_of_slot,
                         partial, stream, partial_bytes);
 }
 
-// ---- sums of rows of at most four features: one lane per slot -----------------
-// With one lane per row a lane group of the run schedule is a single lane: every
-// lane walks a run of its own, so a wave instruction reads 64 separate pieces of the
-// slot-indexed columns and nothing of the walk coalesces (copy_u with one feature on
-// 11.6 M edges: 129 us for 93 MB).  Here a lane owns one SLOT: the wavefront reads 64
-// consecutive slots of the columns with one access each, gathers their rows (a lane
-// holds the row's one to four features), and adds up the slots of each row with a
-// segmented scan over the lanes -- rows are sorted, so lanes with equal row ids at
-// distance d have that id in between, and the scan stops at the first distance at
-// which no lane finds its own row.  A wavefront owns 2^k consecutive chunks of 64
-// slots; the segment that runs into the next chunk is carried in a register.  The
-// first and the last segment of a wavefront's range may be pieces of a longer row:
-// they take the route of the run schedule -- the four wavefronts of a workgroup chain
-// their pieces through LDS, and what crosses the workgroup's slot range leaves the
-// same two partial states per workgroup that runs_kernel leaves, so the second
-// kernel is runs_fixup_kernel of the one-lane-per-row layout, unchanged.  Additions
-// of a row happen in the scan's tree order, fixed by the slot positions.
+// ---- sums of rows of at most eight features: one or two lanes per slot --------
+// With one or two lanes per row a lane group of the run schedule walks a run of its
+// own, so a wave instruction reads 32 or 64 separate pieces of the slot-indexed columns
+// and nothing of the walk coalesces (copy_u with one feature on 11.6 M edges: 129 us
+// for 93 MB).  Here L = 1 or 2 adjacent lanes own one SLOT (a lane holds up to four of
+// the row's features, L apart): the wavefront reads 64 / L consecutive slots of the
+// columns with one access each, gathers their rows, and adds up the slots of each row
+// with a segmented scan over the lanes -- rows are sorted, so lanes with equal row ids
+// at distance d have that id in between: DPP shifts inside rows of 16 lanes, then the
+// totals at the end of a row of lanes go to the lanes of the next one that continue
+// its segment.  A wavefront owns up to 16 consecutive chunks; the segment that runs
+// into the next chunk is carried in registers.  The first and the last segment of a
+// wavefront's range may be pieces of a longer row: they take the route of the run
+// schedule -- the four wavefronts of a workgroup chain their pieces through LDS, and
+// what crosses the workgroup's slot range leaves the same two partial states per
+// workgroup that runs_kernel leaves, so the second kernel is runs_fixup_kernel of the
+// L-lanes-per-row layout, unchanged.  Additions of a row happen in the scan's tree
+// order, fixed by the slot positions.
 constexpr int kSlotUnroll = 4;   // chunks whose loads are in flight together
 
 // One step of the segmented scan inside rows of 16 lanes: a lane whose neighbour OFF
 // lanes down (in its row of lanes) holds the same key adds that neighbour's sums.  Lanes
 // without such a neighbour see the key -3, which no slot has.
 template <int OFF>
-__device__ __forceinline__ void slots_scan16(int key, float (&acc)[4], int feat) {
+__device__ __forceinline__ void slots_scan16(int key, float (&acc)[4], int live) {
   const int pk = __builtin_amdgcn_update_dpp(-3, key, 0x110 + OFF, 0xF, 0xF, false);   // row_shr:OFF
   const bool hit = pk == key;
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
-    if (v < feat) {                          // uniform
+    if (v < live) {                          // uniform: the most features a lane holds
       const float pv = __int_as_float(__builtin_amdgcn_update_dpp(
           0, __float_as_int(acc[v]), 0x110 + OFF, 0xF, 0xF, false));
       if (hit) acc[v] += pv;
     }
   }
 }
-// The lanes of row ROW whose key is that of the last lane of the row before add that
-// lane's (already complete) sums.
-template <int ROW>
-__device__ __forceinline__ void slots_row_carry(int key, float (&acc)[4], int feat, int lane) {
+// The lanes of row ROW whose key is that of the last slot of the row before add that
+// slot's (already complete) sums: lane 16 ROW - L + (lane mod L) holds them.
+template <int ROW, int L>
+__device__ __forceinline__ void slots_row_carry(int key, float (&acc)[4], int live, int lane) {
   const int ck = __builtin_amdgcn_readlane(key, 16 * ROW - 1);
   const bool hit = (lane >> 4) == ROW && key == ck;
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
-    if (v < feat) {
-      const float cv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc[v]), 16 * ROW - 1));
+    if (v < live) {
+      float cv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc[v]), 16 * ROW - 1));
+      if (L == 2) {
+        const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc[v]), 16 * ROW - 2));
+        cv = (lane & 1) ? cv : c0;
+      }
       if (hit) acc[v] += cv;
     }
   }
 }
+// v of lane `from + (lane mod L)` (from: uniform, a multiple of L) in every lane
+template <int L>
+__device__ __forceinline__ float slots_from(float v, int from, int lane) {
+  float r = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), from));
+  if (L == 2) {
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), from + 1));
+    r = (lane & 1) ? r1 : r;
+  }
+  return r;
+}
 
-template <class P, int BOP>
+template <class P, int BOP, int LS>
 __global__ __launch_bounds__(kBlock) void slots_kernel(
     typename P::Args args, const int32_t *__restrict__ pointer,
     const int32_t *__restrict__ row_of_slot, typename P::out_t *__restrict__ out,
@@ -258,19 +273,24 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
   constexpr bool EPI = SF > 4;
   constexpr bool HASW = BOP != 0;
   constexpr int kWaves = kBlock / kWave;
-  if ((int64_t)blockIdx.x >= geo.n_wg) {   // rows without edges, one lane per row
-    const int64_t row = ((int64_t)blockIdx.x - geo.n_wg) * kBlock + threadIdx.x;
+  constexpr int L = 1 << LS;             // lanes per slot
+  constexpr int kChunk = kWave >> LS;    // slots per chunk
+  const int sub = threadIdx.x & (L - 1); // the lane's first feature
+  if ((int64_t)blockIdx.x >= geo.n_wg) {   // rows without edges, L lanes per row
+    const int64_t row = (((int64_t)blockIdx.x - geo.n_wg) * kBlock + threadIdx.x) >> LS;
     if (row < geo.n_rows && pointer[row] == pointer[row + 1])
-      P::emit_empty(args, out, row, geo.feat, 0);
+      P::emit_empty(args, out, row, geo.feat, sub);
     return;
   }
-  __shared__ float piece[kWaves][2][SF];   // [wavefront][A | B][state]
+  __shared__ float piece[kWaves][2][L][SF];   // [wavefront][A | B][lane of the slot][state]
   __shared__ RunFlags flags[kWaves];
   const int lane = threadIdx.x & (kWave - 1);
+  const int slot_lane = lane >> LS;
   const int wave = threadIdx.x / kWave;
   const int feat = geo.feat;
-  const typename IO::lane_t ln = IO::lane(0, feat);
-  const int wg_shift = geo.run_shift + 8;
+  const typename IO::lane_t ln = IO::lane(LS, feat - sub);
+  const int live = (feat + L - 1) >> LS;   // features of the slot's first lane (the most)
+  const int wg_shift = geo.run_shift + 8 - LS;
   const int64_t wave_slots = (int64_t)1 << (wg_shift - 2);
   const int64_t wa = ((int64_t)blockIdx.x << wg_shift) + wave * wave_slots;
   const int64_t wb = min(wa + wave_slots, geo.n_edges);
@@ -293,7 +313,7 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
     auto load_ids = [&](int64_t j0, Ids &I) {
 #pragma unroll
       for (int c = 0; c < kSlotUnroll; ++c) {
-        const int64_t j = j0 + c * kWave + lane;
+        const int64_t j = j0 + c * kChunk + slot_lane;
         const int64_t jc = j < wb ? j : wb - 1;
         I.r[c] = row_of_slot[jc];
         I.rn[c] = jc + 1 < geo.n_edges ? row_of_slot[jc + 1] : -1;
@@ -303,17 +323,18 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
     };
     Ids cur;
     load_ids(wa, cur);
-    for (int64_t j0 = wa; j0 < wb; j0 += kSlotUnroll * kWave) {
+    for (int64_t j0 = wa; j0 < wb; j0 += kSlotUnroll * kChunk) {
       float val[kSlotUnroll][4], rs[kSlotUnroll];
       typename IO::raw_t x[kSlotUnroll];
 #pragma unroll
       for (int c = 0; c < kSlotUnroll; ++c) {
-        x[c] = IO::load(args.u + cur.g[c] * feat, ln);
+        x[c] = IO::load(args.u + cur.g[c] * feat + sub, ln);
         if (EPI) rs[c] = args.row_scale ? args.row_scale[cur.r[c]] : 1.0f;
         if (HASW) {
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
-            const int h = min(v / args.dph, args.heads - 1);   // dead features: any valid weight
+            // the weight of feature sub + v L; dead features: any valid weight
+            const int h = min((sub + (v << LS)) / args.dph, args.heads - 1);
             val[c][v] = args.w[cur.e[c] * args.heads + h];
           }
         }
@@ -324,12 +345,12 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
         r[c] = cur.r[c];
         rn[c] = cur.rn[c];
       }
-      if (j0 + kSlotUnroll * kWave < wb) load_ids(j0 + kSlotUnroll * kWave, cur);
+      if (j0 + kSlotUnroll * kChunk < wb) load_ids(j0 + kSlotUnroll * kChunk, cur);
 #pragma unroll
       for (int c = 0; c < kSlotUnroll; ++c) {
-        const int64_t c0 = j0 + c * kWave;   // uniform
+        const int64_t c0 = j0 + c * kChunk;   // uniform
         if (c0 >= wb) break;
-        const bool valid = c0 + lane < wb;
+        const bool valid = c0 + slot_lane < wb;
         float xf[4];
         IO::widen(x[c], xf);
         int key = valid ? r[c] : -2;         // lanes past the range: a row id no slot has
@@ -339,20 +360,18 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
           const float m = HASW ? bin_apply<BOP>(xf[v], val[c][v]) : xf[v];
           acc[v] = valid ? m : 0.0f;
         }
-        if (lane == 0 && key == carry_key) {
+        if (slot_lane == 0 && key == carry_key) {
 #pragma unroll
           for (int v = 0; v < 4; ++v) acc[v] = carry[v] + acc[v];
         }
-        // inclusive segmented sum over the lanes: inside each row of 16 lanes with
-        // DPP shifts, then the total at the end of a row of lanes goes to the lanes of
-        // the next one that continue its segment (through a scalar register)
-        slots_scan16<1>(key, acc, feat);
-        slots_scan16<2>(key, acc, feat);
-        slots_scan16<4>(key, acc, feat);
-        slots_scan16<8>(key, acc, feat);
-        slots_row_carry<1>(key, acc, feat, lane);
-        slots_row_carry<2>(key, acc, feat, lane);
-        slots_row_carry<3>(key, acc, feat, lane);
+        // inclusive segmented sum over the slots of the chunk
+        if (L == 1) slots_scan16<1>(key, acc, live);
+        slots_scan16<2>(key, acc, live);
+        slots_scan16<4>(key, acc, live);
+        slots_scan16<8>(key, acc, live);
+        slots_row_carry<1, L>(key, acc, live, lane);
+        slots_row_carry<2, L>(key, acc, live, lane);
+        slots_row_carry<3, L>(key, acc, live, lane);
         const bool is_end = valid && rn[c] != key;
         if (is_end) {
           float st[SF];
@@ -361,26 +380,25 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
           if (EPI) st[4] = rs[c];
           if (key == first_key && first_open) {   // the piece of a row that began before this range
 #pragma unroll
-            for (int i = 0; i < SF; ++i) piece[wave][0][i] = st[i];
+            for (int i = 0; i < SF; ++i) piece[wave][0][sub][i] = st[i];
             flags[wave].has_a = 1;
             flags[wave].row_a = key;
           } else {
-            P::emit(args, out, key, feat, 0, st);
+            P::emit(args, out, key, feat, sub, st);
           }
         }
         // the segment of the last slot runs on into the next chunk (or past the range)
-        const int last = (int)min((int64_t)kWave - 1, wb - 1 - c0);   // uniform
+        const int last = (int)min((int64_t)kChunk - 1, wb - 1 - c0) << LS;   // its first lane, uniform
         const bool open = !__builtin_amdgcn_readlane((int)is_end, last);
         carry_key = open ? __builtin_amdgcn_readlane(key, last) : -1;
 #pragma unroll
-        for (int v = 0; v < 4; ++v)
-          carry[v] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc[v]), last));
+        for (int v = 0; v < 4; ++v) carry[v] = slots_from<L>(acc[v], last, lane);
         if (EPI) carry_scale = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rs[c]), last));
       }
     }
-    if (carry_key != -1 && lane == 0) {      // the range ends inside a row
+    if (carry_key != -1 && lane < L) {       // the range ends inside a row
       const bool through = carry_key == first_key && first_open;   // ... that also began before it
-      float *dst = piece[wave][through ? 0 : 1];
+      float *dst = piece[wave][through ? 0 : 1][sub];
 #pragma unroll
       for (int v = 0; v < 4; ++v) dst[v] = carry[v];
       if (EPI) dst[4] = carry_scale;
@@ -394,7 +412,7 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
     }
   }
   __syncthreads();
-  if (lane != 0 || wa >= wb) return;
+  if (lane >= L || wa >= wb) return;
   // the pieces of the workgroup's wavefronts, chained as runs_kernel chains its runs
   auto chain_into = [&](int i, float (&acc)[SF]) -> bool {
     int j = i - 1;
@@ -402,21 +420,21 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
     const bool starts_inside = j >= 0;
     if (starts_inside) {
 #pragma unroll
-      for (int q = 0; q < SF; ++q) acc[q] = piece[j][1][q];
+      for (int q = 0; q < SF; ++q) acc[q] = piece[j][1][sub][q];
     } else {
       P::init(acc);
     }
-    for (int g = j + 1; g <= i; ++g) P::merge(acc, piece[g][0]);
+    for (int g = j + 1; g <= i; ++g) P::merge(acc, piece[g][0][sub]);
     return starts_inside;
   };
-  float *const gp = partial + (int64_t)blockIdx.x * 2 * SF;
+  float *const gp = partial + ((int64_t)blockIdx.x * 2 * L + sub) * SF;   // slot 1: L * SF further
   const int64_t slots_left = geo.n_edges - ((int64_t)blockIdx.x << wg_shift);
   const int last_wave = (int)min((int64_t)kWaves, (slots_left + wave_slots - 1) / wave_slots) - 1;
   const bool has_a = flags[wave].has_a, a_open = flags[wave].a_open, has_b = flags[wave].has_b;
   if (has_a && !a_open) {
     float acc[SF];
     if (chain_into(wave, acc)) {
-      P::emit(args, out, flags[wave].row_a, feat, 0, acc);
+      P::emit(args, out, flags[wave].row_a, feat, sub, acc);
     } else {
 #pragma unroll
       for (int q = 0; q < SF; ++q) gp[q] = acc[q];
@@ -425,23 +443,32 @@ __global__ __launch_bounds__(kBlock) void slots_kernel(
   if (wave == last_wave) {
     if (has_b) {
 #pragma unroll
-      for (int q = 0; q < SF; ++q) gp[SF + q] = piece[wave][1][q];
+      for (int q = 0; q < SF; ++q) gp[L * SF + q] = piece[wave][1][sub][q];
     } else if (has_a && a_open) {
       float acc[SF];
       const bool inside = chain_into(wave, acc);
-      float *p = gp + (inside ? SF : 0);
+      float *p = gp + (inside ? L * SF : 0);
 #pragma unroll
       for (int q = 0; q < SF; ++q) p[q] = acc[q];
     }
   }
 }
 
-// Slots per workgroup: 256 << run_shift -- one chunk per wavefront on small graphs,
-// up to 16 on large ones (measured on 11.6 M edges, one feature, us by slots per
-// workgroup: 256: 189, 512: 129, 1024: 97, 2048: 93, 4096: 95, 8192: 98, 16384: 120);
-// never fewer slots than four runs of the run schedule, whose workspace bound the
-// caller sized.
-template <typename T, int BOP, bool EPI = false, int ACT = GA_ACT_NONE>
+// Slots per workgroup: a power of two from 256 to 4096, for about 2048 workgroups
+// (measured on 11.6 M edges, one feature, us by slots per workgroup: 256: 189, 512:
+// 129, 1024: 97, 2048: 93, 4096: 95, 8192: 98, 16384: 120; on 1 M edges 1024 slots, 977
+// workgroups: 16 against 20 with 256 slots); never fewer slots than four runs of the
+// run schedule, whose workspace bound the caller sized.
+// Where the lanes-per-slot kernel is the faster one: rows of up to four features
+// everywhere (11.6 M edges, us: copy_u with one feature 129 -> 93, three 165 -> 104;
+// 108 k edges: three features 22 -> 14); five to seven features, with two lanes per slot
+// and so twice the chunks, on small graphs only (108 k edges 21 -> 14; 1 M edges 23 -> 26;
+// eight features tile 16-byte accesses and are as fast on the run schedule).
+inline bool slots_preferred(int64_t n_edges, int64_t feat) {
+  return feat <= 4 || (feat <= 7 && n_edges <= 300000);
+}
+
+template <typename T, int BOP, int LS, bool EPI = false, int ACT = GA_ACT_NONE>
 int launch_spmm_slots(const int32_t *pointer, const int32_t *row_of_slot, const int32_t *gidx,
                       const int32_t *eid, const void *u, const float *w, void *out,
                       int64_t n_rows, int64_t n_edges, int feat, int heads, float *partial,
@@ -449,26 +476,28 @@ int launch_spmm_slots(const int32_t *pointer, const int32_t *row_of_slot, const 
                       size_t partial_bytes = SIZE_MAX) {
   typedef SpmmPolicy<T, 4, GA_SUM, BOP, true, EPI, ACT> P;
   constexpr int SF = P::kState;
-  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads, false, 0, row_scale};
+  constexpr int L = 1 << LS;
+  typename P::Args args{gidx, eid, (const T *)u, w, heads, feat / heads, false, LS, row_scale};
   RunGeom geo;
-  int wg_shift = ilog2_ceil((uint64_t)((n_edges + 8191) / 8192));
+  int wg_shift = ilog2_ceil((uint64_t)((n_edges + 2047) / 2048));
   const int floor_shift = std::max(8, run_shift_for(n_edges, feat) + 2);
   wg_shift = std::min(std::max(wg_shift, floor_shift), std::max(12, floor_shift));
-  geo.run_shift = wg_shift - 8;
-  geo.tpr_shift = 0;
-  geo.lanes_total = 1;
+  geo.tpr_shift = LS;
+  geo.run_shift = wg_shift - 8 + LS;       // the second kernel's slots per workgroup: run << (8 - LS)
+  geo.lanes_total = L;
   geo.feat = feat;
   geo.n_edges = n_edges;
   geo.n_rows = n_rows;
   const int64_t n_wg = (n_edges + ((int64_t)1 << wg_shift) - 1) >> wg_shift;
-  geo.n_runs = n_wg * kBlock;
+  geo.n_runs = n_wg * (kBlock >> LS);
   geo.n_wg = n_wg;
-  const int64_t row_blocks = (n_rows + kBlock - 1) / kBlock;
+  const int G = kBlock >> LS;              // rows per block of the trailing blocks and of the second kernel
+  const int64_t row_blocks = (n_rows + G - 1) / G;
   if (n_wg + row_blocks > 0x7fffffff) return GA_EUNSUPPORTED;
-  if ((size_t)n_wg * 2 * SF * sizeof(float) > partial_bytes) return GA_EWORKSPACE;
-  hipLaunchKernelGGL((slots_kernel<P, BOP>), dim3((unsigned)(n_wg + row_blocks)), dim3(kBlock), 0,
-                     stream, args, pointer, row_of_slot, (T *)out, partial, geo);
-  const int64_t fix_blocks = (n_wg + kBlock - 1) / kBlock;
+  if ((size_t)n_wg * 2 * L * SF * sizeof(float) > partial_bytes) return GA_EWORKSPACE;
+  hipLaunchKernelGGL((slots_kernel<P, BOP, LS>), dim3((unsigned)(n_wg + row_blocks)), dim3(kBlock),
+                     0, stream, args, pointer, row_of_slot, (T *)out, partial, geo);
+  const int64_t fix_blocks = (n_wg + G - 1) / G;
   hipLaunchKernelGGL((runs_fixup_kernel<P>), dim3((unsigned)fix_blocks), dim3(kBlock),
                      (size_t)kBlock * SF * sizeof(float), stream, args, pointer, row_of_slot,
                      partial, (T *)out, geo, n_wg, (int)fix_blocks);
@@ -738,12 +767,18 @@ int ga_spmm_csr(const int32_t *pointer, const int32_t *row_of_slot,
   const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
   hipStream_t s = (hipStream_t)stream;
   float *partial = (float *)workspace;
-  // sums of rows of up to four features: one lane per slot
-  if (reduce == GA_SUM && feat <= 4 && n_edges > 0) {
-#define GA_SPMM_SLOTS(T, B)                                                                  \
-  return ga::launch_spmm_slots<T, B>(pointer, row_of_slot, gidx, eid, u, w, out, n_rows,     \
-                                     n_edges, (int)feat, (int)heads, partial, s, nullptr,    \
-                                     workspace_bytes)
+  // sums of rows of up to eight features: one or two lanes per slot
+  if (reduce == GA_SUM && n_edges > 0 && ga::slots_preferred(n_edges, feat)) {
+#define GA_SPMM_SLOTS(T, B)                                                                   \
+  do {                                                                                        \
+    if (feat <= 4)                                                                            \
+      return ga::launch_spmm_slots<T, B, 0>(pointer, row_of_slot, gidx, eid, u, w, out,       \
+                                            n_rows, n_edges, (int)feat, (int)heads, partial,  \
+                                            s, nullptr, workspace_bytes);                     \
+    return ga::launch_spmm_slots<T, B, 1>(pointer, row_of_slot, gidx, eid, u, w, out, n_rows, \
+                                          n_edges, (int)feat, (int)heads, partial, s,         \
+                                          nullptr, workspace_bytes);                          \
+  } while (0)
 #define GA_SPMM_SLOTS_T(T)                                  \
   switch (bop) {                                            \
     case GA_U_MUL_E: GA_SPMM_SLOTS(T, GA_U_MUL_E);          \
@@ -818,11 +853,17 @@ int ga_spmm_csr_scaled(const int32_t *pointer, const int32_t *row_of_slot,
   const bool vec_ok = ga::aligned(out, 16) && (!u || ga::aligned(u, 16));
   hipStream_t s = (hipStream_t)stream;
   float *partial = (float *)workspace;
-  if (feat <= 4 && n_edges > 0) {                        // one lane per slot
-#define GA_SPMM_SLOTS_EPI(T, ACT)                                                            \
-  return ga::launch_spmm_slots<T, 0, true, ACT>(pointer, row_of_slot, gidx, eid, u, nullptr, \
-                                                out, n_rows, n_edges, (int)feat, 1, partial, \
-                                                s, row_scale, workspace_bytes)
+  if (n_edges > 0 && ga::slots_preferred(n_edges, feat)) {   // one or two lanes per slot
+#define GA_SPMM_SLOTS_EPI(T, ACT)                                                                 \
+  do {                                                                                            \
+    if (feat <= 4)                                                                                \
+      return ga::launch_spmm_slots<T, 0, 0, true, ACT>(pointer, row_of_slot, gidx, eid, u,        \
+                                                       nullptr, out, n_rows, n_edges, (int)feat,  \
+                                                       1, partial, s, row_scale, workspace_bytes); \
+    return ga::launch_spmm_slots<T, 0, 1, true, ACT>(pointer, row_of_slot, gidx, eid, u, nullptr, \
+                                                     out, n_rows, n_edges, (int)feat, 1, partial, \
+                                                     s, row_scale, workspace_bytes);              \
+  } while (0)
 #define GA_SPMM_SLOTS_EPI_T(T)                                        \
   do {                                                                \
     if (activation == GA_ACT_RELU) GA_SPMM_SLOTS_EPI(T, GA_ACT_RELU); \

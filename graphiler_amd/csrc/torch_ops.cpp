@@ -345,7 +345,7 @@ torch::Tensor SpMMSrc(torch::Tensor features, std::vector<int64_t> dims,
 // ga_activation.  The kernel takes a factor that is one fp32 number per row, shaped to
 // broadcast over the row ((N, 1) for (N, F) features), on fp32 features; any other
 // factor is multiplied afterwards with torch's own broadcasting and promotion, and so
-// is the tail of a small sum of more than four features that 16-byte accesses do not tile.
+// is the tail of a small sum whose width neither kernel takes at no cost.
 torch::Tensor SpMMScaled(torch::Tensor features, at::optional<torch::Tensor> row_scale,
                          int64_t activation, bool edge_rows, const GraphPtr &graph) {
   TORCH_CHECK(activation >= GA_ACT_NONE && activation <= GA_ACT_ELU, "unknown activation");
@@ -358,12 +358,14 @@ torch::Tensor SpMMScaled(torch::Tensor features, at::optional<torch::Tensor> row
     per_row = f.is_cuda() && f.scalar_type() == at::kFloat && dt == GA_F32 &&
               f.dim() == std::max<int64_t>(features.dim(), 2) && f.size(0) == n && f.numel() == n;
   }
-  // a small result of more than four features whose rows 16-byte accesses do not tile: the
-  // sum alone plus two short elementwise kernels is the faster route (measured at 19,717
-  // nodes x 5 and 7 features)
-  const int64_t row_bytes = feat_dim(features) * features.element_size();
-  const bool tail_pays = feat_dim(features) <= 4 || row_bytes % 16 == 0 ||
-                         n * row_bytes >= (int64_t(8) << 20);
+  // the tail is free on the lanes-per-slot kernel (up to four features; five to seven on
+  // graphs of up to 300,000 edges) and cheap for rows that 16-byte accesses tile; for a
+  // small result of any other width the sum alone plus two short elementwise kernels is
+  // the faster route (measured at 19,717 nodes x 9 features)
+  const int64_t width = feat_dim(features);
+  const int64_t row_bytes = width * features.element_size();
+  const bool on_slots = width <= 4 || (width <= 7 && graph->num_edges <= 300000);
+  const bool tail_pays = on_slots || row_bytes % 16 == 0 || n * row_bytes >= (int64_t(8) << 20);
   const bool has_tail = row_scale.has_value() || activation != GA_ACT_NONE;
   if ((row_scale.has_value() && !per_row) || (has_tail && !tail_pays)) {
     torch::Tensor out = spmm(graph, edge_rows ? GA_COPY_E : GA_COPY_U, GA_SUM, features, at::nullopt, false);

@@ -159,20 +159,23 @@ def SpMMEdge(features, dims: Sequence[int], keep_dim: bool, dtype,
     return spmm(graph, "copy_e", "sum", features)
 
 
-# A row factor / activation in the sum's store is free for rows of up to four features
-# (one lane per slot) and for rows that 16-byte accesses tile.  For the other widths (the
-# one-feature-per-lane layout of the run schedule) it pays from a result of this size on:
-# measured on 19,717 nodes, the 5- or 7-wide sum with the tail takes 31-34 us against
-# 26-27 us for the sum and two elementwise kernels; from 232,965 nodes on the tail in
-# the store wins for every width (4-8 % of the sum).
+# A row factor / activation in the sum's store is free on the lanes-per-slot kernel (rows
+# of up to four features; five to seven features on graphs of up to 300,000 edges, the
+# library's own rule) and cheap for rows that 16-byte accesses tile.  For the other
+# widths (the one-feature-per-lane layout of the run schedule) it pays from a result of
+# SPMM_TAIL_MIN_BYTES on: measured on 19,717 nodes, the 9-wide sum with the tail takes
+# 24 us against 16 us without and 24 us with two elementwise kernels after it; from
+# 232,965 nodes on the tail in the store wins for every width (4-8 % of the sum).
 SPMM_TAIL_MIN_BYTES = 8 << 20
+SPMM_SLOTS_MAX_EDGES_5_TO_7 = 300_000
 
 
 def spmm_tail_preferred(features, graph: DGLGraph) -> bool:
     """Whether ``spmm_scaled`` beats the sum followed by elementwise operators."""
     feat = get_feat_dim(features)
     row_bytes = feat * features.element_size()
-    return feat <= 4 or row_bytes % 16 == 0 or graph.num_nodes * row_bytes >= SPMM_TAIL_MIN_BYTES
+    on_slots = feat <= 4 or (feat <= 7 and graph.num_edges <= SPMM_SLOTS_MAX_EDGES_5_TO_7)
+    return on_slots or row_bytes % 16 == 0 or graph.num_nodes * row_bytes >= SPMM_TAIL_MIN_BYTES
 
 
 def spmm_scaled(features, graph: DGLGraph, row_scale=None, activation=None,

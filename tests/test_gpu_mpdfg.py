@@ -47,7 +47,7 @@ def gcn_both_norms_reduce(nodes: NodeBatchDummy):
 
 
 @pytest.mark.parametrize("level", [0, 1, 2])
-@pytest.mark.parametrize("width", [16, 3, 5])
+@pytest.mark.parametrize("width", [16, 3, 5, 9])
 def test_gcn_plan_with_both_norms(device, level, width):
     """A destination-side norm and elu after the sum (the symmetric normalisation of a
     graph convolution): at level 2 both are arguments of the sum operator."""

@@ -152,10 +152,10 @@ def test_spmm_scaled_is_the_separate_operators(graph, device, feat, op, bf16):
                        (ops.SpMMSrc if op == "copy_u" else ops.SpMMEdge)(xd, [1], False, None, g))
 
 
-@pytest.mark.parametrize("feat", [1, 2, 3, 4])
+@pytest.mark.parametrize("feat", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("bf16", [False, True])
 def test_narrow_sums_with_a_row_across_many_workgroups(device, feat, bf16):
-    """Rows of at most four features take the one-lane-per-slot kernel; a destination
+    """Rows of at most eight features take the lanes-per-slot kernel; a destination
     with 380,000 in-edges spans hundreds of its workgroups (the cooperative fold of the
     second kernel), next to short rows, rows without edges and a shuffled edge order."""
     rng = np.random.default_rng(40 + feat)
