@@ -1351,3 +1351,23 @@ def test_linear_attn_unsupported_shapes(device):
     with pytest.raises(capi.GraphilerError):
         ops.linear_attn(x, torch.ones(8, 16, device=device),
                         torch.ones(2, 8, device=device), torch.ones(2, 8, device=device))
+
+
+def test_graph_without_nodes(device):
+    """Zero nodes and zero edges: every operator returns a tensor with no rows."""
+    none = np.zeros(0, np.int64)
+    g = prepare_graph(none, none, 0, device=device)
+    assert g.num_nodes == 0 and g.num_edges == 0 and g.in_pointer.cpu().tolist() == [0]
+    x = torch.zeros(0, 8, device=device)
+    e1 = torch.zeros(0, 1, device=device)
+    assert ops.SpMMSrc(x, [1], False, None, g).shape == (0, 8)
+    assert ops.SpMMEdge(x, [1], False, None, g).shape == (0, 8)
+    assert ops.gspmm_src_mul_e_sum(x, e1, [1], False, None, g).shape == (0, 8)
+    assert ops.spmm_scaled(x, g, row_scale=e1, activation="relu").shape == (0, 8)
+    assert ops.spmm(g, "copy_u", "max", x).shape == (0, 8)
+    assert ops.gsddmm_u_add_v_mul_alpha(e1, e1, 1, g).shape == (0, 1)
+    assert ops.gsddmm_u_dot_v(x, x, g).shape[0] == 0
+    assert ops.SegmentSoftmax(e1, 1, None, g).shape == (0, 1)
+    assert ops.BroadcastSrcNode(x, g).shape == (0, 8)
+    assert ops.gat_aggregate(e1, e1, x, g, 0.2).shape == (0, 8)
+    assert ops.edge_softmax_sum(e1, x, g).shape == (0, 8)
