@@ -88,13 +88,17 @@ template <> struct XVec<1> { using type = float; };
 // one, the row's last vector) and zero by select at commit time, where the
 // value is consumed anyway; no lane is ever predicated off in the k loop.
 // WAVES: waves per SIMD the register allocation aims at (3 or 2)
-template <bool HAS_ATTN, int VK, int WAVES>
+// NCB: column blocks multiplied and stored, 4 or -- the plain projection onto at most 16
+// columns (a GCN layer's hidden width) -- 1; the W tile is staged 64 columns wide either
+// way, what shrinks is the matrix work and the operand reads.
+template <bool HAS_ATTN, int VK, int WAVES, int NCB = kCB>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void
 linear_attn_kernel(
     const float *__restrict__ X, const float *__restrict__ W,
     const float *__restrict__ a_l, const float *__restrict__ a_r,
     float *__restrict__ Z, float *__restrict__ el, float *__restrict__ er,
     const float *__restrict__ row_scale, int64_t rows, int K, int M, int heads) {
+  static_assert(NCB == kCB || !HAS_ATTN, "the attention epilogue pairs up all four column blocks");
   using xvec_t = typename XVec<VK>::type;
   __shared__ __attribute__((aligned(16))) float xs[kWgRows * kXs];   // wave-private rows, one buffer
   __shared__ __attribute__((aligned(16))) uint32_t wb[2][3][kPassCols * kWb];
@@ -179,11 +183,11 @@ linear_attn_kernel(
     *reinterpret_cast<uint4 *>(&wb[buf][2][wc * kWb + wkg * 4]) = p2;
   };
 
-  floatx4 acc[kRT][kCB];
+  floatx4 acc[kRT][NCB];
 #pragma unroll
   for (int t = 0; t < kRT; ++t)
 #pragma unroll
-    for (int cb = 0; cb < kCB; ++cb) acc[t][cb] = floatx4{0, 0, 0, 0};
+    for (int cb = 0; cb < NCB; ++cb) acc[t][cb] = floatx4{0, 0, 0, 0};
 
   const int xl_ofs = (wave * kWaveRows + lr) * kXs + lk * 8;
   const int wl_ofs = lr * kWb + lk * 4;                  // in uint32 (pairs of bf16)
@@ -213,8 +217,8 @@ linear_attn_kernel(
     }
     constexpr int px[6] = {2, 0, 1, 1, 0, 0}, pw[6] = {0, 2, 1, 0, 1, 0};
 #pragma unroll
-    for (int cb = 0; cb < kCB; ++cb) {
-      if (cb + 1 < kCB) read_w(cb + 1, wf[(cb + 1) & 1]);
+    for (int cb = 0; cb < NCB; ++cb) {
+      if (cb + 1 < NCB) read_w(cb + 1, wf[(cb + 1) & 1]);
 #pragma unroll
       for (int q = 0; q < 6; ++q)
 #pragma unroll
@@ -254,7 +258,7 @@ linear_attn_kernel(
   float al[kCB], ar[kCB];
   const int dph = M / heads;
   const int bph = dph >> 4;                              // column blocks per head
-  if (HAS_ATTN) {
+  if constexpr (HAS_ATTN) {
 #pragma unroll
     for (int cb = 0; cb < kCB; ++cb) {
       const int c = col0 + cb * 16 + lr;
@@ -270,14 +274,14 @@ linear_attn_kernel(
       const bool live = row < rows;
       if (!HAS_ATTN && row_scale) {                      // the plain projection only
 #pragma unroll
-        for (int cb = 0; cb < kCB; ++cb) acc[t][cb][r] *= rsv[t][r];
+        for (int cb = 0; cb < NCB; ++cb) acc[t][cb][r] *= rsv[t][r];
       }
 #pragma unroll
-      for (int cb = 0; cb < kCB; ++cb) {
+      for (int cb = 0; cb < NCB; ++cb) {
         const int c = col0 + cb * 16 + lr;
         if (live && c < M) Z[row * M + c] = acc[t][cb][r];
       }
-      if (HAS_ATTN) {
+      if constexpr (HAS_ATTN) {
         // lane-local products, blocks of one head added, then one 16-lane tree
         float pl[kCB], pr[kCB];
 #pragma unroll
@@ -332,10 +336,15 @@ int launch_linear(const float *X, const float *W, const float *a_l, const float 
   const int64_t gy = (M + kPassCols - 1) / kPassCols;
   if (gx > 0x7fffffff || gy > 65535) return GA_EUNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
-#define GA_LAUNCH_LINEAR(ATTN, VK, WAVES)                                          \
-  hipLaunchKernelGGL((linear_attn_kernel<ATTN, VK, WAVES>), dim3((unsigned)gx, (unsigned)gy), \
-                     dim3(kBlock), 0, s, X, W, a_l, a_r, Z, el, er, row_scale, rows, \
-                     (int)K, (int)M, (int)heads)
+#define GA_LAUNCH_LINEAR_NCB(ATTN, VK, WAVES, NCB)                                  \
+  hipLaunchKernelGGL((linear_attn_kernel<ATTN, VK, WAVES, NCB>),                   \
+                     dim3((unsigned)gx, (unsigned)gy), dim3(kBlock), 0, s, X, W, a_l, a_r, Z, el, \
+                     er, row_scale, rows, (int)K, (int)M, (int)heads)
+#define GA_LAUNCH_LINEAR(ATTN, VK, WAVES)                           \
+  do {                                                              \
+    if (!ATTN && M <= 16) GA_LAUNCH_LINEAR_NCB(false, VK, WAVES, 1); \
+    else GA_LAUNCH_LINEAR_NCB(ATTN, VK, WAVES, kCB);                 \
+  } while (0)
 #define GA_LAUNCH_LINEAR_VK(ATTN, WAVES)                 \
   do {                                                   \
     if (vk == 4) GA_LAUNCH_LINEAR(ATTN, 4, WAVES);       \
@@ -359,6 +368,7 @@ int launch_linear(const float *X, const float *W, const float *a_l, const float 
   }
 #undef GA_LAUNCH_LINEAR_VK
 #undef GA_LAUNCH_LINEAR
+#undef GA_LAUNCH_LINEAR_NCB
   return launch_status();
 }
 }  // namespace
