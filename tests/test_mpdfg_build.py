@@ -303,3 +303,19 @@ def test_stacked_products_skip_operands_overwritten_in_place():
     assert changed and kinds.count("my_ops::SegmentMMNodeStacked") == 1
     changed, kinds = build(inplace=True)
     assert not changed and kinds.count("my_ops::SegmentMMNode") == 2
+
+
+def test_every_operator_the_passes_emit_is_registered():
+    """A rewrite that creates a node of an operator the library does not register fails
+    only when a plan happens to take it: check the names in the passes' source once."""
+    import inspect
+    import re
+    from graphiler_amd import torch_boundary
+    from graphiler_amd.mpdfg import builder, passes
+    torch_boundary.load()
+    names = set()
+    for mod in (builder, passes):
+        names |= set(re.findall(r'"(my_ops::\w+)"', inspect.getsource(mod)))
+    assert len(names) > 20
+    for name in sorted(names):
+        assert len(torch._C._jit_get_schemas_for_operator(name)) == 1, name
