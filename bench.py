@@ -78,9 +78,11 @@ def main():
     ap.add_argument("--reps", type=int, default=30, help="timed calls per operator")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--gather-ceiling", action="store_true",
-                    help="configs[4] only: also run its aggregation kernels on graphs with the same "
+                    help="configs[4]: also run its aggregation kernels on graphs with the same "
                          "destinations and uniformly random sources over tables of several sizes (HBM, "
-                         "Infinity Cache, L2): what the memory system gives a gather of 512-byte rows")
+                         "Infinity Cache, L2): what the memory system gives a gather of 512-byte rows; "
+                         "configs[1] and [4]: u_add_v next to plain gathers of the same rows (torch's "
+                         "index_select, the library's BroadcastSrcNode) and the write of its result alone")
     ap.add_argument("--no-ops", action="store_true",
                     help="time the layers only (shorter kernel traces for profiling)")
     ap.add_argument("--markers", "--calibrate-copy", dest="markers", action="store_true",
@@ -114,6 +116,19 @@ def main():
     def marker():
         if marker_buf is not None:
             marker_buf.add(0.0)        # reads 1 GiB, writes 1 GiB (the result is dropped)
+
+    def u_add_v_reference(g_, el_, er_, src_host):
+        """--gather-ceiling: u_add_v next to gathers of the same (N, H) rows by the same source ids
+        alone -- torch's index_select (the vendor's kernel) and the library's BroadcastSrcNode --
+        and next to the write of the (E, H) result alone."""
+        e_, h_ = g_.num_edges, int(el_.shape[1])
+        src_ = torch.from_numpy(src_host).to(dev)
+        out_ = torch.empty(e_, h_, device=dev)
+        return {"rows": e_, "row_bytes": h_ * 4, "table_MB": round(el_.numel() * 4 / 1e6, 2),
+                "u_add_v_ms": round(ev_time(lambda: ops.gsddmm_u_add_v_mul_alpha(el_, er_, 1, g_), 10), 4),
+                "gather_alone_ms": round(ev_time(lambda: ops.BroadcastSrcNode(el_, g_), 10), 4),
+                "torch_index_select_ms": round(ev_time(lambda: torch.index_select(el_, 0, src_, out=out_), 5), 4),
+                "write_alone_ms": round(ev_time(lambda: out_.copy_(el_[:1].expand(e_, h_)), 10), 4)}
 
     def ev_time(fn, reps=None, warmup=3, key=None):
         reps = reps or args.reps
@@ -367,6 +382,7 @@ def main():
                 del gk
                 torch.cuda.empty_cache()
             rec["gather_ceiling"] = ceil
+            rec["u_add_v_reference"] = u_add_v_reference(g, el1.float().contiguous(), er1.float().contiguous(), wl.src)
 
         if headline == "c5" and not args.no_cpu_baseline:
             # one hidden layer (256 -> 256) of the same network on the host cores: the fp32
@@ -450,6 +466,8 @@ def main():
                 "c2.spmm_copy_u", lambda: ops.SpMMSrc(z, [1], False, None, g),
                 4 * (N + 1) + E * (4 + Fw * b) + N * Fw * b, reps=50, gather=rows)
         rec["ops"] = opsr = kept(opsr)
+        if args.gather_ceiling and not only:
+            rec["u_add_v_reference"] = u_add_v_reference(g, el.float().contiguous(), er.float().contiguous(), wl.src)
         if "gat_aggregate" in opsr:
             rec["roofline"] = dict(opsr["gat_aggregate"],
                                    kernel="gat_aggregate (runs_kernel<GatPolicy<float, 4>> + fix-up)")
