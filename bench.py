@@ -77,12 +77,14 @@ def main():
                          "only these, skip the network steps and the CPU legs (short profiler runs)")
     ap.add_argument("--reps", type=int, default=30, help="timed calls per operator")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--gather-ceiling", action="store_true",
+    ap.add_argument("--gather-ceiling", "--reference-points", dest="gather_ceiling", action="store_true",
                     help="configs[4]: also run its aggregation kernels on graphs with the same "
                          "destinations and uniformly random sources over tables of several sizes (HBM, "
                          "Infinity Cache, L2): what the memory system gives a gather of 512-byte rows; "
                          "configs[1] and [4]: u_add_v next to plain gathers of the same rows (torch's "
-                         "index_select, the library's BroadcastSrcNode) and the write of its result alone")
+                         "index_select, the library's BroadcastSrcNode) and the write of its result alone, "
+                         "and the segment softmax on regular segments of 64 next to torch.softmax over the "
+                         "same view and a copy of the tensor")
     ap.add_argument("--no-ops", action="store_true",
                     help="time the layers only (shorter kernel traces for profiling)")
     ap.add_argument("--markers", "--calibrate-copy", dest="markers", action="store_true",
@@ -129,6 +131,27 @@ def main():
                 "gather_alone_ms": round(ev_time(lambda: ops.BroadcastSrcNode(el_, g_), 10), 4),
                 "torch_index_select_ms": round(ev_time(lambda: torch.index_select(el_, 0, src_, out=out_), 5), 4),
                 "write_alone_ms": round(ev_time(lambda: out_.copy_(el_[:1].expand(e_, h_)), 10), 4)}
+
+    def softmax_reference(g_, heads_):
+        """--reference-points: the segment softmax of the graph's (E, H) logits next to the same
+        number of logits in regular segments of 64 -- through the library and through torch.softmax
+        over the (E / 64, 64, H) view, which knows the segments from the shape -- and next to a
+        copy of the tensor (what reading and writing it once costs)."""
+        e_ = g_.num_edges
+        x_ = torch.randn(e_, heads_, device=dev)
+        e64 = e_ - e_ % 64
+        reg = prepare_graph(np.zeros(e64, np.int64), np.repeat(np.arange(e64 // 64), 64), e64 // 64,
+                            device=dev)
+        reg.in_row_of_slot
+        xr, y_ = x_[:e64].contiguous(), torch.empty_like(x_)
+        out = {"logits": e_ * heads_,
+               "graph_ms": round(ev_time(lambda: ops.SegmentSoftmax(x_, 1, None, g_), 10), 4),
+               "regular_segments_of_64_ms": round(ev_time(lambda: ops.SegmentSoftmax(xr, 1, None, reg), 10), 4),
+               "torch_softmax_regular_segments_of_64_ms":
+                   round(ev_time(lambda: torch.softmax(xr.view(-1, 64, heads_), dim=1), 5), 4),
+               "copy_ms": round(ev_time(lambda: y_.copy_(x_), 10), 4)}
+        out["regular_frac_of_8TBps"] = round(8.0 * e64 * heads_ / out["regular_segments_of_64_ms"] / 1e6 / HBM_PEAK_GBS, 4)
+        return out
 
     def ev_time(fn, reps=None, warmup=3, key=None):
         reps = reps or args.reps
@@ -383,6 +406,7 @@ def main():
                 torch.cuda.empty_cache()
             rec["gather_ceiling"] = ceil
             rec["u_add_v_reference"] = u_add_v_reference(g, el1.float().contiguous(), er1.float().contiguous(), wl.src)
+            rec["softmax_reference"] = softmax_reference(g, H)
 
         if headline == "c5" and not args.no_cpu_baseline:
             # one hidden layer (256 -> 256) of the same network on the host cores: the fp32
@@ -468,6 +492,7 @@ def main():
         rec["ops"] = opsr = kept(opsr)
         if args.gather_ceiling and not only:
             rec["u_add_v_reference"] = u_add_v_reference(g, el.float().contiguous(), er.float().contiguous(), wl.src)
+            rec["softmax_reference"] = softmax_reference(g, H)
         if "gat_aggregate" in opsr:
             rec["roofline"] = dict(opsr["gat_aggregate"],
                                    kernel="gat_aggregate (runs_kernel<GatPolicy<float, 4>> + fix-up)")
