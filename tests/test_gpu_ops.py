@@ -1297,6 +1297,24 @@ def test_linear_with_row_factor(device, rows, K, M):
         ops.linear(x, w, row_scale=s.double())
 
 
+@pytest.mark.parametrize("rows,K,M", [(19717, 500, 16), (16385, 1433, 16), (16400, 128, 3), (20001, 131, 7),
+                                      (17000, 130, 1), (30000, 4096, 16), (16384, 127, 16), (33000, 500, 16)])
+def test_plain_projection_onto_few_columns(device, rows, K, M):
+    """At most 16 columns: the build that multiplies and stores one column block.  Against
+    float64, with and without the row factor, row counts that are no multiple of a tile."""
+    rng = np.random.default_rng(rows + K + M)
+    x = rng.standard_normal((rows, K), dtype=np.float32)
+    w = datasets.glorot(rng, (K, M))
+    sc = rng.uniform(0.5, 1.5, (rows, 1)).astype(np.float32)
+    ref = x.astype(np.float64) @ w.astype(np.float64)
+    xd, wd, sd = _dev(x, device), _dev(w, device), _dev(sc, device)
+    got = ops.linear_attn(xd, wd)
+    assert got.shape == (rows, M)
+    assert_close(got.cpu().numpy(), ref, TOL_F32, f"projection {rows}x{K}x{M}")
+    assert torch.equal(ops.linear(xd, wd, row_scale=sd), got * sd)
+    assert torch.equal(ops.linear_attn(xd, wd), got)          # the same bits every time
+
+
 @pytest.mark.parametrize("offset", [1, 2, 3, 4])
 @pytest.mark.parametrize("K", [66, 602, 64, 37])
 def test_linear_attn_row_alignment(device, K, offset):
